@@ -1,0 +1,110 @@
+"""ctypes front-end of the C restatement in ``slstm_oracle.c``.
+
+TEST INFRASTRUCTURE ONLY (see the header of ``slstm_oracle.c``).  The shared
+object is built by ``make -C oracle`` (``__graft_entry__.build()`` does that);
+if it is missing this module builds it with the same recipe.
+
+Reference lines restated: ``xlstm/blocks/slstm/src/vanilla/__init__.py:17-74``
+(time loop) and ``xlstm/blocks/slstm/src/vanilla/slstm.py:8-37`` (pointwise).
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from typing import Optional, Tuple
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "_build", "libslstm_oracle.so")
+_LIB = None
+
+N0_PER_ELEMENT = 0  # native-kernel rule, slstm_pointwise.cu:79
+N0_WHOLE_TENSOR = 1  # vanilla rule, vanilla/slstm.py:25
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with gcc; returns the path of the shared object."""
+    src = os.path.join(_HERE, "slstm_oracle.c")
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+        subprocess.run(["make", "-C", _HERE, "-B" if force else "-s"], check=True,
+                       stdout=subprocess.DEVNULL)
+    return _SO
+
+
+def _lib():
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(_SO):
+            build()
+        lib = ctypes.CDLL(_SO)
+        for name in ("slstm_oracle_forward_f64", "slstm_oracle_forward_f32"):
+            fn = getattr(lib, name)
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5
+        _LIB = lib
+    return _LIB
+
+
+def slstm_forward(
+    wx: np.ndarray,  # [B, T, 4*H]  external order (gate, head, unit)
+    r_ext: np.ndarray,  # [NH, dh, 4, dh]
+    b_ext: np.ndarray,  # [NH, 4, dh]
+    s0: Optional[np.ndarray] = None,  # [4, B, H]
+    reset: Optional[np.ndarray] = None,  # [B, T] bool / uint8
+    n0_rule: int = N0_PER_ELEMENT,
+    dtype=np.float64,
+) -> Tuple[np.ndarray, np.ndarray]:
+    """Returns ``(h[T,B,H], state[4,B,H])`` computed in ``dtype`` arithmetic."""
+    dtype = np.dtype(dtype)
+    assert dtype in (np.dtype(np.float64), np.dtype(np.float32))
+    NH, dh = int(r_ext.shape[0]), int(r_ext.shape[1])
+    assert r_ext.shape == (NH, dh, 4, dh), r_ext.shape
+    assert b_ext.shape == (NH, 4, dh), b_ext.shape
+    H = NH * dh
+    B, T = int(wx.shape[0]), int(wx.shape[1])
+    assert wx.shape == (B, T, 4 * H), wx.shape
+    wx_c = np.ascontiguousarray(wx, dtype=dtype)
+    r_c = np.ascontiguousarray(r_ext, dtype=dtype)
+    b_c = np.ascontiguousarray(b_ext, dtype=dtype)
+    s0_c = None
+    if s0 is not None:
+        assert s0.shape == (4, B, H), s0.shape
+        s0_c = np.ascontiguousarray(s0, dtype=dtype)
+    reset_c = None
+    if reset is not None:
+        assert reset.shape == (B, T), reset.shape
+        reset_c = np.ascontiguousarray(reset != 0, dtype=np.uint8)
+    h = np.empty((T, B, H), dtype=dtype)
+    s = np.empty((4, B, H), dtype=dtype)
+    fn = _lib().slstm_oracle_forward_f64 if dtype == np.float64 else _lib().slstm_oracle_forward_f32
+    rc = fn(
+        wx_c.ctypes.data, r_c.ctypes.data, b_c.ctypes.data,
+        s0_c.ctypes.data if s0_c is not None else None,
+        reset_c.ctypes.data if reset_c is not None else None,
+        h.ctypes.data, s.ctypes.data, B, T, NH, dh, int(n0_rule),
+    )
+    if rc != 0:
+        raise MemoryError("slstm oracle: allocation failed")
+    return h, s
+
+
+def slstm_forward_per_document(wx, r_ext, b_ext, reset, dtype=np.float64):
+    """Definition of the reset semantics: every document of every row is run
+    ALONE from a zero state and the results are concatenated.  Deliberately a
+    separate code path from the ``reset`` argument of :func:`slstm_forward`."""
+    B, T = wx.shape[0], wx.shape[1]
+    H = r_ext.shape[0] * r_ext.shape[1]
+    h = np.zeros((T, B, H), dtype=dtype)
+    s = np.zeros((4, B, H), dtype=dtype)
+    for b in range(B):
+        starts = [t for t in range(T) if reset[b, t]]
+        if not starts or starts[0] != 0:
+            raise ValueError("per-document oracle needs a document start at t=0 in every row")
+        bounds = starts + [T]
+        for lo, hi in zip(bounds[:-1], bounds[1:]):
+            hd, sd = slstm_forward(wx[b:b + 1, lo:hi], r_ext, b_ext, None, None, dtype=dtype)
+            h[lo:hi, b] = hd[:, 0]
+            s[:, b] = sd[:, 0]
+    return h, s

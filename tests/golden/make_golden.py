@@ -1,0 +1,87 @@
+"""Writes the golden vectors in this folder from the reference's VANILLA sLSTM cell.
+
+Run once, in the build container only (the reference tree never travels):
+
+    python tests/golden/make_golden.py
+
+What the vectors pin that nothing else can: the reference's conventions — gate
+order i,f,z,o inside the ``[B,S,4H]`` input, state order y,c,n,m, the flattening
+``(gate, head, unit)`` of the input, the external parameter views
+``recurrent_kernel[NH,dh_in,4,dh_out]`` / ``bias[NH,4,dh]``, the ``BNSH`` output
+view, and the whole-tensor ``all(n == 0)`` stabiliser rule of the vanilla path.
+
+Parameters are exported through the reference's backend-agnostic external views
+(``cell.recurrent_kernel[:]``, ``cell.bias[:]``), so the fixtures do not depend
+on any backend-internal layout.  Every case stores inputs and outputs as float32.
+"""
+import os
+import sys
+
+import numpy as np
+import torch
+
+REF = "/root/reference"
+OUT = os.path.dirname(os.path.abspath(__file__))
+
+
+def main():
+    sys.path.insert(0, REF)
+    from xlstm.blocks.slstm.cell import sLSTMCell, sLSTMCellConfig  # noqa: E402
+
+    cases = [
+        # name, hidden, heads, B, T, recurrent init, bias init, with state, seed
+        ("ref_test_shape_nostate", 64, 4, 1, 1, "zeros", "powerlaw_blockdependent", False, 42),
+        ("ref_test_shape_state", 64, 4, 1, 1, "zeros", "powerlaw_blockdependent", True, 42),
+        ("seq_standard_nostate", 64, 4, 3, 12, "standard", "small_init", False, 1),
+        ("seq_standard_state", 64, 2, 2, 9, "standard", "standard", True, 2),
+        ("seq_onehead", 32, 1, 2, 7, "standard", "powerlaw_blockdependent", True, 3),
+        ("seq_dh128", 256, 2, 2, 16, "standard", "small_init", False, 4),
+        # row 0 starts with n == 0 but m != 0, row 1 with n > 0: the vanilla path's
+        # whole-tensor test `all(n == 0)` is False, so row 0 takes max(i, m + logsig f)
+        # where the native per-element rule would take i.
+        ("seq_mixed_n", 64, 4, 2, 5, "standard", "small_init", "mixed", 5),
+    ]
+    for name, hidden, heads, B, T, rinit, binit, with_state, seed in cases:
+        torch.manual_seed(seed)
+        cfg = sLSTMCellConfig(
+            hidden_size=hidden, num_heads=heads, backend="vanilla", dtype="float32",
+            recurrent_weight_init=rinit, bias_init=binit,
+        )
+        cell = sLSTMCell(cfg)
+        if rinit == "standard":
+            # U(+-1/sqrt(hidden)) keeps R·y tiny; scale up so that a wrong index,
+            # transposition or gate order in the contraction is far above tolerance.
+            with torch.no_grad():
+                cell._recurrent_kernel_.mul_(6.0)
+        x = torch.randn(B, T, 4 * hidden)
+        state = torch.randn(4, B, hidden) if with_state else None
+        if state is not None:
+            state[2] = state[2].abs() + 0.5  # a normaliser is positive in any reachable state
+            if with_state == "mixed":
+                state[2, 0] = 0.0
+        with torch.no_grad():
+            out, st = cell(x, state)
+        assert out.shape == (B, heads, T, hidden // heads)
+        np.savez(
+            os.path.join(OUT, f"{name}.npz"),
+            wx=x.numpy(),
+            r_ext=cell.recurrent_kernel[:].contiguous().numpy(),
+            b_ext=cell.bias[:].contiguous().numpy(),
+            s0=(state.numpy() if state is not None else np.zeros((0,), np.float32)),
+            out_bnsh=out.contiguous().numpy(),
+            state=st.contiguous().numpy(),
+        )
+        print(name, "out", tuple(out.shape), "state", tuple(st.shape))
+
+    # Notebook shape fixture (notebooks/xlstm/xLSTM_test_notebook.ipynb, cell 2):
+    # zeros[4,4,512] through hidden=128, heads=2 -> out [4,2,4,64], state [4,4,128].
+    torch.manual_seed(0)
+    cell = sLSTMCell(sLSTMCellConfig(hidden_size=128, num_heads=2, backend="vanilla", dtype="float32"))
+    with torch.no_grad():
+        out, st = cell(torch.zeros(4, 4, 512))
+    print("notebook shapes", tuple(out.shape), tuple(st.shape))
+    assert tuple(out.shape) == (4, 2, 4, 64) and tuple(st.shape) == (4, 4, 128)
+
+
+if __name__ == "__main__":
+    main()
