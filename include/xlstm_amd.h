@@ -1,0 +1,135 @@
+/*
+ * xlstm_amd — C ABI of the MI355X (gfx950) sLSTM forward / decode engine.
+ *
+ * Plain C: raw device pointers, sizes, enums and an opaque stream handle.  No
+ * C++ or torch types cross this boundary.  The caller owns every buffer
+ * (inputs, outputs and the workspace); the library allocates nothing and
+ * never synchronises the device.  Every entry point returns 0 on success or a
+ * negative XS_ERR_* code; xs_last_error() gives the text for the calling thread.
+ *
+ * What each entry point replaces in the reference (NX-AI/xlstm, paths relative
+ * to its root) is cited at its declaration.
+ */
+#ifndef XLSTM_AMD_H
+#define XLSTM_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XS_ABI_VERSION 1
+
+/* element types */
+enum { XS_F32 = 0, XS_BF16 = 1 };
+
+/* error codes */
+enum {
+  XS_OK = 0,
+  XS_ERR_NULL = -1,        /* a required pointer is NULL */
+  XS_ERR_SHAPE = -2,       /* a dimension is out of range or inconsistent */
+  XS_ERR_DTYPE = -3,       /* unsupported dtype combination */
+  XS_ERR_ALIGN = -4,       /* pointer or stride not aligned as documented */
+  XS_ERR_UNSUPPORTED = -5, /* shape is valid but not covered by a kernel */
+  XS_ERR_WORKSPACE = -6,   /* workspace missing or too small */
+  XS_ERR_LAUNCH = -7,      /* the HIP runtime refused the launch */
+  XS_ERR_DEVICE = -8       /* device does not fit the grid (co-residency) */
+};
+
+/*
+ * Arguments of one cell call.  All pointers are DEVICE pointers.
+ *
+ *   wx     [B, T, 4, NH, dh]  gate pre-activations (gate order i,f,z,o), element
+ *                             type wx_dtype.  The innermost 4*NH*dh elements are
+ *                             contiguous; rows/steps are addressed through
+ *                             wx_stride_b / wx_stride_t (in ELEMENTS), so the
+ *                             [B,S,4H] tensor the layer produces is read in place
+ *                             (the reference permutes and copies it first:
+ *                             xlstm/blocks/slstm/cell.py:327-352, :768-774).
+ *   r      [NH, 4*dh, dh]     recurrent matrix, r[h][g*dh + a][d] multiplies input
+ *                             unit d of head h into gate g of output unit a —
+ *                             the K-contiguous layout of the reference's vanilla
+ *                             backend (cell.py:601-617).  r_dtype is XS_F32 or
+ *                             XS_BF16; with wx_dtype == XS_F32 it must be XS_F32.
+ *   bias   [NH, 4, dh]        float32 (cell.py:253-257, external view).
+ *   s0     [4, B, NH*dh]      float32 initial y,c,n,m or NULL for zeros (cell.py:441-469).
+ *   reset  [B, T] uint8       or NULL.  Non-zero at (b,t) => y,c,n,m of row b are
+ *                             zeroed before step t (start of a packed document).
+ *                             Row stride reset_stride_b in bytes.  Not in the
+ *                             reference (only the unused `lengths`, cell.py:496).
+ *   h_out  [T, B, NH*dh]      hidden state after every step, element type
+ *                             wx_dtype, contiguous (the reference's
+ *                             all_states[0][1:], cell.py:502).
+ *   s_out  [4, B, NH*dh]      float32 state after the last step (cell.py:471-476).
+ *                             May alias s0.
+ *   workspace                 at least xs_slstm_workspace_bytes() bytes, 256-byte
+ *                             aligned.  Holds the status block (below); two calls
+ *                             that may overlap in time need different workspaces.
+ *   stream                    hipStream_t (NULL = the null stream).
+ *   spin_limit                bound on every wait between compute units, in poll
+ *                             iterations; 0 selects the default.  When a wait
+ *                             runs out the kernel records it in the status block
+ *                             and finishes without waiting any further.
+ */
+typedef struct xs_slstm_args {
+  int32_t B, T, NH, dh;
+  int32_t wx_dtype, r_dtype;
+  const void *wx;
+  int64_t wx_stride_b, wx_stride_t;
+  const void *r;
+  const float *bias;
+  const float *s0;
+  const uint8_t *reset;
+  int64_t reset_stride_b;
+  void *h_out;
+  float *s_out;
+  void *workspace;
+  size_t workspace_bytes;
+  void *stream;
+  int64_t spin_limit;
+} xs_slstm_args;
+
+/* Status block at the start of the workspace, written by the kernels. */
+typedef struct xs_slstm_status {
+  uint32_t aborted;     /* 1 if a bounded wait ran out (results are invalid) */
+  uint32_t abort_wg;    /* workgroup that gave up first */
+  uint32_t abort_step;  /* timestep it was waiting for */
+  uint32_t max_spins;   /* largest number of poll iterations any wait needed */
+  uint32_t xcd_mixed;   /* number of head groups whose workgroups ran on more than one XCD */
+  uint32_t launches;    /* kernel launches the call was split into */
+  uint32_t reserved[10];
+} xs_slstm_status;
+
+/* Library / ABI identification.  Replaces nothing (the reference keys its JIT
+ * modules by config, cell.py:509-534). */
+int xs_abi_version(void);
+
+/* Text of the last error on the calling thread ("" if none). */
+const char *xs_last_error(void);
+
+/* Bytes of workspace a call with these dimensions needs. */
+size_t xs_slstm_workspace_bytes(int32_t B, int32_t T, int32_t NH, int32_t dh);
+
+/*
+ * Sequence forward: T steps in ONE persistent launch (per batch chunk).
+ * Replaces sLSTMFunc.forward -> ForwardPass::Run, i.e. the per-timestep
+ * cuBLAS GEMM + pointwise kernel loop
+ * (xlstm/blocks/slstm/src/cuda/slstm.cc:53-135,
+ *  xlstm/blocks/slstm/src/cuda/slstm_forward.cu:217-267) and the vanilla loop
+ * (xlstm/blocks/slstm/src/vanilla/__init__.py:17-74).
+ */
+int xs_slstm_forward(const xs_slstm_args *args);
+
+/*
+ * Single-token decode step (T must be 1): state in, state out, no waits
+ * between compute units.  Replaces the T == 1 use of the same reference entry
+ * (xlstm/blocks/slstm/layer.py:113-115 calls the cell's forward with S = 1).
+ */
+int xs_slstm_step(const xs_slstm_args *args);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XLSTM_AMD_H */

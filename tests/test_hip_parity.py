@@ -1,0 +1,169 @@
+"""GPU parity tests: the HIP engine (through the C ABI) against the CPU oracle.
+
+Tolerances (|a - ref| <= tol * max(1, |ref|)):
+  float32 path : 1e-5 against the float64 oracle
+  bfloat16 path: 2e-2 against the float64 oracle run on the bf16-rounded inputs
+  resets / chunking / step-by-step: bit-exact against the engine itself
+"""
+import glob
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import slstm_oracle as so
+from tests._util import geometric_reset_mask, make_problem, max_err, r_ext_to_kernel
+
+pytestmark = pytest.mark.gpu
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+TOL_F32 = 1e-5
+TOL_BF16 = 2e-2
+
+
+def _run_hip(wx, r_ext, b_ext, s0=None, reset=None, bf16=False, **kw):
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev)
+    if bf16:
+        wx_t = wx_t.bfloat16()
+    r_t = r_ext_to_kernel(torch.from_numpy(r_ext)).to(dev)
+    b_t = torch.from_numpy(b_ext).to(dev)
+    s0_t = torch.from_numpy(s0).to(dev) if s0 is not None else None
+    m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
+    ws = F.workspace_for(wx.shape[0], wx.shape[1], r_ext.shape[0], r_ext.shape[1], dev)
+    h, s = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t, workspace=ws, **kw)
+    torch.cuda.synchronize()
+    status = F.read_status(ws)
+    return h.float().cpu().numpy(), s.cpu().numpy(), status
+
+
+def _check(h, s, h_ref, s_ref, tol, status):
+    assert status["aborted"] == 0, status
+    assert np.isfinite(h).all() and np.isfinite(s).all()
+    eh, es = max_err(h, h_ref), max_err(s, s_ref)
+    assert eh <= tol, f"h error {eh:.3e} > {tol}"
+    assert es <= tol, f"state error {es:.3e} > {tol}"
+
+
+@pytest.mark.parametrize("path", sorted(glob.glob(os.path.join(GOLDEN, "*.npz"))), ids=lambda p: os.path.basename(p)[:-4])
+def test_reference_golden_vectors_f32(path):
+    """The reference's own vanilla outputs (written by tests/golden/make_golden.py)."""
+    z = np.load(path)
+    if "mixed_n" in path:
+        pytest.skip("vanilla's whole-tensor n==0 rule; the engine uses the native per-element rule")
+    s0 = z["s0"] if z["s0"].size else None
+    NH = z["r_ext"].shape[0]
+    print("case", os.path.basename(path), z["wx"].shape, flush=True)
+    h, s, status = _run_hip(z["wx"], z["r_ext"], z["b_ext"], s0)
+    T, B, H = h.shape
+    out = h.reshape(T, B, NH, H // NH).transpose(1, 2, 0, 3)
+    _check(out, s, z["out_bnsh"], z["state"], TOL_F32, status)
+
+
+def test_mixed_n_golden_matches_per_element_oracle():
+    z = np.load(os.path.join(GOLDEN, "seq_mixed_n.npz"))
+    h_ref, s_ref = so.slstm_forward(z["wx"], z["r_ext"], z["b_ext"], z["s0"], None, n0_rule=so.N0_PER_ELEMENT)
+    h, s, status = _run_hip(z["wx"], z["r_ext"], z["b_ext"], z["s0"])
+    _check(h, s, h_ref, s_ref, TOL_F32, status)
+
+
+F32_CASES = [
+    # B, T, NH, dh, with_state, resets
+    (4, 256, 4, 128, False, False),   # BASELINE config 1
+    (1, 1, 4, 16, True, False),       # the reference test's shape
+    (3, 40, 2, 64, True, True),
+    (5, 33, 3, 24, False, True),      # head dim not a multiple of 16
+    (17, 20, 2, 32, True, True),      # batch not a multiple of 16 -> two tiles
+    (40, 12, 1, 256, False, False),
+    (2, 64, 2, 512, True, True),      # largest fp32 head
+]
+
+
+@pytest.mark.parametrize("B,T,NH,dh,with_state,resets", F32_CASES)
+def test_f32_against_f64_oracle(B, T, NH, dh, with_state, resets):
+    print("case f32", B, T, NH, dh, with_state, resets, flush=True)
+    wx, r, b, s0 = make_problem(11, B, T, NH, dh, rscale=4.0, with_state=with_state)
+    reset = geometric_reset_mask(5, B, T, max(2, T // 3)) if resets else None
+    if reset is not None and with_state:
+        reset[:, 0] = 0  # let the supplied state matter
+    h_ref, s_ref = so.slstm_forward(wx, r, b, s0, reset)
+    h, s, status = _run_hip(wx, r, b, s0, reset)
+    _check(h, s, h_ref, s_ref, TOL_F32, status)
+
+
+BF16_CASES = [
+    (16, 128, 4, 256, False, True),   # BASELINE config 2 shape, short T
+    (4, 50, 2, 128, True, True),
+    (3, 30, 4, 16, True, False),
+    (20, 16, 2, 64, False, True),
+    (64, 8, 1, 1024, False, False),   # config 5 head size, one head
+    (33, 10, 8, 256, True, True),     # config 3 prefill shape, short
+]
+
+
+@pytest.mark.parametrize("B,T,NH,dh,with_state,resets", BF16_CASES)
+def test_bf16_against_f64_oracle(B, T, NH, dh, with_state, resets):
+    print("case bf16", B, T, NH, dh, with_state, resets, flush=True)
+    wx, r, b, s0 = make_problem(12, B, T, NH, dh, rscale=1.0, bf16=True, with_state=with_state)
+    reset = geometric_reset_mask(6, B, T, max(2, T // 3)) if resets else None
+    if reset is not None and with_state:
+        reset[:, 0] = 0
+    h_ref, s_ref = so.slstm_forward(wx, r, b, s0, reset)
+    h, s, status = _run_hip(wx, r, b, s0, reset, bf16=True)
+    _check(h, s, h_ref, s_ref, TOL_BF16, status)
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_packed_documents_equal_documents_run_alone_bit_exact(bf16):
+    B, T, NH, dh = 6, 48, 2, 64
+    wx, r, b, _ = make_problem(13, B, T, NH, dh, rscale=4.0, bf16=bf16)
+    reset = geometric_reset_mask(7, B, T, 12)
+    h, s, status = _run_hip(wx, r, b, None, reset, bf16=bf16)
+    assert status["aborted"] == 0
+    for row in range(B):
+        starts = list(np.flatnonzero(reset[row])) + [T]
+        for lo, hi in zip(starts[:-1], starts[1:]):
+            hd, sd, st = _run_hip(wx[row:row + 1, lo:hi], r, b, None, None, bf16=bf16)
+            assert st["aborted"] == 0
+            np.testing.assert_array_equal(hd[:, 0], h[lo:hi, row])
+            if hi == T:
+                np.testing.assert_array_equal(sd[:, 0], s[:, row])
+
+
+@pytest.mark.parametrize("bf16", [False, True])
+def test_chunked_and_stepwise_equal_whole_bit_exact(bf16):
+    B, T, NH, dh = 5, 24, 2, 128
+    wx, r, b, s0 = make_problem(14, B, T, NH, dh, rscale=4.0, bf16=bf16, with_state=True)
+    h, s, _ = _run_hip(wx, r, b, s0, bf16=bf16)
+    ha, sa, _ = _run_hip(wx[:, :10], r, b, s0, bf16=bf16)
+    hb, sb, _ = _run_hip(wx[:, 10:], r, b, sa, bf16=bf16)
+    np.testing.assert_array_equal(np.concatenate([ha, hb]), h)
+    np.testing.assert_array_equal(sb, s)
+    st = s0
+    for t in range(T):
+        ht, st, status = _run_hip(wx[:, t:t + 1], r, b, st, bf16=bf16, step=True)
+        assert status["aborted"] == 0
+        np.testing.assert_array_equal(ht[0], h[t])
+    np.testing.assert_array_equal(st, s)
+
+
+def test_empty_sequence_returns_initial_state():
+    wx, r, b, s0 = make_problem(15, 3, 0, 2, 32, with_state=True)
+    h, s, _ = _run_hip(wx, r, b, s0)
+    assert h.shape == (0, 3, 64)
+    np.testing.assert_array_equal(s, s0)
+    h, s, _ = _run_hip(wx, r, b, None)
+    np.testing.assert_array_equal(s, np.zeros_like(s0))
+
+
+def test_spin_limit_runs_out_is_reported_not_hung():
+    """Error path forced from the host: a one-iteration bound on the waits
+    between compute units.  The kernel must finish and flag the call."""
+    wx, r, b, _ = make_problem(16, 16, 64, 4, 256, bf16=True)
+    h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
+    assert status["aborted"] in (0, 1)
+    if status["aborted"]:
+        assert status["abort_step"] >= 1

@@ -1,0 +1,90 @@
+"""ctypes binding of the C ABI declared in ``include/xlstm_amd.h``.
+
+The engine has no CPU fallback: if the shared library is missing, loading
+fails loudly with the command that builds it.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(PKG, "lib", "libxlstm_amd.so")
+
+XS_F32, XS_BF16 = 0, 1
+ABI_VERSION = 1
+
+EXPORTS = (
+    "xs_abi_version",
+    "xs_last_error",
+    "xs_slstm_workspace_bytes",
+    "xs_slstm_forward",
+    "xs_slstm_step",
+)
+
+
+class SlstmArgs(ctypes.Structure):
+    """Mirror of ``xs_slstm_args``."""
+
+    _fields_ = [
+        ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("NH", ctypes.c_int32), ("dh", ctypes.c_int32),
+        ("wx_dtype", ctypes.c_int32), ("r_dtype", ctypes.c_int32),
+        ("wx", ctypes.c_void_p),
+        ("wx_stride_b", ctypes.c_int64), ("wx_stride_t", ctypes.c_int64),
+        ("r", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("s0", ctypes.c_void_p),
+        ("reset", ctypes.c_void_p),
+        ("reset_stride_b", ctypes.c_int64),
+        ("h_out", ctypes.c_void_p),
+        ("s_out", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+        ("spin_limit", ctypes.c_int64),
+    ]
+
+
+class SlstmStatus(ctypes.Structure):
+    """Mirror of ``xs_slstm_status`` (first bytes of the workspace)."""
+
+    _fields_ = [
+        ("aborted", ctypes.c_uint32), ("abort_wg", ctypes.c_uint32), ("abort_step", ctypes.c_uint32),
+        ("max_spins", ctypes.c_uint32), ("xcd_mixed", ctypes.c_uint32), ("launches", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32 * 10),
+    ]
+
+
+_LIB: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """Loads the engine; raises if it has not been built."""
+    global _LIB
+    if _LIB is not None:
+        return _LIB
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"xlstm_amd: HIP engine not built ({LIB_PATH} missing). "
+            "Build it with `python -m xlstm_amd.build`; there is no CPU fallback."
+        )
+    lib = ctypes.CDLL(LIB_PATH)
+    lib.xs_abi_version.restype = ctypes.c_int
+    lib.xs_abi_version.argtypes = []
+    lib.xs_last_error.restype = ctypes.c_char_p
+    lib.xs_last_error.argtypes = []
+    lib.xs_slstm_workspace_bytes.restype = ctypes.c_size_t
+    lib.xs_slstm_workspace_bytes.argtypes = [ctypes.c_int32] * 4
+    for name in ("xs_slstm_forward", "xs_slstm_step"):
+        fn = getattr(lib, name)
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(SlstmArgs)]
+    if lib.xs_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"xlstm_amd: ABI version {lib.xs_abi_version()} != expected {ABI_VERSION}; rebuild")
+    _LIB = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().xs_last_error().decode()

@@ -1,0 +1,43 @@
+"""Ahead-of-time build of the HIP engine for gfx950 (replaces the reference's
+per-config JIT build, xlstm/blocks/slstm/src/cuda_init.py:60-117).
+
+``python -m xlstm_amd.build`` compiles ``csrc/*.hip`` with hipcc into
+``xlstm_amd/lib/libxlstm_amd.so``.  hipcc cross-compiles, so no GPU is needed.
+"""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+SOURCES = [os.path.join(PKG, "csrc", "slstm_hip.hip")]
+LIB = os.path.join(PKG, "lib", "libxlstm_amd.so")
+
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-shared", "-fPIC",
+    # the compiler must not form packed-fp32 instructions from scalar float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def build(verbose: bool = False) -> str:
+    hipcc = os.environ.get("HIPCC", "hipcc")
+    os.makedirs(os.path.dirname(LIB), exist_ok=True)
+    cmd = [hipcc, *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *SOURCES]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
+    if verbose and out.strip():
+        print(out)
+    return LIB
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))
+    sys.exit(0)

@@ -1,0 +1,140 @@
+"""Tensor-level entry points of the HIP engine (torch is used for device memory
+and streams only; all arithmetic happens in the HIP kernels).
+
+Layouts are the external ones of the reference cell:
+  wx    [B, S, 4*H]   gate pre-activations, last dim ordered (gate, head, unit)
+                      (xlstm/blocks/slstm/cell.py:339-342, layer.py:151-153)
+  r     [NH, 4*dh, dh] K-contiguous recurrent matrix (the vanilla internal
+                      layout, cell.py:601-617)
+  bias  [NH, 4, dh]   float32 (external view, cell.py:253-257)
+  state [4, B, H]     y, c, n, m (cell.py:441-469)
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: _lib.XS_F32, torch.bfloat16: _lib.XS_BF16}
+
+
+class EngineError(RuntimeError):
+    """The C ABI returned an error code."""
+
+
+def _require_cuda(name: str, t: torch.Tensor) -> None:
+    if not t.is_cuda:
+        raise ValueError(f"{name} must live on the GPU (got {t.device}); the hip backend has no CPU path")
+
+
+def workspace_for(B: int, T: int, NH: int, dh: int, device) -> torch.Tensor:
+    n = _lib.load().xs_slstm_workspace_bytes(B, T, NH, dh)
+    return torch.empty(n, dtype=torch.uint8, device=device)
+
+
+def read_status(workspace: torch.Tensor) -> dict:
+    """Copies the status block back (synchronises the stream)."""
+    raw = bytes(workspace[: ctypes.sizeof(_lib.SlstmStatus)].cpu().numpy().tobytes())
+    st = _lib.SlstmStatus.from_buffer_copy(raw)
+    return {k: getattr(st, k) for k, _ in _lib.SlstmStatus._fields_ if k != "reserved"}
+
+
+def read_placement(workspace: torch.Tensor, max_wg: int = 4096) -> torch.Tensor:
+    """Per-workgroup placement words written by the sequence kernel:
+    bits [3:0] XCD id, bit 8 = workgroup was active, bits [31:16] head group."""
+    off = 256
+    return workspace[off: off + 4 * max_wg].cpu().view(torch.int32)
+
+
+def slstm_forward(
+    wx: torch.Tensor,
+    r: torch.Tensor,
+    bias: torch.Tensor,
+    s0: Optional[torch.Tensor] = None,
+    reset_mask: Optional[torch.Tensor] = None,
+    *,
+    step: bool = False,
+    workspace: Optional[torch.Tensor] = None,
+    h_out: Optional[torch.Tensor] = None,
+    s_out: Optional[torch.Tensor] = None,
+    spin_limit: int = 0,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Runs the cell over ``wx`` and returns ``(h[S,B,H] in wx.dtype, state[4,B,H] float32)``.
+
+    ``reset_mask[B,S]`` (bool/uint8) marks document starts: the row's state is
+    zeroed before that step.  ``step=True`` uses the decode entry point (S == 1).
+    """
+    lib = _lib.load()
+    _require_cuda("wx", wx)
+    if wx.dim() != 3:
+        raise ValueError(f"wx must be [B, S, 4*H], got {tuple(wx.shape)}")
+    if wx.dtype not in _DTYPE_CODE:
+        raise TypeError(f"wx dtype {wx.dtype} not supported by the hip backend (float32 or bfloat16)")
+    if r.dim() != 3 or r.shape[1] != 4 * r.shape[2]:
+        raise ValueError(f"r must be [NH, 4*dh, dh], got {tuple(r.shape)}")
+    NH, dh = int(r.shape[0]), int(r.shape[2])
+    H = NH * dh
+    B, T = int(wx.shape[0]), int(wx.shape[1])
+    if wx.shape[2] != 4 * H:
+        raise ValueError(f"Input size mismatch: Expected input size {4 * H}, but got {wx.shape[2]}.")
+    if r.dtype not in _DTYPE_CODE:
+        raise TypeError(f"r dtype {r.dtype} not supported")
+    if wx.dtype == torch.float32 and r.dtype != torch.float32:
+        r = r.float()
+    if tuple(bias.shape) != (NH, 4, dh):
+        raise ValueError(f"bias must be [NH, 4, dh] = {(NH, 4, dh)}, got {tuple(bias.shape)}")
+    for name, t in (("r", r), ("bias", bias)):
+        _require_cuda(name, t)
+    r = r.contiguous()
+    bias = bias.to(torch.float32).contiguous()
+    if wx.numel() and wx.stride(2) != 1:
+        wx = wx.contiguous()
+    if s0 is not None:
+        _require_cuda("state", s0)
+        if tuple(s0.shape) != (4, B, H):
+            raise ValueError(f"state must be [4, B, H] = {(4, B, H)}, got {tuple(s0.shape)}")
+        s0 = s0.to(torch.float32).contiguous()
+    if reset_mask is not None:
+        _require_cuda("reset_mask", reset_mask)
+        if tuple(reset_mask.shape) != (B, T):
+            raise ValueError(f"reset_mask must be [B, S] = {(B, T)}, got {tuple(reset_mask.shape)}")
+        if reset_mask.dtype == torch.bool:
+            reset_mask = reset_mask.view(torch.uint8) if reset_mask.is_contiguous() else reset_mask.to(torch.uint8)
+        elif reset_mask.dtype != torch.uint8:
+            reset_mask = (reset_mask != 0).to(torch.uint8)
+        if T and reset_mask.stride(1) != 1:
+            reset_mask = reset_mask.contiguous()
+    dev = wx.device
+    if h_out is None:
+        h_out = torch.empty((T, B, H), dtype=wx.dtype, device=dev)
+    if s_out is None:
+        s_out = torch.empty((4, B, H), dtype=torch.float32, device=dev)
+    if workspace is None:
+        workspace = workspace_for(B, T, NH, dh, dev)
+
+    a = _lib.SlstmArgs()
+    a.B, a.T, a.NH, a.dh = B, T, NH, dh
+    a.wx_dtype = _DTYPE_CODE[wx.dtype]
+    a.r_dtype = _DTYPE_CODE[r.dtype]
+    a.wx = wx.data_ptr()
+    a.wx_stride_b = wx.stride(0) if B else 0
+    a.wx_stride_t = wx.stride(1) if T else 0
+    a.r = r.data_ptr()
+    a.bias = bias.data_ptr()
+    a.s0 = s0.data_ptr() if s0 is not None else None
+    a.reset = reset_mask.data_ptr() if reset_mask is not None else None
+    a.reset_stride_b = reset_mask.stride(0) if reset_mask is not None else 0
+    a.h_out = h_out.data_ptr()
+    a.s_out = s_out.data_ptr()
+    a.workspace = workspace.data_ptr()
+    a.workspace_bytes = workspace.numel()
+    a.stream = torch.cuda.current_stream(dev).cuda_stream
+    a.spin_limit = int(spin_limit)
+    with torch.cuda.device(dev):
+        rc = (lib.xs_slstm_step if step else lib.xs_slstm_forward)(ctypes.byref(a))
+    if rc != 0:
+        raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+    return h_out, s_out
