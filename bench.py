@@ -1,0 +1,208 @@
+"""Benchmark of the sLSTM forward hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one forward pass of the cell over one packed batch (BASELINE config 2:
+B=16, T=2048, D=1024, 4 heads, bf16 W.x, documents of geometric length (mean 512)
+packed into every row with a reset mask).  Inputs are resident in HBM before the
+timed region.  Prints ONE JSON line:
+
+  value        tokens/s over the K timed steps (wall clock, synchronised on both sides)
+  roofline     the persistent sequence kernel against the HBM roofline: algorithmic
+               bytes per launch / average launch duration (HIP events on the launch stream)
+  cpu_baseline the vanilla-structured PyTorch CPU port (oracle/vanilla_port.py) timed on
+               a bounded slice of the same workload on this box's host cores
+  decode       BASELINE config 3: us per single-token step at B=256, D=2048 (8 heads),
+               1024 consecutive steps after a 128-token prefill, state carried on device
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+METRIC = "sLSTM fwd tokens/s @ D=1024 packed B16×T2048; decode step µs @ B=256"
+HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+
+
+def algorithmic_bytes(B, T, NH, dh, wx_bytes, h_bytes, r_bytes, with_mask=True):
+    """One read of W.x, one write of h, the reset mask, one read of R and bias, the final state."""
+    H = NH * dh
+    return (B * T * 4 * H * wx_bytes + B * T * H * h_bytes + (B * T if with_mask else 0)
+            + NH * 4 * dh * dh * r_bytes + 4 * H * 4 + 4 * B * H * 4)
+
+
+def make_inputs(B, T, NH, dh, mean_doc, device, seed=0):
+    import numpy as np
+    import torch
+
+    from tests._util import geometric_reset_mask
+
+    g = torch.Generator().manual_seed(seed)
+    H = NH * dh
+    wx = torch.randn(B, T, 4 * H, generator=g).bfloat16()
+    r_ext = (torch.rand(NH, dh, 4, dh, generator=g) * 2 - 1) / float(np.sqrt(H))  # "standard" init
+    bias = torch.zeros(NH, 4, dh)
+    bias[:, 1] = torch.linspace(3.0, 6.0, dh)  # "small_init"
+    mask = torch.from_numpy(geometric_reset_mask(seed, B, T, mean_doc)) if mean_doc else None
+    return wx, r_ext, bias, mask
+
+
+def cpu_baseline(wx, r_ext, bias, mask, budget_s=15.0):
+    """Times the vanilla-structured CPU port on the first T_s steps of the same batch."""
+    import torch
+
+    from oracle import vanilla_port as vp
+
+    B, T = wx.shape[0], wx.shape[1]
+    cores = os.cpu_count() or 1
+    cores = min(cores, 16)  # the GPU box gives one job 16 cores' worth of CPU
+    torch.set_num_threads(cores)
+    wx32 = wx.float()
+    probe = 32
+    t0 = time.perf_counter()
+    vp.slstm_forward(wx32[:, :probe], r_ext, bias, None, mask[:, :probe] if mask is not None else None)
+    per_step = (time.perf_counter() - t0) / probe
+    Ts = int(max(64, min(T, budget_s / max(per_step, 1e-6))))
+    t0 = time.perf_counter()
+    vp.slstm_forward(wx32[:, :Ts], r_ext, bias, None, mask[:, :Ts] if mask is not None else None)
+    dt = time.perf_counter() - t0
+    return {
+        "value": B * Ts / dt, "unit": "tokens/s", "cores": cores, "kind": "port",
+        "sample": f"first {Ts} of {T} steps of the same packed batch (B={B}), fp32, torch {torch.__version__} CPU, "
+                  f"{dt:.1f} s, one run after a {probe}-step warm-up",
+    }
+
+
+def bench_decode(device, steps=1024, prefill=128):
+    """BASELINE config 3: B=256, D=2048 (8 heads x 256), bf16 W.x, state carried on device."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    B, NH, dh = 256, 8, 256
+    H = NH * dh
+    wx_pre, r_ext, bias, _ = make_inputs(B, prefill, NH, dh, 0, device, seed=1)
+    r = r_ext.permute(0, 2, 3, 1).reshape(NH, 4 * dh, dh).contiguous().to(device).bfloat16()  # bf16 R for decode
+    bias = bias.to(device)
+    g = torch.Generator().manual_seed(2)
+    wx_dec = torch.randn(steps, B, 1, 4 * H, generator=g).bfloat16().to(device)  # pre-generated, RNG not timed
+    ws = F.workspace_for(B, prefill, NH, dh, device)
+    _, state = F.slstm_forward(wx_pre.to(device), r, bias, None, None, workspace=ws)
+    h1 = torch.empty(1, B, H, dtype=torch.bfloat16, device=device)
+    s_a, s_b = state.clone(), torch.empty_like(state)  # state ping-pong: s_out must not alias s0
+    for t in range(16):  # warm-up
+        F.slstm_forward(wx_dec[t], r, bias, s_a, None, step=True, workspace=ws, h_out=h1, s_out=s_b)
+        s_a, s_b = s_b, s_a
+    s_a.copy_(state)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record()
+    for t in range(steps):
+        F.slstm_forward(wx_dec[t], r, bias, s_a, None, step=True, workspace=ws, h_out=h1, s_out=s_b)
+        s_a, s_b = s_b, s_a
+    e1.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    gpu_us = e0.elapsed_time(e1) * 1e3 / steps
+    nbytes = algorithmic_bytes(B, 1, NH, dh, 2, 2, 2, with_mask=False) + 4 * B * H * 4  # state is read AND written
+    return {
+        "workload": f"decode B={B} D={H} NH={NH}, {steps} consecutive T=1 steps after a {prefill}-token prefill",
+        "us_per_step": wall * 1e6 / steps, "gpu_us_per_step": gpu_us, "steps": steps,
+        "finite": bool(torch.isfinite(s_a).all()),
+        "roofline": {"bound": "hbm", "achieved": nbytes / (gpu_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / (gpu_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None},
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
+    ap.add_argument("--no-decode", action="store_true", help="skip the decode leg (profiling runs)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures ONE GPU; the path shards over batch rows / heads without "
+                 "communication, and no multi-GPU figure is produced (run with --gpus 1)")
+
+    import torch
+
+    from xlstm_amd import functional as F
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (the hip backend has no CPU path)")
+    device = torch.device("cuda:0")
+    B, T, NH, dh = 16, 2048, 4, 256
+    H = NH * dh
+    wx_c, r_ext_c, bias_c, mask_c = make_inputs(B, T, NH, dh, 512, device)
+    wx = wx_c.to(device)
+    r = r_ext_c.permute(0, 2, 3, 1).reshape(NH, 4 * dh, dh).contiguous().to(device)  # fp32, K-contiguous
+    bias = bias_c.to(device)
+    mask = mask_c.to(device)
+    ws = F.workspace_for(B, T, NH, dh, device)
+    h = torch.empty(T, B, H, dtype=torch.bfloat16, device=device)
+    s = torch.empty(4, B, H, dtype=torch.float32, device=device)
+
+    def step():
+        F.slstm_forward(wx, r, bias, None, mask, workspace=ws, h_out=h, s_out=s)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for e0, e1 in evs:
+        e0.record()  # torch's current stream is the stream the kernel is launched on
+        step()
+        e1.record()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    status = F.read_status(ws)
+    if status["aborted"]:
+        sys.exit(f"bench.py: the engine flagged the run as aborted: {status}")
+    kern_ms = sum(e0.elapsed_time(e1) for e0, e1 in evs) / args.steps
+    nbytes = algorithmic_bytes(B, T, NH, dh, 2, 2, 4)
+    achieved = nbytes / (kern_ms * 1e-3) / 1e9
+    out = {
+        "metric": METRIC,
+        "value": B * T * args.steps / elapsed,
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": elapsed * 1e3 / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "sLSTM cell forward, packed documents (geometric, mean 512) with reset mask, "
+                               "B=16 T=2048 D=1024 NH=4, bf16 W.x/h, fp32 R and state (BASELINE configs[1])",
+                   "tokens_per_step": B * T},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1>", "kernel_ms": kern_ms,
+                     "algorithmic_bytes_per_launch": nbytes, "us_per_timestep": kern_ms * 1e3 / T,
+                     "max_poll_rounds": status["max_spins"]},
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "traffic_seq_cfg2.json")
+    if os.path.exists(traffic_file):
+        out["roofline"]["traffic"] = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
+    if not args.no_decode:
+        out["decode"] = bench_decode(device)
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(wx_c, r_ext_c, bias_c, mask_c)
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -63,9 +63,12 @@ enum {
  *                             wx_dtype, contiguous (the reference's
  *                             all_states[0][1:], cell.py:502).
  *   s_out  [4, B, NH*dh]      float32 state after the last step (cell.py:471-476).
- *                             May alias s0.
+ *                             Must not overlap s0 (other compute units still read it).
  *   workspace                 at least xs_slstm_workspace_bytes() bytes, 256-byte
- *                             aligned.  Holds the status block (below); two calls
+ *                             aligned.  Holds the status block (below), one
+ *                             placement word per workgroup and the exchange
+ *                             ring through which the compute units of a head
+ *                             pass h_t to each other (a few MiB).  Two calls
  *                             that may overlap in time need different workspaces.
  *   stream                    hipStream_t (NULL = the null stream).
  *   spin_limit                bound on every wait between compute units, in poll

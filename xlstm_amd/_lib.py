@@ -10,7 +10,7 @@ import os
 from typing import Optional
 
 PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(PKG, "lib", "libxlstm_amd.so")
+LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
 ABI_VERSION = 1

@@ -1,0 +1,377 @@
+"""sLSTM cell with the ``hip`` backend behind the reference's cell interface.
+
+Mirrors ``xlstm/blocks/slstm/cell.py`` of NX-AI/xlstm for the forward /
+inference path: the same config dataclass (``backend`` gains ``"hip"``,
+cell.py:68), the same external parameter views ``recurrent_kernel
+[NH, dh_in, 4, dh_out]`` / ``bias [NH, 4, dh]`` behind ``ParameterProxy``
+(cell.py:234-261), the same initialisers (cell.py:376-434), the same call
+contract ``cell(input[B,S,4H], state=None) -> (output, state[4,B,H])`` with the
+same input / output shape options (cell.py:327-374, 496-506), and the same
+backend switch ``sLSTMCell(config)`` (cell.py:777-788).
+
+What differs, on purpose:
+  * only the sequence of hidden states and the final state are materialised
+    (the reference keeps ``[4, S+1, B, H]`` states and a gate cache);
+  * ``reset_mask[B,S]`` marks document starts inside packed rows (not in the
+    reference, whose only hook is the unused ``lengths``, cell.py:496);
+  * the stabiliser uses the native kernel's per-element ``n == 0`` rule
+    (slstm_pointwise.cu:79), which equals the vanilla rule for every state the
+    cell itself can produce;
+  * forward only: the hip backend is an inference engine, ``backward`` raises.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from math import sqrt
+from typing import Callable, Literal, Optional, Sequence, Union
+
+import torch
+from torch import nn
+
+from . import functional as F_hip
+
+DTYPE_DICT = {
+    "bfloat16": torch.bfloat16,
+    "float16": torch.float16,
+    "float32": torch.float32,
+}
+DTYPES = Literal["bfloat16", "float16", "float32"]
+
+rnn_function_registry = {"slstm": {"states": 4}}
+
+
+class ParameterProxy:
+    """Backend-agnostic (external) view of a parameter stored in a backend
+    layout; same protocol as ``xlstm/components/util.py:26-74``."""
+
+    def __init__(self, module, parameter_name, internal_to_external: Callable, external_to_internal: Callable):
+        self.module = module
+        self.parameter_name = parameter_name
+        self.internal_to_external = internal_to_external
+        self.external_to_internal = external_to_internal
+
+    def _param(self):
+        return getattr(self.module, self.parameter_name)
+
+    def __getitem__(self, key):
+        return self.internal_to_external(self._param()).detach()[key]
+
+    def __setitem__(self, key, value):
+        with torch.no_grad():
+            ext = self.internal_to_external(self._param())
+            ext[key] = value
+            self._param().data = self.external_to_internal(ext).contiguous()
+
+    def clone(self):
+        return self.internal_to_external(self._param()).clone()
+
+    @property
+    def shape(self):
+        return self.internal_to_external(self._param()).shape
+
+    @property
+    def ndim(self):
+        return self.internal_to_external(self._param()).ndim
+
+    @property
+    def grad(self):
+        return self.internal_to_external(self._param().grad)
+
+    def __getattr__(self, name: str):
+        return getattr(getattr(self.module, self.parameter_name), name)
+
+
+@dataclass
+class sLSTMCellConfig:
+    """Field-for-field the reference's config (cell.py:61-163); the fields that
+    only parameterise its CUDA build (batch_size, constants, gradient clipping)
+    are accepted and ignored by the hip backend."""
+
+    hidden_size: int = -1
+    num_heads: int = 4
+    num_states: int = 4
+    backend: Literal["vanilla", "cuda", "hip"] = "hip"
+    function: str = "slstm"
+    bias_init: Literal["powerlaw_blockdependent", "small_init", "standard", "zeros"] = "powerlaw_blockdependent"
+    recurrent_weight_init: Literal["zeros", "standard"] = "zeros"
+    _block_idx: int = 0
+    _num_blocks: int = 1
+    num_gates: int = 4
+    gradient_recurrent_cut: bool = False
+    gradient_recurrent_clipval: Optional[float] = None
+    forward_clipval: Optional[float] = None
+    batch_size: int = 8
+    input_shape: Literal["BSGNH", "SBGNH"] = "BSGNH"
+    internal_input_shape: Literal["SBNGH", "SBGNH", "SBNHG"] = "SBNGH"
+    output_shape: Literal["BNSH", "SBH", "BSH", "SBNH"] = "BNSH"
+    constants: dict = field(default_factory=dict)
+    dtype: DTYPES = "bfloat16"
+    dtype_b: Optional[DTYPES] = "float32"
+    dtype_r: Optional[DTYPES] = None
+    dtype_w: Optional[DTYPES] = None
+    dtype_g: Optional[DTYPES] = None
+    dtype_s: Optional[DTYPES] = None
+    dtype_a: Optional[DTYPES] = None
+    enable_automatic_mixed_precision: bool = True
+    initial_val: Union[float, Sequence[float]] = 0.0
+
+    @property
+    def head_dim(self):
+        return self.hidden_size // self.num_heads
+
+    @property
+    def input_dim(self):
+        return 4 * self.hidden_size
+
+    @property
+    def torch_dtype(self) -> torch.dtype:
+        return DTYPE_DICT[self.dtype]
+
+    @property
+    def torch_dtype_b(self) -> torch.dtype:
+        return DTYPE_DICT[self.dtype_b]
+
+    @property
+    def torch_dtype_r(self) -> torch.dtype:
+        return DTYPE_DICT[self.dtype_r]
+
+    @property
+    def torch_dtype_w(self) -> torch.dtype:
+        return DTYPE_DICT[self.dtype_w]
+
+    @property
+    def torch_dtype_s(self) -> torch.dtype:
+        return DTYPE_DICT[self.dtype_s]
+
+    def __post_init__(self):
+        if self.num_heads <= 0:
+            self.num_heads = 1
+        if self.dtype_b is None:
+            self.dtype_b = self.dtype
+        if self.dtype_a is None:
+            self.dtype_a = self.dtype_b
+        if self.dtype_r is None:
+            self.dtype_r = self.dtype
+        if self.dtype_w is None:
+            self.dtype_w = self.dtype
+        if self.dtype_s is None:
+            self.dtype_s = self.dtype_w
+        if self.dtype_g is None:
+            self.dtype_g = self.dtype_r
+        assert self.function in rnn_function_registry, f"RNN function {self.function} not in registry"
+        self.num_states = rnn_function_registry[self.function]["states"]
+
+
+class _ForwardOnly(torch.autograd.Function):
+    """Identity on (h, state) whose backward raises: the hip backend has no BPTT kernels
+    (the reference's are slstm_backward.cu, out of this engine's scope)."""
+
+    @staticmethod
+    def forward(ctx, h, s, *deps):
+        return h.view_as(h), s.view_as(s)
+
+    @staticmethod
+    def backward(ctx, *grads):
+        raise RuntimeError(
+            "sLSTMCell backend 'hip' is forward/inference only; use the reference's 'cuda' or 'vanilla' backend to train"
+        )
+
+
+class sLSTMCell_hip(nn.Module):
+    """The cell on the MI355X engine.
+
+    Internal parameter layouts (what the kernels read, no copy per call):
+      ``_recurrent_kernel_`` [NH, 4*dh, dh]  -- r[h, g*dh + a, d] = R_ext[h, d, g, a];
+          identical to the reference's vanilla layout (cell.py:601-617), so a
+          vanilla checkpoint loads as is.
+      ``_bias_`` [4*H] head-major -- b[h*4*dh + g*dh + a] = b_ext[h, g, a];
+          identical to the reference's cuda layout (cell.py:726-733).
+    """
+
+    config_class = sLSTMCellConfig
+
+    def __init__(self, config: sLSTMCellConfig, skip_backend_init: bool = False):
+        super().__init__()
+        self.config = config
+        if self.config.hidden_size % self.config.num_heads != 0:
+            raise ValueError(
+                f"Hidden Size {self.config.hidden_size} must be divisible by head num {self.config.num_heads}"
+            )
+        NH, dh = self.config.num_heads, self.head_dim
+        # master parameters are float32; the bf16 path converts R once per launch inside the kernel
+        self._recurrent_kernel_ = nn.Parameter(torch.zeros(NH, 4 * dh, dh, dtype=torch.float32))
+        self.recurrent_kernel = ParameterProxy(
+            self, "_recurrent_kernel", self._recurrent_kernel_int2ext, self._recurrent_kernel_ext2int
+        )
+        self._bias_ = nn.Parameter(torch.zeros(4 * NH * dh, dtype=torch.float32))
+        self.bias = ParameterProxy(self, "_bias", self._bias_int2ext, self._bias_ext2int)
+        self.config.internal_input_shape = "SBGNH"  # the kernel reads the external (gate, head, unit) order in place
+        # optional: keep the carried state in float32 instead of the input dtype
+        self.keep_state_fp32 = False
+        self.reset_parameters()
+        if not skip_backend_init:
+            from . import _lib
+
+            _lib.load()  # fail loudly here, not at the first forward, if the engine is missing
+
+    def __repr__(self):
+        return (
+            f"{self.__class__.__name__}(function={self.config.function}, "
+            f"hidden_size={self.config.hidden_size}, num_heads={self.config.num_heads})"
+        )
+
+    # ------------------------------------------------------------------ layouts
+    @property
+    def _recurrent_kernel(self):
+        return self._recurrent_kernel_
+
+    @property
+    def _bias(self):
+        return self._bias_
+
+    @property
+    def head_dim(self):
+        return self.config.hidden_size // self.config.num_heads
+
+    def _recurrent_kernel_ext2int(self, recurrent_kernel_ext: torch.Tensor) -> torch.Tensor:
+        NH, dh, G = self.config.num_heads, self.head_dim, self.config.num_gates
+        return recurrent_kernel_ext.reshape(NH, dh, G, dh).permute(0, 2, 3, 1).reshape(NH, G * dh, dh)
+
+    def _recurrent_kernel_int2ext(self, recurrent_kernel_int: torch.Tensor) -> torch.Tensor:
+        NH, dh, G = self.config.num_heads, self.head_dim, self.config.num_gates
+        return recurrent_kernel_int.reshape(NH, G, dh, dh).permute(0, 3, 1, 2)
+
+    def _bias_ext2int(self, bias_ext: torch.Tensor) -> torch.Tensor:
+        return bias_ext.reshape(self.config.num_heads, self.config.num_gates, self.head_dim).reshape(-1)
+
+    def _bias_int2ext(self, bias_int: torch.Tensor) -> torch.Tensor:
+        return bias_int.reshape(self.config.num_heads, self.config.num_gates, self.head_dim)
+
+    # ------------------------------------------------------------------ inits
+    def reset_parameters(self):
+        """Same distributions and loop order as cell.py:376-434."""
+        cfg = self.config
+        dh = self.head_dim
+        for h in range(cfg.num_heads):
+            for i, _gate in enumerate(["i", "f", "z", "o"]):
+                if cfg.recurrent_weight_init == "zeros":
+                    self.recurrent_kernel[h, :, i, :] = torch.zeros(dh, dh)
+                elif cfg.recurrent_weight_init == "standard":
+                    self.recurrent_kernel[h, :, i, :] = nn.init.uniform_(
+                        torch.empty(dh, dh), -1.0 / sqrt(cfg.hidden_size), 1.0 / sqrt(cfg.hidden_size)
+                    )
+                else:
+                    raise ValueError(f"unknown recurrent_weight_init {cfg.recurrent_weight_init}")
+        for h in range(cfg.num_heads):
+            for i, gate in enumerate(["i", "f", "z", "o"]):
+                if cfg.bias_init == "powerlaw_blockdependent":
+                    if gate == "f":
+                        ratio_0_to_1 = cfg._block_idx / (cfg._num_blocks - 1) if cfg._num_blocks > 1 else 0.0
+                        init_values = -(-5.0 + 12.0 * (torch.arange(dh) / (dh - 1)) ** (0.3 + 1.3 * ratio_0_to_1))
+                        self.bias[h, i, :] = init_values
+                    else:
+                        self.bias[h, i] = torch.zeros(dh)
+                elif cfg.bias_init == "small_init":
+                    if gate == "f":
+                        self.bias[h, i] = torch.linspace(3.0, 6.0, dh)
+                    else:
+                        self.bias[h, i] = torch.zeros(dh)
+                elif cfg.bias_init == "zeros":
+                    self.bias[h, i] = torch.zeros(dh)
+                elif cfg.bias_init == "standard":
+                    self.bias[h, i] = nn.init.uniform_(
+                        torch.empty(dh), -1 / sqrt(cfg.hidden_size), 1 / sqrt(cfg.hidden_size)
+                    )
+                else:
+                    raise ValueError(f"unknown bias_init {cfg.bias_init}")
+
+    # ------------------------------------------------------------------ shapes
+    def _check_input(self, input: torch.Tensor) -> None:
+        assert self.config.hidden_size * self.config.num_gates == input.size(-1), (
+            f"Input size mismatch: Expected input size {self.config.hidden_size * self.config.num_gates}, "
+            f"but got {input.size(-1)}."
+        )
+
+    def _input_bs(self, x: torch.Tensor) -> torch.Tensor:
+        """External input -> [B, S, 4H] (a view; the kernel takes strides)."""
+        if x.dim() != 3:
+            raise ValueError(f"input must be 3-dimensional, got {tuple(x.shape)}")
+        if self.config.input_shape == "BSGNH":
+            return x
+        if self.config.input_shape == "SBGNH":
+            return x.permute(1, 0, 2)
+        raise ValueError("Bad input_shape value")
+
+    def _permute_output(self, x: torch.Tensor) -> torch.Tensor:
+        """[S, B, H] -> config.output_shape (cell.py:354-374)."""
+        if self.config.output_shape == "SBH":
+            return x
+        if self.config.output_shape == "BSH":
+            return x.permute(1, 0, 2)
+        if self.config.output_shape == "BNSH":
+            return x.view(x.shape[0], x.shape[1], self.config.num_heads, self.head_dim).permute(1, 2, 0, 3)
+        if self.config.output_shape == "SBNH":
+            return x.view(x.shape[0], x.shape[1], self.config.num_heads, self.head_dim)
+        raise ValueError("Bad output_shape value")
+
+    def _check_state(self, B: int, state: Optional[torch.Tensor]) -> None:
+        if state is not None:
+            assert tuple(state.shape) == (self.config.num_states, B, self.config.hidden_size), (
+                f"state must be {(self.config.num_states, B, self.config.hidden_size)}, got {tuple(state.shape)}"
+            )
+
+    # ------------------------------------------------------------------ forward
+    def _run(self, input, state, reset_mask, step: bool):
+        self._check_input(input)
+        x = self._input_bs(input)
+        B = x.shape[0]
+        self._check_state(B, state)
+        in_dtype = input.dtype
+        if in_dtype == torch.float16:  # no fp16 kernels: compute in float32, round the results back
+            x = x.float()
+        elif in_dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"input dtype {in_dtype} not supported by the hip backend")
+        h, s = F_hip.slstm_forward(
+            x,
+            self._recurrent_kernel_.detach(),
+            self._bias_.detach().view(self.config.num_heads, 4, self.head_dim),
+            state,
+            reset_mask,
+            step=step,
+        )
+        if torch.is_grad_enabled() and (
+            input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
+        ):
+            # forward-only engine: the results join the autograd graph only so that a
+            # backward pass through them fails loudly instead of silently yielding no gradient
+            h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
+        output = self._permute_output(h)
+        if torch.is_autocast_enabled():
+            return output, s
+        return output.to(in_dtype), (s if self.keep_state_fp32 else s.to(in_dtype))
+
+    def forward(self, input, state=None, lengths=None, reset_mask=None):
+        """``input`` [B,S,4H] (or [S,B,4H] for input_shape 'SBGNH'), optional ``state`` [4,B,H],
+        optional ``reset_mask`` [B,S].  Returns ``(output, state)`` like cell.py:496-506."""
+        del lengths  # unused, as in the reference
+        return self._run(input, state, reset_mask, step=False)
+
+    def step(self, input: torch.Tensor, state: Optional[torch.Tensor] = None, reset_mask=None):
+        """One decode step (S == 1) through the step kernel.  Unlike the reference's
+        ``step`` (cell.py:486-494, which hands back the state it was given) this
+        returns the NEW state."""
+        return self._run(input, state, reset_mask, step=True)
+
+
+class sLSTMCell:
+    """Backend switch (cell.py:777-788).  This package implements ``"hip"``."""
+
+    config_class = sLSTMCellConfig
+
+    def __new__(cls, config: sLSTMCellConfig, skip_backend_init: bool = False):
+        if config.backend == "hip":
+            return sLSTMCell_hip(config, skip_backend_init=skip_backend_init)
+        raise RuntimeError(
+            f'sLSTMCell unknown backend {config.backend}, choose from ["hip"] '
+            '("cuda" and "vanilla" live in the reference package)'
+        )

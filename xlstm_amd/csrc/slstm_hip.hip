@@ -6,11 +6,12 @@
 // VGPRs for the whole sequence, computes R.h with MFMA (K split over the 4
 // waves, partial sums reduced through LDS), and runs the exponential-gating
 // pointwise update with c, n, m in fp32 registers.  The only thing exchanged
-// per step is h_t: every workgroup stores its 16 units of h_t straight into
-// the output tensor h_out[t] and the other members of the group poll those
-// very words until none of them carries the "not written yet" pattern the
-// buffer was pre-filled with.  One memory round trip per step, no flags, no
-// atomics-with-return, no grid barrier.
+// per step is h_t: every workgroup stores its 16 units of h_t into a compact
+// exchange buffer (one 512-byte / 1-KiB block per workgroup and step, so that
+// polls and stores move whole cache lines spread over all L2 channels) and
+// the other members of the group poll those very words until none of them
+// carries the "not written yet" pattern the buffer was pre-filled with.  One
+// memory round trip per step, no flags, no atomics-with-return, no grid barrier.
 //
 // Equations follow xlstm/blocks/slstm/src/vanilla/slstm.py:19-37 with the
 // per-element n == 0 rule of xlstm/blocks/slstm/src/cuda/slstm_pointwise.cu:79.
@@ -27,7 +28,7 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kThreads = 256;           // 4 waves
+constexpr int kThreads = 384;           // 4 compute waves + feeder wave + drainer wave
 constexpr int kTileStride = 20;         // floats between unit columns of a partial tile in LDS
 constexpr int kTileFloats = 16 * kTileStride;
 constexpr uint32_t kSentinel32 = 0xFFFFFFFFu;  // fp32 "not written yet"
@@ -47,6 +48,7 @@ struct SeqParams {
   float *s_out;
   xs_slstm_status *status;
   uint32_t *wg_xcc;
+  void *xbuf;    // exchange ring [kRing][head group][G][rows][16 units], pre-filled with the "not written yet" pattern
   int B, T, NH, dh;
   int b0, bend;  // batch rows [b0, bend) handled by this launch
   int G;         // workgroups per head group
@@ -135,20 +137,70 @@ __global__ void copy_state_kernel(const float *s0, float *s_out, size_t n) {
 //   NCH : 16-byte chunks of h each lane holds per batch row; one wave covers
 //         NCH*32 (bf16) or NCH*16 (fp32) input units, the four waves 4x that.
 //   MT  : 16-row batch tiles handled one after the other by a workgroup.
+//
+// Six waves per workgroup, one barrier per (step, tile) iteration shared by all:
+//   waves 0-3  compute: poll h_{t-1}, MFMA, reduce through LDS, gating, publish h_t.
+//              Their vector-memory queue only ever holds L2-resident traffic (the
+//              exchange ring), because vector memory completes in order within a wave
+//              and anything slower would sit in front of the latency-critical polls.
+//   wave 4     feeder: streams W.x and the reset flags of FUTURE iterations from HBM
+//              into an LDS ring (kLookahead iterations in flight).
+//   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
+//              output tensor in HBM.
+//
+// Exchange ring: kRing slots, slot t % kRing holds h_t as [member][row][16 units].
+// A word is either data or the "not written yet" pattern.  A workgroup re-arms its own
+// words of slot (t-2) % kRing after its poll of step t has completed: by then every peer
+// has published h_{t-1}, hence has finished reading h_{t-2}.  The re-arm is acknowledged
+// before the workgroup's poll of step t+1 completes, i.e. before it publishes h_{t+1};
+// a peer polling slot (t-2) % kRing for h_{t-2+kRing} has seen that publication, so it
+// can only ever read the pattern or the new data there, never the stale h_{t-2}.
 // ---------------------------------------------------------------------------
+constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
+constexpr int kRing = 8;       // slots of the exchange ring
+
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <bool FAST>
+__device__ __forceinline__ void slstm_pointwise_t(float iraw, float fraw, float zraw, float oraw, CellState &s) {
+  if (!FAST) {
+    slstm_pointwise(iraw, fraw, zraw, oraw, s);
+    return;
+  }
+  // hardware exp2/log2/rcp: relative error ~1e-6, far inside the bf16 budget
+  const float lfm = s.m + (fminf(fraw, 0.0f) - __logf(1.0f + __expf(-fabsf(fraw))));
+  const float mnew = (s.n == 0.0f) ? iraw : fmaxf(iraw, lfm);
+  const float og = __builtin_amdgcn_rcpf(1.0f + __expf(-oraw));
+  const float ig = fminf(__expf(iraw - mnew), 1.0f);
+  const float fg = fminf(__expf(lfm - mnew), 1.0f);
+  const float tz = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * zraw));
+  const float cnew = fg * s.c + ig * tz;
+  const float nnew = fg * s.n + ig;
+  s.y = og * cnew * __builtin_amdgcn_rcpf(nnew);
+  s.c = cnew; s.n = nnew; s.m = mnew;
+}
+
 template <bool BF16, int NCH, int MT>
 __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int WCH = 16 / EPC;          // 16-byte chunks holding the 16 units of one (row, gate)
+  constexpr int ROWS = 16 * MT;          // batch rows of a workgroup
 
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
+  __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
+  __shared__ float hst[4][256];                 // [slot][row*16 + unit]             h on its way to HBM
+  __shared__ uint32_t rfl[4][16];               // [slot][row]                       reset flags
+  __shared__ uint32_t cross_s;
 
   // ---- role of this workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8,
   //      a head group takes consecutive slots of ONE XCD so its exchange stays in one L2)
   const int wg = blockIdx.x;
   const int ngroups = p.NH * p.NBT;
   int gi, member;  // head group index, position inside the group
-  if (p.G <= 32) {
+  const bool one_xcd_layout = p.G <= 32;
+  if (one_xcd_layout) {
     const int xcd = wg & 7;
     const int local = wg >> 3;
     const int slot = local / p.G;
@@ -158,11 +210,6 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     gi = wg / p.G;
     member = wg - gi * p.G;
   }
-  if (threadIdx.x == 0 && p.wg_xcc) {
-    // XCC_ID hardware register (id 20), bits [3:0]
-    p.wg_xcc[wg] = (gi < ngroups ? 0x100u : 0u) | (uint32_t)(gi << 16) |
-                   (__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu);
-  }
   if (gi >= ngroups) return;
   const int head = gi / p.NBT;
   const int bt = gi - head * p.NBT;
@@ -170,14 +217,201 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
   const int lane = tid & 63;
-  const int q = lane >> 4;     // lane group: which 16-byte chunk of a 4-chunk K slab
-  const int r16 = lane & 15;   // MFMA row (A) / column (B, C)
+  const long long spin_limit = p.spin_limit > 0 ? p.spin_limit : kDefaultSpinLimit;
+
+  // ---- placement handshake: do all members of this head group share one XCD (one L2)?
+  //      If so h is published with plain stores (they land in that L2); otherwise with
+  //      device-scope stores that are written through to memory.
+  if (tid == 0) {
+    const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
+    __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t cross = one_xcd_layout ? 0u : 1u;
+    if (one_xcd_layout) {
+      const int xcd = wg & 7;
+      const int slot = (wg >> 3) / p.G;
+      for (int j = 0; j < p.G; ++j) {
+        const int peer = ((slot * p.G + j) << 3) | xcd;
+        uint32_t w = 0;
+        long long spins = 0;
+        while (((w = __hip_atomic_load(&p.wg_xcc[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & 0x80000000u) == 0u) {
+          if (++spins >= spin_limit) {  // a peer never started: the grid is not co-resident
+            if (atomicExch(&p.status->aborted, 1u) == 0u) {
+              p.status->abort_wg = (uint32_t)wg;
+              p.status->abort_step = 0xFFFFFFFFu;
+            }
+            cross = 1u;
+            break;
+          }
+        }
+        if ((w & 0xFu) != my_xcc) cross = 1u;
+      }
+      if (cross) atomicAdd(&p.status->xcd_mixed, 1u);
+    }
+    cross_s = cross;
+  }
 
   const int dh = p.dh;
   const int H = p.NH * dh;
   const int a0 = member * 16;
   const int rowbase = p.b0 + bt * p.rows_per_wg;
   const long long BH = (long long)p.B * H;
+  const int NIT = p.T * MT;
+  const int NITpad = (NIT + kLookahead - 1) / kLookahead * kLookahead;  // barriers every wave executes
+
+  // =========================================================================
+  // wave 4: feeder.  Every iteration issues exactly WCH + 1 loads (addresses of
+  // rows / chunks / steps that do not exist are clamped to ones that do and the
+  // result is zeroed), so that the outstanding-load count at each use is exact.
+  // =========================================================================
+  if (wave == 4) {
+    const int fb = lane & 15;  // batch row inside the tile
+    const int fg = lane >> 4;  // gate
+    uint4 ring[kLookahead][WCH];
+    uint32_t fring[kLookahead];
+    const char *wxb = reinterpret_cast<const char *>(p.wx);
+    const unsigned char *flagb = p.reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);
+    const long long flag_sb = p.reset ? p.reset_sb : 0;
+    const uint32_t flag_on = p.reset ? 0xFFu : 0u;
+
+    auto issue = [&](int it, uint4 (&dst)[WCH], uint32_t &flag) {
+      const int itc = it < NIT ? it : NIT - 1;
+      const int t = itc / MT;
+      const int mt = itc - t * MT;
+      const int brow = rowbase + mt * 16 + fb;
+      const int browc = brow < p.bend ? brow : p.bend - 1;
+      const long long e0 = (long long)browc * p.wx_sb + (long long)t * p.wx_st + (long long)fg * H + head * dh + a0;
+#ifdef XS_EXP_NOWX
+      for (int c = 0; c < WCH; ++c) dst[c] = make_uint4(e0 & 1, 0, 0, 0);
+      flag = 0;
+#else
+#pragma unroll
+      for (int c = 0; c < WCH; ++c) {
+        const int cc = (a0 + c * EPC < dh) ? c : 0;
+        dst[c] = *reinterpret_cast<const uint4 *>(wxb + (e0 + cc * EPC) * ESZ);
+      }
+      flag = flagb[(long long)browc * flag_sb + (p.reset ? t : 0)];
+#endif
+    };
+    auto put = [&](int it, const uint4 (&src)[WCH], uint32_t flag_next, int it_next) {
+      const int t = it / MT;
+      const int mt = it - t * MT;
+      const bool row_ok = rowbase + mt * 16 + fb < p.bend;
+      float *dst = &wxs[it & 1][fg][fb * kTileStride];
+#pragma unroll
+      for (int c = 0; c < WCH; ++c) {
+        uint4 v = src[c];
+        if (!row_ok || a0 + c * EPC >= dh) v = make_uint4(0, 0, 0, 0);
+        if (BF16) {
+          f32x4 lo, hi;
+          lo[0] = bf16_bits_to_float(v.x & 0xFFFFu); lo[1] = bf16_bits_to_float(v.x >> 16);
+          lo[2] = bf16_bits_to_float(v.y & 0xFFFFu); lo[3] = bf16_bits_to_float(v.y >> 16);
+          hi[0] = bf16_bits_to_float(v.z & 0xFFFFu); hi[1] = bf16_bits_to_float(v.z >> 16);
+          hi[2] = bf16_bits_to_float(v.w & 0xFFFFu); hi[3] = bf16_bits_to_float(v.w >> 16);
+          *reinterpret_cast<f32x4 *>(dst + c * 8) = lo;
+          *reinterpret_cast<f32x4 *>(dst + c * 8 + 4) = hi;
+        } else {
+          *reinterpret_cast<uint4 *>(dst + c * 4) = v;
+        }
+      }
+      // reset flag of the NEXT iteration (needed before that iteration's MFMA)
+      const int tn = it_next / MT;
+      const int mtn = it_next - tn * MT;
+      const bool rown_ok = it_next < NIT && rowbase + mtn * 16 + fb < p.bend;
+      if (fg == 0) rfl[it_next & 3][fb] = rown_ok ? (flag_next & flag_on) : 0u;
+    };
+
+#pragma unroll
+    for (int u = 0; u < kLookahead; ++u) issue(u, ring[u], fring[u]);
+    if (fg == 0) rfl[0][fb] = (rowbase + fb < p.bend) ? (fring[0] & flag_on) : 0u;
+    lds_barrier();  // prologue barrier
+#ifdef XS_PROFILE
+    long long fprof[3] = {0, 0, 0};
+    long long ft = clock64();
+#define XS_FTICK(i) do { const long long now_ = clock64(); fprof[i] += now_ - ft; ft = now_; } while (0)
+#else
+#define XS_FTICK(i) do { } while (0)
+#endif
+    for (int it0 = 0; it0 < NITpad; it0 += kLookahead) {
+#pragma unroll
+      for (int u = 0; u < kLookahead; ++u) {
+        const int it = it0 + u;
+        put(it, ring[u], fring[(u + 1) % kLookahead], it + 1);
+        XS_FTICK(0);
+        issue(it + kLookahead, ring[u], fring[u]);
+        XS_FTICK(1);
+        lds_barrier();  // barrier #it
+        XS_FTICK(2);
+      }
+    }
+    lds_barrier();  // final barrier
+#ifdef XS_PROFILE
+    if (lane == 0 && member == 0 && gi == 0) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 4 * 8;
+      for (int i = 0; i < 3; ++i) dst[i] = fprof[i];
+    }
+#endif
+    return;
+  }
+
+  // =========================================================================
+  // wave 5: drainer.  h of iteration it is staged in LDS by the compute waves
+  // between barriers #it and #it+1; it is written to HBM two iterations later.
+  // =========================================================================
+  if (wave == 5) {
+    const int drow = lane >> 2;   // batch row inside the tile
+    const int dq = lane & 3;      // which 4 of the 16 units
+    auto drain = [&](int it) {
+      const int t = it / MT;
+      const int mt = it - t * MT;
+      const int brow = rowbase + mt * 16 + drow;
+      if (brow < p.bend && a0 + dq * 4 < dh) {
+        const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
+        const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
+#ifdef XS_EXP_NOHOUT
+        if (v[0] == 123.25f)
+#endif
+        if (BF16) {
+          uint2 w;
+          w.x = pack_bf16x2(v[0], v[1]); w.y = pack_bf16x2(v[2], v[3]);
+          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = w;
+        } else {
+          *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.h_out) + o) = v;
+        }
+      }
+    };
+    lds_barrier();  // prologue barrier
+#ifdef XS_PROFILE
+    long long dprof[2] = {0, 0};
+    long long dt = clock64();
+#endif
+    for (int j = 0; j < NITpad; ++j) {
+      if (j >= 2 && j - 2 < NIT) drain(j - 2);
+#ifdef XS_PROFILE
+      { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
+#endif
+      lds_barrier();  // barrier #j
+#ifdef XS_PROFILE
+      { const long long now_ = clock64(); dprof[1] += now_ - dt; dt = now_; }
+#endif
+    }
+    lds_barrier();  // final barrier
+    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it);
+#ifdef XS_PROFILE
+    if (lane == 0 && member == 0 && gi == 0) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
+      for (int i = 0; i < 2; ++i) dst[i] = dprof[i];
+    }
+#endif
+    return;
+  }
+
+  // =========================================================================
+  // waves 0-3: compute
+  // =========================================================================
+  __builtin_amdgcn_s_setprio(3);
+  const int q = lane >> 4;     // lane group: which 16-byte chunk of a 4-chunk K slab
+  const int r16 = lane & 15;   // MFMA row (A) / column (B, C)
 
   // ---- R slice -> registers (once).  B operand: column n = unit a0 + r16 of gate g,
   //      K chunk c of this wave/lane group.
@@ -211,8 +445,8 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   }
 
   // ---- pointwise role: one (batch row, unit) element per thread and batch tile
-  const int pb = tid & 15;
-  const int pa = tid >> 4;
+  const int pa = tid & 15;  // unit inside the workgroup's 16
+  const int pb = tid >> 4;  // batch row inside the tile
   const int ua = a0 + pa;
   const bool unit_ok = ua < dh;
   const int col = head * dh + ua;  // column in [.., H]
@@ -231,26 +465,47 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     }
   }
 
-  const long long spin_limit = p.spin_limit > 0 ? p.spin_limit : kDefaultSpinLimit;
   bool aborted = false;
   uint32_t max_spins = 0;
-  int it = 0;  // (t, mt) iteration counter, selects the LDS buffer
+  int it = 0;  // (t, mt) iteration counter, selects the LDS buffers
+#ifdef XS_PROFILE
+  long long prof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define XS_TICK(i) do { const long long now_ = clock64(); prof[i] += now_ - tick_; tick_ = now_; } while (0)
+  long long tick_ = clock64();
+#else
+#define XS_TICK(i) do { } while (0)
+#endif
+
+  lds_barrier();  // prologue barrier: reset flags of iteration 0 and the placement verdict are in LDS
+  const bool cross = cross_s != 0u;
+
+  // exchange ring layout [head group][member][slot][ROWS][16 units]: the kRing blocks of one
+  // member fill 4 KiB (bf16, one tile), so the members of a group, which are all polled at
+  // once by every peer, sit in different L2 channels (channels interleave at 4 KiB)
+  constexpr int XBLOCK = ROWS * 16 * ESZ;            // bytes one member publishes per step
+  constexpr int XMEMBER = kRing * XBLOCK;            // bytes between members
+  char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * p.G * XMEMBER;
 
   for (int t = 0; t < p.T; ++t) {
+    // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
+    const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
+        xbase + ((t + kRing - 1) % kRing) * XBLOCK, 0, 0x7FFFFFFF, 0x00020000);
+    char *const hcur = xbase + (t % kRing) * XBLOCK;
+    char *const hold = xbase + ((t + kRing - 2) % kRing) * XBLOCK;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt, ++it) {
       // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
+      XS_TICK(5);
       const int arow = rowbase + mt * 16 + r16;
       uint4 areg[NCH];
       bool need[NCH];
       const bool row_ok = arow < p.bend;
-      // a row that starts a document contributes R.0 = 0 exactly
-      const bool row_reset = row_ok && p.reset && p.reset[(long long)arow * p.reset_sb + t] != 0;
+      const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
         areg[c] = make_uint4(0, 0, 0, 0);
-        need[c] = row_ok && !row_reset && k0 < dh;
+        need[c] = row_ok && k0 < dh;
       }
       if (t == 0) {
 #pragma unroll
@@ -269,12 +524,13 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           }
         }
       } else {
-        const char *hprev = reinterpret_cast<const char *>(p.h_out) +
-                            ((long long)(t - 1) * BH + (long long)arow * H + head * dh) * (BF16 ? 2 : 4);
+        // unit k of tile row r lives at member k/16, [mt*16 + r][k%16]
+        int xoff[NCH];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
           const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-          if (need[c]) areg[c] = load16_agent(hprev + (long long)k0 * (BF16 ? 2 : 4));
+          xoff[c] = (k0 >> 4) * XMEMBER + ((mt * 16 + r16) * 16 + (k0 & 15)) * ESZ;
+          if (need[c]) areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xoff[c], 0, 16));
         }
         if (!aborted) {
           uint32_t spins = 0;
@@ -286,8 +542,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
                 const bool bad = BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
                 if (bad) {
                   any_bad = true;
-                  const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-                  areg[c] = load16_agent(hprev + (long long)k0 * (BF16 ? 2 : 4));
+                  areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xoff[c], 0, 16));
                 }
               }
             }
@@ -308,10 +563,18 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
             }
           }
           max_spins = spins > max_spins ? spins : max_spins;
+#ifdef XS_PROFILE
+          prof[6] += spins;
+#endif
         }
+      }
+      if (row_reset) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) areg[c] = make_uint4(0, 0, 0, 0);
       }
 
       // ---- 2. partial R.h over this wave's K slab, all four gates
+      XS_TICK(0);
       f32x4 acc[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -340,7 +603,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g)
         *reinterpret_cast<f32x4 *>(&part[buf][wave][g][r16 * kTileStride + 4 * q]) = acc[g];
-      __syncthreads();
+      XS_TICK(1);
+      lds_barrier();  // barrier #it
+      XS_TICK(2);
 
       // ---- 4. reduce over waves + exponential gating for element (row pb, unit pa)
       const int brow = rowbase + mt * 16 + pb;
@@ -353,30 +618,54 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         ry += part[buf][1][g][pa * kTileStride + pb];
         ry += part[buf][2][g][pa * kTileStride + pb];
         ry += part[buf][3][g][pa * kTileStride + pb];
-        float wxv = 0.0f;
-        if (elem_ok) {
-          const long long o = (long long)brow * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + col;
-          wxv = BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(p.wx)[o])
-                     : reinterpret_cast<const float *>(p.wx)[o];
-        }
-        raw[g] = (wxv + ry) + bias_g[g];
+        raw[g] = (wxs[buf][g][pb * kTileStride + pa] + ry) + bias_g[g];
       }
+      if (rfl[it & 3][pb] != 0u) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+      slstm_pointwise_t<BF16>(raw[0], raw[1], raw[2], raw[3], st[mt]);
+#ifdef XS_PROFILE
+      asm volatile("" :: "v"(st[mt].y));
+#endif
+      XS_TICK(3);
+      // ---- 5. publish h_t to the peers, re-arm the words of h_{t-2}, stage h_t for the drainer
+      float y = st[mt].y;
+      if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
       if (elem_ok) {
-        if (p.reset && p.reset[(long long)brow * p.reset_sb + t] != 0) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
-        slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
-        // ---- 5. publish h_t (this IS the output tensor; peers poll these words)
-        const long long o = (long long)t * BH + (long long)brow * H + col;
+        const long long xo = (long long)member * (XMEMBER / ESZ) + (mt * 16 + pb) * 16 + pa;
         if (BF16) {
-          __hip_atomic_store(reinterpret_cast<uint16_t *>(p.h_out) + o, (uint16_t)float_to_bf16_bits(st[mt].y),
-                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint16_t v = (uint16_t)float_to_bf16_bits(y);
+          uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
+          uint16_t *old = reinterpret_cast<uint16_t *>(hold) + xo;
+          if (cross) {
+            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (t >= 2) __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          } else {
+            *dst = v;
+            if (t >= 2) *old = (uint16_t)kSentinel16;
+          }
         } else {
-          float y = st[mt].y;
-          if (y != y) y = __uint_as_float(0x7FC00000u);
-          __hip_atomic_store(reinterpret_cast<float *>(p.h_out) + o, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          float *dst = reinterpret_cast<float *>(hcur) + xo;
+          float *old = reinterpret_cast<float *>(hold) + xo;
+          if (cross) {
+            __hip_atomic_store(dst, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (t >= 2) __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          } else {
+            *dst = y;
+            if (t >= 2) *old = __uint_as_float(kSentinel32);
+          }
         }
       }
+      hst[it & 3][tid] = y;
+      XS_TICK(4);
     }
   }
+  for (int j = NIT; j < NITpad; ++j) lds_barrier();  // padding iterations of the feeder
+  lds_barrier();                                     // final barrier
+#ifdef XS_PROFILE
+  if (lane == 0 && member == 0 && gi == 0) {
+    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + wave * 8;
+    for (int i = 0; i < 8; ++i) dst[i] = prof[i];
+  }
+#endif
 
   // ---- final state
 #pragma unroll
@@ -405,6 +694,13 @@ int fail(int code, const char *fmt, ...) {
 
 constexpr size_t kStatusBytes = 256;
 constexpr int kMaxWg = 4096;
+constexpr size_t kHeaderBytes = kStatusBytes + (size_t)kMaxWg * 4;  // status block + placement words (multiple of 256)
+
+// upper bound on the elements of the exchange ring [8 slots][head groups][G][rows][16]:
+// the head groups of one launch never cover more than B rounded up to 64 rows per head
+inline size_t xbuf_elems(int B, int NH, int dh) {
+  return (size_t)8 * NH * ((dh + 15) / 16) * ((size_t)(B + 63) / 64 * 64) * 16;
+}
 
 typedef void (*SeqKernel)(SeqParams);
 
@@ -437,6 +733,7 @@ int validate(const xs_slstm_args *a, bool step) {
   if (a->r_dtype != XS_F32 && a->r_dtype != XS_BF16) return fail(XS_ERR_DTYPE, "r_dtype %d not supported", a->r_dtype);
   if (a->wx_dtype == XS_F32 && a->r_dtype != XS_F32) return fail(XS_ERR_DTYPE, "float32 wx needs a float32 recurrent matrix");
   if (!a->r || !a->bias || !a->s_out) return fail(XS_ERR_NULL, "r, bias and s_out are required");
+  if (a->s0 && a->s0 == a->s_out) return fail(XS_ERR_SHAPE, "s_out must not alias s0");
   if (a->B > 0 && a->T > 0 && (!a->wx || !a->h_out)) return fail(XS_ERR_NULL, "wx and h_out are required");
   const int epc = a->wx_dtype == XS_BF16 ? 8 : 4;
   if (a->dh % 8 != 0) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not a multiple of 8", a->dh);
@@ -447,6 +744,10 @@ int validate(const xs_slstm_args *a, bool step) {
     if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
   }
   const uintptr_t al = 16;
+  const long long esz = a->wx_dtype == XS_BF16 ? 2 : 4;
+  if (a->B > 0 && a->T > 0 &&
+      (((uintptr_t)a->wx % al) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16)))
+    return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
   if (((uintptr_t)a->r % al) || ((uintptr_t)a->h_out % al) || ((uintptr_t)a->s0 % al) || ((uintptr_t)a->s_out % al))
     return fail(XS_ERR_ALIGN, "r, h_out, s0 and s_out must be 16-byte aligned");
   if (!a->workspace || a->workspace_bytes < xs_slstm_workspace_bytes(a->B, a->T, a->NH, a->dh))
@@ -479,8 +780,7 @@ int run_forward(const xs_slstm_args *a) {
   if (B == 0) return XS_OK;
   if (T == 0) {
     const size_t n = (size_t)4 * B * H;
-    if (a->s0 != a->s_out)
-      hipLaunchKernelGGL(copy_state_kernel, dim3(256), dim3(256), 0, stream, a->s0, a->s_out, n);
+    hipLaunchKernelGGL(copy_state_kernel, dim3(256), dim3(256), 0, stream, a->s0, a->s_out, n);
     return hipGetLastError() == hipSuccess ? XS_OK : fail(XS_ERR_LAUNCH, "state copy launch failed");
   }
 
@@ -505,14 +805,6 @@ int run_forward(const xs_slstm_args *a) {
   SeqKernel kern = bf16 ? pick_kernel<true>(nch, MT) : pick_kernel<false>(nch, MT);
   if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
 
-  // pre-fill h_out with the "not written yet" pattern
-  {
-    const size_t words = ((size_t)T * B * H * (bf16 ? 2 : 4) + 3) / 4;
-    const int blocks = (int)((words + 256 * 8 - 1) / (256 * 8));
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks < 1 ? 1 : (blocks > 2048 ? 2048 : blocks)), dim3(256), 0, stream,
-                       (uint32_t *)a->h_out, words, kSentinel32);
-  }
-
   uint32_t launches = 0;
   for (int b0 = 0; b0 < B; b0 += rows_per_launch) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
@@ -520,6 +812,12 @@ int run_forward(const xs_slstm_args *a) {
     const int ngroups = NH * NBT;
     const int grid = G <= 32 ? 8 * G * ((ngroups + 7) / 8) : ngroups * G;
     if (grid > kMaxWg) return fail(XS_ERR_UNSUPPORTED, "grid %d too large", grid);
+    {  // every word of the exchange ring starts as "not written yet"
+      const size_t words = ((size_t)kRing * ngroups * G * rows_per_wg * 16 * (bf16 ? 2 : 4) + 3) / 4;
+      const int blocks = (int)((words + 256 * 4 - 1) / (256 * 4));
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks)), dim3(256), 0, stream,
+                         (uint32_t *)((char *)a->workspace + kHeaderBytes), words, kSentinel32);
+    }
     SeqParams p;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.r = a->r; p.r_bf16 = a->r_dtype == XS_BF16;
@@ -528,6 +826,7 @@ int run_forward(const xs_slstm_args *a) {
     p.h_out = a->h_out; p.s_out = a->s_out;
     p.status = (xs_slstm_status *)a->workspace;
     p.wg_xcc = (uint32_t *)((char *)a->workspace + kStatusBytes);
+    p.xbuf = (char *)a->workspace + kHeaderBytes;
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
     p.spin_limit = a->spin_limit;
@@ -548,7 +847,10 @@ int xs_abi_version(void) { return XS_ABI_VERSION; }
 
 const char *xs_last_error(void) { return g_err; }
 
-size_t xs_slstm_workspace_bytes(int32_t, int32_t, int32_t, int32_t) { return kStatusBytes + (size_t)kMaxWg * 4; }
+size_t xs_slstm_workspace_bytes(int32_t B, int32_t T, int32_t NH, int32_t dh) {
+  if (B < 0 || T < 0 || NH <= 0 || dh <= 0) return 0;
+  return kHeaderBytes + xbuf_elems(B, NH, dh) * 4;
+}
 
 int xs_slstm_forward(const xs_slstm_args *args) {
   g_err[0] = 0;

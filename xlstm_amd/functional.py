@@ -44,7 +44,7 @@ def read_status(workspace: torch.Tensor) -> dict:
 
 def read_placement(workspace: torch.Tensor, max_wg: int = 4096) -> torch.Tensor:
     """Per-workgroup placement words written by the sequence kernel:
-    bits [3:0] XCD id, bit 8 = workgroup was active, bits [31:16] head group."""
+    bit 31 = workgroup was active, bits [30:8] head group, bits [3:0] XCD id."""
     off = 256
     return workspace[off: off + 4 * max_wg].cpu().view(torch.int32)
 
@@ -90,8 +90,11 @@ def slstm_forward(
         _require_cuda(name, t)
     r = r.contiguous()
     bias = bias.to(torch.float32).contiguous()
-    if wx.numel() and wx.stride(2) != 1:
-        wx = wx.contiguous()
+    if wx.numel():
+        esz = wx.element_size()
+        if (wx.stride(2) != 1 or wx.data_ptr() % 16 or (wx.stride(0) * esz) % 16 or (wx.stride(1) * esz) % 16
+                or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H)):
+            wx = wx.contiguous()
     if s0 is not None:
         _require_cuda("state", s0)
         if tuple(s0.shape) != (4, B, H):
