@@ -129,6 +129,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode leg (profiling runs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU; the path shards over batch rows / heads without "
@@ -141,6 +143,14 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (the hip backend has no CPU path)")
     device = torch.device("cuda:0")
+    if args.copy_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=device)  # 1 GiB read + 1 GiB written per copy
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"copy_bytes_each_way": src.numel() * 4, "copies": 5}))
+        return
     B, T, NH, dh = 16, 2048, 4, 256
     H = NH * dh
     wx_c, r_ext_c, bias_c, mask_c = make_inputs(B, T, NH, dh, 512, device)
