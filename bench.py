@@ -129,6 +129,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode leg (profiling runs)")
+    ap.add_argument("--decode-only", action="store_true", help="only run the decode leg (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -150,6 +151,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_each_way": src.numel() * 4, "copies": 5}))
+        return
+    if args.decode_only:
+        print(json.dumps({"decode": bench_decode(device)}))
         return
     B, T, NH, dh = 16, 2048, 4, 256
     H = NH * dh

@@ -321,6 +321,16 @@ class sLSTMCell_hip(nn.Module):
             )
 
     # ------------------------------------------------------------------ forward
+    def _bf16_recurrent_kernel(self) -> torch.Tensor:
+        """bf16 copy of R for decoding, refreshed when the parameter changes."""
+        p = self._recurrent_kernel_
+        key = (p.data_ptr(), p._version, p.device)
+        cache = getattr(self, "_r_bf16_cache", None)
+        if cache is None or cache[0] != key:
+            cache = (key, p.detach().to(torch.bfloat16).contiguous())
+            object.__setattr__(self, "_r_bf16_cache", cache)
+        return cache[1]
+
     def _run(self, input, state, reset_mask, step: bool):
         self._check_input(input)
         x = self._input_bs(input)
@@ -331,9 +341,12 @@ class sLSTMCell_hip(nn.Module):
             x = x.float()
         elif in_dtype not in (torch.float32, torch.bfloat16):
             raise TypeError(f"input dtype {in_dtype} not supported by the hip backend")
+        r = self._recurrent_kernel_.detach()
+        if step and x.dtype == torch.bfloat16:
+            r = self._bf16_recurrent_kernel()  # the step kernel reads R every token: keep it in the operand type
         h, s = F_hip.slstm_forward(
             x,
-            self._recurrent_kernel_.detach(),
+            r,
             self._bias_.detach().view(self.config.num_heads, 4, self.head_dim),
             state,
             reset_mask,

@@ -19,6 +19,7 @@
 #include <stdarg.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "xlstm_amd.h"
@@ -255,6 +256,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   const int H = p.NH * dh;
   const int a0 = member * 16;
   const int rowbase = p.b0 + bt * p.rows_per_wg;
+  // rows [rowbase, rend) belong to this workgroup; with few rows per head the batch is cut into
+  // tiles of fewer than 16 rows so that more compute units share the work and every exchange is smaller
+  const int rend = (rowbase + p.rows_per_wg < p.bend) ? rowbase + p.rows_per_wg : p.bend;
   const long long BH = (long long)p.B * H;
   const int NIT = p.T * MT;
   const int NITpad = (NIT + kLookahead - 1) / kLookahead * kLookahead;  // barriers every wave executes
@@ -279,24 +283,19 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       const int t = itc / MT;
       const int mt = itc - t * MT;
       const int brow = rowbase + mt * 16 + fb;
-      const int browc = brow < p.bend ? brow : p.bend - 1;
+      const int browc = brow < rend ? brow : rend - 1;
       const long long e0 = (long long)browc * p.wx_sb + (long long)t * p.wx_st + (long long)fg * H + head * dh + a0;
-#ifdef XS_EXP_NOWX
-      for (int c = 0; c < WCH; ++c) dst[c] = make_uint4(e0 & 1, 0, 0, 0);
-      flag = 0;
-#else
 #pragma unroll
       for (int c = 0; c < WCH; ++c) {
         const int cc = (a0 + c * EPC < dh) ? c : 0;
         dst[c] = *reinterpret_cast<const uint4 *>(wxb + (e0 + cc * EPC) * ESZ);
       }
       flag = flagb[(long long)browc * flag_sb + (p.reset ? t : 0)];
-#endif
     };
     auto put = [&](int it, const uint4 (&src)[WCH], uint32_t flag_next, int it_next) {
       const int t = it / MT;
       const int mt = it - t * MT;
-      const bool row_ok = rowbase + mt * 16 + fb < p.bend;
+      const bool row_ok = rowbase + mt * 16 + fb < rend;
       float *dst = &wxs[it & 1][fg][fb * kTileStride];
 #pragma unroll
       for (int c = 0; c < WCH; ++c) {
@@ -317,13 +316,13 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       // reset flag of the NEXT iteration (needed before that iteration's MFMA)
       const int tn = it_next / MT;
       const int mtn = it_next - tn * MT;
-      const bool rown_ok = it_next < NIT && rowbase + mtn * 16 + fb < p.bend;
+      const bool rown_ok = it_next < NIT && rowbase + mtn * 16 + fb < rend;
       if (fg == 0) rfl[it_next & 3][fb] = rown_ok ? (flag_next & flag_on) : 0u;
     };
 
 #pragma unroll
     for (int u = 0; u < kLookahead; ++u) issue(u, ring[u], fring[u]);
-    if (fg == 0) rfl[0][fb] = (rowbase + fb < p.bend) ? (fring[0] & flag_on) : 0u;
+    if (fg == 0) rfl[0][fb] = (rowbase + fb < rend) ? (fring[0] & flag_on) : 0u;
     lds_barrier();  // prologue barrier
 #ifdef XS_PROFILE
     long long fprof[3] = {0, 0, 0};
@@ -365,12 +364,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       const int t = it / MT;
       const int mt = it - t * MT;
       const int brow = rowbase + mt * 16 + drow;
-      if (brow < p.bend && a0 + dq * 4 < dh) {
+      if (brow < rend && a0 + dq * 4 < dh) {
         const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
         const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
-#ifdef XS_EXP_NOHOUT
-        if (v[0] == 123.25f)
-#endif
         if (BF16) {
           uint2 w;
           w.x = pack_bf16x2(v[0], v[1]); w.y = pack_bf16x2(v[2], v[3]);
@@ -459,7 +455,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   for (int mt = 0; mt < MT; ++mt) {
     const int brow = rowbase + mt * 16 + pb;
     st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
-    if (p.s0 && unit_ok && brow < p.bend) {
+    if (p.s0 && unit_ok && brow < rend) {
       const long long o = (long long)brow * H + col;
       st[mt].y = p.s0[o]; st[mt].c = p.s0[BH + o]; st[mt].n = p.s0[2 * BH + o]; st[mt].m = p.s0[3 * BH + o];
     }
@@ -479,19 +475,20 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   lds_barrier();  // prologue barrier: reset flags of iteration 0 and the placement verdict are in LDS
   const bool cross = cross_s != 0u;
 
-  // exchange ring layout [head group][member][slot][ROWS][16 units]: the kRing blocks of one
-  // member fill 4 KiB (bf16, one tile), so the members of a group, which are all polled at
-  // once by every peer, sit in different L2 channels (channels interleave at 4 KiB)
+  // exchange ring layout [head group][slot][member][ROWS][16 units]: what a group publishes in
+  // one step is contiguous (512 B per member for bf16, one tile), which spreads a step's polls
+  // over all L2 channels (measured: lines 256 B .. 2 KiB apart are served 1.5x faster than
+  // lines 4 KiB or more apart)
   constexpr int XBLOCK = ROWS * 16 * ESZ;            // bytes one member publishes per step
-  constexpr int XMEMBER = kRing * XBLOCK;            // bytes between members
-  char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * p.G * XMEMBER;
+  const int xslot = p.G * XBLOCK;                    // bytes one group publishes per step
+  char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
 
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
     const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
-        xbase + ((t + kRing - 1) % kRing) * XBLOCK, 0, 0x7FFFFFFF, 0x00020000);
-    char *const hcur = xbase + (t % kRing) * XBLOCK;
-    char *const hold = xbase + ((t + kRing - 2) % kRing) * XBLOCK;
+        xbase + ((t + kRing - 1) % kRing) * xslot, 0, 0x7FFFFFFF, 0x00020000);
+    char *const hcur = xbase + (t % kRing) * xslot;
+    char *const hold = xbase + ((t + kRing - 2) % kRing) * xslot;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt, ++it) {
       // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
@@ -499,7 +496,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       const int arow = rowbase + mt * 16 + r16;
       uint4 areg[NCH];
       bool need[NCH];
-      const bool row_ok = arow < p.bend;
+      const bool row_ok = arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
@@ -529,7 +526,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
           const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-          xoff[c] = (k0 >> 4) * XMEMBER + ((mt * 16 + r16) * 16 + (k0 & 15)) * ESZ;
+          xoff[c] = (k0 >> 4) * XBLOCK + ((mt * 16 + r16) * 16 + (k0 & 15)) * ESZ;
           if (need[c]) areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xoff[c], 0, 16));
         }
         if (!aborted) {
@@ -609,7 +606,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 
       // ---- 4. reduce over waves + exponential gating for element (row pb, unit pa)
       const int brow = rowbase + mt * 16 + pb;
-      const bool elem_ok = unit_ok && brow < p.bend;
+      const bool elem_ok = unit_ok && brow < rend;
       float raw[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -630,7 +627,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       float y = st[mt].y;
       if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
       if (elem_ok) {
-        const long long xo = (long long)member * (XMEMBER / ESZ) + (mt * 16 + pb) * 16 + pa;
+        const long long xo = (long long)member * (XBLOCK / ESZ) + (mt * 16 + pb) * 16 + pa;
         if (BF16) {
           const uint16_t v = (uint16_t)float_to_bf16_bits(y);
           uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
@@ -671,12 +668,234 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int brow = rowbase + mt * 16 + pb;
-    if (unit_ok && brow < p.bend) {
+    if (unit_ok && brow < rend) {
       const long long o = (long long)brow * H + col;
       p.s_out[o] = st[mt].y; p.s_out[BH + o] = st[mt].c; p.s_out[2 * BH + o] = st[mt].n; p.s_out[3 * BH + o] = st[mt].m;
     }
   }
   if (lane == 0 && max_spins) atomicMax(&p.status->max_spins, max_spins);
+}
+
+// ---------------------------------------------------------------------------
+// decode step kernel, LDS-staged: a workgroup owns 64 batch rows x 32 units x 4 gates.
+// K is walked in slabs of one MFMA k-step (32 bf16 / 16 fp32 input units); each slab of h
+// (converted to the operand type) and of R is brought to LDS with coalesced 16-byte loads and
+// double-buffered, one barrier per slab.  The product is formed transposed (units on the MFMA
+// M axis), so a lane ends with 4 consecutive units of one batch row and the state, W.x and h
+// move as 16-byte / 8-byte accesses that are issued before the K loop and consumed after it.
+// The slabs are accumulated in the sequence kernel's four K quarters and the quarters are
+// added in its order, so step-by-step decoding reproduces a sequence call bit for bit.
+// ---------------------------------------------------------------------------
+struct StepParams {
+  const void *wx;
+  long long wx_sb;
+  const void *r;
+  int r_bf16;
+  const float *bias;
+  const float *s0;
+  const unsigned char *reset;
+  long long reset_sb;
+  void *h_out;
+  float *s_out;
+  xs_slstm_status *status;
+  int B, NH, dh;
+};
+
+constexpr int kSlabStride = 80;  // bytes per row of an LDS slab: 64 data + 16 pad (conflict-free 16-byte reads)
+
+template <bool BF16>
+__global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  constexpr int SLABK = 4 * EPC;  // input units per slab
+  __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][64 * kSlabStride];
+  __shared__ __attribute__((aligned(16))) unsigned char rbuf[2][128 * kSlabStride];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int q = lane >> 4;
+  const int r16 = lane & 15;
+  const int head = blockIdx.z;
+  const int a0 = blockIdx.x * 32;
+  const int rowbase = blockIdx.y * 64;
+  const int dh = p.dh;
+  const int H = p.NH * dh;
+  const long long BH = (long long)p.B * H;
+  const int KW = nch * SLABK;       // input units per K quarter (as in the sequence kernel)
+  const int nslab = 4 * nch;
+
+  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid < 16)
+    reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
+
+  const bool has_s0 = p.s0 != nullptr;
+  const bool has_reset = p.reset != nullptr;
+  const float *s0p = has_s0 ? p.s0 : reinterpret_cast<const float *>(p.wx);                  // stand-ins are only read
+  const unsigned char *rsp = has_reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);  // in their first 32 bytes
+
+  // ---- staging roles.  h slab: thread -> (row tid/4, 16-byte piece tid%4).  R slab: two (column, piece) items.
+  const int hrow = tid >> 2, hq = tid & 3;
+  const int hbrow = rowbase + hrow;
+  const int hbrowc = hbrow < p.B ? hbrow : p.B - 1;
+  const uint32_t hflag = rsp[has_reset ? (long long)hbrowc * p.reset_sb : 0];
+  const bool hzero = !(hbrow < p.B) || !has_s0 || (has_reset && hflag != 0u);
+  const float *hsrc = s0p + (has_s0 ? (long long)hbrowc * H + head * dh : 0);
+  const char *rsrc[2];
+  bool rok[2];
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const int item = tid + 256 * j;
+    const int colx = item >> 2;            // column of the workgroup's 128: gate colx/32, unit colx%32
+    const int a = a0 + (colx & 31);
+    rok[j] = a < dh;
+    rsrc[j] = reinterpret_cast<const char *>(p.r) +
+              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * (BF16 ? 2 : 4);
+  }
+  uint4 hst0, hst1, rst[2];
+  auto slab_k0 = [&](int sidx) { return (sidx / nch) * KW + (sidx % nch) * SLABK; };
+  auto load_slab = [&](int sidx) {
+    const int k0 = slab_k0(sidx) + hq * EPC;
+    const int k0c = (has_s0 && k0 < dh) ? k0 : 0;
+    hst0 = *reinterpret_cast<const uint4 *>(hsrc + k0c);
+    hst1 = BF16 ? *reinterpret_cast<const uint4 *>(hsrc + k0c + 4) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int kr = slab_k0(sidx) + ((tid + 256 * j) & 3) * EPC;
+      rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(kr < dh ? kr : 0) * (BF16 ? 2 : 4));
+    }
+  };
+  auto store_slab = [&](int sidx, int buf) {
+    const int k0 = slab_k0(sidx) + hq * EPC;
+    uint4 v = hst0;
+    if (BF16) {
+      uint4 t;
+      t.x = pack_bf16x2(__uint_as_float(hst0.x), __uint_as_float(hst0.y)); t.y = pack_bf16x2(__uint_as_float(hst0.z), __uint_as_float(hst0.w));
+      t.z = pack_bf16x2(__uint_as_float(hst1.x), __uint_as_float(hst1.y)); t.w = pack_bf16x2(__uint_as_float(hst1.z), __uint_as_float(hst1.w));
+      v = t;
+    }
+    if (hzero || k0 >= dh) v = make_uint4(0, 0, 0, 0);
+    *reinterpret_cast<uint4 *>(&hbuf[buf][hrow * kSlabStride + hq * 16]) = v;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const int item = tid + 256 * j;
+      const int kr = slab_k0(sidx) + (item & 3) * EPC;
+      uint4 w = rst[j];
+      if (!rok[j] || kr >= dh) w = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4 *>(&rbuf[buf][(item >> 2) * kSlabStride + (item & 3) * 16]) = w;
+    }
+  };
+
+  load_slab(0);
+
+  // ---- pointwise operands of this lane: batch row rowbase + 16*wave + r16, units a0 + ut*16 + 4q .. +3
+  const int brow = rowbase + 16 * wave + r16;
+  const int browc = brow < p.B ? brow : p.B - 1;
+  const uint32_t pflag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+  uint2 wxb[2][4];
+  float4 wxf[2][4], bias4[2][4], c4[2], n4[2], m4[2];
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    const int ua = a0 + ut * 16 + 4 * q;
+    const long long col = (long long)head * dh + (ua < dh ? ua : 0);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
+      if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
+      else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
+      bias4[ut][g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + (ua < dh ? ua : 0));
+    }
+    const long long so = (long long)browc * H + col;
+    c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
+    n4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 2 * BH + so : 0));
+    m4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 3 * BH + so : 0));
+  }
+
+  // ---- K loop
+  f32x4 acc[2][4], tot[2][4];
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
+
+  store_slab(0, 0);
+  __syncthreads();
+  for (int sidx = 0; sidx < nslab; ++sidx) {
+    const int buf = sidx & 1;
+    if (sidx + 1 < nslab) load_slab(sidx + 1);
+    const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[buf][(16 * wave + r16) * kSlabStride + q * 16]);
+#pragma unroll
+    for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + ut * 16 + r16) * kSlabStride + q * 16]);
+        if (BF16) {
+          acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
+        } else {
+          const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+          const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+        }
+      }
+    if ((sidx + 1) % nch == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
+#pragma unroll
+      for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          tot[ut][g] = (sidx + 1 == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+          acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+    if (sidx + 1 < nslab) {
+      store_slab(sidx + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
+      __syncthreads();
+    }
+  }
+
+  // ---- gating
+  const bool reset_row = !has_s0 || (has_reset && pflag != 0u);
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    const int ua = a0 + ut * 16 + 4 * q;
+    const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
+    const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
+    const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
+    float yv[4], cv[4], nv[4], mv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float raw[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float wxv;
+        if (BF16) {
+          const uint32_t wd = i < 2 ? wxb[ut][g].x : wxb[ut][g].y;
+          wxv = bf16_bits_to_float((i & 1) ? (wd >> 16) : (wd & 0xFFFFu));
+        } else {
+          const float wf[4] = {wxf[ut][g].x, wxf[ut][g].y, wxf[ut][g].z, wxf[ut][g].w};
+          wxv = wf[i];
+        }
+        const float bf[4] = {bias4[ut][g].x, bias4[ut][g].y, bias4[ut][g].z, bias4[ut][g].w};
+        raw[g] = (wxv + tot[ut][g][i]) + bf[i];
+      }
+      CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
+      slstm_pointwise_t<BF16>(raw[0], raw[1], raw[2], raw[3], st);
+      yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
+    }
+    if (brow < p.B && ua < dh) {
+      const long long o = (long long)brow * H + head * dh + ua;
+      *reinterpret_cast<float4 *>(p.s_out + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
+      *reinterpret_cast<float4 *>(p.s_out + BH + o) = make_float4(cv[0], cv[1], cv[2], cv[3]);
+      *reinterpret_cast<float4 *>(p.s_out + 2 * BH + o) = make_float4(nv[0], nv[1], nv[2], nv[3]);
+      *reinterpret_cast<float4 *>(p.s_out + 3 * BH + o) = make_float4(mv[0], mv[1], mv[2], mv[3]);
+      if (BF16) {
+        uint2 hw;
+        hw.x = pack_bf16x2(yv[0], yv[1]); hw.y = pack_bf16x2(yv[2], yv[3]);
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = hw;
+      } else {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.h_out) + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
+      }
+    }
+  }
 }
 
 // ---------------------------------------------------------------------------
@@ -699,7 +918,8 @@ constexpr size_t kHeaderBytes = kStatusBytes + (size_t)kMaxWg * 4;  // status bl
 // upper bound on the elements of the exchange ring [8 slots][head groups][G][rows][16]:
 // the head groups of one launch never cover more than B rounded up to 64 rows per head
 inline size_t xbuf_elems(int B, int NH, int dh) {
-  return (size_t)8 * NH * ((dh + 15) / 16) * ((size_t)(B + 63) / 64 * 64) * 16;
+  // (with row tiles of 4 or 8 rows a block still spans 16 rows, hence the factor 4)
+  return (size_t)8 * NH * ((dh + 15) / 16) * ((size_t)(B + 63) / 64 * 64) * 16 * 4;
 }
 
 typedef void (*SeqKernel)(SeqParams);
@@ -729,6 +949,7 @@ int validate(const xs_slstm_args *a, bool step) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
   if (step && a->T != 1) return fail(XS_ERR_SHAPE, "xs_slstm_step needs T == 1, got %d", a->T);
+  if (step && a->r_dtype != a->wx_dtype) return fail(XS_ERR_DTYPE, "xs_slstm_step needs the recurrent matrix in the dtype of wx");
   if (a->wx_dtype != XS_F32 && a->wx_dtype != XS_BF16) return fail(XS_ERR_DTYPE, "wx_dtype %d not supported", a->wx_dtype);
   if (a->r_dtype != XS_F32 && a->r_dtype != XS_BF16) return fail(XS_ERR_DTYPE, "r_dtype %d not supported", a->r_dtype);
   if (a->wx_dtype == XS_F32 && a->r_dtype != XS_F32) return fail(XS_ERR_DTYPE, "float32 wx needs a float32 recurrent matrix");
@@ -768,6 +989,33 @@ int device_cus() {
   return cus;
 }
 
+int run_step(const xs_slstm_args *a) {
+  hipStream_t stream = (hipStream_t)a->stream;
+  const int B = a->B, NH = a->NH, dh = a->dh;
+  const bool bf16 = a->wx_dtype == XS_BF16;
+  if (B == 0) return XS_OK;
+  const int epc = bf16 ? 8 : 4;
+  int nch = 1;
+  while (nch * 16 * epc < dh) nch *= 2;  // the sequence kernel's K quarters are nch slabs wide
+  if (nch > 8) return fail(XS_ERR_UNSUPPORTED, "head dim %d too large for %s operands (max %d)", dh, bf16 ? "bf16" : "fp32", 8 * 16 * epc);
+  if ((long long)B * 4 * NH * dh * (bf16 ? 2 : 4) < 32) return fail(XS_ERR_SHAPE, "wx too small");
+  StepParams p;
+  p.wx = a->wx; p.wx_sb = a->wx_stride_b;
+  p.r = a->r; p.r_bf16 = a->r_dtype == XS_BF16;
+  p.bias = a->bias; p.s0 = a->s0;
+  p.reset = a->reset; p.reset_sb = a->reset_stride_b;
+  p.h_out = a->h_out; p.s_out = a->s_out;
+  p.status = (xs_slstm_status *)a->workspace;
+  p.B = B; p.NH = NH; p.dh = dh;
+  const dim3 grid((dh + 31) / 32, (B + 63) / 64, NH);
+  if (grid.y > 65535 || grid.z > 65535) return fail(XS_ERR_UNSUPPORTED, "batch or head count too large for one step launch");
+  if (bf16) hipLaunchKernelGGL(slstm_step_tile_kernel<true>, grid, dim3(256), 0, stream, p, nch);
+  else hipLaunchKernelGGL(slstm_step_tile_kernel<false>, grid, dim3(256), 0, stream, p, nch);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 int run_forward(const xs_slstm_args *a) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int B = a->B, T = a->T, NH = a->NH, dh = a->dh;
@@ -799,7 +1047,11 @@ int run_forward(const xs_slstm_args *a) {
   const int max_groups_per_head = cus / (NH * G);  // >= 1
   int MT = 1;
   while (MT < 4 && (tiles + MT - 1) / MT > max_groups_per_head) MT *= 2;
-  const int rows_per_wg = 16 * MT;
+  int rows_per_wg = 16 * MT;
+  if (MT == 1) {  // spare compute units: smaller row tiles, smaller exchanges
+    for (int r = 4; r < 16; r *= 2)
+      if ((B + r - 1) / r <= max_groups_per_head) { rows_per_wg = r; break; }
+  }
   const int rows_per_launch = rows_per_wg * max_groups_per_head;
 
   SeqKernel kern = bf16 ? pick_kernel<true>(nch, MT) : pick_kernel<false>(nch, MT);
@@ -813,7 +1065,7 @@ int run_forward(const xs_slstm_args *a) {
     const int grid = G <= 32 ? 8 * G * ((ngroups + 7) / 8) : ngroups * G;
     if (grid > kMaxWg) return fail(XS_ERR_UNSUPPORTED, "grid %d too large", grid);
     {  // every word of the exchange ring starts as "not written yet"
-      const size_t words = ((size_t)kRing * ngroups * G * rows_per_wg * 16 * (bf16 ? 2 : 4) + 3) / 4;
+      const size_t words = ((size_t)kRing * ngroups * G * 16 * MT * 16 * (bf16 ? 2 : 4) + 3) / 4;
       const int blocks = (int)((words + 256 * 4 - 1) / (256 * 4));
       hipLaunchKernelGGL(fill_u32_kernel, dim3(blocks < 1 ? 1 : (blocks > 1024 ? 1024 : blocks)), dim3(256), 0, stream,
                          (uint32_t *)((char *)a->workspace + kHeaderBytes), words, kSentinel32);
@@ -863,7 +1115,7 @@ int xs_slstm_step(const xs_slstm_args *args) {
   g_err[0] = 0;
   const int rc = validate(args, true);
   if (rc != XS_OK) return rc;
-  return run_forward(args);
+  return run_step(args);
 }
 
 }  // extern "C"

@@ -84,6 +84,8 @@ def slstm_forward(
         raise TypeError(f"r dtype {r.dtype} not supported")
     if wx.dtype == torch.float32 and r.dtype != torch.float32:
         r = r.float()
+    if step and r.dtype != wx.dtype:
+        r = r.to(wx.dtype)  # callers that decode many tokens pass a cached copy (see sLSTMCell_hip)
     if tuple(bias.shape) != (NH, 4, dh):
         raise ValueError(f"bias must be [NH, 4, dh] = {(NH, 4, dh)}, got {tuple(bias.shape)}")
     for name, t in (("r", r), ("bias", bias)):
