@@ -122,6 +122,44 @@ def bench_decode(device, steps=1024, prefill=128):
     }
 
 
+def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
+    """Times one forward call of the cell at another BASELINE shape (median of `iters`)."""
+    import numpy as np
+    import torch
+
+    from tests._util import geometric_reset_mask
+    from xlstm_amd import functional as F
+
+    H = NH * dh
+    g = torch.Generator(device=device).manual_seed(7)
+    wx = torch.empty(B, T, 4 * H, dtype=torch.bfloat16 if bf16 else torch.float32, device=device)
+    for row in range(B):
+        wx[row] = torch.randn(T, 4 * H, generator=g, device=device).to(wx.dtype)
+    r = ((torch.rand(NH, 4 * dh, dh, generator=g, device=device) * 2 - 1) / float(np.sqrt(H)))
+    bias = torch.zeros(NH, 4, dh, device=device)
+    bias[:, 1] = torch.linspace(3.0, 6.0, dh, device=device)
+    mask = torch.from_numpy(geometric_reset_mask(7, B, T, mean_doc)).to(device) if mean_doc else None
+    ws = F.workspace_for(B, T, NH, dh, device)
+    h = torch.empty(T, B, H, dtype=wx.dtype, device=device)
+    s = torch.empty(4, B, H, dtype=torch.float32, device=device)
+    times = []
+    for i in range(iters + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        F.slstm_forward(wx, r, bias, None, mask, workspace=ws, h_out=h, s_out=s)
+        e1.record()
+        torch.cuda.synchronize()
+        if i:
+            times.append(e0.elapsed_time(e1))
+    ms = float(np.median(times))
+    esz = 2 if bf16 else 4
+    nbytes = algorithmic_bytes(B, T, NH, dh, esz, esz, 4, with_mask=bool(mean_doc))
+    flops = 8.0 * B * T * H * dh
+    return {"workload": name, "ms": ms, "us_per_timestep": ms * 1e3 / T, "tokens_per_s": B * T / ms * 1e3,
+            "hbm_GBs": nbytes / ms / 1e6, "tflops": flops / ms / 1e9,
+            "aborted": F.read_status(ws)["aborted"]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -130,6 +168,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the CPU leg (profiling runs)")
     ap.add_argument("--no-decode", action="store_true", help="skip the decode leg (profiling runs)")
     ap.add_argument("--decode-only", action="store_true", help="only run the decode leg (profiling runs)")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time the cell at BASELINE configs 1, 4 and 5 (adds an 'all_configs' object)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -211,6 +251,12 @@ def main():
     traffic_file = os.path.join(ROOT, "profiles", "traffic_seq_cfg2.json")
     if os.path.exists(traffic_file):
         out["roofline"]["traffic"] = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
+    if args.all_configs:
+        out["all_configs"] = [
+            bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),
+            bench_config(device, "config 4 (one sLSTM cell): B=8 T=2048 D=1024 NH=4 bf16, documents mean 768", 8, 2048, 4, 256, True, 768),
+            bench_config(device, "config 5: B=64 T=4096 D=4096 NH=4 bf16, no resets", 64, 4096, 4, 1024, True, 0, iters=2),
+        ]
     if not args.no_decode:
         out["decode"] = bench_decode(device)
     if not args.no_cpu_baseline:

@@ -60,16 +60,20 @@ struct SeqParams {
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
 
-// round-to-nearest-even; NaN becomes the canonical quiet NaN so that the
-// "not written yet" pattern 0xFFFF can never be produced by a real value
-__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return 0x7FC0u;
-  return (u + 0x7FFFu + ((u >> 16) & 1u)) >> 16;
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// two floats -> two bf16, round-to-nearest-even, one v_cvt_pk_bf16_f32
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2{lo, hi}, bf16x2));
 }
 
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return float_to_bf16_bits(lo) | (float_to_bf16_bits(hi) << 16);
+// one float -> bf16 for the exchange ring.  A NaN whose payload would round to the
+// "not written yet" pattern 0xFFFF becomes the canonical quiet NaN, so that pattern can
+// never be produced by a value.
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
+  const uint32_t b = pack_bf16x2(f, 0.0f) & 0xFFFFu;
+  return b == 0xFFFFu ? 0x7FC0u : b;
 }
 
 __device__ __forceinline__ bool chunk_has_sentinel_bf16(const uint4 &v) {
@@ -369,7 +373,8 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
         if (BF16) {
           uint2 w;
-          w.x = pack_bf16x2(v[0], v[1]); w.y = pack_bf16x2(v[2], v[3]);
+          w.x = float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16);
+          w.y = float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16);
           *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = w;
         } else {
           *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.h_out) + o) = v;
@@ -678,13 +683,15 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 
 // ---------------------------------------------------------------------------
 // decode step kernel, LDS-staged: a workgroup owns 64 batch rows x 32 units x 4 gates.
-// K is walked in slabs of one MFMA k-step (32 bf16 / 16 fp32 input units); each slab of h
-// (converted to the operand type) and of R is brought to LDS with coalesced 16-byte loads and
-// double-buffered, one barrier per slab.  The product is formed transposed (units on the MFMA
-// M axis), so a lane ends with 4 consecutive units of one batch row and the state, W.x and h
-// move as 16-byte / 8-byte accesses that are issued before the K loop and consumed after it.
-// The slabs are accumulated in the sequence kernel's four K quarters and the quarters are
-// added in its order, so step-by-step decoding reproduces a sequence call bit for bit.
+// K is walked in slabs of SLABCH MFMA k-steps (WIDE: 64 bf16 / 32 fp32 input units, so that
+// every global load instruction moves whole 128-byte lines); each slab of h (converted to the
+// operand type) and of R goes to LDS, double-buffered, one barrier per slab, and the global
+// loads of up to kStepRing slabs are in flight at once (all of them at dh = 256).  The product
+// is formed transposed (units on the MFMA M axis), so a lane ends with 4 consecutive units of
+// one batch row and the state, W.x and h move as 16-byte / 8-byte accesses that are issued
+// before the K loop and consumed after it.  The slabs are accumulated in the sequence kernel's
+// four K quarters and the quarters are added in its order, so step-by-step decoding
+// reproduces a sequence call bit for bit.
 // ---------------------------------------------------------------------------
 struct StepParams {
   const void *wx;
@@ -701,14 +708,20 @@ struct StepParams {
   int B, NH, dh;
 };
 
-constexpr int kSlabStride = 80;  // bytes per row of an LDS slab: 64 data + 16 pad (conflict-free 16-byte reads)
+constexpr int kStepRing = 4;   // slabs of the decode kernel whose loads are in flight
 
-template <bool BF16>
-__global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch) {
+template <bool BF16, bool WIDE>
+__global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
   constexpr int EPC = BF16 ? 8 : 4;
-  constexpr int SLABK = 4 * EPC;  // input units per slab
-  __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][64 * kSlabStride];
-  __shared__ __attribute__((aligned(16))) unsigned char rbuf[2][128 * kSlabStride];
+  constexpr int CHK = 4 * EPC;                // input units per MFMA k-step ("chunk")
+  constexpr int SLABCH = WIDE ? 2 : 1;        // chunks per slab
+  constexpr int SLABK = SLABCH * CHK;         // input units per slab
+  constexpr int RS = SLABCH * 64 + 16;        // bytes per LDS row: data + pad (conflict-free 16-byte reads)
+  constexpr int HITEMS = (SLABK * 4 / 16) / 4;  // 16-byte pieces of fp32 h each thread stages per slab
+  constexpr int RITEMS = SLABCH * 2;            // 16-byte pieces of R each thread stages per slab
+  constexpr int ESZ = BF16 ? 2 : 4;
+  __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][64 * RS];
+  __shared__ __attribute__((aligned(16))) unsigned char rbuf[2][128 * RS];
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -721,8 +734,8 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const int dh = p.dh;
   const int H = p.NH * dh;
   const long long BH = (long long)p.B * H;
-  const int KW = nch * SLABK;       // input units per K quarter (as in the sequence kernel)
-  const int nslab = 4 * nch;
+  const int nch = 1 << nch_log2;              // chunks per K quarter (as in the sequence kernel)
+  const int nslab = (4 * nch) / SLABCH;
 
   if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid < 16)
     reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
@@ -732,59 +745,76 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const float *s0p = has_s0 ? p.s0 : reinterpret_cast<const float *>(p.wx);                  // stand-ins are only read
   const unsigned char *rsp = has_reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);  // in their first 32 bytes
 
-  // ---- staging roles.  h slab: thread -> (row tid/4, 16-byte piece tid%4).  R slab: two (column, piece) items.
-  const int hrow = tid >> 2, hq = tid & 3;
-  const int hbrow = rowbase + hrow;
-  const int hbrowc = hbrow < p.B ? hbrow : p.B - 1;
-  const uint32_t hflag = rsp[has_reset ? (long long)hbrowc * p.reset_sb : 0];
-  const bool hzero = !(hbrow < p.B) || !has_s0 || (has_reset && hflag != 0u);
-  const float *hsrc = s0p + (has_s0 ? (long long)hbrowc * H + head * dh : 0);
-  const char *rsrc[2];
-  bool rok[2];
+  // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row / column
+  constexpr int HPIECES = SLABK * 4 / 16;     // 16-byte pieces of fp32 h per row and slab
+  constexpr int RPIECES = SLABCH * 4;         // 16-byte pieces of R per column and slab
+  const float *hsrc[HITEMS];
+  bool hzero[HITEMS];
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
+  for (int j = 0; j < HITEMS; ++j) {
     const int item = tid + 256 * j;
-    const int colx = item >> 2;            // column of the workgroup's 128: gate colx/32, unit colx%32
+    const int brow = rowbase + item / HPIECES;
+    const int browc = brow < p.B ? brow : p.B - 1;
+    const uint32_t flag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+    hzero[j] = !(brow < p.B) || !has_s0 || (has_reset && flag != 0u);
+    hsrc[j] = s0p + (has_s0 ? (long long)browc * H + head * dh : 0);
+  }
+  const char *rsrc[RITEMS];
+  bool rok[RITEMS];
+#pragma unroll
+  for (int j = 0; j < RITEMS; ++j) {
+    const int colx = (tid + 256 * j) / RPIECES;   // column of the workgroup's 128: gate colx/32, unit colx%32
     const int a = a0 + (colx & 31);
     rok[j] = a < dh;
     rsrc[j] = reinterpret_cast<const char *>(p.r) +
-              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * (BF16 ? 2 : 4);
+              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * ESZ;
   }
-  uint4 hst0, hst1, rst[2];
-  auto slab_k0 = [&](int sidx) { return (sidx / nch) * KW + (sidx % nch) * SLABK; };
-  auto load_slab = [&](int sidx) {
-    const int k0 = slab_k0(sidx) + hq * EPC;
-    const int k0c = (has_s0 && k0 < dh) ? k0 : 0;
-    hst0 = *reinterpret_cast<const uint4 *>(hsrc + k0c);
-    hst1 = BF16 ? *reinterpret_cast<const uint4 *>(hsrc + k0c + 4) : make_uint4(0, 0, 0, 0);
+  uint4 hring[kStepRing][HITEMS], rring[kStepRing][RITEMS];
+  auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS]) {
+    const int kbase = sidx * SLABK;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int kr = slab_k0(sidx) + ((tid + 256 * j) & 3) * EPC;
-      rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(kr < dh ? kr : 0) * (BF16 ? 2 : 4));
+    for (int j = 0; j < HITEMS; ++j) {
+      const int k = kbase + ((tid + 256 * j) % HPIECES) * 4;
+      hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
+    }
+#pragma unroll
+    for (int j = 0; j < RITEMS; ++j) {
+      const int k = kbase + ((tid + 256 * j) % RPIECES) * EPC;
+      rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
     }
   };
-  auto store_slab = [&](int sidx, int buf) {
-    const int k0 = slab_k0(sidx) + hq * EPC;
-    uint4 v = hst0;
-    if (BF16) {
-      uint4 t;
-      t.x = pack_bf16x2(__uint_as_float(hst0.x), __uint_as_float(hst0.y)); t.y = pack_bf16x2(__uint_as_float(hst0.z), __uint_as_float(hst0.w));
-      t.z = pack_bf16x2(__uint_as_float(hst1.x), __uint_as_float(hst1.y)); t.w = pack_bf16x2(__uint_as_float(hst1.z), __uint_as_float(hst1.w));
-      v = t;
-    }
-    if (hzero || k0 >= dh) v = make_uint4(0, 0, 0, 0);
-    *reinterpret_cast<uint4 *>(&hbuf[buf][hrow * kSlabStride + hq * 16]) = v;
+  auto store_slab = [&](int sidx, int buf, const uint4 (&hst)[HITEMS], const uint4 (&rst)[RITEMS]) {
+    const int kbase = sidx * SLABK;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < HITEMS; ++j) {
       const int item = tid + 256 * j;
-      const int kr = slab_k0(sidx) + (item & 3) * EPC;
+      const int piece = item % HPIECES;
+      const bool z = hzero[j] || kbase + piece * 4 >= dh;
+      uint4 v = hst[j];
+      if (z) v = make_uint4(0, 0, 0, 0);
+      unsigned char *dst = &hbuf[buf][(item / HPIECES) * RS];
+      if (BF16) {
+        uint2 w;
+        w.x = pack_bf16x2(__uint_as_float(v.x), __uint_as_float(v.y));
+        w.y = pack_bf16x2(__uint_as_float(v.z), __uint_as_float(v.w));
+        *reinterpret_cast<uint2 *>(dst + piece * 8) = w;
+      } else {
+        *reinterpret_cast<uint4 *>(dst + piece * 16) = v;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < RITEMS; ++j) {
+      const int item = tid + 256 * j;
+      const int piece = item % RPIECES;
       uint4 w = rst[j];
-      if (!rok[j] || kr >= dh) w = make_uint4(0, 0, 0, 0);
-      *reinterpret_cast<uint4 *>(&rbuf[buf][(item >> 2) * kSlabStride + (item & 3) * 16]) = w;
+      if (!rok[j] || kbase + piece * EPC >= dh) w = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4 *>(&rbuf[buf][(item / RPIECES) * RS + piece * 16]) = w;
     }
   };
 
-  load_slab(0);
+#pragma unroll
+  for (int u = 0; u < kStepRing; ++u)
+    if (u < nslab) load_slab(u, hring[u], rring[u]);
 
   // ---- pointwise operands of this lane: batch row rowbase + 16*wave + r16, units a0 + ut*16 + 4q .. +3
   const int brow = rowbase + 16 * wave + r16;
@@ -816,39 +846,51 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #pragma unroll
     for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
 
-  store_slab(0, 0);
+  store_slab(0, 0, hring[0], rring[0]);
   __syncthreads();
-  for (int sidx = 0; sidx < nslab; ++sidx) {
-    const int buf = sidx & 1;
-    if (sidx + 1 < nslab) load_slab(sidx + 1);
-    const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[buf][(16 * wave + r16) * kSlabStride + q * 16]);
+  for (int s0i = 0; s0i < nslab; s0i += kStepRing) {
 #pragma unroll
-    for (int ut = 0; ut < 2; ++ut)
+    for (int u = 0; u < kStepRing; ++u) {
+      const int sidx = s0i + u;
+      if (sidx < nslab) {
+        const int buf = sidx & 1;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + ut * 16 + r16) * kSlabStride + q * 16]);
-        if (BF16) {
-          acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
-        } else {
-          const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
-          const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+        for (int ch = 0; ch < SLABCH; ++ch) {
+          const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[buf][(16 * wave + r16) * RS + ch * 64 + q * 16]);
 #pragma unroll
-          for (int e = 0; e < 4; ++e)
-            acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+          for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + ut * 16 + r16) * RS + ch * 64 + q * 16]);
+              if (BF16) {
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
+              } else {
+                const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+                const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+              }
+            }
+        }
+        const int chunks_done = (sidx + 1) * SLABCH;
+        if ((chunks_done & (nch - 1)) == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
+#pragma unroll
+          for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              tot[ut][g] = (chunks_done == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+              acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+        }
+        // slab sidx went to LDS one iteration ago: its ring entry takes the loads of slab sidx + kStepRing
+        if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u]);
+        if (sidx + 1 < nslab) {
+          const int un = (u + 1) % kStepRing;
+          store_slab(sidx + 1, buf ^ 1, hring[un], rring[un]);  // the other buffer was last read before the previous barrier
+          __syncthreads();
         }
       }
-    if ((sidx + 1) % nch == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
-#pragma unroll
-      for (int ut = 0; ut < 2; ++ut)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          tot[ut][g] = (sidx + 1 == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
-          acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-        }
-    }
-    if (sidx + 1 < nslab) {
-      store_slab(sidx + 1, buf ^ 1);  // the other buffer was last read before the previous barrier
-      __syncthreads();
     }
   }
 
@@ -889,7 +931,8 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
       *reinterpret_cast<float4 *>(p.s_out + 3 * BH + o) = make_float4(mv[0], mv[1], mv[2], mv[3]);
       if (BF16) {
         uint2 hw;
-        hw.x = pack_bf16x2(yv[0], yv[1]); hw.y = pack_bf16x2(yv[2], yv[3]);
+        hw.x = float_to_bf16_bits(yv[0]) | (float_to_bf16_bits(yv[1]) << 16);
+        hw.y = float_to_bf16_bits(yv[2]) | (float_to_bf16_bits(yv[3]) << 16);
         *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = hw;
       } else {
         *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.h_out) + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
@@ -1009,8 +1052,16 @@ int run_step(const xs_slstm_args *a) {
   p.B = B; p.NH = NH; p.dh = dh;
   const dim3 grid((dh + 31) / 32, (B + 63) / 64, NH);
   if (grid.y > 65535 || grid.z > 65535) return fail(XS_ERR_UNSUPPORTED, "batch or head count too large for one step launch");
-  if (bf16) hipLaunchKernelGGL(slstm_step_tile_kernel<true>, grid, dim3(256), 0, stream, p, nch);
-  else hipLaunchKernelGGL(slstm_step_tile_kernel<false>, grid, dim3(256), 0, stream, p, nch);
+  int nch_log2 = 0;
+  while ((1 << nch_log2) < nch) ++nch_log2;
+  const bool wide = nch >= 2;  // two k-steps per slab: every staged row / column is a whole 128-byte line
+  if (bf16) {
+    if (wide) hipLaunchKernelGGL((slstm_step_tile_kernel<true, true>), grid, dim3(256), 0, stream, p, nch_log2);
+    else hipLaunchKernelGGL((slstm_step_tile_kernel<true, false>), grid, dim3(256), 0, stream, p, nch_log2);
+  } else {
+    if (wide) hipLaunchKernelGGL((slstm_step_tile_kernel<false, true>), grid, dim3(256), 0, stream, p, nch_log2);
+    else hipLaunchKernelGGL((slstm_step_tile_kernel<false, false>), grid, dim3(256), 0, stream, p, nch_log2);
+  }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
   return XS_OK;
