@@ -708,20 +708,27 @@ struct StepParams {
   int B, NH, dh;
 };
 
-constexpr int kStepRing = 4;   // slabs of the decode kernel whose loads are in flight
 
-template <bool BF16, bool WIDE>
+// FULL: the tile lies entirely inside the problem (64 rows, 32 units, every K slab), there is an
+// initial state and no reset mask - the decode steady state.  All clamping and masking is then
+// compiled out, which matters: the kernel is bound by the number of instructions a wave issues.
+// SLABCH = MFMA k-steps per slab.  With 4 (dh <= 128) or 8 (dh <= 256, bf16) the whole K range
+// is ONE slab: everything is staged once, one barrier, and the registers that carried the
+// loads are free again before the MFMA loop (which then batches its LDS reads).
+template <bool BF16, int SLABCH, bool FULL>
 __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
   constexpr int EPC = BF16 ? 8 : 4;
   constexpr int CHK = 4 * EPC;                // input units per MFMA k-step ("chunk")
-  constexpr int SLABCH = WIDE ? 2 : 1;        // chunks per slab
   constexpr int SLABK = SLABCH * CHK;         // input units per slab
+  constexpr int kStepRing = SLABCH >= 4 ? 1 : 4;  // slabs whose loads are in flight
+  constexpr int NBUF = SLABCH >= 4 ? 1 : 2;       // LDS buffers
   constexpr int RS = SLABCH * 64 + 16;        // bytes per LDS row: data + pad (conflict-free 16-byte reads)
   constexpr int HITEMS = (SLABK * 4 / 16) / 4;  // 16-byte pieces of fp32 h each thread stages per slab
   constexpr int RITEMS = SLABCH * 2;            // 16-byte pieces of R each thread stages per slab
   constexpr int ESZ = BF16 ? 2 : 4;
-  __shared__ __attribute__((aligned(16))) unsigned char hbuf[2][64 * RS];
-  __shared__ __attribute__((aligned(16))) unsigned char rbuf[2][128 * RS];
+  extern __shared__ __attribute__((aligned(16))) unsigned char step_lds[];
+  unsigned char(*hbuf)[64 * RS] = reinterpret_cast<unsigned char(*)[64 * RS]>(step_lds);
+  unsigned char(*rbuf)[128 * RS] = reinterpret_cast<unsigned char(*)[128 * RS]>(step_lds + NBUF * 64 * RS);
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
@@ -740,8 +747,8 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid < 16)
     reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
 
-  const bool has_s0 = p.s0 != nullptr;
-  const bool has_reset = p.reset != nullptr;
+  const bool has_s0 = FULL || p.s0 != nullptr;
+  const bool has_reset = !FULL && p.reset != nullptr;
   const float *s0p = has_s0 ? p.s0 : reinterpret_cast<const float *>(p.wx);                  // stand-ins are only read
   const unsigned char *rsp = has_reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);  // in their first 32 bytes
 
@@ -754,10 +761,15 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   for (int j = 0; j < HITEMS; ++j) {
     const int item = tid + 256 * j;
     const int brow = rowbase + item / HPIECES;
-    const int browc = brow < p.B ? brow : p.B - 1;
-    const uint32_t flag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
-    hzero[j] = !(brow < p.B) || !has_s0 || (has_reset && flag != 0u);
-    hsrc[j] = s0p + (has_s0 ? (long long)browc * H + head * dh : 0);
+    if (FULL) {
+      hzero[j] = false;
+      hsrc[j] = s0p + (long long)brow * H + head * dh + (item % HPIECES) * 4;
+    } else {
+      const int browc = brow < p.B ? brow : p.B - 1;
+      const uint32_t flag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+      hzero[j] = !(brow < p.B) || !has_s0 || (has_reset && flag != 0u);
+      hsrc[j] = s0p + (has_s0 ? (long long)browc * H + head * dh : 0);
+    }
   }
   const char *rsrc[RITEMS];
   bool rok[RITEMS];
@@ -765,22 +777,31 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   for (int j = 0; j < RITEMS; ++j) {
     const int colx = (tid + 256 * j) / RPIECES;   // column of the workgroup's 128: gate colx/32, unit colx%32
     const int a = a0 + (colx & 31);
-    rok[j] = a < dh;
+    rok[j] = FULL || a < dh;
     rsrc[j] = reinterpret_cast<const char *>(p.r) +
-              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * ESZ;
+              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * ESZ +
+              (FULL ? ((tid + 256 * j) % RPIECES) * 16 : 0);
   }
   uint4 hring[kStepRing][HITEMS], rring[kStepRing][RITEMS];
   auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS]) {
     const int kbase = sidx * SLABK;
 #pragma unroll
     for (int j = 0; j < HITEMS; ++j) {
-      const int k = kbase + ((tid + 256 * j) % HPIECES) * 4;
-      hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
+      if (FULL) {
+        hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase);
+      } else {
+        const int k = kbase + ((tid + 256 * j) % HPIECES) * 4;
+        hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
+      }
     }
 #pragma unroll
     for (int j = 0; j < RITEMS; ++j) {
-      const int k = kbase + ((tid + 256 * j) % RPIECES) * EPC;
-      rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
+      if (FULL) {
+        rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + kbase * ESZ);
+      } else {
+        const int k = kbase + ((tid + 256 * j) % RPIECES) * EPC;
+        rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
+      }
     }
   };
   auto store_slab = [&](int sidx, int buf, const uint4 (&hst)[HITEMS], const uint4 (&rst)[RITEMS]) {
@@ -789,9 +810,8 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
     for (int j = 0; j < HITEMS; ++j) {
       const int item = tid + 256 * j;
       const int piece = item % HPIECES;
-      const bool z = hzero[j] || kbase + piece * 4 >= dh;
       uint4 v = hst[j];
-      if (z) v = make_uint4(0, 0, 0, 0);
+      if (!FULL && (hzero[j] || kbase + piece * 4 >= dh)) v = make_uint4(0, 0, 0, 0);
       unsigned char *dst = &hbuf[buf][(item / HPIECES) * RS];
       if (BF16) {
         uint2 w;
@@ -807,31 +827,36 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
       const int item = tid + 256 * j;
       const int piece = item % RPIECES;
       uint4 w = rst[j];
-      if (!rok[j] || kbase + piece * EPC >= dh) w = make_uint4(0, 0, 0, 0);
+      if (!FULL && (!rok[j] || kbase + piece * EPC >= dh)) w = make_uint4(0, 0, 0, 0);
       *reinterpret_cast<uint4 *>(&rbuf[buf][(item / RPIECES) * RS + piece * 16]) = w;
     }
   };
 
+#ifdef XS_PROFILE
+  long long pstamp[6];
+  pstamp[0] = clock64();
+#endif
 #pragma unroll
   for (int u = 0; u < kStepRing; ++u)
     if (u < nslab) load_slab(u, hring[u], rring[u]);
 
   // ---- pointwise operands of this lane: batch row rowbase + 16*wave + r16, units a0 + ut*16 + 4q .. +3
   const int brow = rowbase + 16 * wave + r16;
-  const int browc = brow < p.B ? brow : p.B - 1;
-  const uint32_t pflag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+  const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
+  const uint32_t pflag = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
   uint2 wxb[2][4];
   float4 wxf[2][4], bias4[2][4], c4[2], n4[2], m4[2];
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
     const int ua = a0 + ut * 16 + 4 * q;
-    const long long col = (long long)head * dh + (ua < dh ? ua : 0);
+    const int uac = (FULL || ua < dh) ? ua : 0;
+    const long long col = (long long)head * dh + uac;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
       if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
       else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
-      bias4[ut][g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + (ua < dh ? ua : 0));
+      bias4[ut][g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
     }
     const long long so = (long long)browc * H + col;
     c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
@@ -846,14 +871,20 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #pragma unroll
     for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
 
+#ifdef XS_PROFILE
+  pstamp[1] = clock64();
+#endif
   store_slab(0, 0, hring[0], rring[0]);
   __syncthreads();
+#ifdef XS_PROFILE
+  pstamp[2] = clock64();
+#endif
   for (int s0i = 0; s0i < nslab; s0i += kStepRing) {
 #pragma unroll
     for (int u = 0; u < kStepRing; ++u) {
       const int sidx = s0i + u;
       if (sidx < nslab) {
-        const int buf = sidx & 1;
+        const int buf = sidx & (NBUF - 1);
 #pragma unroll
         for (int ch = 0; ch < SLABCH; ++ch) {
           const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[buf][(16 * wave + r16) * RS + ch * 64 + q * 16]);
@@ -872,30 +903,36 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
                   acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
               }
             }
-        }
-        const int chunks_done = (sidx + 1) * SLABCH;
-        if ((chunks_done & (nch - 1)) == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
+          const int chunks_done = sidx * SLABCH + ch + 1;
+          if ((chunks_done & (nch - 1)) == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
 #pragma unroll
-          for (int ut = 0; ut < 2; ++ut)
+            for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              tot[ut][g] = (chunks_done == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
-              acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            }
+              for (int g = 0; g < 4; ++g) {
+                tot[ut][g] = (chunks_done == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+                acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+              }
+          }
         }
         // slab sidx went to LDS one iteration ago: its ring entry takes the loads of slab sidx + kStepRing
         if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u]);
         if (sidx + 1 < nslab) {
           const int un = (u + 1) % kStepRing;
-          store_slab(sidx + 1, buf ^ 1, hring[un], rring[un]);  // the other buffer was last read before the previous barrier
+          store_slab(sidx + 1, (sidx + 1) & (NBUF - 1), hring[un], rring[un]);  // the other buffer was last read before the previous barrier
           __syncthreads();
         }
       }
     }
   }
 
+#ifdef XS_PROFILE
+  asm volatile("" :: "v"(tot[0][0][0]), "v"(tot[1][3][3]));
+  pstamp[3] = clock64();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  pstamp[4] = clock64();
+#endif
   // ---- gating
-  const bool reset_row = !has_s0 || (has_reset && pflag != 0u);
+  const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag != 0u));
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
     const int ua = a0 + ut * 16 + 4 * q;
@@ -923,7 +960,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
       slstm_pointwise_t<BF16>(raw[0], raw[1], raw[2], raw[3], st);
       yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
     }
-    if (brow < p.B && ua < dh) {
+    if (FULL || (brow < p.B && ua < dh)) {
       const long long o = (long long)brow * H + head * dh + ua;
       *reinterpret_cast<float4 *>(p.s_out + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
       *reinterpret_cast<float4 *>(p.s_out + BH + o) = make_float4(cv[0], cv[1], cv[2], cv[3]);
@@ -939,6 +976,14 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
       }
     }
   }
+#ifdef XS_PROFILE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (tid == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 1) {
+    pstamp[5] = clock64();
+    long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
+    for (int i = 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
+  }
+#endif
 }
 
 // ---------------------------------------------------------------------------
@@ -1054,14 +1099,23 @@ int run_step(const xs_slstm_args *a) {
   if (grid.y > 65535 || grid.z > 65535) return fail(XS_ERR_UNSUPPORTED, "batch or head count too large for one step launch");
   int nch_log2 = 0;
   while ((1 << nch_log2) < nch) ++nch_log2;
-  const bool wide = nch >= 2;  // two k-steps per slab: every staged row / column is a whole 128-byte line
-  if (bf16) {
-    if (wide) hipLaunchKernelGGL((slstm_step_tile_kernel<true, true>), grid, dim3(256), 0, stream, p, nch_log2);
-    else hipLaunchKernelGGL((slstm_step_tile_kernel<true, false>), grid, dim3(256), 0, stream, p, nch_log2);
-  } else {
-    if (wide) hipLaunchKernelGGL((slstm_step_tile_kernel<false, true>), grid, dim3(256), 0, stream, p, nch_log2);
-    else hipLaunchKernelGGL((slstm_step_tile_kernel<false, false>), grid, dim3(256), 0, stream, p, nch_log2);
+  // steady-state decode: whole tiles, a state, no mask -> the variant without clamping
+  const bool full = a->s0 && !a->reset && B % 64 == 0 && dh % 32 == 0 && dh == nch * 16 * epc;
+  // slab width in MFMA k-steps: the whole K range when it fits LDS (dh <= 256 bf16 / 128 fp32)
+  const int slabch = nch == 1 ? 4 : (nch == 2 ? 8 : 2);
+  const int nbuf = slabch >= 4 ? 1 : 2;
+  const size_t lds = (size_t)nbuf * (64 + 128) * (slabch * 64 + 16);
+  typedef void (*StepKernel)(StepParams, int);
+  StepKernel kern;
+#define XS_PICK(BF, SC) (full ? slstm_step_tile_kernel<BF, SC, true> : slstm_step_tile_kernel<BF, SC, false>)
+  if (bf16) kern = slabch == 4 ? XS_PICK(true, 4) : (slabch == 8 ? XS_PICK(true, 8) : XS_PICK(true, 2));
+  else kern = slabch == 4 ? XS_PICK(false, 4) : (slabch == 8 ? XS_PICK(false, 8) : XS_PICK(false, 2));
+#undef XS_PICK
+  if (lds > 64 * 1024) {  // the single-slab variant at dh = 256 needs 99 KiB of the 160 KiB of LDS
+    const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(ea));
   }
+  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p, nch_log2);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
   return XS_OK;
