@@ -73,6 +73,36 @@ def main():
         )
         print(name, "out", tuple(out.shape), "state", tuple(st.shape))
 
+    # ---- sLSTMLayer (caller of the cell): conv1d + SiLU, headwise gate projections, cell, group norm
+    from xlstm.blocks.slstm.layer import sLSTMLayer, sLSTMLayerConfig  # noqa: E402
+
+    for name, D, NH, B, T, seed in (("layer_d64", 64, 4, 2, 10, 11), ("layer_d128", 128, 2, 3, 7, 12)):
+        torch.manual_seed(seed)
+        cfg = sLSTMLayerConfig(embedding_dim=D, num_heads=NH, conv1d_kernel_size=4, backend="vanilla",
+                               dtype="float32", recurrent_weight_init="standard", bias_init="small_init")
+        layer = sLSTMLayer(cfg)
+        layer.reset_parameters()
+        with torch.no_grad():
+            layer.slstm_cell._recurrent_kernel_.mul_(6.0)
+            layer.group_norm.weight.normal_(0.0, 0.3)
+            for g in (layer.igate, layer.fgate, layer.zgate, layer.ogate):
+                g.weight.mul_(4.0)  # make the gate wiring (which module feeds which slot) matter
+        x = torch.randn(B, T, D)
+        with torch.no_grad():
+            out = layer(x)
+        np.savez(
+            os.path.join(OUT, f"{name}.npz"),
+            x=x.numpy(), out=out.numpy(),
+            conv_weight=layer.conv1d.conv.weight.detach().numpy(), conv_bias=layer.conv1d.conv.bias.detach().numpy(),
+            fgate=layer.fgate.weight.detach().numpy(), igate=layer.igate.weight.detach().numpy(),
+            zgate=layer.zgate.weight.detach().numpy(), ogate=layer.ogate.weight.detach().numpy(),
+            r_ext=layer.slstm_cell.recurrent_kernel[:].contiguous().numpy(),
+            b_ext=layer.slstm_cell.bias[:].contiguous().numpy(),
+            gn_weight=layer.group_norm.weight.detach().numpy(),
+            num_heads=np.array(NH),
+        )
+        print(name, "out", tuple(out.shape))
+
     # Notebook shape fixture (notebooks/xlstm/xLSTM_test_notebook.ipynb, cell 2):
     # zeros[4,4,512] through hidden=128, heads=2 -> out [4,2,4,64], state [4,4,128].
     torch.manual_seed(0)
