@@ -160,6 +160,40 @@ def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
             "aborted": F.read_status(ws)["aborted"]}
 
 
+def bench_config4(device, iters=3):
+    """BASELINE config 4: 24 blocks (sLSTM at 3, 11, 19), D=1024, 4 heads, vocab 50304, bf16, B=8, T=2048,
+    packed documents of mean length 768.  Only the sLSTM cells run on the HIP engine."""
+    import numpy as np
+    import torch
+
+    from tests._util import geometric_reset_mask
+    from xlstm_amd.lm_harness import HarnessConfig, xLSTMLMHarness
+
+    torch.manual_seed(4)
+    B, T = 8, 2048
+    model = xLSTMLMHarness(HarnessConfig()).to(device).bfloat16().eval()
+    idx = torch.randint(0, 50304, (B, T), device=device)
+    mask = torch.from_numpy(geometric_reset_mask(4, B, T, 768)).to(device)
+    total, cells = [], []
+    with torch.no_grad():
+        for i in range(iters + 1):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            logits = model(idx, reset_mask=mask, time_cells=True)
+            e1.record()
+            torch.cuda.synchronize()
+            if i:
+                total.append(e0.elapsed_time(e1))
+                cells.append(list(model.cell_ms))
+    cell_ms = np.median(np.array(cells), axis=0)
+    return {"workload": "config 4: 24-block xLSTM LM harness, sLSTM cells at blocks 3/11/19 on HIP, rest PyTorch-ROCm, "
+                        "B=8 T=2048 D=1024 NH=4 bf16, documents mean 768",
+            "forward_ms": float(np.median(total)), "slstm_cell_ms": [float(c) for c in cell_ms],
+            "slstm_cells_share": float(cell_ms.sum() / np.median(total)),
+            "slstm_tokens_per_s_per_cell": float(B * T / cell_ms.mean() * 1e3),
+            "finite": bool(torch.isfinite(logits.float()).all())}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,6 +204,8 @@ def main():
     ap.add_argument("--decode-only", action="store_true", help="only run the decode leg (profiling runs)")
     ap.add_argument("--all-configs", action="store_true",
                     help="also time the cell at BASELINE configs 1, 4 and 5 (adds an 'all_configs' object)")
+    ap.add_argument("--config4", action="store_true",
+                    help="also run BASELINE config 4: the 24-block LM harness, timing its three sLSTM cells")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -257,6 +293,8 @@ def main():
             bench_config(device, "config 4 (one sLSTM cell): B=8 T=2048 D=1024 NH=4 bf16, documents mean 768", 8, 2048, 4, 256, True, 768),
             bench_config(device, "config 5: B=64 T=4096 D=4096 NH=4 bf16, no resets", 64, 4096, 4, 1024, True, 0, iters=2),
         ]
+    if args.config4:
+        out["config4"] = bench_config4(device)
     if not args.no_decode:
         out["decode"] = bench_decode(device)
     if not args.no_cpu_baseline:
