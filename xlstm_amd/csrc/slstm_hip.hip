@@ -879,6 +879,41 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #ifdef XS_PROFILE
   pstamp[2] = clock64();
 #endif
+  if (SLABCH >= 4) {
+    // single slab: the whole K range is in LDS after one barrier, and the number of chunks per
+    // K quarter is the compile-time constant SLABCH / 4 -> straight-line MFMA code
+    constexpr int NQ = SLABCH / 4;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+#pragma unroll
+      for (int cq = 0; cq < (NQ > 0 ? NQ : 1); ++cq) {
+        const int ch = w * NQ + cq;
+        const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[0][(16 * wave + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + ut * 16 + r16) * RS + ch * 64 + q * 16]);
+            if (BF16) {
+              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
+            } else {
+              const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
+              const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+            }
+          }
+      }
+#pragma unroll
+      for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {  // fold the quarter into the running sum (quarter 0 first)
+          tot[ut][g] = (w == 0) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+          acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+  } else {
   for (int s0i = 0; s0i < nslab; s0i += kStepRing) {
 #pragma unroll
     for (int u = 0; u < kStepRing; ++u) {
@@ -925,6 +960,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
     }
   }
 
+  }
 #ifdef XS_PROFILE
   asm volatile("" :: "v"(tot[0][0][0]), "v"(tot[1][3][3]));
   pstamp[3] = clock64();
