@@ -706,8 +706,31 @@ struct StepParams {
   float *s_out;
   xs_slstm_status *status;
   int B, NH, dh;
+  int n_unit_tiles, n_row_tiles;
 };
 
+// Workgroup i runs on XCD i % 8.  The workgroups of one head share its h rows and its R, so they
+// are placed on as few XCDs as possible (one when there are 8 or more heads): every operand is
+// then fetched from HBM once and re-read from ONE L2 instead of being fetched by all eight.
+__device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &head, int &ut, int &rt) {
+  const int tiles = p.n_unit_tiles * p.n_row_tiles;
+  int tile;
+  if (p.NH % 8 == 0) {
+    const int hpx = p.NH / 8;  // heads per XCD
+    const int m = i >> 3;
+    head = (i & 7) * hpx + m % hpx;
+    tile = m / hpx;
+  } else if (8 % p.NH == 0 && tiles % (8 / p.NH) == 0) {
+    const int xph = 8 / p.NH;  // XCDs per head
+    head = (i & 7) % p.NH;
+    tile = (i >> 3) * xph + (i & 7) / p.NH;
+  } else {
+    head = i / tiles;
+    tile = i - head * tiles;
+  }
+  ut = tile % p.n_unit_tiles;
+  rt = tile / p.n_unit_tiles;
+}
 
 // FULL: the tile lies entirely inside the problem (64 rows, 32 units, every K slab), there is an
 // initial state and no reset mask - the decode steady state.  All clamping and masking is then
@@ -735,16 +758,17 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const int lane = tid & 63;
   const int q = lane >> 4;
   const int r16 = lane & 15;
-  const int head = blockIdx.z;
-  const int a0 = blockIdx.x * 32;
-  const int rowbase = blockIdx.y * 64;
+  int head, unit_tile, row_tile;
+  step_tile_of(p, blockIdx.x, head, unit_tile, row_tile);
+  const int a0 = unit_tile * 32;
+  const int rowbase = row_tile * 64;
   const int dh = p.dh;
   const int H = p.NH * dh;
   const long long BH = (long long)p.B * H;
   const int nch = 1 << nch_log2;              // chunks per K quarter (as in the sequence kernel)
   const int nslab = (4 * nch) / SLABCH;
 
-  if (blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0 && tid < 16)
+  if (blockIdx.x == 0 && tid < 16)
     reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
 
   const bool has_s0 = FULL || p.s0 != nullptr;
@@ -1014,7 +1038,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   }
 #ifdef XS_PROFILE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (tid == 0 && blockIdx.x == 1 && blockIdx.y == 1 && blockIdx.z == 1) {
+  if (tid == 0 && blockIdx.x == 9) {
     pstamp[5] = clock64();
     long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
     for (int i = 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
@@ -1131,8 +1155,11 @@ int run_step(const xs_slstm_args *a) {
   p.h_out = a->h_out; p.s_out = a->s_out;
   p.status = (xs_slstm_status *)a->workspace;
   p.B = B; p.NH = NH; p.dh = dh;
-  const dim3 grid((dh + 31) / 32, (B + 63) / 64, NH);
-  if (grid.y > 65535 || grid.z > 65535) return fail(XS_ERR_UNSUPPORTED, "batch or head count too large for one step launch");
+  p.n_unit_tiles = (dh + 31) / 32;
+  p.n_row_tiles = (B + 63) / 64;
+  const long long nwg = (long long)NH * p.n_unit_tiles * p.n_row_tiles;
+  if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
+  const dim3 grid((unsigned)nwg);
   int nch_log2 = 0;
   while ((1 << nch_log2) < nch) ++nch_log2;
   // steady-state decode: whole tiles, a state, no mask -> the variant without clamping
