@@ -116,12 +116,54 @@ def bench_decode(device, steps=1024, prefill=128):
     wall = time.perf_counter() - t0
     gpu_us = e0.elapsed_time(e1) * 1e3 / steps
     nbytes = algorithmic_bytes(B, 1, NH, dh, 2, 2, 2, with_mask=False) + 4 * B * H * 4  # state is read AND written
+    eager_state = s_a.clone()
+
+    # The same steps replayed from a HIP graph (64 step launches per graph, no host work between them):
+    # what a serving loop that captures its decode step sees.  Every replay is checked against the eager run.
+    per_graph = 64
+    graph_us, graph_ok = None, None
+    if steps % per_graph == 0:
+        g_a, g_b = state.clone(), torch.empty_like(state)
+        wx_g = torch.empty(per_graph, B, 1, 4 * H, dtype=wx_dec.dtype, device=device)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.stream(side):
+            def chain():
+                a, b = g_a, g_b
+                for t in range(per_graph):  # an even count: the state ends in g_a again
+                    F.slstm_forward(wx_g[t], r, bias, a, None, step=True, workspace=ws, h_out=h1, s_out=b)
+                    a, b = b, a
+            chain()  # warm-up outside the capture
+            torch.cuda.synchronize()
+            with torch.cuda.graph(graph, stream=side):
+                chain()
+        torch.cuda.synchronize()
+        g_a.copy_(state)
+        g0, g1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        total = 0.0
+        for rep in range(steps // per_graph):
+            wx_g.copy_(wx_dec[rep * per_graph:(rep + 1) * per_graph])
+            g0.record()
+            graph.replay()
+            g1.record()
+            torch.cuda.synchronize()
+            total += g0.elapsed_time(g1)
+        graph_us = total * 1e3 / steps
+        graph_ok = bool(torch.equal(g_a, eager_state))
+    best_us = min(gpu_us, graph_us) if graph_us else gpu_us
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "traffic_step_cfg3.json")
+    if os.path.exists(traffic_file):
+        traffic = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
     return {
         "workload": f"decode B={B} D={H} NH={NH}, {steps} consecutive T=1 steps after a {prefill}-token prefill",
-        "us_per_step": wall * 1e6 / steps, "gpu_us_per_step": gpu_us, "steps": steps,
+        "us_per_step": wall * 1e6 / steps, "gpu_us_per_step": gpu_us, "graph_us_per_step": graph_us,
+        "graph_equals_eager": graph_ok, "steps": steps,
         "finite": bool(torch.isfinite(s_a).all()),
-        "roofline": {"bound": "hbm", "achieved": nbytes / (gpu_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": nbytes / (gpu_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": None},
+        "roofline": {"bound": "hbm", "achieved": nbytes / (best_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": nbytes / (best_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
+                     "kernel": "slstm_step_tile_kernel<bf16,SLABCH=8,FULL>", "algorithmic_bytes_per_launch": nbytes},
     }
 
 

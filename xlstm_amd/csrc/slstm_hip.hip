@@ -859,6 +859,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #ifdef XS_PROFILE
   long long pstamp[6];
   pstamp[0] = clock64();
+  const long long pwall0 = wall_clock64();
 #endif
 #pragma unroll
   for (int u = 0; u < kStepRing; ++u)
@@ -1042,6 +1043,11 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
     pstamp[5] = clock64();
     long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
     for (int i = 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
+  }
+  if (tid == 0) {
+    long long *wt = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 256);
+    wt[2 * blockIdx.x] = pwall0;
+    wt[2 * blockIdx.x + 1] = wall_clock64();
   }
 #endif
 }
