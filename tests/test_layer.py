@@ -107,3 +107,68 @@ def test_layer_packed_documents_equal_documents_alone_and_step_equals_forward():
             o, st = layer.step(x[:, t:t + 1], conv_state=conv_state, slstm_state=cell_state)
             conv_state, cell_state = st["conv_state"], st["slstm_state"]
             assert max_err(o[:, 0].cpu().numpy(), full[:, t].cpu().numpy()) <= 1e-5
+
+
+def test_conv_step_accepts_the_state_a_prefill_returns():
+    from xlstm_amd.layer import CausalConv1d
+
+    torch.manual_seed(2)
+    conv = CausalConv1d(5, 4)
+    x = torch.randn(2, 9, 5)
+    with torch.no_grad():
+        y = conv(x)
+        _, cs = conv(x[:, :5], return_last_state=True)  # [B, k-1, D], conv.py:126-127
+        st = cs
+        for t in range(5, 9):
+            yt, st = conv.step(x[:, t:t + 1], st)
+            np.testing.assert_allclose(yt[:, 0].numpy(), y[:, t].numpy(), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_prefill_then_steps_equals_one_forward(dtype):
+    """forward(x[:, :k], return_last_state=True) followed by step() per token = forward(x)."""
+    from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
+
+    torch.manual_seed(3)
+    dev = torch.device("cuda:0")
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=128, num_heads=4, backend="hip",
+                                        recurrent_weight_init="standard")).to(dev).to(dtype)
+    layer.slstm_cell.keep_state_fp32 = True
+    x = torch.randn(3, 12, 128, device=dev).to(dtype)
+    with torch.no_grad():
+        whole = layer(x)
+        pre, st = layer(x[:, :7], return_last_state=True)
+        outs = [pre]
+        for t in range(7, 12):
+            o, st = layer.step(x[:, t:t + 1], conv_state=st["conv_state"], slstm_state=st["slstm_state"])
+            outs.append(o)
+    tol = 1e-5 if dtype == torch.float32 else 2e-2
+    assert max_err(torch.cat(outs, 1).float().cpu().numpy(), whole.float().cpu().numpy()) <= tol
+
+
+@pytest.mark.gpu
+def test_graphed_decoder_replays_equal_eager_steps():
+    """Two alternating HIP graphs of layer.step against the eager loop, with host work between replays."""
+    from xlstm_amd.decode import GraphedLayerDecoder
+    from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
+
+    torch.manual_seed(4)
+    dev = torch.device("cuda:0")
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=4, backend="hip",
+                                        recurrent_weight_init="standard")).to(dev).bfloat16()
+    layer.slstm_cell.keep_state_fp32 = True
+    B = 8
+    x = torch.randn(B, 16, 256, device=dev).bfloat16()
+    with torch.no_grad():
+        _, st0 = layer(x[:, :5], return_last_state=True)
+        dec = GraphedLayerDecoder(layer, B)
+        for trial in range(2):  # the second pass re-uses the graphs after a state reload
+            dec.load_state(st0["conv_state"], st0["slstm_state"])
+            st = st0
+            for t in range(5, 16):
+                want, st = layer.step(x[:, t:t + 1], conv_state=st["conv_state"], slstm_state=st["slstm_state"])
+                got = dec.step(x[:, t:t + 1])
+                torch.cuda.synchronize()
+                assert torch.equal(got, want), (trial, t)
+                assert torch.equal(dec.state()["slstm_state"], st["slstm_state"]), (trial, t)

@@ -331,7 +331,7 @@ class sLSTMCell_hip(nn.Module):
             object.__setattr__(self, "_r_bf16_cache", cache)
         return cache[1]
 
-    def _run(self, input, state, reset_mask, step: bool):
+    def _run(self, input, state, reset_mask, step: bool, state_out=None):
         self._check_input(input)
         x = self._input_bs(input)
         B = x.shape[0]
@@ -351,6 +351,7 @@ class sLSTMCell_hip(nn.Module):
             state,
             reset_mask,
             step=step,
+            s_out=state_out,
         )
         if torch.is_grad_enabled() and (
             input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
@@ -369,11 +370,18 @@ class sLSTMCell_hip(nn.Module):
         del lengths  # unused, as in the reference
         return self._run(input, state, reset_mask, step=False)
 
-    def step(self, input: torch.Tensor, state: Optional[torch.Tensor] = None, reset_mask=None):
+    def step(self, input: torch.Tensor, state: Optional[torch.Tensor] = None, reset_mask=None,
+             state_out: Optional[torch.Tensor] = None):
         """One decode step (S == 1) through the step kernel.  Unlike the reference's
         ``step`` (cell.py:486-494, which hands back the state it was given) this
-        returns the NEW state."""
-        return self._run(input, state, reset_mask, step=True)
+        returns the NEW state.  ``state_out`` (float32 [4,B,H], not overlapping ``state``)
+        receives it without an allocation, for decode loops that alternate two buffers."""
+        if state_out is not None:
+            B = self._input_bs(input).shape[0]
+            if state_out.dtype != torch.float32 or not state_out.is_contiguous() or tuple(state_out.shape) != (
+                    self.config.num_states, B, self.config.hidden_size):
+                raise ValueError("state_out must be a contiguous float32 [4, B, H] tensor")
+        return self._run(input, state, reset_mask, step=True, state_out=state_out)
 
 
 class sLSTMCell:

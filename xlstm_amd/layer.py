@@ -91,13 +91,19 @@ class CausalConv1d(nn.Module):
             y = y + self.conv.bias
         return y
 
-    def step(self, x: torch.Tensor, conv_state: Optional[tuple] = None):
-        """One token, ring state [B,k,D] in a 1-tuple as in conv.py:131-157."""
+    def step(self, x: torch.Tensor, conv_state=None):
+        """One token, ring state [B,k,D] in a 1-tuple as in conv.py:131-157.  Also accepted: the
+        bare [B,k-1,D] tensor that ``forward(..., return_last_state=True)`` hands back
+        (conv.py:126-127), so that a prefill can be followed by steps."""
         B, S, D = x.shape
         assert S == 1, f"x has sequence length {S} but it should be 1"
         if conv_state is None:
             conv_state = (torch.zeros(B, self.kernel_size, D, device=x.device, dtype=x.dtype),)
-        state = torch.roll(conv_state[0], shifts=-1, dims=1)
+        prev = conv_state[0] if isinstance(conv_state, (tuple, list)) else conv_state
+        if prev.shape[1] == self.kernel_size - 1:
+            prev = F.pad(prev, (0, 0, 1, 0))  # the oldest slot is dropped by the roll below
+        assert prev.shape[1] == self.kernel_size, f"conv state holds {prev.shape[1]} inputs, expected {self.kernel_size}"
+        state = torch.roll(prev, shifts=-1, dims=1)
         state[:, -1:, :] = x
         y = torch.sum(state * self.conv.weight[:, 0, :].transpose(0, 1), dim=1, keepdim=True)
         if self.conv.bias is not None:
@@ -188,14 +194,16 @@ class sLSTMLayer(nn.Module):
             return out, {"conv_state": conv_state, "slstm_state": slstm_state}
         return out
 
-    def step(self, x: torch.Tensor, conv_state: Optional[tuple] = None, slstm_state: Optional[torch.Tensor] = None):
+    def step(self, x: torch.Tensor, conv_state: Optional[tuple] = None, slstm_state: Optional[torch.Tensor] = None,
+             slstm_state_out: Optional[torch.Tensor] = None):
+        """One token (layer.py:92-121).  ``slstm_state_out`` is handed to the cell's ``step``."""
         B, S, _ = x.shape
         if self.config.conv1d_kernel_size > 0:
             x_conv, conv_state = self.conv1d.step(x, conv_state=conv_state)
             x_conv = self.conv_act_fn(x_conv)
         else:
             x_conv = x
-        y, slstm_state = self.slstm_cell.step(self._gates(x, x_conv), slstm_state)
+        y, slstm_state = self.slstm_cell.step(self._gates(x, x_conv), slstm_state, state_out=slstm_state_out)
         y = self.dropout(y)
         out = self.group_norm(y).transpose(1, 2).reshape(B, S, -1)
         return out, {"conv_state": conv_state, "slstm_state": slstm_state}
