@@ -103,6 +103,8 @@ def main():
         )
         print(name, "out", tuple(out.shape))
 
+    write_checkpoint_layouts()
+
     # Notebook shape fixture (notebooks/xlstm/xLSTM_test_notebook.ipynb, cell 2):
     # zeros[4,4,512] through hidden=128, heads=2 -> out [4,2,4,64], state [4,4,128].
     torch.manual_seed(0)
@@ -113,5 +115,33 @@ def main():
     assert tuple(out.shape) == (4, 2, 4, 64) and tuple(st.shape) == (4, 4, 128)
 
 
+def write_checkpoint_layouts():
+    """The same external parameters as each reference backend stores them (its ``state_dict``
+    tensors ``_recurrent_kernel_`` / ``_bias_``): what a checkpoint written with backend
+    "vanilla" or "cuda" holds.  The cuda cell is built with ``skip_backend_init=True`` as in
+    the reference's own doctests (cell.py:712-716), so nothing is compiled."""
+    sys.path.insert(0, REF)
+    from xlstm.blocks.slstm.cell import sLSTMCell_cuda, sLSTMCell_vanilla, sLSTMCellConfig  # noqa: E402
+
+    torch.manual_seed(21)
+    hidden, heads = 48, 3
+    r_ext = torch.randn(heads, hidden // heads, 4, hidden // heads)
+    b_ext = torch.randn(heads, 4, hidden // heads)
+    out = {"r_ext": r_ext.numpy(), "b_ext": b_ext.numpy(), "num_heads": np.array(heads)}
+    for backend, cls in (("vanilla", sLSTMCell_vanilla), ("cuda", sLSTMCell_cuda)):
+        cell = cls(sLSTMCellConfig(hidden_size=hidden, num_heads=heads, backend=backend, dtype="float32"),
+                   skip_backend_init=True)
+        cell.recurrent_kernel[:] = r_ext
+        cell.bias[:] = b_ext
+        sd = cell.state_dict()
+        out[f"r_{backend}"] = sd["_recurrent_kernel_"].contiguous().numpy()
+        out[f"b_{backend}"] = sd["_bias_"].contiguous().numpy()
+        print("checkpoint layout", backend, out[f"r_{backend}"].shape, out[f"b_{backend}"].shape)
+    np.savez(os.path.join(OUT, "ckpt_layouts.npz"), **out)
+
+
 if __name__ == "__main__":
-    main()
+    if len(sys.argv) > 1 and sys.argv[1] == "--checkpoint-layouts-only":
+        write_checkpoint_layouts()
+    else:
+        main()

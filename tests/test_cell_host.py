@@ -103,3 +103,36 @@ def test_bad_input_size_and_cpu_tensor_fail_loudly():
 
 def test_state_dict_names_match_reference():
     assert set(_cell().state_dict().keys()) == {"_recurrent_kernel_", "_bias_"}
+
+
+def test_reference_checkpoint_layouts_convert_to_hip():
+    """Internal tensors as the reference's vanilla and cuda cells store them (fixture written from
+    those classes) land in the hip cell with the same EXTERNAL view."""
+    import os
+
+    import numpy as np
+    import torch
+
+    from xlstm_amd.cell import reference_cell_params_to_hip, reference_state_dict_to_hip, sLSTMCell, sLSTMCellConfig
+
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "ckpt_layouts.npz"))
+    NH = int(z["num_heads"])
+    r_ext, b_ext = torch.from_numpy(z["r_ext"]), torch.from_numpy(z["b_ext"])
+    for backend in ("vanilla", "cuda"):
+        cell = sLSTMCell(sLSTMCellConfig(hidden_size=r_ext.shape[0] * r_ext.shape[1], num_heads=NH, backend="hip",
+                                         dtype="float32"), skip_backend_init=True)
+        sd = {"slstm_cell._recurrent_kernel_": torch.from_numpy(z[f"r_{backend}"]),
+              "slstm_cell._bias_": torch.from_numpy(z[f"b_{backend}"]), "other.weight": torch.ones(2)}
+        conv = reference_state_dict_to_hip(sd, backend, NH)
+        assert conv["other.weight"] is sd["other.weight"]
+        cell.load_state_dict({"_recurrent_kernel_": conv["slstm_cell._recurrent_kernel_"],
+                              "_bias_": conv["slstm_cell._bias_"]})
+        assert torch.equal(cell.recurrent_kernel[:], r_ext), backend
+        assert torch.equal(cell.bias[:], b_ext), backend
+    # the two source layouts really differ from each other (the fixture is not vacuous)
+    assert z["r_vanilla"].shape != z["r_cuda"].shape and not np.array_equal(z["b_vanilla"], z["b_cuda"])
+    import pytest
+    with pytest.raises(ValueError):
+        reference_cell_params_to_hip(torch.from_numpy(z["r_cuda"]), torch.from_numpy(z["b_cuda"]), "vanilla", NH)
+    with pytest.raises(ValueError):
+        reference_cell_params_to_hip(torch.from_numpy(z["r_cuda"]), torch.from_numpy(z["b_cuda"]), "triton", NH)

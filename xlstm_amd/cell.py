@@ -384,6 +384,43 @@ class sLSTMCell_hip(nn.Module):
         return self._run(input, state, reset_mask, step=True, state_out=state_out)
 
 
+def reference_cell_params_to_hip(recurrent_kernel_int: torch.Tensor, bias_int: torch.Tensor, source_backend: str,
+                                 num_heads: int):
+    """``_recurrent_kernel_`` / ``_bias_`` as a reference checkpoint of backend ``source_backend``
+    stores them -> the hip cell's layouts (R ``[NH, 4dh, dh]``, bias ``[4H]`` head-major).
+
+    vanilla keeps R as ``[NH, 4dh, dh]`` (cell.py:601-617, the hip layout) and the bias gate-major
+    (cell.py:635-642); cuda keeps R as ``[NH, dh, 4dh]`` (cell.py:694-706) and the bias head-major
+    (cell.py:726-733, the hip layout)."""
+    NH = num_heads
+    if source_backend == "hip":
+        return recurrent_kernel_int, bias_int
+    if source_backend == "vanilla":
+        if recurrent_kernel_int.dim() != 3 or recurrent_kernel_int.shape[1] != 4 * recurrent_kernel_int.shape[2]:
+            raise ValueError(f"a vanilla checkpoint holds R as [NH, 4*dh, dh], got {tuple(recurrent_kernel_int.shape)}")
+        dh = recurrent_kernel_int.shape[2]
+        return recurrent_kernel_int, bias_int.reshape(4, NH, dh).permute(1, 0, 2).reshape(-1)
+    if source_backend == "cuda":
+        if recurrent_kernel_int.dim() != 3 or recurrent_kernel_int.shape[2] != 4 * recurrent_kernel_int.shape[1]:
+            raise ValueError(f"a cuda checkpoint holds R as [NH, dh, 4*dh], got {tuple(recurrent_kernel_int.shape)}")
+        return recurrent_kernel_int.permute(0, 2, 1).contiguous(), bias_int
+    raise ValueError(f'unknown source backend {source_backend!r}, choose from ["vanilla", "cuda", "hip"]')
+
+
+def reference_state_dict_to_hip(state_dict: dict, source_backend: str, num_heads: int) -> dict:
+    """A state dict of any module that contains reference sLSTM cells (a cell, an ``sLSTMLayer``,
+    a block stack) with every ``..._recurrent_kernel_`` / ``..._bias_`` pair rewritten for the hip
+    cell; all other entries pass through untouched."""
+    out = dict(state_dict)
+    for key in state_dict:
+        if key.endswith("_recurrent_kernel_"):
+            bkey = key[: -len("_recurrent_kernel_")] + "_bias_"
+            if bkey not in state_dict:
+                raise KeyError(f"{key} has no matching {bkey}")
+            out[key], out[bkey] = reference_cell_params_to_hip(state_dict[key], state_dict[bkey], source_backend, num_heads)
+    return out
+
+
 class sLSTMCell:
     """Backend switch (cell.py:777-788).  This package implements ``"hip"``."""
 
