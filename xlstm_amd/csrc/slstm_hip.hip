@@ -776,18 +776,26 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const float *s0p = has_s0 ? p.s0 : reinterpret_cast<const float *>(p.wx);                  // stand-ins are only read
   const unsigned char *rsp = has_reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);  // in their first 32 bytes
 
-  // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row / column
+  // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row / column.
+  // A single slab is staged in NSPLIT phases (K halves): a thread's first HITEMS / NSPLIT items
+  // lie in the first half of K, so the MFMA loop can start on it while the second half lands.
   constexpr int HPIECES = SLABK * 4 / 16;     // 16-byte pieces of fp32 h per row and slab
   constexpr int RPIECES = SLABCH * 4;         // 16-byte pieces of R per column and slab
+  constexpr int NSPLIT = SLABCH >= 4 ? 2 : 1;
+  constexpr int HPP = HPIECES / NSPLIT, HIP = HITEMS / NSPLIT;  // pieces per row, items per thread: per phase
+  constexpr int RPP = RPIECES / NSPLIT, RIP = RITEMS / NSPLIT;
+  auto hrow_of = [&](int j) { return (tid + 256 * (j % HIP)) / HPP; };
+  auto hpiece_of = [&](int j) { return (j / HIP) * HPP + (tid + 256 * (j % HIP)) % HPP; };
+  auto rcol_of = [&](int j) { return (tid + 256 * (j % RIP)) / RPP; };
+  auto rpiece_of = [&](int j) { return (j / RIP) * RPP + (tid + 256 * (j % RIP)) % RPP; };
   const float *hsrc[HITEMS];
   bool hzero[HITEMS];
 #pragma unroll
   for (int j = 0; j < HITEMS; ++j) {
-    const int item = tid + 256 * j;
-    const int brow = rowbase + item / HPIECES;
+    const int brow = rowbase + hrow_of(j);
     if (FULL) {
       hzero[j] = false;
-      hsrc[j] = s0p + (long long)brow * H + head * dh + (item % HPIECES) * 4;
+      hsrc[j] = s0p + (long long)brow * H + head * dh + hpiece_of(j) * 4;
     } else {
       const int browc = brow < p.B ? brow : p.B - 1;
       const uint32_t flag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
@@ -799,44 +807,48 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   bool rok[RITEMS];
 #pragma unroll
   for (int j = 0; j < RITEMS; ++j) {
-    const int colx = (tid + 256 * j) / RPIECES;   // column of the workgroup's 128: gate colx/32, unit colx%32
+    const int colx = rcol_of(j);                  // column of the workgroup's 128: gate colx/32, unit colx%32
     const int a = a0 + (colx & 31);
     rok[j] = FULL || a < dh;
     rsrc[j] = reinterpret_cast<const char *>(p.r) +
               ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * ESZ +
-              (FULL ? ((tid + 256 * j) % RPIECES) * 16 : 0);
+              (FULL ? rpiece_of(j) * 16 : 0);
   }
   uint4 hring[kStepRing][HITEMS], rring[kStepRing][RITEMS];
   auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS]) {
     const int kbase = sidx * SLABK;
 #pragma unroll
-    for (int j = 0; j < HITEMS; ++j) {
-      if (FULL) {
-        hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase);
-      } else {
-        const int k = kbase + ((tid + 256 * j) % HPIECES) * 4;
-        hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
-      }
-    }
+    for (int ph = 0; ph < NSPLIT; ++ph) {
 #pragma unroll
-    for (int j = 0; j < RITEMS; ++j) {
-      if (FULL) {
-        rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + kbase * ESZ);
-      } else {
-        const int k = kbase + ((tid + 256 * j) % RPIECES) * EPC;
-        rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
+      for (int j = ph * HIP; j < (ph + 1) * HIP; ++j) {
+        if (FULL) {
+          hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase);
+        } else {
+          const int k = kbase + hpiece_of(j) * 4;
+          hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
+        }
+      }
+#pragma unroll
+      for (int j = ph * RIP; j < (ph + 1) * RIP; ++j) {
+        if (FULL) {
+          rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + kbase * ESZ);
+        } else {
+          const int k = kbase + rpiece_of(j) * EPC;
+          rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
+        }
       }
     }
   };
-  auto store_slab = [&](int sidx, int buf, const uint4 (&hst)[HITEMS], const uint4 (&rst)[RITEMS]) {
+  // phase < 0: the whole slab; otherwise the items of that K phase only
+  auto store_slab = [&](int sidx, int buf, const uint4 (&hst)[HITEMS], const uint4 (&rst)[RITEMS], int phase) {
     const int kbase = sidx * SLABK;
 #pragma unroll
     for (int j = 0; j < HITEMS; ++j) {
-      const int item = tid + 256 * j;
-      const int piece = item % HPIECES;
+      if (phase >= 0 && j / HIP != phase) continue;
+      const int piece = hpiece_of(j);
       uint4 v = hst[j];
       if (!FULL && (hzero[j] || kbase + piece * 4 >= dh)) v = make_uint4(0, 0, 0, 0);
-      unsigned char *dst = &hbuf[buf][(item / HPIECES) * RS];
+      unsigned char *dst = &hbuf[buf][hrow_of(j) * RS];
       if (BF16) {
         uint2 w;
         w.x = pack_bf16x2(__uint_as_float(v.x), __uint_as_float(v.y));
@@ -848,11 +860,11 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
     }
 #pragma unroll
     for (int j = 0; j < RITEMS; ++j) {
-      const int item = tid + 256 * j;
-      const int piece = item % RPIECES;
+      if (phase >= 0 && j / RIP != phase) continue;
+      const int piece = rpiece_of(j);
       uint4 w = rst[j];
       if (!FULL && (!rok[j] || kbase + piece * EPC >= dh)) w = make_uint4(0, 0, 0, 0);
-      *reinterpret_cast<uint4 *>(&rbuf[buf][(item / RPIECES) * RS + piece * 16]) = w;
+      *reinterpret_cast<uint4 *>(&rbuf[buf][rcol_of(j) * RS + piece * 16]) = w;
     }
   };
 
@@ -899,17 +911,21 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #ifdef XS_PROFILE
   pstamp[1] = clock64();
 #endif
-  store_slab(0, 0, hring[0], rring[0]);
+  store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
   __syncthreads();
 #ifdef XS_PROFILE
   pstamp[2] = clock64();
 #endif
   if (SLABCH >= 4) {
-    // single slab: the whole K range is in LDS after one barrier, and the number of chunks per
-    // K quarter is the compile-time constant SLABCH / 4 -> straight-line MFMA code
+    // single slab: the number of chunks per K quarter is the compile-time constant SLABCH / 4 ->
+    // straight-line MFMA code; the second K half goes to LDS after the MFMAs of the first
     constexpr int NQ = SLABCH / 4;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
+      if (w == 2) {
+        store_slab(0, 0, hring[0], rring[0], 1);
+        __syncthreads();
+      }
 #pragma unroll
       for (int cq = 0; cq < (NQ > 0 ? NQ : 1); ++cq) {
         const int ch = w * NQ + cq;
@@ -978,7 +994,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
         if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u]);
         if (sidx + 1 < nslab) {
           const int un = (u + 1) % kStepRing;
-          store_slab(sidx + 1, (sidx + 1) & (NBUF - 1), hring[un], rring[un]);  // the other buffer was last read before the previous barrier
+          store_slab(sidx + 1, (sidx + 1) & (NBUF - 1), hring[un], rring[un], -1);  // the other buffer was last read before the previous barrier
           __syncthreads();
         }
       }
