@@ -877,23 +877,30 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   for (int u = 0; u < kStepRing; ++u)
     if (u < nslab) load_slab(u, hring[u], rring[u]);
 
-  // ---- pointwise operands of this lane: batch row rowbase + 16*wave + r16, units a0 + ut*16 + 4q .. +3
-  const int brow = rowbase + 16 * wave + r16;
-  const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
-  const uint32_t pflag = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+  // ---- wave tiling 2 x 2: wave (wr, wu) owns rows 32*wr .. +31 (two MFMA row tiles, index ut below)
+  // and units 16*wu .. +15 of all four gates, so a k-step reads 2 h and 4 R fragments from LDS for
+  // its 8 MFMAs.  Pointwise operands of this lane: batch rows rowbase + 32*wr + 16*ut + r16,
+  // units a0 + 16*wu + 4q .. +3.
+  const int wr = wave >> 1, wu = wave & 1;
+  const int ua = a0 + wu * 16 + 4 * q;
+  const int uac = (FULL || ua < dh) ? ua : 0;
+  const long long col = (long long)head * dh + uac;
   uint2 wxb[2][4];
-  float4 wxf[2][4], bias4[2][4], c4[2], n4[2], m4[2];
+  float4 wxf[2][4], bias4[4], c4[2], n4[2], m4[2];
+  uint32_t pflag[2];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+    bias4[g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
-    const int ua = a0 + ut * 16 + 4 * q;
-    const int uac = (FULL || ua < dh) ? ua : 0;
-    const long long col = (long long)head * dh + uac;
+    const int brow = rowbase + 32 * wr + 16 * ut + r16;
+    const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
+    pflag[ut] = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
       if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
       else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
-      bias4[ut][g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
     }
     const long long so = (long long)browc * H + col;
     c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
@@ -929,17 +936,22 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #pragma unroll
       for (int cq = 0; cq < (NQ > 0 ? NQ : 1); ++cq) {
         const int ch = w * NQ + cq;
-        const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[0][(16 * wave + r16) * RS + ch * 64 + q * 16]);
+        uint4 hv[2], rv[4];
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut)
+          hv[ut] = *reinterpret_cast<const uint4 *>(&hbuf[0][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          rv[g] = *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
 #pragma unroll
         for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
-            const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + ut * 16 + r16) * RS + ch * 64 + q * 16]);
             if (BF16) {
-              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
+              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
             } else {
-              const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
-              const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+              const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w};
+              const uint32_t hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
 #pragma unroll
               for (int e = 0; e < 4; ++e)
                 acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
@@ -963,17 +975,22 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
         const int buf = sidx & (NBUF - 1);
 #pragma unroll
         for (int ch = 0; ch < SLABCH; ++ch) {
-          const uint4 hv = *reinterpret_cast<const uint4 *>(&hbuf[buf][(16 * wave + r16) * RS + ch * 64 + q * 16]);
+          uint4 hv[2], rv[4];
+#pragma unroll
+          for (int ut = 0; ut < 2; ++ut)
+            hv[ut] = *reinterpret_cast<const uint4 *>(&hbuf[buf][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            rv[g] = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
 #pragma unroll
           for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-              const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + ut * 16 + r16) * RS + ch * 64 + q * 16]);
               if (BF16) {
-                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, hv), acc[ut][g], 0, 0, 0);
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
               } else {
-                const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w};
-                const uint32_t hw[4] = {hv.x, hv.y, hv.z, hv.w};
+                const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w};
+                const uint32_t hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
 #pragma unroll
                 for (int e = 0; e < 4; ++e)
                   acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
@@ -1009,10 +1026,10 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   pstamp[4] = clock64();
 #endif
   // ---- gating
-  const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag != 0u));
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
-    const int ua = a0 + ut * 16 + 4 * q;
+    const int brow = rowbase + 32 * wr + 16 * ut + r16;
+    const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag[ut] != 0u));
     const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
     const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
     const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
@@ -1030,7 +1047,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
           const float wf[4] = {wxf[ut][g].x, wxf[ut][g].y, wxf[ut][g].z, wxf[ut][g].w};
           wxv = wf[i];
         }
-        const float bf[4] = {bias4[ut][g].x, bias4[ut][g].y, bias4[ut][g].z, bias4[ut][g].w};
+        const float bf[4] = {bias4[g].x, bias4[g].y, bias4[g].z, bias4[g].w};
         raw[g] = (wxv + tot[ut][g][i]) + bf[i];
       }
       CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
