@@ -79,6 +79,7 @@ F32_CASES = [
     (17, 20, 2, 32, True, True),      # batch not a multiple of 16 -> two tiles
     (40, 12, 1, 256, False, False),
     (2, 64, 2, 512, True, True),      # largest fp32 head
+    (70, 6, 4, 512, False, True),     # four row tiles per workgroup (ragged), the drainer wave publishes
 ]
 
 
@@ -101,6 +102,10 @@ BF16_CASES = [
     (20, 16, 2, 64, False, True),
     (64, 8, 1, 1024, False, False),   # config 5 head size, one head
     (33, 10, 8, 256, True, True),     # config 3 prefill shape, short
+    (50, 12, 4, 1024, True, True),    # config 5 shape, ragged batch: four row tiles, groups over two XCDs
+    (100, 6, 8, 256, True, True),     # four row tiles inside one XCD, two row groups, ragged
+    (40, 8, 4, 768, True, False),     # 48 members per head: 24 + 24 on an XCD pair
+    (24, 8, 3, 1000, False, True),    # odd member count (spread placement), partial last member, two row tiles
 ]
 
 

@@ -192,6 +192,11 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int WCH = 16 / EPC;          // 16-byte chunks holding the 16 units of one (row, gate)
   constexpr int ROWS = 16 * MT;          // batch rows of a workgroup
+  // With four row tiles a tile is polled by the peers three iterations after it was computed, so
+  // it can leave through the drainer wave (two iterations late) and the compute waves issue no
+  // stores at all: their waits for poll data then never include a store acknowledgement (loads
+  // and stores share one counter and complete out of order with each other).
+  constexpr bool kDrainerPublishes = MT >= 4;
 
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
   __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
@@ -211,7 +216,16 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     const int slot = local / p.G;
     member = local - slot * p.G;
     gi = slot * 8 + xcd;
-  } else {  // a group larger than one XCD is spread over all of them
+  } else if (p.G <= 64 && (p.G & 1) == 0) {
+    // two XCDs per group (workgroup i runs on XCD i % 8): members 0 .. G/2-1 on the even XCD of a
+    // pair, the rest on the odd one, so that half of a member's polls stay inside its own L2
+    const int xcd = wg & 7;
+    const int local = wg >> 3;
+    const int half = p.G >> 1;
+    const int slot = local / half;
+    member = (xcd & 1) * half + (local - slot * half);
+    gi = slot * 4 + (xcd >> 1);
+  } else {  // larger groups are spread over all XCDs
     gi = wg / p.G;
     member = wg - gi * p.G;
   }
@@ -364,12 +378,43 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   if (wave == 5) {
     const int drow = lane >> 2;   // batch row inside the tile
     const int dq = lane & 3;      // which 4 of the 16 units
-    auto drain = [&](int it) {
+    bool dcross = false;
+    auto drain = [&](int it, bool publish) {
       const int t = it / MT;
       const int mt = it - t * MT;
       const int brow = rowbase + mt * 16 + drow;
+      const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
+      if (kDrainerPublishes && publish) {
+        // h_t of this tile goes to the exchange ring from here, and the words of h_{t-2} are re-armed,
+        // so the compute waves wait on nothing but their polls.  Every lane stores: words outside
+        // the batch or the head belong to this member's block and are never polled.
+        constexpr int XB = ROWS * 16 * ESZ;
+        const int xsl = p.G * XB;
+        char *const blk = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xsl + (long long)member * XB +
+                          ((mt * 16 + drow) * 16 + dq * 4) * ESZ;
+        unsigned long long *cur = reinterpret_cast<unsigned long long *>(blk + (t % kRing) * xsl);
+        unsigned long long *old = reinterpret_cast<unsigned long long *>(blk + ((t + kRing - 2) % kRing) * xsl);
+        unsigned long long w0, w1 = 0;
+        if (BF16) {
+          w0 = (unsigned long long)(float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16)) |
+               ((unsigned long long)(float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16)) << 32);
+        } else {
+          w0 = (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32);
+          w1 = (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32);
+        }
+        if (dcross) {
+          __hip_atomic_store(cur, w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (!BF16) __hip_atomic_store(cur + 1, w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(old, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (!BF16) __hip_atomic_store(old + 1, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          cur[0] = w0;
+          if (!BF16) cur[1] = w1;
+          old[0] = ~0ull;
+          if (!BF16) old[1] = ~0ull;
+        }
+      }
       if (brow < rend && a0 + dq * 4 < dh) {
-        const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
         const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
         if (BF16) {
           uint2 w;
@@ -382,12 +427,13 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       }
     };
     lds_barrier();  // prologue barrier
+    dcross = cross_s != 0u;
 #ifdef XS_PROFILE
     long long dprof[2] = {0, 0};
     long long dt = clock64();
 #endif
     for (int j = 0; j < NITpad; ++j) {
-      if (j >= 2 && j - 2 < NIT) drain(j - 2);
+      if (j >= 2 && j - 2 < NIT) drain(j - 2, true);
 #ifdef XS_PROFILE
       { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
 #endif
@@ -397,7 +443,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #endif
     }
     lds_barrier();  // final barrier
-    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it);
+    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it, false);
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
@@ -488,6 +534,18 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   const int xslot = p.G * XBLOCK;                    // bytes one group publishes per step
   char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
 
+  // With several row tiles per workgroup (MT > 1) the polls of the NEXT (t, mt) iteration are
+  // issued right after the MFMAs of the current one have consumed the operand registers: the
+  // peers published that tile MT - 1 iterations ago, so the data is there and the exchange
+  // latency hides behind barrier, gating and publish.  The completion check, the re-arm and
+  // their order are unchanged.  (With MT == 1 the tile is published only at the end of the
+  // peers' current iteration, so there is nothing to fetch early.)
+  uint4 areg[NCH];
+  bool prefetched = false;
+  // poll address of chunk c of row tile mt = per-lane part (one register) + a compile-time constant:
+  // unit k of tile row r lives at member k/16, [mt*16 + r][k%16]
+  const int xlane = ((wave * KW + q * EPC) >> 4) * XBLOCK + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
+  auto xconst = [](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XBLOCK + mt_ * 256 * ESZ; };
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
     const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
@@ -499,14 +557,13 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
       XS_TICK(5);
       const int arow = rowbase + mt * 16 + r16;
-      uint4 areg[NCH];
       bool need[NCH];
       const bool row_ok = arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-        areg[c] = make_uint4(0, 0, 0, 0);
+        if (!(MT > 1 && prefetched)) areg[c] = make_uint4(0, 0, 0, 0);
         need[c] = row_ok && k0 < dh;
       }
       if (t == 0) {
@@ -526,13 +583,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           }
         }
       } else {
-        // unit k of tile row r lives at member k/16, [mt*16 + r][k%16]
-        int xoff[NCH];
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
-          const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-          xoff[c] = (k0 >> 4) * XBLOCK + ((mt * 16 + r16) * 16 + (k0 & 15)) * ESZ;
-          if (need[c]) areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xoff[c], 0, 16));
+          if (!(MT > 1 && prefetched) && need[c])
+            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
         }
         if (!aborted) {
           uint32_t spins = 0;
@@ -544,7 +598,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
                 const bool bad = BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
                 if (bad) {
                   any_bad = true;
-                  areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xoff[c], 0, 16));
+                  areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
                 }
               }
             }
@@ -570,10 +624,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #endif
         }
       }
-      if (row_reset) {
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) areg[c] = make_uint4(0, 0, 0, 0);
-      }
+      for (int c = 0; c < NCH; ++c)
+        if (row_reset || (MT > 1 && !need[c])) areg[c] = make_uint4(0, 0, 0, 0);
 
       // ---- 2. partial R.h over this wave's K slab, all four gates
       XS_TICK(0);
@@ -600,6 +653,23 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         }
       }
 
+      if (MT > 1) {
+        // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
+        const int nmt = (mt + 1) % MT;
+        const int nt = t + (mt + 1 == MT ? 1 : 0);
+        prefetched = nt >= 1 && nt < p.T;
+        if (prefetched) {
+          // unconditional loads (a select on the loaded value would make the wave wait for it right
+          // here); the descriptor ends with the slot, so a chunk past the last member reads zeros,
+          // and chunks that are not needed are zeroed when consumed
+          const __amdgpu_buffer_rsrc_t hrn = __builtin_amdgcn_make_buffer_rsrc(
+              xbase + ((nt + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrn, xlane, xconst(c, nmt), 16));
+        }
+      }
+
       // ---- 3. partial tiles -> LDS.  C layout: lane holds unit column r16, batch rows 4q..4q+3
       const int buf = it & 1;
 #pragma unroll
@@ -611,7 +681,6 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 
       // ---- 4. reduce over waves + exponential gating for element (row pb, unit pa)
       const int brow = rowbase + mt * 16 + pb;
-      const bool elem_ok = unit_ok && brow < rend;
       float raw[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -631,7 +700,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       // ---- 5. publish h_t to the peers, re-arm the words of h_{t-2}, stage h_t for the drainer
       float y = st[mt].y;
       if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
-      if (elem_ok) {
+      // (With four row tiles the drainer wave publishes: see there.)  Every lane stores, every
+      // iteration: lanes outside the batch or the head write words of their own block that nobody
+      // polls, and the re-arm of steps 0 and 1 hits slots that still hold the pattern.
+      if (!kDrainerPublishes) {
         const long long xo = (long long)member * (XBLOCK / ESZ) + (mt * 16 + pb) * 16 + pa;
         if (BF16) {
           const uint16_t v = (uint16_t)float_to_bf16_bits(y);
@@ -639,20 +711,20 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           uint16_t *old = reinterpret_cast<uint16_t *>(hold) + xo;
           if (cross) {
             __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (t >= 2) __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           } else {
             *dst = v;
-            if (t >= 2) *old = (uint16_t)kSentinel16;
+            *old = (uint16_t)kSentinel16;
           }
         } else {
           float *dst = reinterpret_cast<float *>(hcur) + xo;
           float *old = reinterpret_cast<float *>(hold) + xo;
           if (cross) {
             __hip_atomic_store(dst, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (t >= 2) __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           } else {
             *dst = y;
-            if (t >= 2) *old = __uint_as_float(kSentinel32);
+            *old = __uint_as_float(kSentinel32);
           }
         }
       }
@@ -1269,7 +1341,9 @@ int run_forward(const xs_slstm_args *a) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NH * NBT;
-    const int grid = G <= 32 ? 8 * G * ((ngroups + 7) / 8) : ngroups * G;
+    // grid shapes of the three placements the kernel knows: one XCD per group, two XCDs per group, spread
+    const int grid = G <= 32 ? 8 * G * ((ngroups + 7) / 8)
+                             : ((G <= 64 && G % 2 == 0) ? 8 * (G / 2) * ((ngroups + 3) / 4) : ngroups * G);
     if (grid > kMaxWg) return fail(XS_ERR_UNSUPPORTED, "grid %d too large", grid);
     {  // every word of the exchange ring starts as "not written yet"
       const size_t words = ((size_t)kRing * ngroups * G * 16 * MT * 16 * (bf16 ? 2 : 4) + 3) / 4;
