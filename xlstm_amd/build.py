@@ -20,6 +20,8 @@ HIPCC_FLAGS = [
     # the compiler must not form packed-fp32 instructions from scalar float code
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the LDS-direct loads are inline assembly that sets M0 and says so in its clobber list
+    "-Wno-inline-asm",
 ]
 
 

@@ -166,6 +166,22 @@ constexpr int kRing = 8;       // slots of the exchange ring
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+// 16 bytes per lane from a buffer straight into LDS (no registers): lane i's bytes land at
+// lds_addr + 16 * i.  Issued as inline assembly on purpose: the compiler then knows nothing of
+// these loads, and the waits for them are written by hand with exact counts (s_waitcnt vmcnt).
+__device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  // descriptor and LDS address are the same for all lanes of a wave: move them to scalar registers
+  rsrc.x = __builtin_amdgcn_readfirstlane(rsrc.x);
+  rsrc.y = __builtin_amdgcn_readfirstlane(rsrc.y);
+  rsrc.z = __builtin_amdgcn_readfirstlane(rsrc.z);
+  rsrc.w = __builtin_amdgcn_readfirstlane(rsrc.w);
+  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
+
 template <bool FAST>
 __device__ __forceinline__ void slstm_pointwise_t(float iraw, float fraw, float zraw, float oraw, CellState &s) {
   if (!FAST) {
@@ -197,12 +213,18 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   // stores at all: their waits for poll data then never include a store acknowledgement (loads
   // and stores share one counter and complete out of order with each other).
   constexpr bool kDrainerPublishes = MT >= 4;
+  // ... and the polls of a tile are then issued TWO iterations ahead, straight into LDS (dynamic
+  // shared memory, [2][compute wave][NCH][lane] 16-byte pieces), because the load latency of a
+  // freshly published tile (about 3000 to 5000 cycles) is longer than one iteration.
+  constexpr bool kDeepPrefetch = kDrainerPublishes;
+  extern __shared__ __attribute__((aligned(16))) unsigned char seq_dyn_lds[];
 
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
   __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
   __shared__ float hst[4][256];                 // [slot][row*16 + unit]             h on its way to HBM
   __shared__ uint32_t rfl[4][16];               // [slot][row]                       reset flags
   __shared__ uint32_t cross_s;
+  __shared__ uint32_t pubflag[4];               // [compute wave] iterations whose h is staged in hst
 
   // ---- role of this workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8,
   //      a head group takes consecutive slots of ONE XCD so its exchange stays in one L2)
@@ -269,6 +291,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     }
     cross_s = cross;
   }
+  if (tid < 4) pubflag[tid] = 0u;
 
   const int dh = p.dh;
   const int H = p.NH * dh;
@@ -432,6 +455,41 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     long long dprof[2] = {0, 0};
     long long dt = clock64();
 #endif
+    if (kDrainerPublishes) {
+      // iteration j leaves as soon as the four compute waves have staged it (they raise their
+      // counters after the LDS write): the peers fetch a tile two iterations before they use it
+      bool gave_up = false;
+      for (int j = 0; j < NITpad; ++j) {
+        lds_barrier();  // barrier #j
+#ifdef XS_PROFILE
+        { const long long now_ = clock64(); dprof[1] += now_ - dt; dt = now_; }
+#endif
+        if (j < NIT) {
+          long long spins = 0;
+          while (!gave_up) {
+            const uint32_t want = (uint32_t)j + 1u;
+            const uint32_t f0 = __hip_atomic_load(&pubflag[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f1 = __hip_atomic_load(&pubflag[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f2 = __hip_atomic_load(&pubflag[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f3 = __hip_atomic_load(&pubflag[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (f0 >= want && f1 >= want && f2 >= want && f3 >= want) break;
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins >= spin_limit) {  // cannot happen while the compute waves run; never wait forever
+              gave_up = true;
+              if (lane == 0 && atomicExch(&p.status->aborted, 1u) == 0u) {
+                p.status->abort_wg = (uint32_t)wg;
+                p.status->abort_step = (uint32_t)(j / MT);
+              }
+            }
+          }
+          drain(j, true);
+        }
+#ifdef XS_PROFILE
+        { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
+#endif
+      }
+      lds_barrier();  // final barrier
+    } else {
     for (int j = 0; j < NITpad; ++j) {
       if (j >= 2 && j - 2 < NIT) drain(j - 2, true);
 #ifdef XS_PROFILE
@@ -444,6 +502,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
     }
     lds_barrier();  // final barrier
     for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it, false);
+    }
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
@@ -546,6 +605,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   // unit k of tile row r lives at member k/16, [mt*16 + r][k%16]
   const int xlane = ((wave * KW + q * EPC) >> 4) * XBLOCK + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
   auto xconst = [](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XBLOCK + mt_ * 256 * ESZ; };
+  auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
     const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
@@ -583,12 +643,29 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           }
         }
       } else {
+        if (kDeepPrefetch) {
+          // this tile was requested two iterations ago; the only younger requests are the NCH of the next tile
+          if (it + 1 < NIT) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NCH) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-          if (!(MT > 1 && prefetched) && need[c])
-            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
+          for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
+        } else {
+#pragma unroll
+          for (int c = 0; c < NCH; ++c) {
+            if (!(MT > 1 && prefetched) && need[c])
+              areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
+          }
         }
-        if (!aborted) {
+        // (tiles fetched ahead through LDS are checked once outside the loop: inside it the wave
+        // waits for ALL of its outstanding loads, the next tile's requests included)
+        bool repoll = true;
+        if (kDeepPrefetch) {
+          repoll = false;
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            if (need[c]) repoll |= BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
+        }
+        if (!aborted && repoll) {
           uint32_t spins = 0;
           for (;;) {
             bool any_bad = false;
@@ -653,7 +730,20 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         }
       }
 
-      if (MT > 1) {
+      if (kDeepPrefetch) {
+        // request the tile of iteration it + 2 (its LDS slot is the one just read); step 0 takes its
+        // operand from s0.  A chunk past the last member reads zeros (the descriptor ends with the slot).
+        const int nmt = (mt + 2) % MT;
+        const int nt = t + (mt + 2 >= MT ? 1 : 0);
+        if (nt >= 1 && nt < p.T) {
+          const unsigned long long sb = reinterpret_cast<unsigned long long>(xbase + ((nt + kRing - 1) % kRing) * xslot);
+          const u32x4_t rs = {(uint32_t)sb, (uint32_t)(sb >> 32) & 0xFFFFu, (uint32_t)xslot, 0x00020000u};
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            lds_direct_load_b128(rs, (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(it, c)),
+                                 xlane, xconst(c, nmt));
+        }
+      } else if (MT > 1) {
         // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
         const int nmt = (mt + 1) % MT;
         const int nt = t + (mt + 1 == MT ? 1 : 0);
@@ -729,6 +819,8 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         }
       }
       hst[it & 3][tid] = y;
+      if (kDrainerPublishes && lane == 0)
+        __hip_atomic_store(&pubflag[wave], (uint32_t)it + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       XS_TICK(4);
     }
   }
@@ -1363,7 +1455,13 @@ int run_forward(const xs_slstm_args *a) {
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
     p.spin_limit = a->spin_limit;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), 0, stream, p);
+    // with four row tiles the polled tiles are staged in dynamic LDS: [2][4 waves][nch] KiB
+    const size_t dyn_lds = MT >= 4 ? (size_t)nch * 8192 : 0;
+    if (dyn_lds) {
+      const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn_lds);
+      if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", dyn_lds, hipGetErrorString(ea));
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), dyn_lds, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
     ++launches;
