@@ -76,13 +76,27 @@ __device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
   return b == 0xFFFFu ? 0x7FC0u : b;
 }
 
-__device__ __forceinline__ bool chunk_has_sentinel_bf16(const uint4 &v) {
-  auto bad = [](uint32_t w) { return ((w & 0xFFFFu) == kSentinel16) || ((w >> 16) == kSentinel16); };
-  return bad(v.x) || bad(v.y) || bad(v.z) || bad(v.w);
+// "Not written yet" tests without branches (they sit on the critical path between the arrival of
+// h and the MFMAs).  A mark is the element-wise unsigned maximum of words: the pattern is all
+// ones, so an element of the maximum equals the pattern iff one of the inputs did.
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+template <bool BF16>
+__device__ __forceinline__ uint32_t mark_join(uint32_t a, uint32_t b) {
+  if (BF16)  // v_pk_max_u16
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_max(__builtin_bit_cast(u16x2_t, a), __builtin_bit_cast(u16x2_t, b)));
+  return a > b ? a : b;
 }
-__device__ __forceinline__ bool chunk_has_sentinel_f32(const uint4 &v) {
-  return v.x == kSentinel32 || v.y == kSentinel32 || v.z == kSentinel32 || v.w == kSentinel32;
+template <bool BF16>
+__device__ __forceinline__ uint32_t chunk_mark(const uint4 &v) {
+  return mark_join<BF16>(mark_join<BF16>(v.x, v.y), mark_join<BF16>(v.z, v.w));
 }
+template <bool BF16>
+__device__ __forceinline__ bool mark_has_sentinel(uint32_t m) {
+  if (BF16) return (int)((m & 0xFFFFu) == kSentinel16) | (int)(m >= 0xFFFF0000u);
+  return m == kSentinel32;
+}
+__device__ __forceinline__ bool chunk_has_sentinel_bf16(const uint4 &v) { return mark_has_sentinel<true>(chunk_mark<true>(v)); }
+__device__ __forceinline__ bool chunk_has_sentinel_f32(const uint4 &v) { return mark_has_sentinel<false>(chunk_mark<false>(v)); }
 
 // 16-byte load that is served beyond this compute unit's vector L1
 __device__ __forceinline__ uint4 load16_agent(const void *p) {
@@ -153,7 +167,7 @@ __global__ void copy_state_kernel(const float *s0, float *s_out, size_t n) {
 //   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
 //              output tensor in HBM.
 //
-// Exchange ring: kRing slots, slot t % kRing holds h_t as [member][row][16 units].
+// Exchange ring: kRing slots, slot t % kRing holds h_t as [row tile][member][16 rows][16 units].
 // A word is either data or the "not written yet" pattern.  A workgroup re-arms its own
 // words of slot (t-2) % kRing after its poll of step t has completed: by then every peer
 // has published h_{t-1}, hence has finished reading h_{t-2}.  The re-arm is acknowledged
@@ -411,10 +425,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         // h_t of this tile goes to the exchange ring from here, and the words of h_{t-2} are re-armed,
         // so the compute waves wait on nothing but their polls.  Every lane stores: words outside
         // the batch or the head belong to this member's block and are never polled.
-        constexpr int XB = ROWS * 16 * ESZ;
-        const int xsl = p.G * XB;
-        char *const blk = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xsl + (long long)member * XB +
-                          ((mt * 16 + drow) * 16 + dq * 4) * ESZ;
+        constexpr int TB = 16 * 16 * ESZ;  // one member's tile; a ring slot is [row tile][member][16 rows][16 units]
+        const int xsl = p.G * MT * TB;
+        char *const blk = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xsl + ((long long)mt * p.G + member) * TB +
+                          (drow * 16 + dq * 4) * ESZ;
         unsigned long long *cur = reinterpret_cast<unsigned long long *>(blk + (t % kRing) * xsl);
         unsigned long long *old = reinterpret_cast<unsigned long long *>(blk + ((t + kRing - 2) % kRing) * xsl);
         unsigned long long w0, w1 = 0;
@@ -590,7 +604,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   // over all L2 channels (measured: lines 256 B .. 2 KiB apart are served 1.5x faster than
   // lines 4 KiB or more apart)
   constexpr int XBLOCK = ROWS * 16 * ESZ;            // bytes one member publishes per step
+  constexpr int XTILE = 16 * 16 * ESZ;               // ... per row tile
   const int xslot = p.G * XBLOCK;                    // bytes one group publishes per step
+  // a slot is laid out [row tile][member][16 rows][16 units]: what the group publishes for one row
+  // tile is contiguous, so the polls of an iteration spread over all L2 channels
   char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
 
   // With several row tiles per workgroup (MT > 1) the polls of the NEXT (t, mt) iteration are
@@ -602,9 +619,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   uint4 areg[NCH];
   bool prefetched = false;
   // poll address of chunk c of row tile mt = per-lane part (one register) + a compile-time constant:
-  // unit k of tile row r lives at member k/16, [mt*16 + r][k%16]
-  const int xlane = ((wave * KW + q * EPC) >> 4) * XBLOCK + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
-  auto xconst = [](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XBLOCK + mt_ * 256 * ESZ; };
+  // unit k of row r of row tile mt lives at [mt][member k/16][r][k%16]
+  const int xlane = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
+  const int xtile_stride = p.G * XTILE;
+  auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
   auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
@@ -645,8 +663,14 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       } else {
         if (kDeepPrefetch) {
           // this tile was requested two iterations ago; the only younger requests are the NCH of the next tile
+#ifdef XS_PROFILE
+          const long long w0_ = clock64();
+#endif
           if (it + 1 < NIT) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NCH) : "memory");
           else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef XS_PROFILE
+          prof[7] += clock64() - w0_;
+#endif
 #pragma unroll
           for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
         } else {
@@ -658,14 +682,11 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         }
         // (tiles fetched ahead through LDS are checked once outside the loop: inside it the wave
         // waits for ALL of its outstanding loads, the next tile's requests included)
-        bool repoll = true;
-        if (kDeepPrefetch) {
-          repoll = false;
+        // first look at everything at once: one mark over all chunks this lane needs
+        uint32_t mark = 0u;
 #pragma unroll
-          for (int c = 0; c < NCH; ++c)
-            if (need[c]) repoll |= BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
-        }
-        if (!aborted && repoll) {
+        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+        if (!aborted && mark_has_sentinel<BF16>(mark)) {
           uint32_t spins = 0;
           for (;;) {
             bool any_bad = false;
@@ -794,7 +815,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       // iteration: lanes outside the batch or the head write words of their own block that nobody
       // polls, and the re-arm of steps 0 and 1 hits slots that still hold the pattern.
       if (!kDrainerPublishes) {
-        const long long xo = (long long)member * (XBLOCK / ESZ) + (mt * 16 + pb) * 16 + pa;
+        const long long xo = ((long long)mt * p.G + member) * (XTILE / ESZ) + pb * 16 + pa;
         if (BF16) {
           const uint16_t v = (uint16_t)float_to_bf16_bits(y);
           uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
