@@ -626,8 +626,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
+    // (the descriptor ends with the slot: a chunk past the last member reads zeros)
     const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
-        xbase + ((t + kRing - 1) % kRing) * xslot, 0, 0x7FFFFFFF, 0x00020000);
+        xbase + ((t + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
     char *const hcur = xbase + (t % kRing) * xslot;
     char *const hold = xbase + ((t + kRing - 2) % kRing) * xslot;
 #pragma unroll
@@ -674,9 +675,11 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
           for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
         } else {
+          // every lane loads every chunk (no divergent branches on the way to the MFMAs); what is
+          // not needed is left out of the test below and zeroed afterwards
+          if (!(MT > 1 && prefetched)) {
 #pragma unroll
-          for (int c = 0; c < NCH; ++c) {
-            if (!(MT > 1 && prefetched) && need[c])
+            for (int c = 0; c < NCH; ++c)
               areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
           }
         }
@@ -724,7 +727,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       }
 #pragma unroll
       for (int c = 0; c < NCH; ++c)
-        if (row_reset || (MT > 1 && !need[c])) areg[c] = make_uint4(0, 0, 0, 0);
+        if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
 
       // ---- 2. partial R.h over this wave's K slab, all four gates
       XS_TICK(0);
