@@ -181,17 +181,13 @@ constexpr int kRing = 8;       // slots of the exchange ring
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // 16 bytes per lane from a buffer straight into LDS (no registers): lane i's bytes land at
 // lds_addr + 16 * i.  Issued as inline assembly on purpose: the compiler then knows nothing of
 // these loads, and the waits for them are written by hand with exact counts (s_waitcnt vmcnt).
+// rsrc and lds_addr must be wave-uniform values (see uniform()).
 __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_addr, int voffset, int soffset) {
-  // descriptor and LDS address are the same for all lanes of a wave: move them to scalar registers
-  rsrc.x = __builtin_amdgcn_readfirstlane(rsrc.x);
-  rsrc.y = __builtin_amdgcn_readfirstlane(rsrc.y);
-  rsrc.z = __builtin_amdgcn_readfirstlane(rsrc.z);
-  rsrc.w = __builtin_amdgcn_readfirstlane(rsrc.w);
-  lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
                :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
@@ -725,9 +721,15 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #endif
         }
       }
+      // (a whole wave rarely has anything to clear: one uniform branch instead of 4 selects per chunk)
+      bool clear_any = row_reset;
 #pragma unroll
-      for (int c = 0; c < NCH; ++c)
-        if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
+      for (int c = 0; c < NCH; ++c) clear_any |= !need[c];
+      if (__builtin_amdgcn_ballot_w64(clear_any) != 0ull) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c)
+          if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
+      }
 
       // ---- 2. partial R.h over this wave's K slab, all four gates
       XS_TICK(0);
@@ -761,11 +763,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         const int nt = t + (mt + 2 >= MT ? 1 : 0);
         if (nt >= 1 && nt < p.T) {
           const unsigned long long sb = reinterpret_cast<unsigned long long>(xbase + ((nt + kRing - 1) % kRing) * xslot);
-          const u32x4_t rs = {(uint32_t)sb, (uint32_t)(sb >> 32) & 0xFFFFu, (uint32_t)xslot, 0x00020000u};
+          const u32x4_t rs = {uniform((uint32_t)sb), uniform((uint32_t)(sb >> 32) & 0xFFFFu), uniform((uint32_t)xslot), 0x00020000u};
+          const uint32_t lds0 = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(it, 0)));
 #pragma unroll
-          for (int c = 0; c < NCH; ++c)
-            lds_direct_load_b128(rs, (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(it, c)),
-                                 xlane, xconst(c, nmt));
+          for (int c = 0; c < NCH; ++c) lds_direct_load_b128(rs, lds0 + (c << 10), xlane, xconst(c, nmt));
         }
       } else if (MT > 1) {
         // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
