@@ -172,3 +172,12 @@ def test_spin_limit_runs_out_is_reported_not_hung():
     assert status["aborted"] in (0, 1)
     if status["aborted"]:
         assert status["abort_step"] >= 1
+    # four row tiles per workgroup: the drainer wave's wait for the compute waves is bounded the same way
+    wx, r, b, _ = make_problem(17, 64, 6, 4, 1024, bf16=True)
+    h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
+    assert status["aborted"] in (0, 1)
+    # and the next call on the same device is unaffected
+    h2, s2, status2 = _run_hip(wx, r, b, bf16=True)
+    assert status2["aborted"] == 0
+    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
+    assert max_err(h2, h_ref) <= TOL_BF16
