@@ -49,7 +49,7 @@ struct SeqParams {
   float *s_out;
   xs_slstm_status *status;
   uint32_t *wg_xcc;
-  void *xbuf;    // exchange ring [kRing][head group][G][rows][16 units], pre-filled with the "not written yet" pattern
+  void *xbuf;    // exchange ring [head group][kRing][row tile][member][16 rows][16 units], pre-filled with the "not written yet" pattern
   int B, T, NH, dh;
   int b0, bend;  // batch rows [b0, bend) handled by this launch
   int G;         // workgroups per head group
@@ -97,16 +97,6 @@ __device__ __forceinline__ bool mark_has_sentinel(uint32_t m) {
 }
 __device__ __forceinline__ bool chunk_has_sentinel_bf16(const uint4 &v) { return mark_has_sentinel<true>(chunk_mark<true>(v)); }
 __device__ __forceinline__ bool chunk_has_sentinel_f32(const uint4 &v) { return mark_has_sentinel<false>(chunk_mark<false>(v)); }
-
-// 16-byte load that is served beyond this compute unit's vector L1
-__device__ __forceinline__ uint4 load16_agent(const void *p) {
-  const unsigned long long *q = reinterpret_cast<const unsigned long long *>(p);
-  unsigned long long lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  unsigned long long hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  uint4 v;
-  v.x = (uint32_t)lo; v.y = (uint32_t)(lo >> 32); v.z = (uint32_t)hi; v.w = (uint32_t)(hi >> 32);
-  return v;
-}
 
 __device__ __forceinline__ float logsigmoid_f(float x) {
   // min(x,0) - log1p(exp(-|x|))
@@ -795,7 +785,6 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       XS_TICK(2);
 
       // ---- 4. reduce over waves + exponential gating for element (row pb, unit pa)
-      const int brow = rowbase + mt * 16 + pb;
       float raw[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
