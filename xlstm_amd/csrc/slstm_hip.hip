@@ -167,6 +167,7 @@ __global__ void copy_state_kernel(const float *s0, float *s_out, size_t n) {
 // ---------------------------------------------------------------------------
 constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
 constexpr int kRing = 8;       // slots of the exchange ring
+constexpr int kPollStagger = 6;  // s_sleep units (64 cycles) between the two polls of a step (measured best of 2 .. 16)
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -660,6 +661,63 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #endif
 #pragma unroll
           for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
+        } else if (MT == 1) {
+          // Two polls in flight, about half a round trip apart (kPollStagger), re-issued alternately:
+          // a poll returns every ~300 cycles instead of every ~600, which halves both the wait for h
+          // and the skew between the four waves at the barrier.  Lanes whose batch row does not exist
+          // ask for an offset past the descriptor's end: zeros, no memory traffic, so the doubled poll
+          // rate stays far below what a compute unit can pull from the L2.  The decisions are
+          // wave-uniform (ballot) so that the waits keep exact counts.
+          const int xl = row_ok ? xlane : 0x7FFFFF00;
+          uint4 breg[NCH];
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+          __builtin_amdgcn_s_sleep(kPollStagger);
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+          if (!aborted) {
+            uint32_t spins = 0;
+            for (;;) {
+              uint32_t ma = 0u;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c) ma = mark_join<BF16>(ma, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(ma)) == 0ull) break;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c)
+                areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+              uint32_t mb = 0u;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, need[c] ? chunk_mark<BF16>(breg[c]) : 0u);
+              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mb)) == 0ull) {
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) areg[c] = breg[c];
+                break;
+              }
+#pragma unroll
+              for (int c = 0; c < NCH; ++c)
+                breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+              spins += 2;
+              if ((spins & 1023u) == 0u &&
+                  __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+                aborted = true;
+                break;
+              }
+              if ((long long)spins >= spin_limit) {
+                aborted = true;
+                if (atomicExch(&p.status->aborted, 1u) == 0u) {
+                  p.status->abort_wg = (uint32_t)wg;
+                  p.status->abort_step = (uint32_t)t;
+                }
+                break;
+              }
+            }
+            max_spins = spins > max_spins ? spins : max_spins;
+#ifdef XS_PROFILE
+            prof[6] += spins;
+#endif
+          }
         } else {
           // every lane loads every chunk (no divergent branches on the way to the MFMAs); what is
           // not needed is left out of the test below and zeroed afterwards
