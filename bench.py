@@ -71,7 +71,7 @@ def cpu_baseline(wx, r_ext, bias, mask, budget_s=15.0):
     per_step = (time.perf_counter() - t0) / probe
     Ts = int(max(64, min(T, budget_s / max(per_step, 1e-6))))
     runs = []
-    while sum(runs) < 10.0 and len(runs) < 3:  # 10-30 s of CPU work in total
+    while (sum(runs) < 10.0 and len(runs) < 40) or len(runs) < 2:  # 10-30 s of CPU work in total, whatever the host's speed
         t0 = time.perf_counter()
         vp.slstm_forward(wx32[:, :Ts], r_ext, bias, None, mask[:, :Ts] if mask is not None else None)
         runs.append(time.perf_counter() - t0)
