@@ -105,11 +105,14 @@ def bench_decode(device, steps=1024, prefill=128):
         s_a, s_b = s_b, s_a
     s_a.copy_(state)
     torch.cuda.synchronize()
+    # eager loop: one xs_slstm_step call per token from Python through a StepPlan (arguments validated once)
+    plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16, workspace=ws)
+    stream = torch.cuda.current_stream().cuda_stream
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
     for t in range(steps):
-        F.slstm_forward(wx_dec[t], r, bias, s_a, None, step=True, workspace=ws, h_out=h1, s_out=s_b)
+        plan(wx_dec[t], s_a, s_b, h1, stream)
         s_a, s_b = s_b, s_a
     e1.record()
     torch.cuda.synchronize()

@@ -119,3 +119,33 @@ def test_unsupported_head_dim_is_an_error_not_a_wrong_answer():
     with pytest.raises(EngineError, match="multiple of 8"):
         with torch.no_grad():
             cell(torch.from_numpy(wx).cuda())
+
+
+@pytest.mark.gpu
+def test_step_plan_equals_the_generic_step_call():
+    """The pre-validated fast host path launches the same kernel with the same arguments."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(5)
+    B, NH, dh = 64, 2, 128
+    H = NH * dh
+    r = (torch.rand(NH, 4 * dh, dh, device=dev) - 0.5) * 0.2
+    bias = torch.randn(NH, 4, dh, device=dev)
+    wx = torch.randn(6, B, 1, 4 * H, device=dev).bfloat16()
+    s = torch.randn(4, B, H, device=dev)
+    s[2] = s[2].abs() + 0.5
+    plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16)
+    a, b = s.clone(), torch.empty_like(s)
+    h = torch.empty(1, B, H, dtype=torch.bfloat16, device=dev)
+    ref = s.clone()
+    for t in range(6):
+        plan(wx[t], a, b, h)
+        h_ref, ref = F.slstm_forward(wx[t], r.bfloat16(), bias, ref, None, step=True)
+        a, b = b, a
+        torch.cuda.synchronize()
+        assert torch.equal(h, h_ref) and torch.equal(a, ref), t
+    with pytest.raises(ValueError):
+        plan(wx[0].float(), a, b, h)

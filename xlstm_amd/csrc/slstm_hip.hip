@@ -22,6 +22,9 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+#include <vector>
+
 #include "xlstm_amd.h"
 
 namespace {
@@ -1415,6 +1418,23 @@ int device_cus() {
   return cus;
 }
 
+// Raises a kernel's dynamic-LDS limit once per (kernel, device); the attribute call is not free and
+// a decode loop would otherwise pay it every token.
+int ensure_dynamic_lds(const void *kernel, size_t bytes) {
+  struct Done { const void *kernel; int device; size_t bytes; };
+  static std::mutex mu;
+  static std::vector<Done> done;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(XS_ERR_DEVICE, "cannot query the current device");
+  std::lock_guard<std::mutex> lock(mu);
+  for (const Done &d : done)
+    if (d.kernel == kernel && d.device == dev && d.bytes >= bytes) return XS_OK;
+  const hipError_t ea = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(ea));
+  done.push_back(Done{kernel, dev, bytes});
+  return XS_OK;
+}
+
 int run_step(const xs_slstm_args *a) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int B = a->B, NH = a->NH, dh = a->dh;
@@ -1453,8 +1473,8 @@ int run_step(const xs_slstm_args *a) {
   else kern = slabch == 4 ? XS_PICK(false, 4) : (slabch == 8 ? XS_PICK(false, 8) : XS_PICK(false, 2));
 #undef XS_PICK
   if (lds > 64 * 1024) {  // the single-slab variant at dh = 256 needs 99 KiB of the 160 KiB of LDS
-    const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(ea));
+    const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
+    if (rc != XS_OK) return rc;
   }
   hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p, nch_log2);
   const hipError_t e = hipGetLastError();
@@ -1533,8 +1553,8 @@ int run_forward(const xs_slstm_args *a) {
     // with four row tiles the polled tiles are staged in dynamic LDS: [2][4 waves][nch] KiB
     const size_t dyn_lds = MT >= 4 ? (size_t)nch * 8192 : 0;
     if (dyn_lds) {
-      const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn_lds);
-      if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", dyn_lds, hipGetErrorString(ea));
+      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), dyn_lds);
+      if (rc != XS_OK) return rc;
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), dyn_lds, stream, p);
     const hipError_t e = hipGetLastError();

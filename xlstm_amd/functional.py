@@ -143,3 +143,62 @@ def slstm_forward(
     if rc != 0:
         raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
     return h_out, s_out
+
+
+class StepPlan:
+    """Single-token steps with fixed shapes, validated once.
+
+    ``slstm_forward(..., step=True)`` checks and normalises every argument on every call, which costs
+    more host time than the step kernel runs.  A plan does that work once; calling it only swaps
+    the five pointers that change between tokens and launches ``xs_slstm_step``::
+
+        plan = StepPlan(B, r, bias, wx_dtype=torch.bfloat16)
+        for x_t in tokens:                       # x_t: [B, 1, 4H], contiguous
+            plan(x_t, s_in, s_out, h_out)        # s_in / s_out: float32 [4, B, H], distinct buffers
+            s_in, s_out = s_out, s_in
+
+    The caller keeps the plan's contract: tensors on the plan's device, which is the current one,
+    the dtypes and shapes given at construction, contiguous, ``s_out`` not overlapping ``s_in``.
+    """
+
+    def __init__(self, B: int, r: torch.Tensor, bias: torch.Tensor, wx_dtype: torch.dtype = torch.bfloat16,
+                 workspace: Optional[torch.Tensor] = None):
+        lib = _lib.load()
+        _require_cuda("r", r)
+        if wx_dtype not in _DTYPE_CODE:
+            raise TypeError(f"wx dtype {wx_dtype} not supported by the hip backend (float32 or bfloat16)")
+        if r.dim() != 3 or r.shape[1] != 4 * r.shape[2]:
+            raise ValueError(f"r must be [NH, 4*dh, dh], got {tuple(r.shape)}")
+        NH, dh = int(r.shape[0]), int(r.shape[2])
+        if tuple(bias.shape) != (NH, 4, dh):
+            raise ValueError(f"bias must be [NH, 4, dh] = {(NH, 4, dh)}, got {tuple(bias.shape)}")
+        self.B, self.NH, self.dh, self.H = int(B), NH, dh, NH * dh
+        self.wx_dtype = wx_dtype
+        self.device = r.device
+        # the plan owns what it points to: R in the operand type, float32 bias, the workspace
+        self.r = r.detach().to(wx_dtype).contiguous()
+        self.bias = bias.detach().to(torch.float32).contiguous()
+        self.workspace = workspace if workspace is not None else workspace_for(self.B, 1, NH, dh, self.device)
+        a = _lib.SlstmArgs()
+        a.B, a.T, a.NH, a.dh = self.B, 1, NH, dh
+        a.wx_dtype = a.r_dtype = _DTYPE_CODE[wx_dtype]
+        a.wx_stride_b, a.wx_stride_t = 4 * self.H, 4 * self.H
+        a.r, a.bias = self.r.data_ptr(), self.bias.data_ptr()
+        a.reset, a.reset_stride_b = None, 0
+        a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
+        a.spin_limit = 0
+        self._args, self._ref, self._fn = a, ctypes.byref(a), lib.xs_slstm_step
+        self._wx_numel, self._s_numel = self.B * 4 * self.H, 4 * self.B * self.H
+
+    def __call__(self, wx: torch.Tensor, s_in: torch.Tensor, s_out: torch.Tensor, h_out: torch.Tensor,
+                 stream: Optional[int] = None) -> None:
+        if (wx.dtype != self.wx_dtype or wx.numel() != self._wx_numel or s_in.numel() != self._s_numel
+                or s_out.numel() != self._s_numel or s_in.dtype != torch.float32 or s_out.dtype != torch.float32
+                or h_out.dtype != self.wx_dtype or h_out.numel() * 4 != self._s_numel):
+            raise ValueError("tensor does not fit the plan (dtype or size)")
+        a = self._args
+        a.wx, a.s0, a.s_out, a.h_out = wx.data_ptr(), s_in.data_ptr(), s_out.data_ptr(), h_out.data_ptr()
+        a.stream = stream if stream is not None else torch.cuda.current_stream().cuda_stream
+        rc = self._fn(self._ref)
+        if rc != 0:
+            raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
