@@ -381,7 +381,38 @@ class sLSTMCell_hip(nn.Module):
             if state_out.dtype != torch.float32 or not state_out.is_contiguous() or tuple(state_out.shape) != (
                     self.config.num_states, B, self.config.hidden_size):
                 raise ValueError("state_out must be a contiguous float32 [4, B, H] tensor")
+        fast = self._step_fast(input, state, reset_mask, state_out)
+        if fast is not None:
+            return fast
         return self._run(input, state, reset_mask, step=True, state_out=state_out)
+
+    def _step_fast(self, input, state, reset_mask, state_out):
+        """The decode steady state (float32 state carried over, no mask, no autograd) through a cached
+        ``StepPlan``: the generic path spends more host time per token than the kernel runs."""
+        if (reset_mask is not None or state is None or state.dtype != torch.float32 or not state.is_contiguous()
+                or input.dtype not in (torch.float32, torch.bfloat16) or self.config.input_shape != "BSGNH"
+                or input.dim() != 3 or input.shape[1] != 1 or not input.is_contiguous() or not input.is_cuda
+                or torch.is_autocast_enabled()):
+            return None
+        if torch.is_grad_enabled() and (
+                input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad):
+            return None
+        self._check_input(input)
+        B = input.shape[0]
+        self._check_state(B, state)
+        r, b = self._recurrent_kernel_, self._bias_
+        key = (B, input.dtype, input.device, r.data_ptr(), r._version, b.data_ptr(), b._version)
+        cached = getattr(self, "_step_plan_cache", None)
+        if cached is None or cached[0] != key:
+            plan = F_hip.StepPlan(B, r.detach(), b.detach().view(self.config.num_heads, 4, self.head_dim), wx_dtype=input.dtype)
+            cached = (key, plan)
+            object.__setattr__(self, "_step_plan_cache", cached)
+        H = self.config.hidden_size
+        h = torch.empty((1, B, H), dtype=input.dtype, device=input.device)
+        s_out = state_out if state_out is not None else torch.empty((4, B, H), dtype=torch.float32, device=input.device)
+        with torch.cuda.device(input.device):
+            cached[1](input, state, s_out, h)
+        return self._permute_output(h), (s_out if self.keep_state_fp32 else s_out.to(input.dtype))
 
 
 def reference_cell_params_to_hip(recurrent_kernel_int: torch.Tensor, bias_int: torch.Tensor, source_backend: str,
