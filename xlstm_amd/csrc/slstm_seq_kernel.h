@@ -1,0 +1,788 @@
+// The persistent sequence kernel: all T timesteps of a call in one launch.
+// Included by slstm_hip.hip only (one translation unit), after slstm_device_common.h.
+#pragma once
+
+namespace {
+
+struct SeqParams {
+  const void *wx;
+  long long wx_sb, wx_st;
+  const void *r;
+  int r_bf16;
+  const float *bias;
+  const float *s0;
+  const unsigned char *reset;
+  long long reset_sb;
+  void *h_out;
+  float *s_out;
+  xs_slstm_status *status;
+  uint32_t *wg_xcc;
+  void *xbuf;    // exchange ring [head group][kRing][row tile][member][16 rows][16 units], pre-filled with the "not written yet" pattern
+  int B, T, NH, dh;
+  int b0, bend;  // batch rows [b0, bend) handled by this launch
+  int G;         // workgroups per head group
+  int NBT;       // batch tiles (independent groups) per head
+  int rows_per_wg;
+  long long spin_limit;
+};
+
+// ---------------------------------------------------------------------------
+// persistent sequence kernel
+//   BF16: wx / h_out / MFMA operands are bf16 (fp32 accumulate, fp32 c,n,m);
+//         otherwise everything is fp32 (v_mfma_f32_16x16x4_f32).
+//   NCH : 16-byte chunks of h each lane holds per batch row; one wave covers
+//         NCH*32 (bf16) or NCH*16 (fp32) input units, the four waves 4x that.
+//   MT  : 16-row batch tiles handled one after the other by a workgroup.
+//
+// Six waves per workgroup, one barrier per (step, tile) iteration shared by all:
+//   waves 0-3  compute: poll h_{t-1}, MFMA, reduce through LDS, gating, publish h_t.
+//              Their vector-memory queue only ever holds L2-resident traffic (the
+//              exchange ring), because vector memory completes in order within a wave
+//              and anything slower would sit in front of the latency-critical polls.
+//   wave 4     feeder: streams W.x and the reset flags of FUTURE iterations from HBM
+//              into an LDS ring (kLookahead iterations in flight).
+//   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
+//              output tensor in HBM.
+//
+// Exchange ring: kRing slots, slot t % kRing holds h_t as [row tile][member][16 rows][16 units].
+// A word is either data or the "not written yet" pattern.  A workgroup re-arms its own
+// words of slot (t-2) % kRing after its poll of step t has completed: by then every peer
+// has published h_{t-1}, hence has finished reading h_{t-2}.  The re-arm is acknowledged
+// before the workgroup's poll of step t+1 completes, i.e. before it publishes h_{t+1};
+// a peer polling slot (t-2) % kRing for h_{t-2+kRing} has seen that publication, so it
+// can only ever read the pattern or the new data there, never the stale h_{t-2}.
+// ---------------------------------------------------------------------------
+constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
+constexpr int kRing = 8;       // slots of the exchange ring
+constexpr int kPollStagger = 6;  // s_sleep units (64 cycles) between the two polls of a step (measured best of 2 .. 16)
+
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
+
+// 16 bytes per lane from a buffer straight into LDS (no registers): lane i's bytes land at
+// lds_addr + 16 * i.  Issued as inline assembly on purpose: the compiler then knows nothing of
+// these loads, and the waits for them are written by hand with exact counts (s_waitcnt vmcnt).
+// rsrc and lds_addr must be wave-uniform values (see uniform()).
+__device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_addr, int voffset, int soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
+}
+
+template <bool BF16, int NCH, int MT>
+__global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
+  constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
+  constexpr int KW = NCH * 4 * EPC;      // input units per wave
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int WCH = 16 / EPC;          // 16-byte chunks holding the 16 units of one (row, gate)
+  constexpr int ROWS = 16 * MT;          // batch rows of a workgroup
+  // With four row tiles a tile is polled by the peers three iterations after it was computed, so
+  // it can leave through the drainer wave (two iterations late) and the compute waves issue no
+  // stores at all: their waits for poll data then never include a store acknowledgement (loads
+  // and stores share one counter and complete out of order with each other).
+  constexpr bool kDrainerPublishes = MT >= 4;
+  // ... and the polls of a tile are then issued TWO iterations ahead, straight into LDS (dynamic
+  // shared memory, [2][compute wave][NCH][lane] 16-byte pieces), because the load latency of a
+  // freshly published tile (about 3000 to 5000 cycles) is longer than one iteration.
+  constexpr bool kDeepPrefetch = kDrainerPublishes;
+  extern __shared__ __attribute__((aligned(16))) unsigned char seq_dyn_lds[];
+
+  __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
+  __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
+  __shared__ float hst[4][256];                 // [slot][row*16 + unit]             h on its way to HBM
+  __shared__ uint32_t rfl[4][16];               // [slot][row]                       reset flags
+  __shared__ uint32_t cross_s;
+  __shared__ uint32_t pubflag[4];               // [compute wave] iterations whose h is staged in hst
+
+  // ---- role of this workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8,
+  //      a head group takes consecutive slots of ONE XCD so its exchange stays in one L2)
+  const int wg = blockIdx.x;
+  const int ngroups = p.NH * p.NBT;
+  int gi, member;  // head group index, position inside the group
+  const bool one_xcd_layout = p.G <= 32;
+  if (one_xcd_layout) {
+    const int xcd = wg & 7;
+    const int local = wg >> 3;
+    const int slot = local / p.G;
+    member = local - slot * p.G;
+    gi = slot * 8 + xcd;
+  } else if (p.G <= 64 && (p.G & 1) == 0) {
+    // two XCDs per group (workgroup i runs on XCD i % 8): members 0 .. G/2-1 on the even XCD of a
+    // pair, the rest on the odd one, so that half of a member's polls stay inside its own L2
+    const int xcd = wg & 7;
+    const int local = wg >> 3;
+    const int half = p.G >> 1;
+    const int slot = local / half;
+    member = (xcd & 1) * half + (local - slot * half);
+    gi = slot * 4 + (xcd >> 1);
+  } else {  // larger groups are spread over all XCDs
+    gi = wg / p.G;
+    member = wg - gi * p.G;
+  }
+  if (gi >= ngroups) return;
+  const int head = gi / p.NBT;
+  const int bt = gi - head * p.NBT;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const long long spin_limit = p.spin_limit > 0 ? p.spin_limit : kDefaultSpinLimit;
+
+  // ---- placement handshake: do all members of this head group share one XCD (one L2)?
+  //      If so h is published with plain stores (they land in that L2); otherwise with
+  //      device-scope stores that are written through to memory.
+  if (tid == 0) {
+    const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
+    __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t cross = one_xcd_layout ? 0u : 1u;
+    if (one_xcd_layout) {
+      const int xcd = wg & 7;
+      const int slot = (wg >> 3) / p.G;
+      for (int j = 0; j < p.G; ++j) {
+        const int peer = ((slot * p.G + j) << 3) | xcd;
+        uint32_t w = 0;
+        long long spins = 0;
+        while (((w = __hip_atomic_load(&p.wg_xcc[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & 0x80000000u) == 0u) {
+          if (++spins >= spin_limit) {  // a peer never started: the grid is not co-resident
+            if (atomicExch(&p.status->aborted, 1u) == 0u) {
+              p.status->abort_wg = (uint32_t)wg;
+              p.status->abort_step = 0xFFFFFFFFu;
+            }
+            cross = 1u;
+            break;
+          }
+        }
+        if ((w & 0xFu) != my_xcc) cross = 1u;
+      }
+      if (cross) atomicAdd(&p.status->xcd_mixed, 1u);
+    }
+    cross_s = cross;
+  }
+  if (tid < 4) pubflag[tid] = 0u;
+
+  const int dh = p.dh;
+  const int H = p.NH * dh;
+  const int a0 = member * 16;
+  const int rowbase = p.b0 + bt * p.rows_per_wg;
+  // rows [rowbase, rend) belong to this workgroup; with few rows per head the batch is cut into
+  // tiles of fewer than 16 rows so that more compute units share the work and every exchange is smaller
+  const int rend = (rowbase + p.rows_per_wg < p.bend) ? rowbase + p.rows_per_wg : p.bend;
+  const long long BH = (long long)p.B * H;
+  const int NIT = p.T * MT;
+  const int NITpad = (NIT + kLookahead - 1) / kLookahead * kLookahead;  // barriers every wave executes
+
+  // =========================================================================
+  // wave 4: feeder.  Every iteration issues exactly WCH + 1 loads (addresses of
+  // rows / chunks / steps that do not exist are clamped to ones that do and the
+  // result is zeroed), so that the outstanding-load count at each use is exact.
+  // =========================================================================
+  if (wave == 4) {
+    const int fb = lane & 15;  // batch row inside the tile
+    const int fg = lane >> 4;  // gate
+    uint4 ring[kLookahead][WCH];
+    uint32_t fring[kLookahead];
+    const char *wxb = reinterpret_cast<const char *>(p.wx);
+    const unsigned char *flagb = p.reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);
+    const long long flag_sb = p.reset ? p.reset_sb : 0;
+    const uint32_t flag_on = p.reset ? 0xFFu : 0u;
+
+    auto issue = [&](int it, uint4 (&dst)[WCH], uint32_t &flag) {
+      const int itc = it < NIT ? it : NIT - 1;
+      const int t = itc / MT;
+      const int mt = itc - t * MT;
+      const int brow = rowbase + mt * 16 + fb;
+      const int browc = brow < rend ? brow : rend - 1;
+      const long long e0 = (long long)browc * p.wx_sb + (long long)t * p.wx_st + (long long)fg * H + head * dh + a0;
+#pragma unroll
+      for (int c = 0; c < WCH; ++c) {
+        const int cc = (a0 + c * EPC < dh) ? c : 0;
+        dst[c] = *reinterpret_cast<const uint4 *>(wxb + (e0 + cc * EPC) * ESZ);
+      }
+      flag = flagb[(long long)browc * flag_sb + (p.reset ? t : 0)];
+    };
+    auto put = [&](int it, const uint4 (&src)[WCH], uint32_t flag_next, int it_next) {
+      const int t = it / MT;
+      const int mt = it - t * MT;
+      const bool row_ok = rowbase + mt * 16 + fb < rend;
+      float *dst = &wxs[it & 1][fg][fb * kTileStride];
+#pragma unroll
+      for (int c = 0; c < WCH; ++c) {
+        uint4 v = src[c];
+        if (!row_ok || a0 + c * EPC >= dh) v = make_uint4(0, 0, 0, 0);
+        if (BF16) {
+          f32x4 lo, hi;
+          lo[0] = bf16_bits_to_float(v.x & 0xFFFFu); lo[1] = bf16_bits_to_float(v.x >> 16);
+          lo[2] = bf16_bits_to_float(v.y & 0xFFFFu); lo[3] = bf16_bits_to_float(v.y >> 16);
+          hi[0] = bf16_bits_to_float(v.z & 0xFFFFu); hi[1] = bf16_bits_to_float(v.z >> 16);
+          hi[2] = bf16_bits_to_float(v.w & 0xFFFFu); hi[3] = bf16_bits_to_float(v.w >> 16);
+          *reinterpret_cast<f32x4 *>(dst + c * 8) = lo;
+          *reinterpret_cast<f32x4 *>(dst + c * 8 + 4) = hi;
+        } else {
+          *reinterpret_cast<uint4 *>(dst + c * 4) = v;
+        }
+      }
+      // reset flag of the NEXT iteration (needed before that iteration's MFMA)
+      const int tn = it_next / MT;
+      const int mtn = it_next - tn * MT;
+      const bool rown_ok = it_next < NIT && rowbase + mtn * 16 + fb < rend;
+      if (fg == 0) rfl[it_next & 3][fb] = rown_ok ? (flag_next & flag_on) : 0u;
+    };
+
+#pragma unroll
+    for (int u = 0; u < kLookahead; ++u) issue(u, ring[u], fring[u]);
+    if (fg == 0) rfl[0][fb] = (rowbase + fb < rend) ? (fring[0] & flag_on) : 0u;
+    lds_barrier();  // prologue barrier
+#ifdef XS_PROFILE
+    long long fprof[3] = {0, 0, 0};
+    long long ft = clock64();
+#define XS_FTICK(i) do { const long long now_ = clock64(); fprof[i] += now_ - ft; ft = now_; } while (0)
+#else
+#define XS_FTICK(i) do { } while (0)
+#endif
+    for (int it0 = 0; it0 < NITpad; it0 += kLookahead) {
+#pragma unroll
+      for (int u = 0; u < kLookahead; ++u) {
+        const int it = it0 + u;
+        put(it, ring[u], fring[(u + 1) % kLookahead], it + 1);
+        XS_FTICK(0);
+        issue(it + kLookahead, ring[u], fring[u]);
+        XS_FTICK(1);
+        lds_barrier();  // barrier #it
+        XS_FTICK(2);
+      }
+    }
+    lds_barrier();  // final barrier
+#ifdef XS_PROFILE
+    if (lane == 0 && member == 0 && gi == 0) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 4 * 8;
+      for (int i = 0; i < 3; ++i) dst[i] = fprof[i];
+    }
+#endif
+    return;
+  }
+
+  // =========================================================================
+  // wave 5: drainer.  h of iteration it is staged in LDS by the compute waves
+  // between barriers #it and #it+1; it is written to HBM two iterations later.
+  // =========================================================================
+  if (wave == 5) {
+    const int drow = lane >> 2;   // batch row inside the tile
+    const int dq = lane & 3;      // which 4 of the 16 units
+    bool dcross = false;
+    auto drain = [&](int it, bool publish) {
+      const int t = it / MT;
+      const int mt = it - t * MT;
+      const int brow = rowbase + mt * 16 + drow;
+      const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
+      if (kDrainerPublishes && publish) {
+        // h_t of this tile goes to the exchange ring from here, and the words of h_{t-2} are re-armed,
+        // so the compute waves wait on nothing but their polls.  Every lane stores: words outside
+        // the batch or the head belong to this member's block and are never polled.
+        constexpr int TB = 16 * 16 * ESZ;  // one member's tile; a ring slot is [row tile][member][16 rows][16 units]
+        const int xsl = p.G * MT * TB;
+        char *const blk = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xsl + ((long long)mt * p.G + member) * TB +
+                          (drow * 16 + dq * 4) * ESZ;
+        unsigned long long *cur = reinterpret_cast<unsigned long long *>(blk + (t % kRing) * xsl);
+        unsigned long long *old = reinterpret_cast<unsigned long long *>(blk + ((t + kRing - 2) % kRing) * xsl);
+        unsigned long long w0, w1 = 0;
+        if (BF16) {
+          w0 = (unsigned long long)(float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16)) |
+               ((unsigned long long)(float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16)) << 32);
+        } else {
+          w0 = (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32);
+          w1 = (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32);
+        }
+        if (dcross) {
+          __hip_atomic_store(cur, w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (!BF16) __hip_atomic_store(cur + 1, w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(old, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (!BF16) __hip_atomic_store(old + 1, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          cur[0] = w0;
+          if (!BF16) cur[1] = w1;
+          old[0] = ~0ull;
+          if (!BF16) old[1] = ~0ull;
+        }
+      }
+      if (brow < rend && a0 + dq * 4 < dh) {
+        const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
+        if (BF16) {
+          uint2 w;
+          w.x = float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16);
+          w.y = float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16);
+          *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = w;
+        } else {
+          *reinterpret_cast<f32x4 *>(reinterpret_cast<float *>(p.h_out) + o) = v;
+        }
+      }
+    };
+    lds_barrier();  // prologue barrier
+    dcross = cross_s != 0u;
+#ifdef XS_PROFILE
+    long long dprof[2] = {0, 0};
+    long long dt = clock64();
+#endif
+    if (kDrainerPublishes) {
+      // iteration j leaves as soon as the four compute waves have staged it (they raise their
+      // counters after the LDS write): the peers fetch a tile two iterations before they use it
+      bool gave_up = false;
+      for (int j = 0; j < NITpad; ++j) {
+        lds_barrier();  // barrier #j
+#ifdef XS_PROFILE
+        { const long long now_ = clock64(); dprof[1] += now_ - dt; dt = now_; }
+#endif
+        if (j < NIT) {
+          long long spins = 0;
+          while (!gave_up) {
+            const uint32_t want = (uint32_t)j + 1u;
+            const uint32_t f0 = __hip_atomic_load(&pubflag[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f1 = __hip_atomic_load(&pubflag[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f2 = __hip_atomic_load(&pubflag[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            const uint32_t f3 = __hip_atomic_load(&pubflag[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (f0 >= want && f1 >= want && f2 >= want && f3 >= want) break;
+            __builtin_amdgcn_s_sleep(1);
+            if (++spins >= spin_limit) {  // cannot happen while the compute waves run; never wait forever
+              gave_up = true;
+              if (lane == 0 && atomicExch(&p.status->aborted, 1u) == 0u) {
+                p.status->abort_wg = (uint32_t)wg;
+                p.status->abort_step = (uint32_t)(j / MT);
+              }
+            }
+          }
+          drain(j, true);
+        }
+#ifdef XS_PROFILE
+        { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
+#endif
+      }
+      lds_barrier();  // final barrier
+    } else {
+    for (int j = 0; j < NITpad; ++j) {
+      if (j >= 2 && j - 2 < NIT) drain(j - 2, true);
+#ifdef XS_PROFILE
+      { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
+#endif
+      lds_barrier();  // barrier #j
+#ifdef XS_PROFILE
+      { const long long now_ = clock64(); dprof[1] += now_ - dt; dt = now_; }
+#endif
+    }
+    lds_barrier();  // final barrier
+    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it, false);
+    }
+#ifdef XS_PROFILE
+    if (lane == 0 && member == 0 && gi == 0) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
+      for (int i = 0; i < 2; ++i) dst[i] = dprof[i];
+    }
+#endif
+    return;
+  }
+
+  // =========================================================================
+  // waves 0-3: compute
+  // =========================================================================
+  __builtin_amdgcn_s_setprio(3);
+  const int q = lane >> 4;     // lane group: which 16-byte chunk of a 4-chunk K slab
+  const int r16 = lane & 15;   // MFMA row (A) / column (B, C)
+
+  // ---- R slice -> registers (once).  B operand: column n = unit a0 + r16 of gate g,
+  //      K chunk c of this wave/lane group.
+  uint4 rreg[4][NCH];
+  {
+    const int a = a0 + r16;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int k0 = wave * KW + c * 4 * EPC + q * EPC;
+        uint4 v = make_uint4(0, 0, 0, 0);
+        if (a < dh && k0 < dh) {
+          const long long off = ((long long)head * 4 * dh + (long long)g * dh + a) * dh + k0;
+          if (BF16) {
+            if (p.r_bf16) {
+              v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.r) + off);
+            } else {
+              const float4 lo = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.r) + off);
+              const float4 hi = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.r) + off + 4);
+              v.x = pack_bf16x2(lo.x, lo.y); v.y = pack_bf16x2(lo.z, lo.w);
+              v.z = pack_bf16x2(hi.x, hi.y); v.w = pack_bf16x2(hi.z, hi.w);
+            }
+          } else {
+            v = *reinterpret_cast<const uint4 *>(reinterpret_cast<const float *>(p.r) + off);
+          }
+        }
+        rreg[g][c] = v;
+      }
+    }
+  }
+
+  // ---- pointwise role: one (batch row, unit) element per thread and batch tile
+  const int pa = tid & 15;  // unit inside the workgroup's 16
+  const int pb = tid >> 4;  // batch row inside the tile
+  const int ua = a0 + pa;
+  const bool unit_ok = ua < dh;
+  const int col = head * dh + ua;  // column in [.., H]
+  float bias_g[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) bias_g[g] = unit_ok ? p.bias[((long long)head * 4 + g) * dh + ua] : 0.0f;
+
+  CellState st[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int brow = rowbase + mt * 16 + pb;
+    st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+    if (p.s0 && unit_ok && brow < rend) {
+      const long long o = (long long)brow * H + col;
+      st[mt].y = p.s0[o]; st[mt].c = p.s0[BH + o]; st[mt].n = p.s0[2 * BH + o]; st[mt].m = p.s0[3 * BH + o];
+    }
+  }
+
+  bool aborted = false;
+  uint32_t max_spins = 0;
+  int it = 0;  // (t, mt) iteration counter, selects the LDS buffers
+#ifdef XS_PROFILE
+  long long prof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+#define XS_TICK(i) do { const long long now_ = clock64(); prof[i] += now_ - tick_; tick_ = now_; } while (0)
+  long long tick_ = clock64();
+#else
+#define XS_TICK(i) do { } while (0)
+#endif
+
+  lds_barrier();  // prologue barrier: reset flags of iteration 0 and the placement verdict are in LDS
+  const bool cross = cross_s != 0u;
+
+  // exchange ring layout [head group][slot][member][ROWS][16 units]: what a group publishes in
+  // one step is contiguous (512 B per member for bf16, one tile), which spreads a step's polls
+  // over all L2 channels (measured: lines 256 B .. 2 KiB apart are served 1.5x faster than
+  // lines 4 KiB or more apart)
+  constexpr int XBLOCK = ROWS * 16 * ESZ;            // bytes one member publishes per step
+  constexpr int XTILE = 16 * 16 * ESZ;               // ... per row tile
+  const int xslot = p.G * XBLOCK;                    // bytes one group publishes per step
+  // a slot is laid out [row tile][member][16 rows][16 units]: what the group publishes for one row
+  // tile is contiguous, so the polls of an iteration spread over all L2 channels
+  char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
+
+  // With several row tiles per workgroup (MT > 1) the polls of the NEXT (t, mt) iteration are
+  // issued right after the MFMAs of the current one have consumed the operand registers: the
+  // peers published that tile MT - 1 iterations ago, so the data is there and the exchange
+  // latency hides behind barrier, gating and publish.  The completion check, the re-arm and
+  // their order are unchanged.  (With MT == 1 the tile is published only at the end of the
+  // peers' current iteration, so there is nothing to fetch early.)
+  uint4 areg[NCH];
+  bool prefetched = false;
+  // poll address of chunk c of row tile mt = per-lane part (one register) + a compile-time constant:
+  // unit k of row r of row tile mt lives at [mt][member k/16][r][k%16]
+  const int xlane = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
+  const int xtile_stride = p.G * XTILE;
+  auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
+  auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
+  for (int t = 0; t < p.T; ++t) {
+    // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
+    // (the descriptor ends with the slot: a chunk past the last member reads zeros)
+    const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
+        xbase + ((t + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
+    char *const hcur = xbase + (t % kRing) * xslot;
+    char *const hold = xbase + ((t + kRing - 2) % kRing) * xslot;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt, ++it) {
+      // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
+      XS_TICK(5);
+      const int arow = rowbase + mt * 16 + r16;
+      bool need[NCH];
+      const bool row_ok = arow < rend;
+      const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        const int k0 = wave * KW + c * 4 * EPC + q * EPC;
+        if (!(MT > 1 && prefetched)) areg[c] = make_uint4(0, 0, 0, 0);
+        need[c] = row_ok && k0 < dh;
+      }
+      if (t == 0) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          const int k0 = wave * KW + c * 4 * EPC + q * EPC;
+          if (need[c] && p.s0) {
+            const float *src = p.s0 + (long long)arow * H + head * dh + k0;
+            if (BF16) {
+              const float4 lo = *reinterpret_cast<const float4 *>(src);
+              const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
+              areg[c].x = pack_bf16x2(lo.x, lo.y); areg[c].y = pack_bf16x2(lo.z, lo.w);
+              areg[c].z = pack_bf16x2(hi.x, hi.y); areg[c].w = pack_bf16x2(hi.z, hi.w);
+            } else {
+              areg[c] = *reinterpret_cast<const uint4 *>(src);
+            }
+          }
+        }
+      } else {
+        if (kDeepPrefetch) {
+          // this tile was requested two iterations ago; the only younger requests are the NCH of the next tile
+#ifdef XS_PROFILE
+          const long long w0_ = clock64();
+#endif
+          if (it + 1 < NIT) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NCH) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#ifdef XS_PROFILE
+          prof[7] += clock64() - w0_;
+#endif
+#pragma unroll
+          for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
+        } else if (MT == 1) {
+          // Two polls in flight, about half a round trip apart (kPollStagger), re-issued alternately:
+          // a poll returns every ~300 cycles instead of every ~600, which halves both the wait for h
+          // and the skew between the four waves at the barrier.  Lanes whose batch row does not exist
+          // ask for an offset past the descriptor's end: zeros, no memory traffic, so the doubled poll
+          // rate stays far below what a compute unit can pull from the L2.  The decisions are
+          // wave-uniform (ballot) so that the waits keep exact counts.
+          const int xl = row_ok ? xlane : 0x7FFFFF00;
+          uint4 breg[NCH];
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+          __builtin_amdgcn_s_sleep(kPollStagger);
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+          if (!aborted) {
+            uint32_t spins = 0;
+            for (;;) {
+              uint32_t ma = 0u;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c) ma = mark_join<BF16>(ma, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(ma)) == 0ull) break;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c)
+                areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+              uint32_t mb = 0u;
+#pragma unroll
+              for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, need[c] ? chunk_mark<BF16>(breg[c]) : 0u);
+              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mb)) == 0ull) {
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) areg[c] = breg[c];
+                break;
+              }
+#pragma unroll
+              for (int c = 0; c < NCH; ++c)
+                breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+              spins += 2;
+              if ((spins & 1023u) == 0u &&
+                  __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+                aborted = true;
+                break;
+              }
+              if ((long long)spins >= spin_limit) {
+                aborted = true;
+                if (atomicExch(&p.status->aborted, 1u) == 0u) {
+                  p.status->abort_wg = (uint32_t)wg;
+                  p.status->abort_step = (uint32_t)t;
+                }
+                break;
+              }
+            }
+            max_spins = spins > max_spins ? spins : max_spins;
+#ifdef XS_PROFILE
+            prof[6] += spins;
+#endif
+          }
+        } else {
+          // every lane loads every chunk (no divergent branches on the way to the MFMAs); what is
+          // not needed is left out of the test below and zeroed afterwards
+          if (!(MT > 1 && prefetched)) {
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+              areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
+          }
+        }
+        // (tiles fetched ahead through LDS are checked once outside the loop: inside it the wave
+        // waits for ALL of its outstanding loads, the next tile's requests included)
+        // first look at everything at once: one mark over all chunks this lane needs
+        uint32_t mark = 0u;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+        if (!aborted && mark_has_sentinel<BF16>(mark)) {
+          uint32_t spins = 0;
+          for (;;) {
+            bool any_bad = false;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+              if (need[c]) {
+                const bool bad = BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
+                if (bad) {
+                  any_bad = true;
+                  areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
+                }
+              }
+            }
+            if (!any_bad) break;
+            ++spins;
+            if ((spins & 1023u) == 0u &&
+                __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+              aborted = true;
+              break;
+            }
+            if ((long long)spins >= spin_limit) {
+              aborted = true;
+              if (atomicExch(&p.status->aborted, 1u) == 0u) {
+                p.status->abort_wg = (uint32_t)wg;
+                p.status->abort_step = (uint32_t)t;
+              }
+              break;
+            }
+          }
+          max_spins = spins > max_spins ? spins : max_spins;
+#ifdef XS_PROFILE
+          prof[6] += spins;
+#endif
+        }
+      }
+      // (a whole wave rarely has anything to clear: one uniform branch instead of 4 selects per chunk)
+      bool clear_any = row_reset;
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) clear_any |= !need[c];
+      if (__builtin_amdgcn_ballot_w64(clear_any) != 0ull) {
+#pragma unroll
+        for (int c = 0; c < NCH; ++c)
+          if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
+      }
+
+      // ---- 2. partial R.h over this wave's K slab, all four gates
+      XS_TICK(0);
+      f32x4 acc[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < NCH; ++c) {
+        if (BF16) {
+          const bf16x8 av = __builtin_bit_cast(bf16x8, areg[c]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, rreg[g][c]), acc[g], 0, 0, 0);
+        } else {
+          const uint32_t aw[4] = {areg[c].x, areg[c].y, areg[c].z, areg[c].w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const uint32_t bw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
+              acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[g], 0, 0, 0);
+            }
+          }
+        }
+      }
+
+      if (kDeepPrefetch) {
+        // request the tile of iteration it + 2 (its LDS slot is the one just read); step 0 takes its
+        // operand from s0.  A chunk past the last member reads zeros (the descriptor ends with the slot).
+        const int nmt = (mt + 2) % MT;
+        const int nt = t + (mt + 2 >= MT ? 1 : 0);
+        if (nt >= 1 && nt < p.T) {
+          const unsigned long long sb = reinterpret_cast<unsigned long long>(xbase + ((nt + kRing - 1) % kRing) * xslot);
+          const u32x4_t rs = {uniform((uint32_t)sb), uniform((uint32_t)(sb >> 32) & 0xFFFFu), uniform((uint32_t)xslot), 0x00020000u};
+          const uint32_t lds0 = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(it, 0)));
+#pragma unroll
+          for (int c = 0; c < NCH; ++c) lds_direct_load_b128(rs, lds0 + (c << 10), xlane, xconst(c, nmt));
+        }
+      } else if (MT > 1) {
+        // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
+        const int nmt = (mt + 1) % MT;
+        const int nt = t + (mt + 1 == MT ? 1 : 0);
+        prefetched = nt >= 1 && nt < p.T;
+        if (prefetched) {
+          // unconditional loads (a select on the loaded value would make the wave wait for it right
+          // here); the descriptor ends with the slot, so a chunk past the last member reads zeros,
+          // and chunks that are not needed are zeroed when consumed
+          const __amdgpu_buffer_rsrc_t hrn = __builtin_amdgcn_make_buffer_rsrc(
+              xbase + ((nt + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrn, xlane, xconst(c, nmt), 16));
+        }
+      }
+
+      // ---- 3. partial tiles -> LDS.  C layout: lane holds unit column r16, batch rows 4q..4q+3
+      const int buf = it & 1;
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<f32x4 *>(&part[buf][wave][g][r16 * kTileStride + 4 * q]) = acc[g];
+      XS_TICK(1);
+      lds_barrier();  // barrier #it
+      XS_TICK(2);
+
+      // ---- 4. reduce over waves + exponential gating for element (row pb, unit pa)
+      float raw[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
+        float ry = part[buf][0][g][pa * kTileStride + pb];
+        ry += part[buf][1][g][pa * kTileStride + pb];
+        ry += part[buf][2][g][pa * kTileStride + pb];
+        ry += part[buf][3][g][pa * kTileStride + pb];
+        raw[g] = (wxs[buf][g][pb * kTileStride + pa] + ry) + bias_g[g];
+      }
+      if (rfl[it & 3][pb] != 0u) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+      slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
+#ifdef XS_PROFILE
+      asm volatile("" :: "v"(st[mt].y));
+#endif
+      XS_TICK(3);
+      // ---- 5. publish h_t to the peers, re-arm the words of h_{t-2}, stage h_t for the drainer
+      float y = st[mt].y;
+      if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
+      // (With four row tiles the drainer wave publishes: see there.)  Every lane stores, every
+      // iteration: lanes outside the batch or the head write words of their own block that nobody
+      // polls, and the re-arm of steps 0 and 1 hits slots that still hold the pattern.
+      if (!kDrainerPublishes) {
+        const long long xo = ((long long)mt * p.G + member) * (XTILE / ESZ) + pb * 16 + pa;
+        if (BF16) {
+          const uint16_t v = (uint16_t)float_to_bf16_bits(y);
+          uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
+          uint16_t *old = reinterpret_cast<uint16_t *>(hold) + xo;
+          if (cross) {
+            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          } else {
+            *dst = v;
+            *old = (uint16_t)kSentinel16;
+          }
+        } else {
+          float *dst = reinterpret_cast<float *>(hcur) + xo;
+          float *old = reinterpret_cast<float *>(hold) + xo;
+          if (cross) {
+            __hip_atomic_store(dst, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          } else {
+            *dst = y;
+            *old = __uint_as_float(kSentinel32);
+          }
+        }
+      }
+      hst[it & 3][tid] = y;
+      if (kDrainerPublishes && lane == 0)
+        __hip_atomic_store(&pubflag[wave], (uint32_t)it + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      XS_TICK(4);
+    }
+  }
+  for (int j = NIT; j < NITpad; ++j) lds_barrier();  // padding iterations of the feeder
+  lds_barrier();                                     // final barrier
+#ifdef XS_PROFILE
+  if (lane == 0 && member == 0 && gi == 0) {
+    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + wave * 8;
+    for (int i = 0; i < 8; ++i) dst[i] = prof[i];
+  }
+#endif
+
+  // ---- final state
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int brow = rowbase + mt * 16 + pb;
+    if (unit_ok && brow < rend) {
+      const long long o = (long long)brow * H + col;
+      p.s_out[o] = st[mt].y; p.s_out[BH + o] = st[mt].c; p.s_out[2 * BH + o] = st[mt].n; p.s_out[3 * BH + o] = st[mt].m;
+    }
+  }
+  if (lane == 0 && max_spins) atomicMax(&p.status->max_spins, max_spins);
+}
+
+}  // namespace

@@ -1,0 +1,414 @@
+// The decode step kernel (T = 1).  Included by slstm_hip.hip only (one translation unit),
+// after slstm_device_common.h.
+#pragma once
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// decode step kernel, LDS-staged: a workgroup owns 64 batch rows x 32 units x 4 gates.
+// K is walked in slabs of SLABCH MFMA k-steps (WIDE: 64 bf16 / 32 fp32 input units, so that
+// every global load instruction moves whole 128-byte lines); each slab of h (converted to the
+// operand type) and of R goes to LDS, double-buffered, one barrier per slab, and the global
+// loads of up to kStepRing slabs are in flight at once (all of them at dh = 256).  The product
+// is formed transposed (units on the MFMA M axis), so a lane ends with 4 consecutive units of
+// one batch row and the state, W.x and h move as 16-byte / 8-byte accesses that are issued
+// before the K loop and consumed after it.  The slabs are accumulated in the sequence kernel's
+// four K quarters and the quarters are added in its order, so step-by-step decoding
+// reproduces a sequence call bit for bit.
+// ---------------------------------------------------------------------------
+struct StepParams {
+  const void *wx;
+  long long wx_sb;
+  const void *r;
+  int r_bf16;
+  const float *bias;
+  const float *s0;
+  const unsigned char *reset;
+  long long reset_sb;
+  void *h_out;
+  float *s_out;
+  xs_slstm_status *status;
+  int B, NH, dh;
+  int n_unit_tiles, n_row_tiles;
+};
+
+// Workgroup i runs on XCD i % 8.  The workgroups of one head share its h rows and its R, so they
+// are placed on as few XCDs as possible (one when there are 8 or more heads): every operand is
+// then fetched from HBM once and re-read from ONE L2 instead of being fetched by all eight.
+__device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &head, int &ut, int &rt) {
+  const int tiles = p.n_unit_tiles * p.n_row_tiles;
+  int tile;
+  if (p.NH % 8 == 0) {
+    const int hpx = p.NH / 8;  // heads per XCD
+    const int m = i >> 3;
+    head = (i & 7) * hpx + m % hpx;
+    tile = m / hpx;
+  } else if (8 % p.NH == 0 && tiles % (8 / p.NH) == 0) {
+    const int xph = 8 / p.NH;  // XCDs per head
+    head = (i & 7) % p.NH;
+    tile = (i >> 3) * xph + (i & 7) / p.NH;
+  } else {
+    head = i / tiles;
+    tile = i - head * tiles;
+  }
+  ut = tile % p.n_unit_tiles;
+  rt = tile / p.n_unit_tiles;
+}
+
+// FULL: the tile lies entirely inside the problem (64 rows, 32 units, every K slab), there is an
+// initial state and no reset mask - the decode steady state.  All clamping and masking is then
+// compiled out, which matters: the kernel is bound by the number of instructions a wave issues.
+// SLABCH = MFMA k-steps per slab.  With 4 (dh <= 128) or 8 (dh <= 256, bf16) the whole K range
+// is ONE slab: everything is staged once, one barrier, and the registers that carried the
+// loads are free again before the MFMA loop (which then batches its LDS reads).
+template <bool BF16, int SLABCH, bool FULL>
+__global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
+  constexpr int EPC = BF16 ? 8 : 4;
+  constexpr int CHK = 4 * EPC;                // input units per MFMA k-step ("chunk")
+  constexpr int SLABK = SLABCH * CHK;         // input units per slab
+  constexpr int kStepRing = SLABCH >= 4 ? 1 : 4;  // slabs whose loads are in flight
+  constexpr int NBUF = SLABCH >= 4 ? 1 : 2;       // LDS buffers
+  constexpr int RS = SLABCH * 64 + 16;        // bytes per LDS row: data + pad (conflict-free 16-byte reads)
+  constexpr int HITEMS = (SLABK * 4 / 16) / 4;  // 16-byte pieces of fp32 h each thread stages per slab
+  constexpr int RITEMS = SLABCH * 2;            // 16-byte pieces of R each thread stages per slab
+  constexpr int ESZ = BF16 ? 2 : 4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char step_lds[];
+  unsigned char(*hbuf)[64 * RS] = reinterpret_cast<unsigned char(*)[64 * RS]>(step_lds);
+  unsigned char(*rbuf)[128 * RS] = reinterpret_cast<unsigned char(*)[128 * RS]>(step_lds + NBUF * 64 * RS);
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6;
+  const int lane = tid & 63;
+  const int q = lane >> 4;
+  const int r16 = lane & 15;
+  int head, unit_tile, row_tile;
+  step_tile_of(p, blockIdx.x, head, unit_tile, row_tile);
+  const int a0 = unit_tile * 32;
+  const int rowbase = row_tile * 64;
+  const int dh = p.dh;
+  const int H = p.NH * dh;
+  const long long BH = (long long)p.B * H;
+  const int nch = 1 << nch_log2;              // chunks per K quarter (as in the sequence kernel)
+  const int nslab = (4 * nch) / SLABCH;
+
+  if (blockIdx.x == 0 && tid < 16)
+    reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
+
+  const bool has_s0 = FULL || p.s0 != nullptr;
+  const bool has_reset = !FULL && p.reset != nullptr;
+  const float *s0p = has_s0 ? p.s0 : reinterpret_cast<const float *>(p.wx);                  // stand-ins are only read
+  const unsigned char *rsp = has_reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);  // in their first 32 bytes
+
+  // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row / column.
+  // A single slab is staged in NSPLIT phases (K halves): a thread's first HITEMS / NSPLIT items
+  // lie in the first half of K, so the MFMA loop can start on it while the second half lands.
+  constexpr int HPIECES = SLABK * 4 / 16;     // 16-byte pieces of fp32 h per row and slab
+  constexpr int RPIECES = SLABCH * 4;         // 16-byte pieces of R per column and slab
+  constexpr int NSPLIT = SLABCH >= 4 ? 2 : 1;
+  constexpr int HPP = HPIECES / NSPLIT, HIP = HITEMS / NSPLIT;  // pieces per row, items per thread: per phase
+  constexpr int RPP = RPIECES / NSPLIT, RIP = RITEMS / NSPLIT;
+  auto hrow_of = [&](int j) { return (tid + 256 * (j % HIP)) / HPP; };
+  auto hpiece_of = [&](int j) { return (j / HIP) * HPP + (tid + 256 * (j % HIP)) % HPP; };
+  auto rcol_of = [&](int j) { return (tid + 256 * (j % RIP)) / RPP; };
+  auto rpiece_of = [&](int j) { return (j / RIP) * RPP + (tid + 256 * (j % RIP)) % RPP; };
+  const float *hsrc[HITEMS];
+  bool hzero[HITEMS];
+#pragma unroll
+  for (int j = 0; j < HITEMS; ++j) {
+    const int brow = rowbase + hrow_of(j);
+    if (FULL) {
+      hzero[j] = false;
+      hsrc[j] = s0p + (long long)brow * H + head * dh + hpiece_of(j) * 4;
+    } else {
+      const int browc = brow < p.B ? brow : p.B - 1;
+      const uint32_t flag = rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+      hzero[j] = !(brow < p.B) || !has_s0 || (has_reset && flag != 0u);
+      hsrc[j] = s0p + (has_s0 ? (long long)browc * H + head * dh : 0);
+    }
+  }
+  const char *rsrc[RITEMS];
+  bool rok[RITEMS];
+#pragma unroll
+  for (int j = 0; j < RITEMS; ++j) {
+    const int colx = rcol_of(j);                  // column of the workgroup's 128: gate colx/32, unit colx%32
+    const int a = a0 + (colx & 31);
+    rok[j] = FULL || a < dh;
+    rsrc[j] = reinterpret_cast<const char *>(p.r) +
+              ((long long)head * 4 * dh + (long long)(colx >> 5) * dh + (rok[j] ? a : 0)) * dh * ESZ +
+              (FULL ? rpiece_of(j) * 16 : 0);
+  }
+  uint4 hring[kStepRing][HITEMS], rring[kStepRing][RITEMS];
+  auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS]) {
+    const int kbase = sidx * SLABK;
+#pragma unroll
+    for (int ph = 0; ph < NSPLIT; ++ph) {
+#pragma unroll
+      for (int j = ph * HIP; j < (ph + 1) * HIP; ++j) {
+        if (FULL) {
+          hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase);
+        } else {
+          const int k = kbase + hpiece_of(j) * 4;
+          hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + ((has_s0 && k < dh) ? k : 0));
+        }
+      }
+#pragma unroll
+      for (int j = ph * RIP; j < (ph + 1) * RIP; ++j) {
+        if (FULL) {
+          rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + kbase * ESZ);
+        } else {
+          const int k = kbase + rpiece_of(j) * EPC;
+          rst[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)(k < dh ? k : 0) * ESZ);
+        }
+      }
+    }
+  };
+  // phase < 0: the whole slab; otherwise the items of that K phase only
+  auto store_slab = [&](int sidx, int buf, const uint4 (&hst)[HITEMS], const uint4 (&rst)[RITEMS], int phase) {
+    const int kbase = sidx * SLABK;
+#pragma unroll
+    for (int j = 0; j < HITEMS; ++j) {
+      if (phase >= 0 && j / HIP != phase) continue;
+      const int piece = hpiece_of(j);
+      uint4 v = hst[j];
+      if (!FULL && (hzero[j] || kbase + piece * 4 >= dh)) v = make_uint4(0, 0, 0, 0);
+      unsigned char *dst = &hbuf[buf][hrow_of(j) * RS];
+      if (BF16) {
+        uint2 w;
+        w.x = pack_bf16x2(__uint_as_float(v.x), __uint_as_float(v.y));
+        w.y = pack_bf16x2(__uint_as_float(v.z), __uint_as_float(v.w));
+        *reinterpret_cast<uint2 *>(dst + piece * 8) = w;
+      } else {
+        *reinterpret_cast<uint4 *>(dst + piece * 16) = v;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < RITEMS; ++j) {
+      if (phase >= 0 && j / RIP != phase) continue;
+      const int piece = rpiece_of(j);
+      uint4 w = rst[j];
+      if (!FULL && (!rok[j] || kbase + piece * EPC >= dh)) w = make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4 *>(&rbuf[buf][rcol_of(j) * RS + piece * 16]) = w;
+    }
+  };
+
+#ifdef XS_PROFILE
+  long long pstamp[6];
+  pstamp[0] = clock64();
+  const long long pwall0 = wall_clock64();
+#endif
+#pragma unroll
+  for (int u = 0; u < kStepRing; ++u)
+    if (u < nslab) load_slab(u, hring[u], rring[u]);
+
+  // ---- wave tiling 2 x 2: wave (wr, wu) owns rows 32*wr .. +31 (two MFMA row tiles, index ut below)
+  // and units 16*wu .. +15 of all four gates, so a k-step reads 2 h and 4 R fragments from LDS for
+  // its 8 MFMAs.  Pointwise operands of this lane: batch rows rowbase + 32*wr + 16*ut + r16,
+  // units a0 + 16*wu + 4q .. +3.
+  const int wr = wave >> 1, wu = wave & 1;
+  const int ua = a0 + wu * 16 + 4 * q;
+  const int uac = (FULL || ua < dh) ? ua : 0;
+  const long long col = (long long)head * dh + uac;
+  uint2 wxb[2][4];
+  float4 wxf[2][4], bias4[4], c4[2], n4[2], m4[2];
+  uint32_t pflag[2];
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+    bias4[g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    const int brow = rowbase + 32 * wr + 16 * ut + r16;
+    const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
+    pflag[ut] = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
+      if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
+      else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
+    }
+    const long long so = (long long)browc * H + col;
+    c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
+    n4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 2 * BH + so : 0));
+    m4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 3 * BH + so : 0));
+  }
+
+  // ---- K loop
+  f32x4 acc[2][4], tot[2][4];
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
+
+#ifdef XS_PROFILE
+  pstamp[1] = clock64();
+#endif
+  store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
+  __syncthreads();
+#ifdef XS_PROFILE
+  pstamp[2] = clock64();
+#endif
+  if (SLABCH >= 4) {
+    // single slab: the number of chunks per K quarter is the compile-time constant SLABCH / 4 ->
+    // straight-line MFMA code; the second K half goes to LDS after the MFMAs of the first
+    constexpr int NQ = SLABCH / 4;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      if (w == 2) {
+        store_slab(0, 0, hring[0], rring[0], 1);
+        __syncthreads();
+      }
+#pragma unroll
+      for (int cq = 0; cq < (NQ > 0 ? NQ : 1); ++cq) {
+        const int ch = w * NQ + cq;
+        uint4 hv[2], rv[4];
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut)
+          hv[ut] = *reinterpret_cast<const uint4 *>(&hbuf[0][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          rv[g] = *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            if (BF16) {
+              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
+            } else {
+              const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w};
+              const uint32_t hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+            }
+          }
+      }
+#pragma unroll
+      for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {  // fold the quarter into the running sum (quarter 0 first)
+          tot[ut][g] = (w == 0) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+          acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+  } else {
+  for (int s0i = 0; s0i < nslab; s0i += kStepRing) {
+#pragma unroll
+    for (int u = 0; u < kStepRing; ++u) {
+      const int sidx = s0i + u;
+      if (sidx < nslab) {
+        const int buf = sidx & (NBUF - 1);
+#pragma unroll
+        for (int ch = 0; ch < SLABCH; ++ch) {
+          uint4 hv[2], rv[4];
+#pragma unroll
+          for (int ut = 0; ut < 2; ++ut)
+            hv[ut] = *reinterpret_cast<const uint4 *>(&hbuf[buf][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            rv[g] = *reinterpret_cast<const uint4 *>(&rbuf[buf][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
+#pragma unroll
+          for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              if (BF16) {
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
+              } else {
+                const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w};
+                const uint32_t hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+              }
+            }
+          const int chunks_done = sidx * SLABCH + ch + 1;
+          if ((chunks_done & (nch - 1)) == 0) {  // end of a K quarter: fold it into the running sum (quarter 0 first)
+#pragma unroll
+            for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+              for (int g = 0; g < 4; ++g) {
+                tot[ut][g] = (chunks_done == nch) ? acc[ut][g] : tot[ut][g] + acc[ut][g];
+                acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+              }
+          }
+        }
+        // slab sidx went to LDS one iteration ago: its ring entry takes the loads of slab sidx + kStepRing
+        if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u]);
+        if (sidx + 1 < nslab) {
+          const int un = (u + 1) % kStepRing;
+          store_slab(sidx + 1, (sidx + 1) & (NBUF - 1), hring[un], rring[un], -1);  // the other buffer was last read before the previous barrier
+          __syncthreads();
+        }
+      }
+    }
+  }
+
+  }
+#ifdef XS_PROFILE
+  asm volatile("" :: "v"(tot[0][0][0]), "v"(tot[1][3][3]));
+  pstamp[3] = clock64();
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  pstamp[4] = clock64();
+#endif
+  // ---- gating
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    const int brow = rowbase + 32 * wr + 16 * ut + r16;
+    const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag[ut] != 0u));
+    const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
+    const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
+    const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
+    float yv[4], cv[4], nv[4], mv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float raw[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float wxv;
+        if (BF16) {
+          const uint32_t wd = i < 2 ? wxb[ut][g].x : wxb[ut][g].y;
+          wxv = bf16_bits_to_float((i & 1) ? (wd >> 16) : (wd & 0xFFFFu));
+        } else {
+          const float wf[4] = {wxf[ut][g].x, wxf[ut][g].y, wxf[ut][g].z, wxf[ut][g].w};
+          wxv = wf[i];
+        }
+        const float bf[4] = {bias4[g].x, bias4[g].y, bias4[g].z, bias4[g].w};
+        raw[g] = (wxv + tot[ut][g][i]) + bf[i];
+      }
+      CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
+      slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
+      yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
+    }
+    if (FULL || (brow < p.B && ua < dh)) {
+      const long long o = (long long)brow * H + head * dh + ua;
+      // streaming stores: the lines leave the L2 while the kernel still runs instead of being
+      // written back when it ends (measured: 0.65 us per step at B = 256, D = 2048)
+      __builtin_nontemporal_store(f32x4{yv[0], yv[1], yv[2], yv[3]}, reinterpret_cast<f32x4 *>(p.s_out + o));
+      __builtin_nontemporal_store(f32x4{cv[0], cv[1], cv[2], cv[3]}, reinterpret_cast<f32x4 *>(p.s_out + BH + o));
+      __builtin_nontemporal_store(f32x4{nv[0], nv[1], nv[2], nv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 2 * BH + o));
+      __builtin_nontemporal_store(f32x4{mv[0], mv[1], mv[2], mv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 3 * BH + o));
+      if (BF16) {
+        uint2 hw;
+        hw.x = float_to_bf16_bits(yv[0]) | (float_to_bf16_bits(yv[1]) << 16);
+        hw.y = float_to_bf16_bits(yv[2]) | (float_to_bf16_bits(yv[3]) << 16);
+        // (h stays an ordinary store: as a streaming store its 8-byte pieces cost 0.8 us per step)
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = hw;
+      } else {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.h_out) + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
+      }
+    }
+  }
+#ifdef XS_PROFILE
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  if (tid == 0 && blockIdx.x == 9) {
+    pstamp[5] = clock64();
+    long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
+    for (int i = 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
+  }
+  if (tid == 0) {
+    long long *wt = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 256);
+    wt[2 * blockIdx.x] = pwall0;
+    wt[2 * blockIdx.x + 1] = wall_clock64();
+  }
+#endif
+}
+
+}  // namespace
