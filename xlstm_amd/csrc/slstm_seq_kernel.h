@@ -492,6 +492,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       XS_TICK(5);
       const int arow = rowbase + mt * 16 + r16;
       bool need[NCH];
+      uint32_t needmask[NCH];
       const bool row_ok = arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
@@ -499,6 +500,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
         if (!(MT > 1 && prefetched)) areg[c] = make_uint4(0, 0, 0, 0);
         need[c] = row_ok && k0 < dh;
+        needmask[c] = need[c] ? 0xFFFFFFFFu : 0u;  // (masks, not selects: the tests below stay straight-line code)
       }
       if (t == 0) {
 #pragma unroll
@@ -550,14 +552,14 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
             for (;;) {
               uint32_t ma = 0u;
 #pragma unroll
-              for (int c = 0; c < NCH; ++c) ma = mark_join<BF16>(ma, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+              for (int c = 0; c < NCH; ++c) ma = mark_join<BF16>(ma, chunk_mark<BF16>(areg[c]) & needmask[c]);
               if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(ma)) == 0ull) break;
 #pragma unroll
               for (int c = 0; c < NCH; ++c)
                 areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
               uint32_t mb = 0u;
 #pragma unroll
-              for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, need[c] ? chunk_mark<BF16>(breg[c]) : 0u);
+              for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, chunk_mark<BF16>(breg[c]) & needmask[c]);
               if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mb)) == 0ull) {
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) areg[c] = breg[c];
@@ -600,7 +602,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         // first look at everything at once: one mark over all chunks this lane needs
         uint32_t mark = 0u;
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, need[c] ? chunk_mark<BF16>(areg[c]) : 0u);
+        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[c]) & needmask[c]);
         if (!aborted && mark_has_sentinel<BF16>(mark)) {
           uint32_t spins = 0;
           for (;;) {
