@@ -265,7 +265,9 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 
   // =========================================================================
   // wave 5: drainer.  h of iteration it is staged in LDS by the compute waves
-  // between barriers #it and #it+1; it is written to HBM two iterations later.
+  // between barriers #it and #it+1; it is written to HBM two iterations later
+  // (with four row tiles: as soon as it is staged, together with the publication
+  // of the tile in the exchange ring).
   // =========================================================================
   if (wave == 5) {
     const int drow = lane >> 2;   // batch row inside the tile
@@ -454,23 +456,23 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   lds_barrier();  // prologue barrier: reset flags of iteration 0 and the placement verdict are in LDS
   const bool cross = cross_s != 0u;
 
-  // exchange ring layout [head group][slot][member][ROWS][16 units]: what a group publishes in
-  // one step is contiguous (512 B per member for bf16, one tile), which spreads a step's polls
-  // over all L2 channels (measured: lines 256 B .. 2 KiB apart are served 1.5x faster than
-  // lines 4 KiB or more apart)
+  // exchange ring layout [head group][slot][row tile][member][16 rows][16 units]: what a group
+  // publishes for one row tile is contiguous (512 B per member for bf16), which spreads the polls
+  // of an iteration over all L2 channels (measured: lines 256 B .. 2 KiB apart are served 1.5x
+  // faster than lines 4 KiB or more apart)
   constexpr int XBLOCK = ROWS * 16 * ESZ;            // bytes one member publishes per step
   constexpr int XTILE = 16 * 16 * ESZ;               // ... per row tile
   const int xslot = p.G * XBLOCK;                    // bytes one group publishes per step
-  // a slot is laid out [row tile][member][16 rows][16 units]: what the group publishes for one row
-  // tile is contiguous, so the polls of an iteration spread over all L2 channels
   char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
 
-  // With several row tiles per workgroup (MT > 1) the polls of the NEXT (t, mt) iteration are
-  // issued right after the MFMAs of the current one have consumed the operand registers: the
-  // peers published that tile MT - 1 iterations ago, so the data is there and the exchange
-  // latency hides behind barrier, gating and publish.  The completion check, the re-arm and
-  // their order are unchanged.  (With MT == 1 the tile is published only at the end of the
-  // peers' current iteration, so there is nothing to fetch early.)
+  // How h_{t-1} is fetched depends on the number of row tiles per workgroup:
+  //   MT == 1  nothing can be fetched early (the peers publish the tile at the end of their current
+  //            iteration): two staggered polls in flight, see below;
+  //   MT == 2  the polls of the NEXT (t, mt) iteration are issued right after the MFMAs of the
+  //            current one have consumed the operand registers (the peers published that tile one
+  //            iteration ago);
+  //   MT == 4  the tile of iteration it + 2 is requested straight into LDS (kDeepPrefetch).
+  // The completion test, the re-arm and their order are the same in all three.
   uint4 areg[NCH];
   bool prefetched = false;
   // poll address of chunk c of row tile mt = per-lane part (one register) + a compile-time constant:
