@@ -127,9 +127,11 @@ int xs_slstm_forward(const xs_slstm_args *args);
 
 /*
  * Single-token decode step (T must be 1): state in, state out, no waits
- * between compute units.  The recurrent matrix must be in the dtype of wx
- * (keep a bf16 copy for bf16 decoding instead of converting it every token).  Replaces the T == 1 use of the same reference entry
- * (xlstm/blocks/slstm/layer.py:113-115 calls the cell's forward with S = 1).
+ * between compute units; bit-identical to the same step inside a sequence
+ * call.  The recurrent matrix must be in the dtype of wx (keep a bf16 copy
+ * for bf16 decoding instead of converting it every token).  Replaces the
+ * T == 1 use of the same reference entry (xlstm/blocks/slstm/layer.py:113-115
+ * calls the cell's forward with S = 1).
  */
 int xs_slstm_step(const xs_slstm_args *args);
 

@@ -46,6 +46,15 @@ def test_argument_errors_without_touching_the_gpu():
     a.T = 2
     assert lib.xs_slstm_step(ctypes.byref(a)) == -2  # step needs T == 1
     assert b"T == 1" in lib.xs_last_error()
+    # s_out may not overlap s0 anywhere (fake, never dereferenced addresses: validation comes before any launch)
+    a.T = 1
+    a.r, a.bias = 0x10000, 0x20000
+    a.s0, a.s_out = 0x100000, 0x100000 + 64  # 16 * B * NH * dh = 128 bytes each
+    assert lib.xs_slstm_step(ctypes.byref(a)) == -2 and b"overlap" in lib.xs_last_error()
+    a.s_out = 0x100000 - 64
+    assert lib.xs_slstm_step(ctypes.byref(a)) == -2 and b"overlap" in lib.xs_last_error()
+    a.s_out = 0x100000 + 128  # adjacent is fine: the next complaint is about wx / h_out
+    assert lib.xs_slstm_step(ctypes.byref(a)) == -1
 
 
 def test_workspace_bytes_is_bounded_and_monotone():

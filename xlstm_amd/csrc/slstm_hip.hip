@@ -89,7 +89,11 @@ int validate(const xs_slstm_args *a, bool step) {
   if (a->r_dtype != XS_F32 && a->r_dtype != XS_BF16) return fail(XS_ERR_DTYPE, "r_dtype %d not supported", a->r_dtype);
   if (a->wx_dtype == XS_F32 && a->r_dtype != XS_F32) return fail(XS_ERR_DTYPE, "float32 wx needs a float32 recurrent matrix");
   if (!a->r || !a->bias || !a->s_out) return fail(XS_ERR_NULL, "r, bias and s_out are required");
-  if (a->s0 && a->s0 == a->s_out) return fail(XS_ERR_SHAPE, "s_out must not alias s0");
+  if (a->s0) {  // other workgroups still read s0 while the first ones write s_out
+    const uintptr_t lo0 = (uintptr_t)a->s0, lo1 = (uintptr_t)a->s_out;
+    const uintptr_t bytes = (uintptr_t)16 * (uintptr_t)a->B * (uintptr_t)a->NH * (uintptr_t)a->dh;
+    if (lo0 < lo1 + bytes && lo1 < lo0 + bytes && bytes) return fail(XS_ERR_SHAPE, "s_out must not overlap s0");
+  }
   if (a->B > 0 && a->T > 0 && (!a->wx || !a->h_out)) return fail(XS_ERR_NULL, "wx and h_out are required");
   const int epc = a->wx_dtype == XS_BF16 ? 8 : 4;
   if (a->dh % 8 != 0) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not a multiple of 8", a->dh);
