@@ -99,7 +99,8 @@ def bench_decode(device, steps=1024, prefill=128):
     ws = F.workspace_for(B, prefill, NH, dh, device)
     _, state = F.slstm_forward(wx_pre.to(device), r, bias, None, None, workspace=ws)
     h1 = torch.empty(1, B, H, dtype=torch.bfloat16, device=device)
-    s_a, s_b = state.clone(), torch.empty_like(state)  # state ping-pong: s_out must not alias s0
+    h2 = [torch.empty(1, B, H, dtype=torch.bfloat16, device=device) for _ in range(2)]  # h ping-pong: h of step t is the
+    s_a, s_b = state.clone(), torch.empty_like(state)  # bf16 operand of step t+1.  State ping-pong: s_out must not alias s0
     for t in range(16):  # warm-up
         F.slstm_forward(wx_dec[t], r, bias, s_a, None, step=True, workspace=ws, h_out=h1, s_out=s_b)
         s_a, s_b = s_b, s_a
@@ -112,7 +113,7 @@ def bench_decode(device, steps=1024, prefill=128):
     t0 = time.perf_counter()
     e0.record()
     for t in range(steps):
-        plan(wx_dec[t], s_a, s_b, h1, stream)
+        plan(wx_dec[t], s_a, s_b, h2[t & 1], stream, h2[(t + 1) & 1] if t else None)
         s_a, s_b = s_b, s_a
     e1.record()
     torch.cuda.synchronize()
@@ -135,7 +136,8 @@ def bench_decode(device, steps=1024, prefill=128):
             def chain():
                 a, b = g_a, g_b
                 for t in range(per_graph):  # an even count: the state ends in g_a again
-                    F.slstm_forward(wx_g[t], r, bias, a, None, step=True, workspace=ws, h_out=h1, s_out=b)
+                    F.slstm_forward(wx_g[t], r, bias, a, None, step=True, workspace=ws, h_out=h2[t & 1], s_out=b,
+                                    h_prev=h2[(t + 1) & 1] if t else None)
                     a, b = b, a
             chain()  # warm-up outside the capture
             torch.cuda.synchronize()

@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 1
+#define XS_ABI_VERSION 2
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -75,6 +75,14 @@ enum {
  *                             iterations; 0 selects the default.  When a wait
  *                             runs out the kernel records it in the status block
  *                             and finishes without waiting any further.
+ *   h_prev [B, NH*dh]         optional, xs_slstm_step with bf16 wx only (ignored
+ *                             otherwise): the y plane of s0 rounded to bf16, i.e.
+ *                             the h_out of the previous step.  The kernel rounds
+ *                             y to bf16 anyway before it multiplies by r; given
+ *                             this copy it reads half the bytes and the result is
+ *                             bit for bit the same.  The caller vouches for the
+ *                             copy: it is not compared with s0.  Not in the
+ *                             reference.
  */
 typedef struct xs_slstm_args {
   int32_t B, T, NH, dh;
@@ -92,6 +100,7 @@ typedef struct xs_slstm_args {
   size_t workspace_bytes;
   void *stream;
   int64_t spin_limit;
+  const void *h_prev;
 } xs_slstm_args;
 
 /* Status block at the start of the workspace, written by the kernels. */

@@ -25,8 +25,8 @@ def test_header_symbols_are_exported():
 def test_abi_version_and_struct_mirror():
     lib = _lib.load()
     assert lib.xs_abi_version() == _lib.ABI_VERSION
-    # xs_slstm_args: 6 int32, pointers/int64 after -> 8-byte aligned, 14 more 8-byte fields
-    assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 14 * 8
+    # xs_slstm_args: 6 int32, pointers/int64 after -> 8-byte aligned, 15 more 8-byte fields
+    assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 15 * 8
     assert ctypes.sizeof(_lib.SlstmStatus) == 64
 
 

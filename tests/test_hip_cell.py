@@ -149,3 +149,33 @@ def test_step_plan_equals_the_generic_step_call():
         assert torch.equal(h, h_ref) and torch.equal(a, ref), t
     with pytest.raises(ValueError):
         plan(wx[0].float(), a, b, h)
+
+
+@pytest.mark.gpu
+def test_bf16_operand_hint_gives_the_same_bits():
+    """A decode chain that hands each step the previous step's h (already bfloat16) equals the chain without it."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(6)
+    for B, NH, dh in ((64, 2, 256), (128, 1, 128), (64, 1, 512)):  # one slab (8 and 4 k-steps), slab ring
+        H = NH * dh
+        r = ((torch.rand(NH, 4 * dh, dh, device=dev) - 0.5) * 0.3).bfloat16()
+        bias = torch.randn(NH, 4, dh, device=dev)
+        wx = torch.randn(5, B, 1, 4 * H, device=dev).bfloat16()
+        s = torch.randn(4, B, H, device=dev)
+        s[2] = s[2].abs() + 0.5
+        plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16)
+        a, b = s.clone(), torch.empty_like(s)
+        h = [torch.empty(1, B, H, dtype=torch.bfloat16, device=dev) for _ in range(2)]
+        ref = s.clone()
+        prev = None
+        for t in range(5):
+            plan(wx[t], a, b, h[t & 1], h_prev=prev)
+            h_ref, ref = F.slstm_forward(wx[t], r, bias, ref, None, step=True)
+            a, b = b, a
+            prev = h[t & 1]
+            torch.cuda.synchronize()
+            assert torch.equal(prev, h_ref) and torch.equal(a, ref), (B, NH, dh, t)

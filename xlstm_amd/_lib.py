@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 EXPORTS = (
     "xs_abi_version",
@@ -43,6 +43,7 @@ class SlstmArgs(ctypes.Structure):
         ("workspace_bytes", ctypes.c_size_t),
         ("stream", ctypes.c_void_p),
         ("spin_limit", ctypes.c_int64),
+        ("h_prev", ctypes.c_void_p),
     ]
 
 

@@ -108,8 +108,10 @@ int validate(const xs_slstm_args *a, bool step) {
   if (a->B > 0 && a->T > 0 &&
       (((uintptr_t)a->wx % al) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16)))
     return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
-  if (((uintptr_t)a->r % al) || ((uintptr_t)a->h_out % al) || ((uintptr_t)a->s0 % al) || ((uintptr_t)a->s_out % al))
-    return fail(XS_ERR_ALIGN, "r, h_out, s0 and s_out must be 16-byte aligned");
+  if (((uintptr_t)a->r % al) || ((uintptr_t)a->h_out % al) || ((uintptr_t)a->s0 % al) || ((uintptr_t)a->s_out % al) ||
+      ((uintptr_t)a->h_prev % al))
+    return fail(XS_ERR_ALIGN, "r, h_out, s0, s_out and h_prev must be 16-byte aligned");
+  if (a->h_prev && !a->s0) return fail(XS_ERR_NULL, "h_prev is a copy of the y plane of s0: s0 is required with it");
   if (!a->workspace || a->workspace_bytes < xs_slstm_workspace_bytes(a->B, a->T, a->NH, a->dh))
     return fail(XS_ERR_WORKSPACE, "workspace missing or smaller than xs_slstm_workspace_bytes()");
   if ((uintptr_t)a->workspace % 256) return fail(XS_ERR_ALIGN, "workspace must be 256-byte aligned");
@@ -178,9 +180,13 @@ int run_step(const xs_slstm_args *a) {
   const size_t lds = (size_t)nbuf * (64 + 128) * (slabch * 64 + 16);
   typedef void (*StepKernel)(StepParams, int);
   StepKernel kern;
+  const bool hint = full && bf16 && a->h_prev != nullptr;  // operand already in bf16 (h_out of the previous step)
+  p.h_prev = hint ? a->h_prev : nullptr;
 #define XS_PICK(BF, SC) (full ? slstm_step_tile_kernel<BF, SC, true> : slstm_step_tile_kernel<BF, SC, false>)
-  if (bf16) kern = slabch == 4 ? XS_PICK(true, 4) : (slabch == 8 ? XS_PICK(true, 8) : XS_PICK(true, 2));
+#define XS_PICK_HINT(SC) (hint ? slstm_step_tile_kernel<true, SC, true, true> : XS_PICK(true, SC))
+  if (bf16) kern = slabch == 4 ? XS_PICK_HINT(4) : (slabch == 8 ? XS_PICK_HINT(8) : XS_PICK_HINT(2));
   else kern = slabch == 4 ? XS_PICK(false, 4) : (slabch == 8 ? XS_PICK(false, 8) : XS_PICK(false, 2));
+#undef XS_PICK_HINT
 #undef XS_PICK
   if (lds > 64 * 1024) {  // the single-slab variant at dh = 256 needs 99 KiB of the 160 KiB of LDS
     const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);

@@ -30,6 +30,7 @@ struct StepParams {
   xs_slstm_status *status;
   int B, NH, dh;
   int n_unit_tiles, n_row_tiles;
+  const void *h_prev;  // optional bf16 copy of the y plane of s0 (see the HB variant)
 };
 
 // Workgroup i runs on XCD i % 8.  The workgroups of one head share its h rows and its R, so they
@@ -61,15 +62,20 @@ __device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &he
 // SLABCH = MFMA k-steps per slab.  With 4 (dh <= 128) or 8 (dh <= 256, bf16) the whole K range
 // is ONE slab: everything is staged once, one barrier, and the registers that carried the
 // loads are free again before the MFMA loop (which then batches its LDS reads).
-template <bool BF16, int SLABCH, bool FULL>
+// HB (only with BF16 and FULL): the recurrent operand comes from StepParams::h_prev, a bf16 copy of
+// the y plane of s0 (the h_out of the previous step), instead of being converted from float32:
+// half the bytes of the most re-read operand (every unit tile of a row tile reads all of it).
+template <bool BF16, int SLABCH, bool FULL, bool HB = false>
 __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
+  static_assert(!HB || (BF16 && FULL), "the bf16 operand hint is a steady-state bf16 path");
+  constexpr int HBYTES = HB ? 2 : 4;          // bytes per element of the recurrent operand as it is read
   constexpr int EPC = BF16 ? 8 : 4;
   constexpr int CHK = 4 * EPC;                // input units per MFMA k-step ("chunk")
   constexpr int SLABK = SLABCH * CHK;         // input units per slab
   constexpr int kStepRing = SLABCH >= 4 ? 1 : 4;  // slabs whose loads are in flight
   constexpr int NBUF = SLABCH >= 4 ? 1 : 2;       // LDS buffers
   constexpr int RS = SLABCH * 64 + 16;        // bytes per LDS row: data + pad (conflict-free 16-byte reads)
-  constexpr int HITEMS = (SLABK * 4 / 16) / 4;  // 16-byte pieces of fp32 h each thread stages per slab
+  constexpr int HITEMS = (SLABK * HBYTES / 16) / 4;  // 16-byte pieces of h each thread stages per slab
   constexpr int RITEMS = SLABCH * 2;            // 16-byte pieces of R each thread stages per slab
   constexpr int ESZ = BF16 ? 2 : 4;
   extern __shared__ __attribute__((aligned(16))) unsigned char step_lds[];
@@ -102,7 +108,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row / column.
   // A single slab is staged in NSPLIT phases (K halves): a thread's first HITEMS / NSPLIT items
   // lie in the first half of K, so the MFMA loop can start on it while the second half lands.
-  constexpr int HPIECES = SLABK * 4 / 16;     // 16-byte pieces of fp32 h per row and slab
+  constexpr int HPIECES = SLABK * HBYTES / 16;  // 16-byte pieces of h per row and slab
   constexpr int RPIECES = SLABCH * 4;         // 16-byte pieces of R per column and slab
   constexpr int NSPLIT = SLABCH >= 4 ? 2 : 1;
   constexpr int HPP = HPIECES / NSPLIT, HIP = HITEMS / NSPLIT;  // pieces per row, items per thread: per phase
@@ -116,7 +122,11 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #pragma unroll
   for (int j = 0; j < HITEMS; ++j) {
     const int brow = rowbase + hrow_of(j);
-    if (FULL) {
+    if (HB) {  // hsrc counts in float units below: a bf16 row is half as long, a 16-byte piece is 4 floats wide
+      hzero[j] = false;
+      hsrc[j] = reinterpret_cast<const float *>(reinterpret_cast<const uint16_t *>(p.h_prev) + (long long)brow * H + head * dh) +
+                hpiece_of(j) * 4;
+    } else if (FULL) {
       hzero[j] = false;
       hsrc[j] = s0p + (long long)brow * H + head * dh + hpiece_of(j) * 4;
     } else {
@@ -144,7 +154,9 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
     for (int ph = 0; ph < NSPLIT; ++ph) {
 #pragma unroll
       for (int j = ph * HIP; j < (ph + 1) * HIP; ++j) {
-        if (FULL) {
+        if (HB) {
+          hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase / 2);
+        } else if (FULL) {
           hst[j] = *reinterpret_cast<const uint4 *>(hsrc[j] + kbase);
         } else {
           const int k = kbase + hpiece_of(j) * 4;
@@ -172,7 +184,9 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
       uint4 v = hst[j];
       if (!FULL && (hzero[j] || kbase + piece * 4 >= dh)) v = make_uint4(0, 0, 0, 0);
       unsigned char *dst = &hbuf[buf][hrow_of(j) * RS];
-      if (BF16) {
+      if (HB) {
+        *reinterpret_cast<uint4 *>(dst + piece * 16) = v;  // already in the operand type
+      } else if (BF16) {
         uint2 w;
         w.x = pack_bf16x2(__uint_as_float(v.x), __uint_as_float(v.y));
         w.y = pack_bf16x2(__uint_as_float(v.z), __uint_as_float(v.w));

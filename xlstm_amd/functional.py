@@ -61,11 +61,14 @@ def slstm_forward(
     h_out: Optional[torch.Tensor] = None,
     s_out: Optional[torch.Tensor] = None,
     spin_limit: int = 0,
+    h_prev: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Runs the cell over ``wx`` and returns ``(h[S,B,H] in wx.dtype, state[4,B,H] float32)``.
 
     ``reset_mask[B,S]`` (bool/uint8) marks document starts: the row's state is
     zeroed before that step.  ``step=True`` uses the decode entry point (S == 1).
+    ``h_prev`` (bfloat16 decode steps only): the ``h`` the previous step returned, i.e.
+    ``s0[0]`` already rounded to bfloat16; the kernel then reads half the operand bytes.
     """
     lib = _lib.load()
     _require_cuda("wx", wx)
@@ -138,6 +141,11 @@ def slstm_forward(
     a.workspace_bytes = workspace.numel()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
     a.spin_limit = int(spin_limit)
+    a.h_prev = None
+    if h_prev is not None and step and wx.dtype == torch.bfloat16 and s0 is not None:
+        if h_prev.dtype != torch.bfloat16 or h_prev.numel() != B * H or not h_prev.is_contiguous():
+            raise ValueError(f"h_prev must be a contiguous bfloat16 tensor of {B * H} elements")
+        a.h_prev = h_prev.data_ptr()
     with torch.cuda.device(dev):
         rc = (lib.xs_slstm_step if step else lib.xs_slstm_forward)(ctypes.byref(a))
     if rc != 0:
@@ -191,13 +199,21 @@ class StepPlan:
         self._wx_numel, self._s_numel = self.B * 4 * self.H, 4 * self.B * self.H
 
     def __call__(self, wx: torch.Tensor, s_in: torch.Tensor, s_out: torch.Tensor, h_out: torch.Tensor,
-                 stream: Optional[int] = None) -> None:
+                 stream: Optional[int] = None, h_prev: Optional[torch.Tensor] = None) -> None:
+        """``h_prev`` (bfloat16 plans): the ``h_out`` buffer the previous call filled, a different buffer
+        than this call's ``h_out``; it must hold ``s_in[0]`` rounded to bfloat16."""
         if (wx.dtype != self.wx_dtype or wx.numel() != self._wx_numel or s_in.numel() != self._s_numel
                 or s_out.numel() != self._s_numel or s_in.dtype != torch.float32 or s_out.dtype != torch.float32
                 or h_out.dtype != self.wx_dtype or h_out.numel() * 4 != self._s_numel):
             raise ValueError("tensor does not fit the plan (dtype or size)")
         a = self._args
         a.wx, a.s0, a.s_out, a.h_out = wx.data_ptr(), s_in.data_ptr(), s_out.data_ptr(), h_out.data_ptr()
+        if h_prev is not None and self.wx_dtype == torch.bfloat16:
+            if h_prev.dtype != torch.bfloat16 or h_prev.numel() * 4 != self._s_numel:
+                raise ValueError("h_prev does not fit the plan (dtype or size)")
+            a.h_prev = h_prev.data_ptr()
+        else:
+            a.h_prev = None
         a.stream = stream if stream is not None else torch.cuda.current_stream().cuda_stream
         rc = self._fn(self._ref)
         if rc != 0:
