@@ -181,3 +181,21 @@ def test_spin_limit_runs_out_is_reported_not_hung():
     assert status2["aborted"] == 0
     h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
     assert max_err(h2, h_ref) <= TOL_BF16
+
+
+def test_status_reports_the_number_of_launches():
+    """A batch that does not fit the compute units at once runs as several launches of row chunks."""
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(9)
+    for B, NH, dh, want in ((16, 4, 256, 1), (256, 8, 256, 2)):
+        H = NH * dh
+        wx = torch.randn(B, 3, 4 * H, device=dev).bfloat16()
+        r = (torch.rand(NH, 4 * dh, dh, device=dev) - 0.5) * 0.1
+        bias = torch.zeros(NH, 4, dh, device=dev)
+        ws = F.workspace_for(B, 3, NH, dh, dev)
+        F.slstm_forward(wx, r, bias, None, None, workspace=ws)
+        torch.cuda.synchronize()
+        st = F.read_status(ws)
+        assert st["aborted"] == 0 and st["launches"] == want, st

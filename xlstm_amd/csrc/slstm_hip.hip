@@ -239,7 +239,6 @@ int run_forward(const xs_slstm_args *a) {
   SeqKernel kern = bf16 ? pick_kernel<true>(nch, MT) : pick_kernel<false>(nch, MT);
   if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
 
-  uint32_t launches = 0;
   for (int b0 = 0; b0 < B; b0 += rows_per_launch) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
@@ -275,9 +274,7 @@ int run_forward(const xs_slstm_args *a) {
     hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), dyn_lds, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
-    ++launches;
   }
-  (void)launches;
   return XS_OK;
 }
 

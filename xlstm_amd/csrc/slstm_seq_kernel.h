@@ -133,6 +133,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   //      If so h is published with plain stores (they land in that L2); otherwise with
   //      device-scope stores that are written through to memory.
   if (tid == 0) {
+    if (wg == 0) atomicAdd(&p.status->launches, 1u);  // a long batch is run as several launches of row chunks
     const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
     __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);

@@ -98,7 +98,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const int nslab = (4 * nch) / SLABCH;
 
   if (blockIdx.x == 0 && tid < 16)
-    reinterpret_cast<uint32_t *>(p.status)[tid] = 0u;  // a step never waits, so it never aborts
+    reinterpret_cast<uint32_t *>(p.status)[tid] = tid == 5 ? 1u : 0u;  // a step never waits, so it never aborts; one launch
 
   const bool has_s0 = FULL || p.s0 != nullptr;
   const bool has_reset = !FULL && p.reset != nullptr;
