@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 2
+#define XS_ABI_VERSION 3
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -69,7 +69,11 @@ enum {
  *                             placement word per workgroup and the exchange
  *                             ring through which the compute units of a head
  *                             pass h_t to each other (a few MiB).  Two calls
- *                             that may overlap in time need different workspaces.
+ *                             that may overlap in time need different workspaces;
+ *                             two sequence calls that overlap on one GPU also
+ *                             compete for its compute units (each needs all of
+ *                             its workgroups running at once), so one of them
+ *                             waits, within spin_limit, until the other is done.
  *   stream                    hipStream_t (NULL = the null stream).
  *   spin_limit                bound on every wait between compute units, in poll
  *                             iterations; 0 selects the default.  When a wait
@@ -143,6 +147,58 @@ int xs_slstm_forward(const xs_slstm_args *args);
  * calls the cell's forward with S = 1).
  */
 int xs_slstm_step(const xs_slstm_args *args);
+
+/*
+ * The two operations in front of the cell inside an sLSTM layer (bf16 only; the layer keeps its
+ * PyTorch path for everything else).  They enqueue one kernel each and allocate nothing.
+ *
+ * xs_causal_conv_silu: out[b,t,c] = silu(bias[c] + sum_j weight[c,j] * x[b, t-(K-1)+j, c]),
+ * the causal depthwise convolution of xlstm/components/conv.py:113-127 followed by the
+ * activation of xlstm/blocks/slstm/layer.py:136-137.  Inputs before t = 0 are read from
+ * conv_state (the K-1 tokens before this call, conv.py:118-122) or are zero.  With a reset
+ * mask (not in the reference) a tap that would reach before the start of the token's document
+ * reads zero.
+ */
+typedef struct xs_conv_args {
+  int32_t B, T, D, K;        /* K taps, 2..4; D a multiple of 8 */
+  int32_t dtype;             /* XS_BF16 */
+  const void *x;             /* [B,T,D], strides in elements, innermost contiguous */
+  int64_t x_stride_b, x_stride_t;
+  const void *conv_state;    /* [B,K-1,D] or NULL; tokens contiguous, rows conv_state_stride_b apart */
+  int64_t conv_state_stride_b; /* in elements; 0 = (K-1)*D */
+  const void *weight;        /* [D,K] (nn.Conv1d's [D,1,K]) */
+  const void *bias;          /* [D] or NULL */
+  const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes */
+  int64_t reset_stride_b;
+  void *out;                 /* [B,T,D] contiguous */
+  void *stream;
+} xs_conv_args;
+
+int xs_causal_conv_silu(const xs_conv_args *args);
+
+/*
+ * xs_headwise_gates: the four block-diagonal gate projections and their concatenation,
+ *   out[m, g*H + h*dh + o] = sum_d A_g[m, h*dh + d] * w[g][h, o, d],   H = NH*dh,
+ * with A_g = x_conv for the slots g = i, f and x for g = z, o
+ * (xlstm/blocks/slstm/layer.py:144-153: four LinearHeadwiseExpand modules,
+ * xlstm/components/linear_headwise.py:75-82, then torch.cat).  `out` is the cell's wx.
+ * w[] is in SLOT order i, f, z, o; the reference wires its module named fgate to the i slot
+ * and igate to the f slot (layer.py:144-149).
+ */
+typedef struct xs_gates_args {
+  int32_t M, NH, dh;         /* M = B*T tokens; dh a multiple of 64 */
+  int32_t dtype;             /* XS_BF16 */
+  const void *x;             /* [M, H], row stride in elements */
+  int64_t x_stride_row;
+  const void *x_conv;        /* [M, H] */
+  int64_t x_conv_stride_row;
+  const void *w[4];          /* each [NH, dh, dh] contiguous */
+  void *out;                 /* [M, 4*H] */
+  int64_t out_stride_row;
+  void *stream;
+} xs_gates_args;
+
+int xs_headwise_gates(const xs_gates_args *args);
 
 #ifdef __cplusplus
 }

@@ -28,6 +28,9 @@ def test_abi_version_and_struct_mirror():
     # xs_slstm_args: 6 int32, pointers/int64 after -> 8-byte aligned, 15 more 8-byte fields
     assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 15 * 8
     assert ctypes.sizeof(_lib.SlstmStatus) == 64
+    # xs_conv_args: 5 int32 (+4 padding), then 11 8-byte fields; xs_gates_args: 4 int32, then 11 8-byte fields
+    assert ctypes.sizeof(_lib.ConvArgs) == 24 + 11 * 8
+    assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
 
 
 def test_argument_errors_without_touching_the_gpu():
@@ -55,6 +58,36 @@ def test_argument_errors_without_touching_the_gpu():
     assert lib.xs_slstm_step(ctypes.byref(a)) == -2 and b"overlap" in lib.xs_last_error()
     a.s_out = 0x100000 + 128  # adjacent is fine: the next complaint is about wx / h_out
     assert lib.xs_slstm_step(ctypes.byref(a)) == -1
+
+
+def test_layer_op_argument_errors_without_touching_the_gpu():
+    lib = _lib.load()
+    assert lib.xs_causal_conv_silu(None) == -1 and lib.xs_headwise_gates(None) == -1
+    c = _lib.ConvArgs()
+    c.B, c.T, c.D, c.K, c.dtype = 1, 4, 16, 4, _lib.XS_F32
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == -3  # bf16 only
+    c.dtype, c.K = _lib.XS_BF16, 5
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == -5 and b"taps" in lib.xs_last_error()
+    c.K, c.D = 4, 12
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == -5  # D not a multiple of 8
+    c.D = 16
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == -1  # x / weight / out missing
+    c.x, c.weight, c.out, c.x_stride_b, c.x_stride_t = 0x1000, 0x2000, 0x3008, 64, 16
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == -4  # out not 16-byte aligned
+    c.T = 0
+    assert lib.xs_causal_conv_silu(ctypes.byref(c)) == 0  # nothing to do, nothing launched
+    g = _lib.GatesArgs()
+    g.M, g.NH, g.dh, g.dtype = 4, 2, 32, _lib.XS_BF16
+    assert lib.xs_headwise_gates(ctypes.byref(g)) == -5 and b"multiple of 64" in lib.xs_last_error()
+    g.dh = 64
+    assert lib.xs_headwise_gates(ctypes.byref(g)) == -1
+    g.x, g.x_conv, g.out = 0x1000, 0x2000, 0x3000
+    for i in range(4):
+        g.w[i] = 0x4000
+    g.x_stride_row, g.x_conv_stride_row, g.out_stride_row = 128, 128, 128
+    assert lib.xs_headwise_gates(ctypes.byref(g)) == -2  # out rows overlap
+    g.M = 0
+    assert lib.xs_headwise_gates(ctypes.byref(g)) == 0
 
 
 def test_workspace_bytes_is_bounded_and_monotone():

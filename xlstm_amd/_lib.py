@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 EXPORTS = (
     "xs_abi_version",
@@ -21,6 +21,8 @@ EXPORTS = (
     "xs_slstm_workspace_bytes",
     "xs_slstm_forward",
     "xs_slstm_step",
+    "xs_causal_conv_silu",
+    "xs_headwise_gates",
 )
 
 
@@ -44,6 +46,42 @@ class SlstmArgs(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("spin_limit", ctypes.c_int64),
         ("h_prev", ctypes.c_void_p),
+    ]
+
+
+class ConvArgs(ctypes.Structure):
+    """Mirror of ``xs_conv_args``."""
+
+    _fields_ = [
+        ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("D", ctypes.c_int32), ("K", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("x", ctypes.c_void_p),
+        ("x_stride_b", ctypes.c_int64), ("x_stride_t", ctypes.c_int64),
+        ("conv_state", ctypes.c_void_p),
+        ("conv_state_stride_b", ctypes.c_int64),
+        ("weight", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("reset", ctypes.c_void_p),
+        ("reset_stride_b", ctypes.c_int64),
+        ("out", ctypes.c_void_p),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
+class GatesArgs(ctypes.Structure):
+    """Mirror of ``xs_gates_args``."""
+
+    _fields_ = [
+        ("M", ctypes.c_int32), ("NH", ctypes.c_int32), ("dh", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("x", ctypes.c_void_p),
+        ("x_stride_row", ctypes.c_int64),
+        ("x_conv", ctypes.c_void_p),
+        ("x_conv_stride_row", ctypes.c_int64),
+        ("w", ctypes.c_void_p * 4),
+        ("out", ctypes.c_void_p),
+        ("out_stride_row", ctypes.c_int64),
+        ("stream", ctypes.c_void_p),
     ]
 
 
@@ -81,6 +119,10 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmArgs)]
+    lib.xs_causal_conv_silu.restype = ctypes.c_int
+    lib.xs_causal_conv_silu.argtypes = [ctypes.POINTER(ConvArgs)]
+    lib.xs_headwise_gates.restype = ctypes.c_int
+    lib.xs_headwise_gates.argtypes = [ctypes.POINTER(GatesArgs)]
     if lib.xs_abi_version() != ABI_VERSION:
         raise RuntimeError(f"xlstm_amd: ABI version {lib.xs_abi_version()} != expected {ABI_VERSION}; rebuild")
     _LIB = lib

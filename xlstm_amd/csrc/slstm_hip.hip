@@ -6,12 +6,13 @@
 // VGPRs for the whole sequence, computes R.h with MFMA (K split over the 4
 // waves, partial sums reduced through LDS), and runs the exponential-gating
 // pointwise update with c, n, m in fp32 registers.  The only thing exchanged
-// per step is h_t: every workgroup stores its 16 units of h_t into a compact
-// exchange buffer (one 512-byte / 1-KiB block per workgroup and step, so that
-// polls and stores move whole cache lines spread over all L2 channels) and
-// the other members of the group poll those very words until none of them
-// carries the "not written yet" pattern the buffer was pre-filled with.  One
-// memory round trip per step, no flags, no atomics-with-return, no grid barrier.
+// per step is h_t: every workgroup stores its 16 units of h_t into a ring of
+// 8 step slots in the workspace (laid out [row tile][member][16 rows][16 units],
+// so that polls and stores move whole cache lines) and the other members of the
+// group poll those very words until none of them carries the "not written yet"
+// pattern the ring was pre-filled with.  One memory round trip per step, no
+// flags, no atomics-with-return, no grid barrier.  A decode step (T = 1) is a
+// different kernel: a tiled GEMM + gating with no waits between workgroups.
 //
 // Equations follow xlstm/blocks/slstm/src/vanilla/slstm.py:19-37 with the
 // per-element n == 0 rule of xlstm/blocks/slstm/src/cuda/slstm_pointwise.cu:79.
@@ -30,6 +31,7 @@
 #include "slstm_device_common.h"
 #include "slstm_seq_kernel.h"
 #include "slstm_step_kernel.h"
+#include "slstm_layer_kernels.h"
 
 namespace {
 
@@ -95,7 +97,6 @@ int validate(const xs_slstm_args *a, bool step) {
     if (lo0 < lo1 + bytes && lo1 < lo0 + bytes && bytes) return fail(XS_ERR_SHAPE, "s_out must not overlap s0");
   }
   if (a->B > 0 && a->T > 0 && (!a->wx || !a->h_out)) return fail(XS_ERR_NULL, "wx and h_out are required");
-  const int epc = a->wx_dtype == XS_BF16 ? 8 : 4;
   if (a->dh % 8 != 0) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not a multiple of 8", a->dh);
   const long long H = (long long)a->NH * a->dh;
   if (a->B > 0 && a->T > 0) {
@@ -115,18 +116,15 @@ int validate(const xs_slstm_args *a, bool step) {
   if (!a->workspace || a->workspace_bytes < xs_slstm_workspace_bytes(a->B, a->T, a->NH, a->dh))
     return fail(XS_ERR_WORKSPACE, "workspace missing or smaller than xs_slstm_workspace_bytes()");
   if ((uintptr_t)a->workspace % 256) return fail(XS_ERR_ALIGN, "workspace must be 256-byte aligned");
-  (void)epc;
   return XS_OK;
 }
 
+// compute units of the current device (an attribute query: no device synchronisation, cheap per call)
 int device_cus() {
-  static int cus = -1;
-  if (cus < 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -1;
-    cus = prop.multiProcessorCount;
-  }
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess ||
+      hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+    return -1;
   return cus;
 }
 
@@ -278,6 +276,77 @@ int run_forward(const xs_slstm_args *a) {
   return XS_OK;
 }
 
+int run_conv(const xs_conv_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->B < 0 || a->T < 0 || a->D <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d D=%d", a->B, a->T, a->D);
+  if (a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "xs_causal_conv_silu computes on bf16 tensors only");
+  if (a->K < 2 || a->K > 4) return fail(XS_ERR_UNSUPPORTED, "convolution of %d taps not supported (2..4)", a->K);
+  if (a->D % 8 != 0) return fail(XS_ERR_UNSUPPORTED, "D = %d is not a multiple of 8", a->D);
+  if (a->B == 0 || a->T == 0) return XS_OK;
+  if (!a->x || !a->weight || !a->out) return fail(XS_ERR_NULL, "x, weight and out are required");
+  if (a->x_stride_t < a->D || (a->B > 1 && a->x_stride_b < a->D)) return fail(XS_ERR_SHAPE, "x strides overlap the innermost D elements");
+  if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
+  if (a->conv_state && a->conv_state_stride_b && (a->conv_state_stride_b < (long long)(a->K - 1) * a->D || a->conv_state_stride_b % 8))
+    return fail(XS_ERR_SHAPE, "conv_state row stride %lld too small or not 16-byte aligned", (long long)a->conv_state_stride_b);
+  if (((uintptr_t)a->x % 16) || ((a->x_stride_b * 2) % 16) || ((a->x_stride_t * 2) % 16) || ((uintptr_t)a->conv_state % 16) ||
+      ((uintptr_t)a->weight % 16) || ((uintptr_t)a->bias % 16) || ((uintptr_t)a->out % 16))
+    return fail(XS_ERR_ALIGN, "x and its strides, conv_state, weight, bias and out must be 16-byte aligned");
+  const long long threads = (long long)a->B * a->T * (a->D / 8);
+  const long long blocks = (threads + 255) / 256;
+  if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tokens for one launch");
+  ConvParams p;
+  p.x = (const uint16_t *)a->x; p.x_sb = a->x_stride_b; p.x_st = a->x_stride_t;
+  p.state = (const uint16_t *)a->conv_state;
+  p.state_sb = a->conv_state_stride_b ? a->conv_state_stride_b : (long long)(a->K - 1) * a->D;
+  p.w = (const uint16_t *)a->weight; p.bias = (const uint16_t *)a->bias;
+  p.reset = a->reset; p.reset_sb = a->reset_stride_b;
+  p.out = (uint16_t *)a->out;
+  p.B = a->B; p.T = a->T; p.D = a->D;
+  hipStream_t stream = (hipStream_t)a->stream;
+  void (*kern)(ConvParams) = a->K == 2 ? causal_conv_silu_kernel<2> : (a->K == 3 ? causal_conv_silu_kernel<3> : causal_conv_silu_kernel<4>);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "convolution kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
+int run_gates(const xs_gates_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->M < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims M=%d NH=%d dh=%d", a->M, a->NH, a->dh);
+  if (a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "xs_headwise_gates computes on bf16 tensors only");
+  if (a->dh % 64 != 0) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not a multiple of 64", a->dh);
+  if (a->M == 0) return XS_OK;
+  const long long H = (long long)a->NH * a->dh;
+  if (!a->x || !a->x_conv || !a->out || !a->w[0] || !a->w[1] || !a->w[2] || !a->w[3])
+    return fail(XS_ERR_NULL, "x, x_conv, the four weights and out are required");
+  if (a->x_stride_row < H || a->x_conv_stride_row < H || a->out_stride_row < 4 * H)
+    return fail(XS_ERR_SHAPE, "a row stride is smaller than the row");
+  if (((uintptr_t)a->x % 16) || ((uintptr_t)a->x_conv % 16) || ((uintptr_t)a->out % 16) || ((a->x_stride_row * 2) % 16) ||
+      ((a->x_conv_stride_row * 2) % 16) || ((a->out_stride_row * 2) % 16) || ((uintptr_t)a->w[0] % 16) ||
+      ((uintptr_t)a->w[1] % 16) || ((uintptr_t)a->w[2] % 16) || ((uintptr_t)a->w[3] % 16))
+    return fail(XS_ERR_ALIGN, "x, x_conv, out, their row strides and the weights must be 16-byte aligned");
+  GatesParams p;
+  p.x = (const uint16_t *)a->x; p.xc = (const uint16_t *)a->x_conv;
+  p.x_sr = a->x_stride_row; p.xc_sr = a->x_conv_stride_row;
+  for (int g = 0; g < 4; ++g) p.w[g] = (const uint16_t *)a->w[g];
+  p.out = (uint16_t *)a->out; p.out_sr = a->out_stride_row;
+  p.M = a->M; p.NH = a->NH; p.dh = a->dh;
+  // tile: 128 tokens when there are enough of them to fill the compute units, 128 units when dh allows
+  const int bn = a->dh % 128 == 0 ? 128 : 64;
+  const int bm = a->M >= 4096 ? 128 : 64;
+  p.m_tiles = (a->M + bm - 1) / bm;
+  p.n_tiles = 4 * a->NH * (a->dh / bn);
+  const long long grid = (long long)8 * ((p.m_tiles + 7) / 8) * p.n_tiles;
+  if (grid > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one launch");
+  void (*kern)(GatesParams) = bm == 128 ? (bn == 128 ? headwise_gates_kernel<128, 128> : headwise_gates_kernel<128, 64>)
+                                        : (bn == 128 ? headwise_gates_kernel<64, 128> : headwise_gates_kernel<64, 64>);
+  hipStream_t stream = (hipStream_t)a->stream;
+  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), 0, stream, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "gate projection kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -303,6 +372,16 @@ int xs_slstm_step(const xs_slstm_args *args) {
   const int rc = validate(args, true);
   if (rc != XS_OK) return rc;
   return run_step(args);
+}
+
+int xs_causal_conv_silu(const xs_conv_args *args) {
+  g_err[0] = 0;
+  return run_conv(args);
+}
+
+int xs_headwise_gates(const xs_gates_args *args) {
+  g_err[0] = 0;
+  return run_gates(args);
 }
 
 }  // extern "C"

@@ -1,0 +1,237 @@
+// The two kernels in front of the cell inside an sLSTM layer: causal depthwise convolution + SiLU,
+// and the four block-diagonal gate projections that produce the cell's input W.x.  bf16 operands,
+// float32 arithmetic.  Included by slstm_hip.hip only (one translation unit), after
+// slstm_device_common.h.
+#pragma once
+
+namespace {
+
+// ---------------------------------------------------------------------------
+// causal depthwise convolution over time + SiLU (xlstm/components/conv.py:113-127 followed by
+// the activation of xlstm/blocks/slstm/layer.py:136-137).  One thread: 8 channels of one token.
+// Tap j of a kernel of KS taps multiplies the input KS-1-j tokens back; inputs before t = 0 come
+// from `state` (the KS-1 tokens before this call) or are zero; with a reset mask a tap that
+// would reach before the start of the token's document reads zero.
+// ---------------------------------------------------------------------------
+struct ConvParams {
+  const uint16_t *x;
+  long long x_sb, x_st;
+  const uint16_t *state;  // [B, KS-1, D] or null; rows state_sb elements apart
+  long long state_sb;
+  const uint16_t *w;      // [D, KS]
+  const uint16_t *bias;   // [D] or null
+  const unsigned char *reset;
+  long long reset_sb;
+  uint16_t *out;          // [B, T, D]
+  int B, T, D;
+};
+
+template <int KS>
+__global__ __launch_bounds__(256) void causal_conv_silu_kernel(ConvParams p) {
+  const int pieces = p.D >> 3;
+  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (long long)p.B * p.T * pieces) return;
+  const int piece = (int)(idx % pieces);
+  const long long bt = idx / pieces;
+  const int t = (int)(bt % p.T);
+  const int b = (int)(bt / p.T);
+  const int c0 = piece * 8;
+
+  // weights of the 8 channels: 8 * KS consecutive bf16
+  uint16_t wv[8 * KS];
+  {
+    const uint4 *wp = reinterpret_cast<const uint4 *>(p.w + (long long)c0 * KS);
+#pragma unroll
+    for (int j = 0; j < KS; ++j) {
+      const uint4 v = wp[j];
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        wv[8 * j + 2 * e] = (uint16_t)(d[e] & 0xFFFFu);
+        wv[8 * j + 2 * e + 1] = (uint16_t)(d[e] >> 16);
+      }
+    }
+  }
+  float acc[8];
+  if (p.bias) {
+    const uint4 v = *reinterpret_cast<const uint4 *>(p.bias + c0);
+    const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      acc[2 * e] = bf16_bits_to_float(d[e] & 0xFFFFu);
+      acc[2 * e + 1] = bf16_bits_to_float(d[e] >> 16);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.0f;
+  }
+  bool alive = true;  // no document start between the tap and the token so far
+#pragma unroll
+  for (int back = 0; back < KS; ++back) {
+    const int j = KS - 1 - back;
+    const int ts = t - back;
+    if (back > 0 && p.reset) {  // the tap at `back` is dropped if a document starts in (t - back, t]
+      const int tm = t - back + 1;
+      if (tm >= 0 && p.reset[(long long)b * p.reset_sb + tm] != 0) alive = false;
+    }
+    const uint16_t *src = nullptr;
+    if (alive) {
+      if (ts >= 0) src = p.x + (long long)b * p.x_sb + (long long)ts * p.x_st + c0;
+      else if (p.state) src = p.state + (long long)b * p.state_sb + (long long)(KS - 1 + ts) * p.D + c0;
+    }
+    if (src) {
+      const uint4 v = *reinterpret_cast<const uint4 *>(src);
+      const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] += bf16_bits_to_float(wv[(2 * e) * KS + j]) * bf16_bits_to_float(d[e] & 0xFFFFu);
+        acc[2 * e + 1] += bf16_bits_to_float(wv[(2 * e + 1) * KS + j]) * bf16_bits_to_float(d[e] >> 16);
+      }
+    }
+  }
+  uint32_t o[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const float a = acc[2 * e], c = acc[2 * e + 1];
+    o[e] = pack_bf16x2(a * __builtin_amdgcn_rcpf(1.0f + __expf(-a)), c * __builtin_amdgcn_rcpf(1.0f + __expf(-c)));
+  }
+  *reinterpret_cast<uint4 *>(p.out + ((long long)b * p.T + t) * p.D + c0) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+
+// ---------------------------------------------------------------------------
+// the four headwise gate projections and their concatenation
+// (xlstm/blocks/slstm/layer.py:144-153, xlstm/components/linear_headwise.py:75-82):
+//   out[m, g*H + h*dh + o] = sum_d A_g[m, h*dh + d] * W_g[h, o, d]
+// with A_g = x_conv for the slots i and f, x for z and o.  A workgroup computes BM tokens x BN output
+// units of one (slot, head); K = dh is walked in stages of 64 inputs (128-byte rows), each staged
+// through LDS once; the loads of the next stage are in flight during the MFMAs of the current one.
+// Four waves as 2 x 2.  The product is formed transposed (units on the MFMA M axis), so a lane ends
+// with 4 consecutive units of one token.  Workgroup i runs on XCD i % 8: the tiles of one block of
+// tokens are given to ONE XCD, so that x and x_conv are fetched from HBM once.
+// ---------------------------------------------------------------------------
+struct GatesParams {
+  const uint16_t *x, *xc;
+  long long x_sr, xc_sr;
+  const uint16_t *w[4];
+  uint16_t *out;
+  long long out_sr;
+  int M, NH, dh;
+  int m_tiles, n_tiles;
+};
+
+constexpr int kGateRowBytes = 144;  // 128 bytes of data + 16 of padding: conflict-free 16-byte reads
+
+template <int BM, int BN>
+__global__ __launch_bounds__(256) void headwise_gates_kernel(GatesParams p) {
+  constexpr int AI = BM * 8 / 256;  // 16-byte pieces of the token tile a thread stages per K stage
+  constexpr int WI = BN * 8 / 256;  // ... of the weight tile
+  constexpr int TM = BM / 32, TN = BN / 32;  // MFMA tiles of a wave: TM token tiles x TN unit tiles
+  __shared__ __attribute__((aligned(16))) unsigned char abuf[BM * kGateRowBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char wbuf[BN * kGateRowBytes];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  const int xcd = blockIdx.x & 7;
+  const int jj = blockIdx.x >> 3;
+  const int mtile = (jj / p.n_tiles) * 8 + xcd;
+  if (mtile >= p.m_tiles) return;  // the whole workgroup leaves before any barrier
+  int nt = jj % p.n_tiles;
+  const int npu = p.dh / BN;  // unit tiles per (slot, head)
+  const int ut = nt % npu; nt /= npu;
+  const int slot_in_pair = nt & 1; nt >>= 1;
+  const int pair = nt & 1;
+  const int head = nt >> 1;
+  const int slot = pair * 2 + slot_in_pair;
+  const int m0 = mtile * BM;
+  const int n0 = ut * BN;
+  const int dh = p.dh;
+
+  const uint16_t *abase = pair ? p.x : p.xc;
+  const long long asr = pair ? p.x_sr : p.xc_sr;
+  const uint16_t *wbase = p.w[slot] + ((long long)head * dh + n0) * dh;
+
+  const uint16_t *asrc[AI];
+  int adst[AI];
+#pragma unroll
+  for (int j = 0; j < AI; ++j) {
+    const int e = tid + 256 * j;
+    const int row = e >> 3, pc = e & 7;
+    const int m = m0 + row < p.M ? m0 + row : p.M - 1;
+    asrc[j] = abase + (long long)m * asr + (long long)head * dh + pc * 8;
+    adst[j] = row * kGateRowBytes + pc * 16;
+  }
+  const uint16_t *wsrc[WI];
+  int wdst[WI];
+#pragma unroll
+  for (int j = 0; j < WI; ++j) {
+    const int e = tid + 256 * j;
+    const int row = e >> 3, pc = e & 7;
+    wsrc[j] = wbase + (long long)row * dh + pc * 8;
+    wdst[j] = row * kGateRowBytes + pc * 16;
+  }
+
+  f32x4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  uint4 areg[AI], wreg[WI];
+#pragma unroll
+  for (int j = 0; j < AI; ++j) areg[j] = *reinterpret_cast<const uint4 *>(asrc[j]);
+#pragma unroll
+  for (int j = 0; j < WI; ++j) wreg[j] = *reinterpret_cast<const uint4 *>(wsrc[j]);
+
+  const int nstage = dh >> 6;
+  for (int s = 0; s < nstage; ++s) {
+    if (s) __syncthreads();  // every wave is done reading the previous stage
+#pragma unroll
+    for (int j = 0; j < AI; ++j) *reinterpret_cast<uint4 *>(&abuf[adst[j]]) = areg[j];
+#pragma unroll
+    for (int j = 0; j < WI; ++j) *reinterpret_cast<uint4 *>(&wbuf[wdst[j]]) = wreg[j];
+    __syncthreads();
+    if (s + 1 < nstage) {
+#pragma unroll
+      for (int j = 0; j < AI; ++j) areg[j] = *reinterpret_cast<const uint4 *>(asrc[j] + (s + 1) * 64);
+#pragma unroll
+      for (int j = 0; j < WI; ++j) wreg[j] = *reinterpret_cast<const uint4 *>(wsrc[j] + (s + 1) * 64);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      uint4 av[TM], wv[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[i] = *reinterpret_cast<const uint4 *>(&abuf[(wm * (BM / 2) + 16 * i + r16) * kGateRowBytes + ks * 64 + q * 16]);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        wv[j] = *reinterpret_cast<const uint4 *>(&wbuf[(wn * (BN / 2) + 16 * j + r16) * kGateRowBytes + ks * 64 + q * 16]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[j]), __builtin_bit_cast(bf16x8, av[i]), acc[i][j], 0, 0, 0);
+    }
+  }
+
+  // lane (r16, q) holds token m0 + wm*BM/2 + 16 i + r16, units n0 + wn*BN/2 + 16 j + 4 q .. +3
+  const long long colbase = (long long)slot * p.NH * dh + (long long)head * dh + n0 + wn * (BN / 2) + 4 * q;
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * (BM / 2) + 16 * i + r16;
+    if (m < p.M) {
+      uint16_t *orow = p.out + (long long)m * p.out_sr + colbase;
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        uint2 v;
+        v.x = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+        v.y = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        *reinterpret_cast<uint2 *>(orow + 16 * j) = v;
+      }
+    }
+  }
+}
+
+}  // namespace

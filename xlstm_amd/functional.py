@@ -218,3 +218,119 @@ class StepPlan:
         rc = self._fn(self._ref)
         if rc != 0:
             raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+
+
+def _mask_u8(reset_mask: torch.Tensor, B: int, T: int) -> torch.Tensor:
+    _require_cuda("reset_mask", reset_mask)
+    if tuple(reset_mask.shape) != (B, T):
+        raise ValueError(f"reset_mask must be [B, S] = {(B, T)}, got {tuple(reset_mask.shape)}")
+    if reset_mask.dtype == torch.bool:
+        reset_mask = reset_mask.view(torch.uint8) if reset_mask.is_contiguous() else reset_mask.to(torch.uint8)
+    elif reset_mask.dtype != torch.uint8:
+        reset_mask = (reset_mask != 0).to(torch.uint8)
+    if T and reset_mask.stride(1) != 1:
+        reset_mask = reset_mask.contiguous()
+    return reset_mask
+
+
+def fused_layer_ops_supported(x: torch.Tensor, num_heads: int, kernel_size: int) -> bool:
+    """Whether :func:`causal_conv_silu` and :func:`headwise_gates` cover this input (bfloat16 on the GPU,
+    head dim a multiple of 64, 2..4 taps)."""
+    D = int(x.shape[-1])
+    return (x.is_cuda and x.dtype == torch.bfloat16 and D % num_heads == 0 and (D // num_heads) % 64 == 0
+            and (kernel_size == 0 or 2 <= kernel_size <= 4))
+
+
+def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
+                     conv_state: Optional[torch.Tensor] = None, reset_mask: Optional[torch.Tensor] = None,
+                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``silu(causal_conv1d(x))`` of an sLSTM layer (xlstm/components/conv.py:113-127,
+    xlstm/blocks/slstm/layer.py:136-137) in one kernel.  ``x`` [B,S,D] bfloat16, ``weight`` [D,1,K] or [D,K],
+    ``conv_state`` [B,K-1,D] = the inputs before ``x``; ``reset_mask`` [B,S] stops the taps at document starts."""
+    lib = _lib.load()
+    _require_cuda("x", x)
+    if x.dim() != 3 or x.dtype != torch.bfloat16:
+        raise TypeError(f"x must be a bfloat16 [B, S, D] tensor, got {x.dtype} {tuple(x.shape)}")
+    B, T, D = (int(v) for v in x.shape)
+    w = weight.reshape(D, -1)
+    K = int(w.shape[1])
+    if w.dtype != torch.bfloat16 or not w.is_contiguous():
+        w = w.to(torch.bfloat16).contiguous()
+    if bias is not None and (bias.dtype != torch.bfloat16 or not bias.is_contiguous()):
+        bias = bias.to(torch.bfloat16).contiguous()
+    if x.numel() and (x.stride(2) != 1 or x.data_ptr() % 16 or x.stride(0) % 8 or x.stride(1) % 8
+                      or x.stride(1) < D or (B > 1 and x.stride(0) < D)):
+        x = x.contiguous()
+    if conv_state is not None:
+        if tuple(conv_state.shape) != (B, K - 1, D):
+            raise ValueError(f"conv_state must be [B, K-1, D] = {(B, K - 1, D)}, got {tuple(conv_state.shape)}")
+        if (conv_state.dtype != torch.bfloat16 or conv_state.stride(2) != 1 or conv_state.stride(1) != D
+                or conv_state.stride(0) % 8 or conv_state.data_ptr() % 16):  # a [:, :K-1] view of a ring is taken as it is
+            conv_state = conv_state.to(torch.bfloat16).contiguous()
+    if reset_mask is not None:
+        reset_mask = _mask_u8(reset_mask, B, T)
+    if out is None:
+        out = torch.empty((B, T, D), dtype=torch.bfloat16, device=x.device)
+    a = _lib.ConvArgs()
+    a.B, a.T, a.D, a.K = B, T, D, K
+    a.dtype = _lib.XS_BF16
+    a.x = x.data_ptr()
+    a.x_stride_b = x.stride(0) if B else 0
+    a.x_stride_t = x.stride(1) if T else 0
+    a.conv_state = conv_state.data_ptr() if conv_state is not None else None
+    a.conv_state_stride_b = conv_state.stride(0) if conv_state is not None and B > 1 else 0
+    a.weight = w.data_ptr()
+    a.bias = bias.data_ptr() if bias is not None else None
+    a.reset = reset_mask.data_ptr() if reset_mask is not None else None
+    a.reset_stride_b = reset_mask.stride(0) if reset_mask is not None else 0
+    a.out = out.data_ptr()
+    a.stream = torch.cuda.current_stream(x.device).cuda_stream
+    with torch.cuda.device(x.device):
+        rc = lib.xs_causal_conv_silu(ctypes.byref(a))
+    if rc != 0:
+        raise EngineError(f"xs_causal_conv_silu failed ({rc}): {_lib.last_error()}")
+    return out
+
+
+def headwise_gates(x: torch.Tensor, x_conv: torch.Tensor, weights, num_heads: int,
+                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The cell input of an sLSTM layer in one kernel: ``cat([W_i x_conv, W_f x_conv, W_z x, W_o x], -1)`` with
+    block-diagonal ("headwise") matrices (xlstm/blocks/slstm/layer.py:144-153,
+    xlstm/components/linear_headwise.py:75-82).  ``weights``: four [NH, dh, dh] tensors in slot order i, f, z, o."""
+    lib = _lib.load()
+    _require_cuda("x", x)
+    if x.dtype != torch.bfloat16 or x_conv.dtype != torch.bfloat16 or x.shape != x_conv.shape:
+        raise TypeError("x and x_conv must be bfloat16 tensors of one shape")
+    H = int(x.shape[-1])
+    dh = H // num_heads
+    x2 = x.reshape(-1, H)
+    xc2 = x_conv.reshape(-1, H)
+    if x2.stride(1) != 1 or x2.stride(0) % 8 or x2.data_ptr() % 16:
+        x2 = x2.contiguous()
+    if xc2.stride(1) != 1 or xc2.stride(0) % 8 or xc2.data_ptr() % 16:
+        xc2 = xc2.contiguous()
+    M = int(x2.shape[0])
+    ws = []
+    for w in weights:
+        if tuple(w.shape) != (num_heads, dh, dh):
+            raise ValueError(f"gate weight must be [NH, dh, dh] = {(num_heads, dh, dh)}, got {tuple(w.shape)}")
+        ws.append(w if (w.dtype == torch.bfloat16 and w.is_contiguous()) else w.to(torch.bfloat16).contiguous())
+    if out is None:
+        out = torch.empty(tuple(x.shape[:-1]) + (4 * H,), dtype=torch.bfloat16, device=x.device)
+    a = _lib.GatesArgs()
+    a.M, a.NH, a.dh = M, num_heads, dh
+    a.dtype = _lib.XS_BF16
+    a.x = x2.data_ptr()
+    a.x_stride_row = x2.stride(0) if M else H
+    a.x_conv = xc2.data_ptr()
+    a.x_conv_stride_row = xc2.stride(0) if M else H
+    for g in range(4):
+        a.w[g] = ws[g].data_ptr()
+    a.out = out.data_ptr()
+    a.out_stride_row = 4 * H
+    a.stream = torch.cuda.current_stream(x.device).cuda_stream
+    with torch.cuda.device(x.device):
+        rc = lib.xs_headwise_gates(ctypes.byref(a))
+    if rc != 0:
+        raise EngineError(f"xs_headwise_gates failed ({rc}): {_lib.last_error()}")
+    return out

@@ -10,7 +10,10 @@ reference's (``conv1d.conv``, ``fgate``, ``igate``, ``zgate``, ``ogate``,
 reference state dict maps one to one (the cell's two tensors go through the
 external views).
 
-The pre/post ops stay in PyTorch-ROCm; only the cell runs on the HIP engine.
+For bfloat16 inputs with a head dim that is a multiple of 64 the ops in front of the cell run
+as two HIP kernels of the engine (convolution + SiLU; the four projections written straight into the
+cell's input), see ``functional.causal_conv_silu`` / ``functional.headwise_gates``; otherwise, and for
+the group norm behind the cell, they are PyTorch-ROCm ops.
 New: ``reset_mask[B,S]`` (document starts of packed rows) reaches the cell, and
 the causal convolution does not look across a document start either.
 """
@@ -24,6 +27,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
+from . import functional as hipF
 from .cell import sLSTMCell, sLSTMCellConfig
 
 
@@ -91,20 +95,23 @@ class CausalConv1d(nn.Module):
             y = y + self.conv.bias
         return y
 
+    def advance(self, x: torch.Tensor, conv_state=None) -> torch.Tensor:
+        """The ring state after one more token: [B,k,D], oldest input first, ``x`` last (conv.py:142-149)."""
+        B, S, D = x.shape
+        assert S == 1, f"x has sequence length {S} but it should be 1"
+        if conv_state is None:
+            return torch.cat([torch.zeros(B, self.kernel_size - 1, D, device=x.device, dtype=x.dtype), x], dim=1)
+        prev = conv_state[0] if isinstance(conv_state, (tuple, list)) else conv_state
+        if prev.shape[1] == self.kernel_size:
+            prev = prev[:, 1:]  # the oldest slot is dropped
+        assert prev.shape[1] == self.kernel_size - 1, f"conv state holds {prev.shape[1]} inputs, expected {self.kernel_size}"
+        return torch.cat([prev.to(x.dtype), x], dim=1)
+
     def step(self, x: torch.Tensor, conv_state=None):
         """One token, ring state [B,k,D] in a 1-tuple as in conv.py:131-157.  Also accepted: the
         bare [B,k-1,D] tensor that ``forward(..., return_last_state=True)`` hands back
         (conv.py:126-127), so that a prefill can be followed by steps."""
-        B, S, D = x.shape
-        assert S == 1, f"x has sequence length {S} but it should be 1"
-        if conv_state is None:
-            conv_state = (torch.zeros(B, self.kernel_size, D, device=x.device, dtype=x.dtype),)
-        prev = conv_state[0] if isinstance(conv_state, (tuple, list)) else conv_state
-        if prev.shape[1] == self.kernel_size - 1:
-            prev = F.pad(prev, (0, 0, 1, 0))  # the oldest slot is dropped by the roll below
-        assert prev.shape[1] == self.kernel_size, f"conv state holds {prev.shape[1]} inputs, expected {self.kernel_size}"
-        state = torch.roll(prev, shifts=-1, dims=1)
-        state[:, -1:, :] = x
+        state = self.advance(x, conv_state)
         y = torch.sum(state * self.conv.weight[:, 0, :].transpose(0, 1), dim=1, keepdim=True)
         if self.conv.bias is not None:
             y = y + self.conv.bias
@@ -161,6 +168,7 @@ class sLSTMLayer(nn.Module):
         self.slstm_cell = sLSTMCell(config)
         self.group_norm = MultiHeadLayerNorm(ndim=D, weight=config.group_norm_weight)
         self.dropout = nn.Dropout(config.dropout)
+        self.fused_pre_ops = True  # use the engine's conv and projection kernels where they apply
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -173,13 +181,26 @@ class sLSTMLayer(nn.Module):
 
     def _gates(self, x, x_conv):
         # the module named fgate feeds the i slot, igate the f slot (layer.py:144-149)
+        if self._fused(x):
+            return hipF.headwise_gates(x, x_conv, (self.fgate.weight, self.igate.weight, self.zgate.weight, self.ogate.weight),
+                                       self.config.num_heads)
         return torch.cat([self.fgate(x_conv), self.igate(x_conv), self.zgate(x), self.ogate(x)], dim=-1)
+
+    def _fused(self, x) -> bool:
+        return (self.fused_pre_ops and self.fgate.weight.dtype == torch.bfloat16
+                and hipF.fused_layer_ops_supported(x, self.config.num_heads, self.config.conv1d_kernel_size))
 
     def forward(self, x: torch.Tensor, conv_state: Optional[torch.Tensor] = None,
                 slstm_state: Optional[torch.Tensor] = None, return_last_state: bool = False,
                 reset_mask: Optional[torch.Tensor] = None, **kwargs):
         B, S, _ = x.shape
-        if self.config.conv1d_kernel_size > 0:
+        if self.config.conv1d_kernel_size > 0 and self._fused(x):
+            conv = self.conv1d.conv
+            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, conv_state, reset_mask)
+            if return_last_state:  # the last k-1 inputs (conv.py:126-127)
+                x_all = x if conv_state is None else torch.cat([conv_state.to(x.dtype), x], dim=1)
+                conv_state = x_all[:, -self.conv1d.pad:]
+        elif self.config.conv1d_kernel_size > 0:
             if return_last_state:
                 x_conv, conv_state = self.conv1d(x, conv_state, return_last_state=True, reset_mask=reset_mask)
             else:
@@ -198,7 +219,12 @@ class sLSTMLayer(nn.Module):
              slstm_state_out: Optional[torch.Tensor] = None):
         """One token (layer.py:92-121).  ``slstm_state_out`` is handed to the cell's ``step``."""
         B, S, _ = x.shape
-        if self.config.conv1d_kernel_size > 0:
+        if self.config.conv1d_kernel_size > 0 and self._fused(x):
+            ring = self.conv1d.advance(x, conv_state)  # [B,k,D]: the k-1 inputs before x, then x
+            conv = self.conv1d.conv
+            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, ring[:, :-1])
+            conv_state = (ring,)
+        elif self.config.conv1d_kernel_size > 0:
             x_conv, conv_state = self.conv1d.step(x, conv_state=conv_state)
             x_conv = self.conv_act_fn(x_conv)
         else:
