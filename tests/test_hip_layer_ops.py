@@ -93,6 +93,10 @@ def test_causal_conv_silu_reads_a_ring_view_and_strided_input():
     ((4100,), 4, 64),      # 128 x 64, ragged
     ((256, 1), 8, 256),    # the decode shape of BASELINE config 3
     ((1, 1), 1, 192),      # one token, three 64-unit tiles per slot
+    ((8, 2048), 4, 256),   # the layer of BASELINE config 4: weights resident, 8 token partitions of 16 tiles
+    ((5, 999), 16, 256),   # 128 combinations: two token partitions, no XCD grouping, ragged
+    ((3, 1000), 3, 128),   # 12 combinations, 16 partitions of one or two tiles
+    ((2, 3), 1, 128),      # fewer token tiles than partitions
 ])
 def test_headwise_gates_equal_float32_einsum(lead, NH, dh):
     from xlstm_amd import functional as hipF

@@ -331,17 +331,34 @@ int run_gates(const xs_gates_args *a) {
   for (int g = 0; g < 4; ++g) p.w[g] = (const uint16_t *)a->w[g];
   p.out = (uint16_t *)a->out; p.out_sr = a->out_stride_row;
   p.M = a->M; p.NH = a->NH; p.dh = a->dh;
-  // tile: 128 tokens when there are enough of them to fill the compute units, 128 units when dh allows
-  const int bn = a->dh % 128 == 0 ? 128 : 64;
-  const int bm = a->M >= 4096 ? 128 : 64;
-  p.m_tiles = (a->M + bm - 1) / bm;
-  p.n_tiles = 4 * a->NH * (a->dh / bn);
-  const long long grid = (long long)8 * ((p.m_tiles + 7) / 8) * p.n_tiles;
-  if (grid > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one launch");
-  void (*kern)(GatesParams) = bm == 128 ? (bn == 128 ? headwise_gates_kernel<128, 128> : headwise_gates_kernel<128, 64>)
-                                        : (bn == 128 ? headwise_gates_kernel<64, 128> : headwise_gates_kernel<64, 64>);
   hipStream_t stream = (hipStream_t)a->stream;
-  hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), 0, stream, p);
+  if (a->dh == 128 || a->dh == 256) {
+    // weights resident in registers, workgroups walk over token tiles
+    const int cus = device_cus();
+    if (cus <= 0) return fail(XS_ERR_DEVICE, "cannot query the device");
+    const int combos = 2 * a->NH;  // (head, operand)
+    const int bm = a->dh == 256 ? 64 : 32;  // tokens per tile: threads / 8
+    p.m_tiles = (a->M + bm - 1) / bm;
+    p.n_tiles = combos;
+    int parts = cus / combos;
+    if (parts < 1) parts = 1;
+    if (parts > p.m_tiles) parts = p.m_tiles;
+    if (a->dh == 256)
+      hipLaunchKernelGGL(headwise_gates_resident_kernel<4>, dim3((unsigned)(combos * parts)), dim3(512), 0, stream, p, combos, parts);
+    else
+      hipLaunchKernelGGL(headwise_gates_resident_kernel<2>, dim3((unsigned)(combos * parts)), dim3(256), 0, stream, p, combos, parts);
+  } else {
+    // tile: 128 tokens when there are enough of them to fill the compute units, 128 units when dh allows
+    const int bn = a->dh % 128 == 0 ? 128 : 64;
+    const int bm = a->M >= 4096 ? 128 : 64;
+    p.m_tiles = (a->M + bm - 1) / bm;
+    p.n_tiles = 4 * a->NH * (a->dh / bn);
+    const long long grid = (long long)8 * ((p.m_tiles + 7) / 8) * p.n_tiles;
+    if (grid > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one launch");
+    void (*kern)(GatesParams) = bm == 128 ? (bn == 128 ? headwise_gates_kernel<128, 128> : headwise_gates_kernel<128, 64>)
+                                          : (bn == 128 ? headwise_gates_kernel<64, 128> : headwise_gates_kernel<64, 64>);
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), 0, stream, p);
+  }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "gate projection kernel launch failed: %s", hipGetErrorString(e));
   return XS_OK;

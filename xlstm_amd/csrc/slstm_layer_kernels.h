@@ -4,6 +4,8 @@
 // slstm_device_common.h.
 #pragma once
 
+#include <type_traits>
+
 namespace {
 
 // ---------------------------------------------------------------------------
@@ -230,6 +232,129 @@ __global__ __launch_bounds__(256) void headwise_gates_kernel(GatesParams p) {
         v.y = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
         *reinterpret_cast<uint2 *>(orow + 16 * j) = v;
       }
+    }
+  }
+}
+
+// The same projections for head dims 128 and 256 with the weights RESIDENT in registers.  A workgroup
+// owns one (head, operand) pair - all units of the slots i and f (operand x_conv) or z and o (operand x)
+// of one head - and walks over tiles of 64 tokens (32 at dh = 128).  Each of its 2 * dh / 64 waves keeps the MFMA
+// fragments of 64 units of one slot for the whole K range in VGPRs (128 at dh = 256), so the weights are
+// read once per workgroup, every token tile is read from memory exactly once in the whole launch, and LDS
+// carries the token fragments only: global -> registers -> LDS, two buffers, one barrier per K stage of
+// 64 inputs, the loads of stage k + 2 issued before the MFMAs of stage k.  (The kernel above reads a
+// token tile once per 128 output units - eight times at dh = 256 - and is bound by the fill rate of
+// the L1, the workgroups that share a tile asking the same L2 channel at the same time.)
+template <int I, typename T>
+__device__ __forceinline__ T &pick_set(T &a, T &b) {
+  if constexpr (I != 0) return b;
+  else return a;
+}
+
+template <int NST>
+__global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(GatesParams p, int combos, int parts) {
+  constexpr int NW = 2 * NST;        // waves
+  constexpr int NT = 64 * NW;        // threads
+  constexpr int BM = NT / 8;         // tokens per tile: a thread stages ONE 16-byte piece per K stage
+  constexpr int TM = BM / 16;
+  constexpr int dh = NST * 64;
+  __shared__ __attribute__((aligned(16))) unsigned char abuf[2][BM * kGateRowBytes];
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int combo = blockIdx.x % combos, part = blockIdx.x / combos;
+  const int pair = combo & 1, head = combo >> 1;
+  const int slot = pair * 2 + wave / NST;
+  const int u0 = (wave % NST) * 64;  // this wave's units of the slot
+
+  const int my_tiles = part < p.m_tiles ? (p.m_tiles - part + parts - 1) / parts : 0;
+  if (my_tiles == 0) return;  // the whole workgroup leaves before any barrier
+
+  // resident weight fragments: units u0 + 16 j + r16, inputs 64 s + 32 ks + 8 q .. +7
+  uint4 wfrag[NST][2][4];
+  {
+    const uint16_t *wbase = p.w[slot] + ((long long)head * dh + u0 + r16) * dh + 8 * q;
+#pragma unroll
+    for (int s = 0; s < NST; ++s)
+#pragma unroll
+      for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          wfrag[s][ks][j] = *reinterpret_cast<const uint4 *>(wbase + (long long)(16 * j) * dh + s * 64 + ks * 32);
+  }
+
+  const uint16_t *abase = (pair ? p.x : p.xc) + (long long)head * dh;
+  const long long asr = pair ? p.x_sr : p.xc_sr;
+  const int arow = tid >> 3;
+  const int adst = arow * kGateRowBytes + (tid & 7) * 16;
+  const int apc = (tid & 7) * 8;
+  // stage k of this workgroup: token tile part + parts * (k / NST), inputs 64 * (k % NST) .. +63
+  const int nstages = my_tiles * NST;
+  auto load_stage = [&](int k) -> uint4 {
+    const int m0 = (part + parts * (k / NST)) * BM;
+    const int m = m0 + arow < p.M ? m0 + arow : p.M - 1;
+    return *reinterpret_cast<const uint4 *>(abase + (long long)m * asr + (k % NST) * 64 + apc);
+  };
+
+  f32x4 acc[TM][4];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+
+  uint4 areg0 = load_stage(0), areg1 = make_uint4(0, 0, 0, 0);  // two named registers, not an array (it would be placed in LDS)
+  if (nstages > 1) areg1 = load_stage(1);
+  *reinterpret_cast<uint4 *>(&abuf[0][adst]) = areg0;
+  __syncthreads();
+
+  const long long colbase = (long long)slot * p.NH * dh + (long long)head * dh + u0 + 4 * q;
+  // NST is even, so stage k lives in LDS buffer k & 1 = s & 1 and in register set k & 1 alike
+  auto stage = [&](int k, auto sc) {
+    constexpr int s = decltype(sc)::value;
+    uint4 &mine = pick_set<s & 1>(areg0, areg1);         // held stage k, in LDS since the previous stage
+    uint4 &other = pick_set<(s + 1) & 1>(areg0, areg1);  // holds stage k + 1, loaded one stage ago
+    if (k + 2 < nstages) mine = load_stage(k + 2);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      uint4 av[TM];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        av[i] = *reinterpret_cast<const uint4 *>(&abuf[s & 1][(16 * i + r16) * kGateRowBytes + ks * 64 + q * 16]);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wfrag[s][ks][j]), __builtin_bit_cast(bf16x8, av[i]), acc[i][j], 0, 0, 0);
+    }
+    if (k + 1 < nstages)  // stage k + 1 goes to the other buffer, last read at stage k - 1
+      *reinterpret_cast<uint4 *>(&abuf[(s + 1) & 1][adst]) = other;
+    __syncthreads();
+  };
+  for (int k0 = 0; k0 < nstages; k0 += NST) {
+    stage(k0, std::integral_constant<int, 0>{});
+    stage(k0 + 1, std::integral_constant<int, 1>{});
+    if constexpr (NST > 2) {
+      stage(k0 + 2, std::integral_constant<int, 2>{});
+      stage(k0 + 3, std::integral_constant<int, 3>{});
+    }
+    // the token tile is complete: lane (r16, q) holds token m0 + 16 i + r16, units u0 + 16 j + 4 q .. +3
+    const int m0 = (part + parts * (k0 / NST)) * BM;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+      const int m = m0 + 16 * i + r16;
+      if (m < p.M) {
+        uint16_t *orow = p.out + (long long)m * p.out_sr + colbase;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint2 v;
+          v.x = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+          v.y = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+          *reinterpret_cast<uint2 *>(orow + 16 * j) = v;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     }
   }
 }
