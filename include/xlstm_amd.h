@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 3
+#define XS_ABI_VERSION 4
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -149,7 +149,7 @@ int xs_slstm_forward(const xs_slstm_args *args);
 int xs_slstm_step(const xs_slstm_args *args);
 
 /*
- * The two operations in front of the cell inside an sLSTM layer (bf16 only; the layer keeps its
+ * The operations around the cell inside an sLSTM layer (bf16 only; the layer keeps its
  * PyTorch path for everything else).  They enqueue one kernel each and allocate nothing.
  *
  * xs_causal_conv_silu: out[b,t,c] = silu(bias[c] + sum_j weight[c,j] * x[b, t-(K-1)+j, c]),
@@ -199,6 +199,27 @@ typedef struct xs_gates_args {
 } xs_gates_args;
 
 int xs_headwise_gates(const xs_gates_args *args);
+
+/*
+ * xs_headwise_group_norm: the per-head group norm behind the cell,
+ *   out[b,t,h,:] = (x[b,t,h,:] - mean) / sqrt(var + eps) * (1 + weight[h,:])
+ * with mean and (biased) variance over the dh units of head h of one token
+ * (MultiHeadLayerNorm.forward, xlstm/components/ln.py:51-68, with the residual weight of
+ * ln.py:29-33, as called by xlstm/blocks/slstm/layer.py:159).  x is addressed by strides so that
+ * the cell's [T,B,H] output is read where it lies; out is token-major, the layer's output layout.
+ */
+typedef struct xs_norm_args {
+  int32_t B, T, NH, dh;      /* dh a multiple of 4, at most 1024 */
+  int32_t dtype;             /* XS_BF16 */
+  float eps;
+  const void *x;             /* element (b,t,h,d) at b*x_stride_b + t*x_stride_t + h*x_stride_h + d */
+  int64_t x_stride_b, x_stride_t, x_stride_h;
+  const void *weight;        /* [NH*dh] or NULL (scale 1) */
+  void *out;                 /* [B,T,NH*dh] contiguous */
+  void *stream;
+} xs_norm_args;
+
+int xs_headwise_group_norm(const xs_norm_args *args);
 
 #ifdef __cplusplus
 }

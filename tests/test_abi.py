@@ -31,6 +31,7 @@ def test_abi_version_and_struct_mirror():
     # xs_conv_args: 5 int32 (+4 padding), then 11 8-byte fields; xs_gates_args: 4 int32, then 11 8-byte fields
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 11 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
+    assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
 
 
 def test_argument_errors_without_touching_the_gpu():
@@ -88,6 +89,18 @@ def test_layer_op_argument_errors_without_touching_the_gpu():
     assert lib.xs_headwise_gates(ctypes.byref(g)) == -2  # out rows overlap
     g.M = 0
     assert lib.xs_headwise_gates(ctypes.byref(g)) == 0
+    assert lib.xs_headwise_group_norm(None) == -1
+    n = _lib.NormArgs()
+    n.B, n.T, n.NH, n.dh, n.dtype = 2, 3, 4, 6, _lib.XS_BF16
+    assert lib.xs_headwise_group_norm(ctypes.byref(n)) == -5  # head dim not a multiple of 4
+    n.dh = 2048
+    assert lib.xs_headwise_group_norm(ctypes.byref(n)) == -5
+    n.dh = 64
+    assert lib.xs_headwise_group_norm(ctypes.byref(n)) == -1  # x / out missing
+    n.x, n.out, n.x_stride_b, n.x_stride_t, n.x_stride_h = 0x1000, 0x2000, 256, 514, 64
+    assert lib.xs_headwise_group_norm(ctypes.byref(n)) == -4  # stride not 8-byte aligned
+    n.B = 0
+    assert lib.xs_headwise_group_norm(ctypes.byref(n)) == 0
 
 
 def test_workspace_bytes_is_bounded_and_monotone():

@@ -135,6 +135,30 @@ def test_headwise_gates_slot_wiring_one_hot():
             assert torch.equal(got[m, s * H:(s + 1) * H], want), (m, s)
 
 
+@pytest.mark.parametrize("B,NH,T,dh,with_weight,cell_layout", [
+    (3, 4, 17, 64, True, True),
+    (2, 2, 5, 256, True, True),
+    (2, 3, 9, 36, False, False),    # 9 pieces of 4 units: part of a wave idles
+    (1, 1, 4, 1024, True, True),    # four pieces per lane
+    (5, 2, 1, 520, True, False),    # three pieces used of four
+])
+def test_headwise_group_norm_equals_float32_group_norm(B, NH, T, dh, with_weight, cell_layout):
+    from xlstm_amd import functional as hipF
+
+    g = torch.Generator().manual_seed(B + NH + T + dh)
+    H = NH * dh
+    if cell_layout:  # the cell's output: [S,B,H] storage seen as [B,NH,S,DH] (cell.py:354-374)
+        y = (torch.randn(T, B, H, generator=g) * 3 + 0.5).bfloat16().view(T, B, NH, dh).permute(1, 2, 0, 3)
+    else:
+        y = (torch.randn(B, NH, T, dh, generator=g) * 3 + 0.5).bfloat16()
+    w = (torch.randn(H, generator=g) * 0.2).bfloat16() if with_weight else None
+    want = F.group_norm(y.float().transpose(1, 2).reshape(B * T, H), NH, None if w is None else 1.0 + w.float(), None, 1e-5)
+    got = hipF.headwise_group_norm(y.to(DEV), None if w is None else w.to(DEV), 1e-5)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (B, T, H)
+    assert max_err(got.float().cpu().numpy(), want.view(B, T, H).numpy()) <= TOL
+
+
 def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
     """sLSTMLayer.forward and .step: the HIP conv / projection kernels against the PyTorch ops they replace."""
     from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig

@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 EXPORTS = (
     "xs_abi_version",
@@ -23,6 +23,7 @@ EXPORTS = (
     "xs_slstm_step",
     "xs_causal_conv_silu",
     "xs_headwise_gates",
+    "xs_headwise_group_norm",
 )
 
 
@@ -85,6 +86,21 @@ class GatesArgs(ctypes.Structure):
     ]
 
 
+class NormArgs(ctypes.Structure):
+    """Mirror of ``xs_norm_args``."""
+
+    _fields_ = [
+        ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("NH", ctypes.c_int32), ("dh", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("eps", ctypes.c_float),
+        ("x", ctypes.c_void_p),
+        ("x_stride_b", ctypes.c_int64), ("x_stride_t", ctypes.c_int64), ("x_stride_h", ctypes.c_int64),
+        ("weight", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
 class SlstmStatus(ctypes.Structure):
     """Mirror of ``xs_slstm_status`` (first bytes of the workspace)."""
 
@@ -123,6 +139,8 @@ def load() -> ctypes.CDLL:
     lib.xs_causal_conv_silu.argtypes = [ctypes.POINTER(ConvArgs)]
     lib.xs_headwise_gates.restype = ctypes.c_int
     lib.xs_headwise_gates.argtypes = [ctypes.POINTER(GatesArgs)]
+    lib.xs_headwise_group_norm.restype = ctypes.c_int
+    lib.xs_headwise_group_norm.argtypes = [ctypes.POINTER(NormArgs)]
     if lib.xs_abi_version() != ABI_VERSION:
         raise RuntimeError(f"xlstm_amd: ABI version {lib.xs_abi_version()} != expected {ABI_VERSION}; rebuild")
     _LIB = lib

@@ -343,7 +343,18 @@ int run_gates(const xs_gates_args *a) {
     int parts = cus / combos;
     if (parts < 1) parts = 1;
     if (parts > p.m_tiles) parts = p.m_tiles;
-    if (a->dh == 256)
+    if ((long long)((a->M + 63) / 64) * combos < cus) {
+      // too few token tiles to fill the device that way (a decode step): split the units instead
+      p.m_tiles = (a->M + 63) / 64;
+      p.n_tiles = 4 * a->NH * (a->dh / 64);
+      const size_t lds = (size_t)128 * (a->dh * 2 + 16);
+      void (*kern)(GatesParams) = a->dh == 256 ? headwise_gates_slab_kernel<4> : headwise_gates_slab_kernel<2>;
+      if (lds > 64 * 1024) {
+        const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
+        if (rc != XS_OK) return rc;
+      }
+      hipLaunchKernelGGL(kern, dim3((unsigned)(p.m_tiles * p.n_tiles)), dim3(256), lds, stream, p);
+    } else if (a->dh == 256)
       hipLaunchKernelGGL(headwise_gates_resident_kernel<4>, dim3((unsigned)(combos * parts)), dim3(512), 0, stream, p, combos, parts);
     else
       hipLaunchKernelGGL(headwise_gates_resident_kernel<2>, dim3((unsigned)(combos * parts)), dim3(256), 0, stream, p, combos, parts);
@@ -361,6 +372,30 @@ int run_gates(const xs_gates_args *a) {
   }
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "gate projection kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
+int run_group_norm(const xs_norm_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
+  if (a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "xs_headwise_group_norm computes on bf16 tensors only");
+  if (a->dh % 4 != 0 || a->dh > 1024) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not a multiple of 4 up to 1024", a->dh);
+  if (a->B == 0 || a->T == 0) return XS_OK;
+  if (!a->x || !a->out) return fail(XS_ERR_NULL, "x and out are required");
+  if (((uintptr_t)a->x % 8) || ((uintptr_t)a->out % 8) || ((uintptr_t)a->weight % 8) || (a->x_stride_b % 4) || (a->x_stride_t % 4) || (a->x_stride_h % 4))
+    return fail(XS_ERR_ALIGN, "x, weight, out and the strides of x must be 8-byte aligned");
+  const long long groups = (long long)a->B * a->T * a->NH;
+  const long long blocks = (groups + 3) / 4;
+  if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tokens for one launch");
+  NormParams p;
+  p.x = (const uint16_t *)a->x; p.x_sb = a->x_stride_b; p.x_st = a->x_stride_t; p.x_sh = a->x_stride_h;
+  p.weight = (const uint16_t *)a->weight; p.out = (uint16_t *)a->out; p.eps = a->eps;
+  p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
+  const int pieces = (a->dh + 255) / 256;
+  void (*kern)(NormParams) = pieces == 1 ? headwise_group_norm_kernel<1> : (pieces == 2 ? headwise_group_norm_kernel<2> : headwise_group_norm_kernel<4>);
+  hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)a->stream, p);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "group norm kernel launch failed: %s", hipGetErrorString(e));
   return XS_OK;
 }
 
@@ -399,6 +434,11 @@ int xs_causal_conv_silu(const xs_conv_args *args) {
 int xs_headwise_gates(const xs_gates_args *args) {
   g_err[0] = 0;
   return run_gates(args);
+}
+
+int xs_headwise_group_norm(const xs_norm_args *args) {
+  g_err[0] = 0;
+  return run_group_norm(args);
 }
 
 }  // extern "C"

@@ -1,5 +1,5 @@
-// The two kernels in front of the cell inside an sLSTM layer: causal depthwise convolution + SiLU,
-// and the four block-diagonal gate projections that produce the cell's input W.x.  bf16 operands,
+// The kernels around the cell inside an sLSTM layer: causal depthwise convolution + SiLU, the four
+// block-diagonal gate projections that produce the cell's input W.x, and the per-head group norm behind it.  bf16 operands,
 // float32 arithmetic.  Included by slstm_hip.hip only (one translation unit), after
 // slstm_device_common.h.
 #pragma once
@@ -291,7 +291,10 @@ __global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(Gate
   const int apc = (tid & 7) * 8;
   // stage k of this workgroup: token tile part + parts * (k / NST), inputs 64 * (k % NST) .. +63
   const int nstages = my_tiles * NST;
+  // (no branches around the loads and LDS writes of the pipeline: past the last stage they repeat it, so the
+  // compiler can count outstanding loads exactly instead of waiting for all of them at every join)
   auto load_stage = [&](int k) -> uint4 {
+    k = k < nstages ? k : nstages - 1;
     const int m0 = (part + parts * (k / NST)) * BM;
     const int m = m0 + arow < p.M ? m0 + arow : p.M - 1;
     return *reinterpret_cast<const uint4 *>(abase + (long long)m * asr + (k % NST) * 64 + apc);
@@ -303,8 +306,7 @@ __global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(Gate
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 
-  uint4 areg0 = load_stage(0), areg1 = make_uint4(0, 0, 0, 0);  // two named registers, not an array (it would be placed in LDS)
-  if (nstages > 1) areg1 = load_stage(1);
+  uint4 areg0 = load_stage(0), areg1 = load_stage(1);  // two named registers, not an array (it would be placed in LDS)
   *reinterpret_cast<uint4 *>(&abuf[0][adst]) = areg0;
   __syncthreads();
 
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(Gate
     constexpr int s = decltype(sc)::value;
     uint4 &mine = pick_set<s & 1>(areg0, areg1);         // held stage k, in LDS since the previous stage
     uint4 &other = pick_set<(s + 1) & 1>(areg0, areg1);  // holds stage k + 1, loaded one stage ago
-    if (k + 2 < nstages) mine = load_stage(k + 2);
+    mine = load_stage(k + 2);
 #pragma unroll
     for (int ks = 0; ks < 2; ++ks) {
       uint4 av[TM];
@@ -327,8 +329,7 @@ __global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(Gate
         for (int j = 0; j < 4; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wfrag[s][ks][j]), __builtin_bit_cast(bf16x8, av[i]), acc[i][j], 0, 0, 0);
     }
-    if (k + 1 < nstages)  // stage k + 1 goes to the other buffer, last read at stage k - 1
-      *reinterpret_cast<uint4 *>(&abuf[(s + 1) & 1][adst]) = other;
+    *reinterpret_cast<uint4 *>(&abuf[(s + 1) & 1][adst]) = other;  // stage k + 1 goes to the other buffer, last read at stage k - 1
     __syncthreads();
   };
   for (int k0 = 0; k0 < nstages; k0 += NST) {
@@ -355,6 +356,164 @@ __global__ __launch_bounds__(128 * NST) void headwise_gates_resident_kernel(Gate
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    }
+  }
+}
+
+// The same projections for FEW tokens (a decode step: M = batch size), head dims 128 and 256.  There the
+// weights are the traffic (4 * H * dh elements against M * H of x) and every compute unit should fetch its
+// share of them once: a workgroup computes 64 tokens x 64 units of one (slot, head) with the WHOLE K range
+// staged through LDS in one go - all global loads of the two operand tiles are in flight together, one
+// barrier, then 4 * NST MFMA k-steps per wave (four waves as 2 x 2, 32 x 32 outputs each).
+template <int NST>
+__global__ __launch_bounds__(256) void headwise_gates_slab_kernel(GatesParams p) {
+  constexpr int dh = NST * 64;
+  constexpr int RB = dh * 2 + 16;           // bytes per LDS row: data + pad (conflict-free 16-byte reads)
+  constexpr int PPR = dh / 8;               // 16-byte pieces per row
+  constexpr int ITEMS = 64 * PPR / 256;     // pieces of each operand tile a thread stages
+  extern __shared__ __attribute__((aligned(16))) unsigned char slab_lds[];
+  unsigned char *abuf = slab_lds, *wbuf = slab_lds + 64 * RB;
+
+  const int tid = threadIdx.x;
+  const int wave = tid >> 6, lane = tid & 63;
+  const int q = lane >> 4, r16 = lane & 15;
+  const int wm = wave >> 1, wn = wave & 1;
+  // blockIdx -> (token tile, slot, head, unit tile); unit tiles fastest so that neighbours share x rows in one L2
+  constexpr int npu = dh / 64;
+  int nt = blockIdx.x % p.n_tiles;
+  const int mtile = blockIdx.x / p.n_tiles;
+  const int ut = nt % npu; nt /= npu;
+  const int slot = nt & 3;
+  const int head = nt >> 2;
+  const int m0 = mtile * 64, n0 = ut * 64;
+
+  const uint16_t *abase = (slot >= 2 ? p.x : p.xc) + (long long)head * dh;
+  const long long asr = slot >= 2 ? p.x_sr : p.xc_sr;
+  const uint16_t *wbase = p.w[slot] + ((long long)head * dh + n0) * dh;
+  uint4 areg[ITEMS], wreg[ITEMS];
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const int e = tid + 256 * j;
+    const int row = e / PPR, pc = e % PPR;
+    const int m = m0 + row < p.M ? m0 + row : p.M - 1;
+    areg[j] = *reinterpret_cast<const uint4 *>(abase + (long long)m * asr + pc * 8);
+    wreg[j] = *reinterpret_cast<const uint4 *>(wbase + (long long)row * dh + pc * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < ITEMS; ++j) {
+    const int e = tid + 256 * j;
+    const int row = e / PPR, pc = e % PPR;
+    *reinterpret_cast<uint4 *>(&abuf[row * RB + pc * 16]) = areg[j];
+    *reinterpret_cast<uint4 *>(&wbuf[row * RB + pc * 16]) = wreg[j];
+  }
+  __syncthreads();
+
+  f32x4 acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+  for (int ks = 0; ks < 2 * NST; ++ks) {
+    uint4 av[2], wv[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) av[i] = *reinterpret_cast<const uint4 *>(&abuf[(wm * 32 + 16 * i + r16) * RB + ks * 64 + q * 16]);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) wv[j] = *reinterpret_cast<const uint4 *>(&wbuf[(wn * 32 + 16 * j + r16) * RB + ks * 64 + q * 16]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, wv[j]), __builtin_bit_cast(bf16x8, av[i]), acc[i][j], 0, 0, 0);
+  }
+  // lane (r16, q) holds token m0 + 32 wm + 16 i + r16, units n0 + 32 wn + 16 j + 4 q .. +3
+  const long long colbase = (long long)slot * p.NH * dh + (long long)head * dh + n0 + wn * 32 + 4 * q;
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + wm * 32 + 16 * i + r16;
+    if (m < p.M) {
+      uint16_t *orow = p.out + (long long)m * p.out_sr + colbase;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        uint2 v;
+        v.x = pack_bf16x2(acc[i][j][0], acc[i][j][1]);
+        v.y = pack_bf16x2(acc[i][j][2], acc[i][j][3]);
+        *reinterpret_cast<uint2 *>(orow + 16 * j) = v;
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// per-head group norm behind the cell (xlstm/components/ln.py:51-68 as called by
+// xlstm/blocks/slstm/layer.py:159): for every token and head, (x - mean) / sqrt(var + eps) * (1 + weight)
+// over the dh units of the head, biased variance, float32 arithmetic.  One wave per (token, head); a lane
+// holds 4 consecutive units per 256 units of head dim.  The input is addressed by strides, so the cell's
+// [S,B,H] output is read as it lies in memory and the result is written token-major [B,S,H].
+// ---------------------------------------------------------------------------
+struct NormParams {
+  const uint16_t *x;
+  long long x_sb, x_st, x_sh;
+  const uint16_t *weight;  // [NH*dh] or null
+  uint16_t *out;           // [B, T, NH*dh]
+  float eps;
+  int B, T, NH, dh;
+};
+
+template <int PIECES>  // 8-byte pieces per lane: ceil(dh / 256)
+__global__ __launch_bounds__(256) void headwise_group_norm_kernel(NormParams p) {
+  const int lane = threadIdx.x & 63;
+  const long long g = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);  // (b, t, head)
+  if (g >= (long long)p.B * p.T * p.NH) return;
+  const int head = (int)(g % p.NH);
+  const long long bt = g / p.NH;
+  const int t = (int)(bt % p.T);
+  const int b = (int)(bt / p.T);
+  const uint16_t *src = p.x + (long long)b * p.x_sb + (long long)t * p.x_st + (long long)head * p.x_sh;
+  float v[PIECES][4];
+  float sum = 0.0f;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int u = (lane + 64 * j) * 4;
+    if (u < p.dh) {
+      const uint2 w = *reinterpret_cast<const uint2 *>(src + u);
+      v[j][0] = bf16_bits_to_float(w.x & 0xFFFFu); v[j][1] = bf16_bits_to_float(w.x >> 16);
+      v[j][2] = bf16_bits_to_float(w.y & 0xFFFFu); v[j][3] = bf16_bits_to_float(w.y >> 16);
+    } else {
+      v[j][0] = v[j][1] = v[j][2] = v[j][3] = 0.0f;
+    }
+    sum += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o, 64);
+  const float mean = sum / (float)p.dh;
+  float sq = 0.0f;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int u = (lane + 64 * j) * 4;
+    if (u < p.dh) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { const float d = v[j][e] - mean; sq += d * d; }
+    }
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) sq += __shfl_xor(sq, o, 64);
+  const float rstd = rsqrtf(sq / (float)p.dh + p.eps);
+  uint16_t *dst = p.out + ((long long)b * p.T + t) * p.NH * p.dh + (long long)head * p.dh;
+#pragma unroll
+  for (int j = 0; j < PIECES; ++j) {
+    const int u = (lane + 64 * j) * 4;
+    if (u < p.dh) {
+      float sc[4] = {1.0f, 1.0f, 1.0f, 1.0f};
+      if (p.weight) {
+        const uint2 w = *reinterpret_cast<const uint2 *>(p.weight + (long long)head * p.dh + u);
+        sc[0] += bf16_bits_to_float(w.x & 0xFFFFu); sc[1] += bf16_bits_to_float(w.x >> 16);
+        sc[2] += bf16_bits_to_float(w.y & 0xFFFFu); sc[3] += bf16_bits_to_float(w.y >> 16);
+      }
+      uint2 o2;
+      o2.x = pack_bf16x2((v[j][0] - mean) * rstd * sc[0], (v[j][1] - mean) * rstd * sc[1]);
+      o2.y = pack_bf16x2((v[j][2] - mean) * rstd * sc[2], (v[j][3] - mean) * rstd * sc[3]);
+      *reinterpret_cast<uint2 *>(dst + u) = o2;
     }
   }
 }

@@ -334,3 +334,35 @@ def headwise_gates(x: torch.Tensor, x_conv: torch.Tensor, weights, num_heads: in
     if rc != 0:
         raise EngineError(f"xs_headwise_gates failed ({rc}): {_lib.last_error()}")
     return out
+
+
+def headwise_group_norm(y: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 1e-5,
+                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The layer's group norm behind the cell in one kernel (xlstm/components/ln.py:51-68 with the residual
+    weight, then the transpose + view of xlstm/blocks/slstm/layer.py:159): ``y`` [B,NH,S,DH] bfloat16 - the cell's
+    output, any strides with a contiguous last dim - to ``[B,S,NH*DH]``."""
+    lib = _lib.load()
+    _require_cuda("y", y)
+    if y.dim() != 4 or y.dtype != torch.bfloat16:
+        raise TypeError(f"y must be a bfloat16 [B, NH, S, DH] tensor, got {y.dtype} {tuple(y.shape)}")
+    B, NH, T, dh = (int(v) for v in y.shape)
+    if y.numel() and (y.stride(3) != 1 or y.data_ptr() % 8 or any(y.stride(i) % 4 for i in range(3))):
+        y = y.contiguous()
+    if weight is not None and (weight.dtype != torch.bfloat16 or not weight.is_contiguous()):
+        weight = weight.to(torch.bfloat16).contiguous()
+    if out is None:
+        out = torch.empty((B, T, NH * dh), dtype=torch.bfloat16, device=y.device)
+    a = _lib.NormArgs()
+    a.B, a.T, a.NH, a.dh = B, T, NH, dh
+    a.dtype = _lib.XS_BF16
+    a.eps = float(eps)
+    a.x = y.data_ptr()
+    a.x_stride_b, a.x_stride_h, a.x_stride_t = y.stride(0), y.stride(1), y.stride(2)
+    a.weight = weight.data_ptr() if weight is not None else None
+    a.out = out.data_ptr()
+    a.stream = torch.cuda.current_stream(y.device).cuda_stream
+    with torch.cuda.device(y.device):
+        rc = lib.xs_headwise_group_norm(ctypes.byref(a))
+    if rc != 0:
+        raise EngineError(f"xs_headwise_group_norm failed ({rc}): {_lib.last_error()}")
+    return out

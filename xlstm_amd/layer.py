@@ -8,12 +8,12 @@ reference's (``conv1d.conv``, ``fgate``, ``igate``, ``zgate``, ``ogate``,
 ``slstm_cell``, ``group_norm``), including its wiring of the module called
 ``fgate`` to the i slot and ``igate`` to the f slot (layer.py:144-149), so a
 reference state dict maps one to one (the cell's two tensors go through the
-external views).
+external views, ``cell.reference_state_dict_to_hip``).
 
 For bfloat16 inputs with a head dim that is a multiple of 64 the ops in front of the cell run
 as two HIP kernels of the engine (convolution + SiLU; the four projections written straight into the
-cell's input), see ``functional.causal_conv_silu`` / ``functional.headwise_gates``; otherwise, and for
-the group norm behind the cell, they are PyTorch-ROCm ops.
+cell's input), see ``functional.causal_conv_silu`` / ``functional.headwise_gates``, and so does the
+group norm behind it (``functional.headwise_group_norm``); otherwise they are PyTorch-ROCm ops.
 New: ``reset_mask[B,S]`` (document starts of packed rows) reaches the cell, and
 the causal convolution does not look across a document start either.
 """
@@ -186,6 +186,13 @@ class sLSTMLayer(nn.Module):
                                        self.config.num_heads)
         return torch.cat([self.fgate(x_conv), self.igate(x_conv), self.zgate(x), self.ogate(x)], dim=-1)
 
+    def _norm(self, y, B, S):
+        """Group norm per head of the cell output [B,NH,S,DH] -> [B,S,D] (layer.py:159)."""
+        if (self.fused_pre_ops and y.is_cuda and y.dtype == torch.bfloat16 and y.shape[-1] % 4 == 0 and y.shape[-1] <= 1024
+                and (self.group_norm.weight is None or self.group_norm.weight.dtype == torch.bfloat16)):
+            return hipF.headwise_group_norm(y, self.group_norm.weight, self.group_norm.eps)
+        return self.group_norm(y).transpose(1, 2).reshape(B, S, -1)
+
     def _fused(self, x) -> bool:
         return (self.fused_pre_ops and self.fgate.weight.dtype == torch.bfloat16
                 and hipF.fused_layer_ops_supported(x, self.config.num_heads, self.config.conv1d_kernel_size))
@@ -209,8 +216,7 @@ class sLSTMLayer(nn.Module):
         else:
             x_conv = x
         y, slstm_state = self.slstm_cell(self._gates(x, x_conv), state=slstm_state, reset_mask=reset_mask)
-        y = self.dropout(y)
-        out = self.group_norm(y).transpose(1, 2).reshape(B, S, -1)
+        out = self._norm(self.dropout(y), B, S)
         if return_last_state:
             return out, {"conv_state": conv_state, "slstm_state": slstm_state}
         return out
@@ -230,6 +236,5 @@ class sLSTMLayer(nn.Module):
         else:
             x_conv = x
         y, slstm_state = self.slstm_cell.step(self._gates(x, x_conv), slstm_state, state_out=slstm_state_out)
-        y = self.dropout(y)
-        out = self.group_norm(y).transpose(1, 2).reshape(B, S, -1)
+        out = self._norm(self.dropout(y), B, S)
         return out, {"conv_state": conv_state, "slstm_state": slstm_state}
