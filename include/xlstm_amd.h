@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 4
+#define XS_ABI_VERSION 5
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -172,6 +172,8 @@ typedef struct xs_conv_args {
   int64_t reset_stride_b;
   void *out;                 /* [B,T,D] contiguous */
   void *stream;
+  void *ring_out;            /* NULL, or with T == 1 a [B,K,D] contiguous buffer that receives the K-1 inputs
+                                before x followed by x: the state of the next step (conv.py:142-149) */
 } xs_conv_args;
 
 int xs_causal_conv_silu(const xs_conv_args *args);

@@ -28,8 +28,8 @@ def test_abi_version_and_struct_mirror():
     # xs_slstm_args: 6 int32, pointers/int64 after -> 8-byte aligned, 15 more 8-byte fields
     assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 15 * 8
     assert ctypes.sizeof(_lib.SlstmStatus) == 64
-    # xs_conv_args: 5 int32 (+4 padding), then 11 8-byte fields; xs_gates_args: 4 int32, then 11 8-byte fields
-    assert ctypes.sizeof(_lib.ConvArgs) == 24 + 11 * 8
+    # xs_conv_args: 5 int32 (+4 padding), then 12 8-byte fields; xs_gates_args: 4 int32, then 11 8-byte fields
+    assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
 

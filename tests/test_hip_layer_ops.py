@@ -86,6 +86,26 @@ def test_causal_conv_silu_reads_a_ring_view_and_strided_input():
     assert max_err(got.float().cpu().numpy(), want.numpy()) <= TOL
 
 
+def test_causal_conv_silu_step_writes_the_next_ring():
+    from xlstm_amd import functional as hipF
+
+    g = torch.Generator().manual_seed(6)
+    B, D, K = 3, 64, 4
+    ring = torch.randn(B, K, D, generator=g).bfloat16().to(DEV)
+    x = torch.randn(B, 1, D, generator=g).bfloat16().to(DEV)
+    w = torch.randn(D, K, generator=g).bfloat16().to(DEV)
+    new_ring = torch.full((B, K, D), 7.0, dtype=torch.bfloat16, device=DEV)
+    got = hipF.causal_conv_silu(x, w, None, ring[:, 1:], ring_out=new_ring)
+    want = hipF.causal_conv_silu(x, w, None, ring[:, 1:].contiguous())
+    assert torch.equal(got, want)
+    assert torch.equal(new_ring, torch.cat([ring[:, 1:], x], 1))
+    first = torch.full((B, K, D), 7.0, dtype=torch.bfloat16, device=DEV)  # no state yet: zeros, then x
+    hipF.causal_conv_silu(x, w, None, None, ring_out=first)
+    assert torch.equal(first, torch.cat([torch.zeros(B, K - 1, D, dtype=torch.bfloat16, device=DEV), x], 1))
+    with pytest.raises(hipF.EngineError):
+        hipF.causal_conv_silu(x, w, None, ring[:, 1:], ring_out=ring)  # in place is refused
+
+
 @pytest.mark.parametrize("lead,NH,dh", [
     ((2, 37), 4, 64),      # 64-token x 64-unit tiles, ragged token count
     ((3, 50), 2, 256),     # 64 x 128

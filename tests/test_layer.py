@@ -148,18 +148,21 @@ def test_prefill_then_steps_equals_one_forward(dtype):
 
 
 @pytest.mark.gpu
-def test_graphed_decoder_replays_equal_eager_steps():
-    """Two alternating HIP graphs of layer.step against the eager loop, with host work between replays."""
+@pytest.mark.parametrize("B,D,NH", [(8, 256, 4), (64, 512, 4), (5, 96, 3)],
+                         ids=["engine-ops", "engine-ops-operand-hint", "torch-ops"])
+def test_graphed_decoder_replays_equal_eager_steps(B, D, NH):
+    """Two alternating HIP graphs of layer.step against the eager loop, with host work between replays.
+    (64, 512, 4) is a shape where the step kernel takes the previous h as its bf16 operand; (5, 96, 3)
+    one where the ops around the cell are PyTorch's."""
     from xlstm_amd.decode import GraphedLayerDecoder
     from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
 
     torch.manual_seed(4)
     dev = torch.device("cuda:0")
-    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=4, backend="hip",
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=D, num_heads=NH, backend="hip",
                                         recurrent_weight_init="standard")).to(dev).bfloat16()
     layer.slstm_cell.keep_state_fp32 = True
-    B = 8
-    x = torch.randn(B, 16, 256, device=dev).bfloat16()
+    x = torch.randn(B, 16, D, device=dev).bfloat16()
     with torch.no_grad():
         _, st0 = layer(x[:, :5], return_last_state=True)
         dec = GraphedLayerDecoder(layer, B)

@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 EXPORTS = (
     "xs_abi_version",
@@ -66,6 +66,7 @@ class ConvArgs(ctypes.Structure):
         ("reset_stride_b", ctypes.c_int64),
         ("out", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
+        ("ring_out", ctypes.c_void_p),
     ]
 
 

@@ -371,22 +371,27 @@ class sLSTMCell_hip(nn.Module):
         return self._run(input, state, reset_mask, step=False)
 
     def step(self, input: torch.Tensor, state: Optional[torch.Tensor] = None, reset_mask=None,
-             state_out: Optional[torch.Tensor] = None):
+             state_out: Optional[torch.Tensor] = None, h_out: Optional[torch.Tensor] = None,
+             h_prev: Optional[torch.Tensor] = None):
         """One decode step (S == 1) through the step kernel.  Unlike the reference's
         ``step`` (cell.py:486-494, which hands back the state it was given) this
         returns the NEW state.  ``state_out`` (float32 [4,B,H], not overlapping ``state``)
-        receives it without an allocation, for decode loops that alternate two buffers."""
+        receives it without an allocation, for decode loops that alternate two buffers.
+        ``h_out`` ([1,B,H] in the input dtype) likewise receives the hidden state; ``h_prev`` is the
+        ``h_out`` of the previous step (bfloat16 inputs: the kernel then reads half the operand bytes,
+        see ``functional.StepPlan``).  Both only take effect on the steady-state path (float32 state carried
+        over, no mask); otherwise they are ignored and fresh tensors are returned."""
         if state_out is not None:
             B = self._input_bs(input).shape[0]
             if state_out.dtype != torch.float32 or not state_out.is_contiguous() or tuple(state_out.shape) != (
                     self.config.num_states, B, self.config.hidden_size):
                 raise ValueError("state_out must be a contiguous float32 [4, B, H] tensor")
-        fast = self._step_fast(input, state, reset_mask, state_out)
+        fast = self._step_fast(input, state, reset_mask, state_out, h_out, h_prev)
         if fast is not None:
             return fast
         return self._run(input, state, reset_mask, step=True, state_out=state_out)
 
-    def _step_fast(self, input, state, reset_mask, state_out):
+    def _step_fast(self, input, state, reset_mask, state_out, h_out=None, h_prev=None):
         """The decode steady state (float32 state carried over, no mask, no autograd) through a cached
         ``StepPlan``: the generic path spends more host time per token than the kernel runs."""
         if (reset_mask is not None or state is None or state.dtype != torch.float32 or not state.is_contiguous()
@@ -408,10 +413,12 @@ class sLSTMCell_hip(nn.Module):
             cached = (key, plan)
             object.__setattr__(self, "_step_plan_cache", cached)
         H = self.config.hidden_size
-        h = torch.empty((1, B, H), dtype=input.dtype, device=input.device)
+        h = h_out if h_out is not None else torch.empty((1, B, H), dtype=input.dtype, device=input.device)
+        if h.dtype != input.dtype or h.numel() != B * H or not h.is_contiguous():
+            raise ValueError("h_out must be a contiguous [1, B, H] tensor in the input dtype")
         s_out = state_out if state_out is not None else torch.empty((4, B, H), dtype=torch.float32, device=input.device)
         with torch.cuda.device(input.device):
-            cached[1](input, state, s_out, h)
+            cached[1](input, state, s_out, h, h_prev=h_prev)
         return self._permute_output(h), (s_out if self.keep_state_fp32 else s_out.to(input.dtype))
 
 

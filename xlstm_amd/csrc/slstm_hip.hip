@@ -282,8 +282,16 @@ int run_conv(const xs_conv_args *a) {
   if (a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "xs_causal_conv_silu computes on bf16 tensors only");
   if (a->K < 2 || a->K > 4) return fail(XS_ERR_UNSUPPORTED, "convolution of %d taps not supported (2..4)", a->K);
   if (a->D % 8 != 0) return fail(XS_ERR_UNSUPPORTED, "D = %d is not a multiple of 8", a->D);
+  if (a->ring_out && (a->T != 1 || a->reset)) return fail(XS_ERR_SHAPE, "ring_out goes with a single unmasked token (T == 1, no reset mask)");
   if (a->B == 0 || a->T == 0) return XS_OK;
   if (!a->x || !a->weight || !a->out) return fail(XS_ERR_NULL, "x, weight and out are required");
+  if ((uintptr_t)a->ring_out % 16) return fail(XS_ERR_ALIGN, "ring_out must be 16-byte aligned");
+  if (a->ring_out && a->conv_state) {  // other threads still read the old ring while the first ones write the new one
+    const uintptr_t lo0 = (uintptr_t)a->conv_state, lo1 = (uintptr_t)a->ring_out;
+    const uintptr_t sb = (uintptr_t)(a->conv_state_stride_b ? a->conv_state_stride_b : (long long)(a->K - 1) * a->D) * 2;
+    const uintptr_t n0 = sb * (uintptr_t)(a->B - 1) + (uintptr_t)(a->K - 1) * a->D * 2, n1 = (uintptr_t)a->B * a->K * a->D * 2;
+    if (lo0 < lo1 + n1 && lo1 < lo0 + n0) return fail(XS_ERR_SHAPE, "ring_out must not overlap conv_state");
+  }
   if (a->x_stride_t < a->D || (a->B > 1 && a->x_stride_b < a->D)) return fail(XS_ERR_SHAPE, "x strides overlap the innermost D elements");
   if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
   if (a->conv_state && a->conv_state_stride_b && (a->conv_state_stride_b < (long long)(a->K - 1) * a->D || a->conv_state_stride_b % 8))
@@ -301,6 +309,7 @@ int run_conv(const xs_conv_args *a) {
   p.w = (const uint16_t *)a->weight; p.bias = (const uint16_t *)a->bias;
   p.reset = a->reset; p.reset_sb = a->reset_stride_b;
   p.out = (uint16_t *)a->out;
+  p.ring_out = (uint16_t *)a->ring_out;
   p.B = a->B; p.T = a->T; p.D = a->D;
   hipStream_t stream = (hipStream_t)a->stream;
   void (*kern)(ConvParams) = a->K == 2 ? causal_conv_silu_kernel<2> : (a->K == 3 ? causal_conv_silu_kernel<3> : causal_conv_silu_kernel<4>);

@@ -13,7 +13,8 @@ namespace {
 // the activation of xlstm/blocks/slstm/layer.py:136-137).  One thread: 8 channels of one token.
 // Tap j of a kernel of KS taps multiplies the input KS-1-j tokens back; inputs before t = 0 come
 // from `state` (the KS-1 tokens before this call) or are zero; with a reset mask a tap that
-// would reach before the start of the token's document reads zero.
+// would reach before the start of the token's document reads zero.  A decode step (T = 1) can also
+// write the ring of the next step: the inputs of its taps, oldest first.
 // ---------------------------------------------------------------------------
 struct ConvParams {
   const uint16_t *x;
@@ -25,6 +26,7 @@ struct ConvParams {
   const unsigned char *reset;
   long long reset_sb;
   uint16_t *out;          // [B, T, D]
+  uint16_t *ring_out;     // [B, KS, D] or null (T == 1): the inputs of the taps, oldest first
   int B, T, D;
 };
 
@@ -80,6 +82,10 @@ __global__ __launch_bounds__(256) void causal_conv_silu_kernel(ConvParams p) {
     if (alive) {
       if (ts >= 0) src = p.x + (long long)b * p.x_sb + (long long)ts * p.x_st + c0;
       else if (p.state) src = p.state + (long long)b * p.state_sb + (long long)(KS - 1 + ts) * p.D + c0;
+    }
+    if (p.ring_out) {  // (T == 1, no mask: `alive` holds; a missing state reads as zeros)
+      const uint4 v = src ? *reinterpret_cast<const uint4 *>(src) : make_uint4(0, 0, 0, 0);
+      *reinterpret_cast<uint4 *>(p.ring_out + ((long long)b * KS + j) * p.D + c0) = v;
     }
     if (src) {
       const uint4 v = *reinterpret_cast<const uint4 *>(src);

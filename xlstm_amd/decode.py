@@ -36,6 +36,7 @@ class GraphedLayerDecoder:
         self.out = torch.zeros(B, 1, D, dtype=dtype, device=device)
         self.conv = [torch.zeros(B, K, D, dtype=dtype, device=device) for _ in range(2)]
         self.slstm = [torch.zeros(4, B, D, dtype=torch.float32, device=device) for _ in range(2)]
+        self.h = [torch.zeros(1, B, D, dtype=dtype, device=device) for _ in range(2)]  # hidden state of each set in dtype
         self.cur = 0
         self.graphs = [None, None]
         side = torch.cuda.Stream(device=device)
@@ -55,13 +56,16 @@ class GraphedLayerDecoder:
 
     def _one_step(self, k: int) -> None:
         out, st = self.layer.step(self.x, conv_state=(self.conv[k],), slstm_state=self.slstm[k],
-                                  slstm_state_out=self.slstm[1 - k])
-        self.conv[1 - k].copy_(st["conv_state"][0])
-        self.out.copy_(out)
+                                  slstm_state_out=self.slstm[1 - k], conv_state_out=self.conv[1 - k],
+                                  h_out=self.h[1 - k], h_prev=self.h[k], out=self.out)
+        if st["conv_state"][0].data_ptr() != self.conv[1 - k].data_ptr():  # a path that did not use the buffers
+            self.conv[1 - k].copy_(st["conv_state"][0])
+        if out.data_ptr() != self.out.data_ptr():
+            self.out.copy_(out)
 
     def reset(self) -> None:
         """Zero state: the start of a document."""
-        for t in self.conv + self.slstm:
+        for t in self.conv + self.slstm + self.h:
             t.zero_()
         self.cur = 0
 
@@ -73,6 +77,7 @@ class GraphedLayerDecoder:
         buf.zero_()
         buf[:, K - prev.shape[1]:].copy_(prev)
         self.slstm[self.cur].copy_(slstm_state)
+        self.h[self.cur].copy_(self.slstm[self.cur][0:1])  # the step kernel's operand hint: y rounded to dtype
 
     def step(self, x: torch.Tensor) -> torch.Tensor:
         """``x`` [B,1,D] -> the layer's output for this token (a buffer that the next call overwrites)."""

@@ -243,10 +243,12 @@ def fused_layer_ops_supported(x: torch.Tensor, num_heads: int, kernel_size: int)
 
 def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      conv_state: Optional[torch.Tensor] = None, reset_mask: Optional[torch.Tensor] = None,
-                     out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     out: Optional[torch.Tensor] = None, ring_out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """``silu(causal_conv1d(x))`` of an sLSTM layer (xlstm/components/conv.py:113-127,
     xlstm/blocks/slstm/layer.py:136-137) in one kernel.  ``x`` [B,S,D] bfloat16, ``weight`` [D,1,K] or [D,K],
-    ``conv_state`` [B,K-1,D] = the inputs before ``x``; ``reset_mask`` [B,S] stops the taps at document starts."""
+    ``conv_state`` [B,K-1,D] = the inputs before ``x``; ``reset_mask`` [B,S] stops the taps at document starts.
+    ``ring_out`` (S == 1): a contiguous bfloat16 [B,K,D] buffer, not overlapping ``conv_state``, that receives the
+    state of the next step (``conv_state`` followed by ``x``, conv.py:142-149)."""
     lib = _lib.load()
     _require_cuda("x", x)
     if x.dim() != 3 or x.dtype != torch.bfloat16:
@@ -271,6 +273,8 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
         reset_mask = _mask_u8(reset_mask, B, T)
     if out is None:
         out = torch.empty((B, T, D), dtype=torch.bfloat16, device=x.device)
+    elif out.dtype != torch.bfloat16 or out.numel() != B * T * D or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous bfloat16 tensor of {B * T * D} elements")
     a = _lib.ConvArgs()
     a.B, a.T, a.D, a.K = B, T, D, K
     a.dtype = _lib.XS_BF16
@@ -284,6 +288,11 @@ def causal_conv_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch
     a.reset = reset_mask.data_ptr() if reset_mask is not None else None
     a.reset_stride_b = reset_mask.stride(0) if reset_mask is not None else 0
     a.out = out.data_ptr()
+    a.ring_out = None
+    if ring_out is not None:
+        if ring_out.dtype != torch.bfloat16 or tuple(ring_out.shape) != (B, K, D) or not ring_out.is_contiguous():
+            raise ValueError(f"ring_out must be a contiguous bfloat16 [B, K, D] = {(B, K, D)} tensor")
+        a.ring_out = ring_out.data_ptr()
     a.stream = torch.cuda.current_stream(x.device).cuda_stream
     with torch.cuda.device(x.device):
         rc = lib.xs_causal_conv_silu(ctypes.byref(a))
@@ -317,6 +326,8 @@ def headwise_gates(x: torch.Tensor, x_conv: torch.Tensor, weights, num_heads: in
         ws.append(w if (w.dtype == torch.bfloat16 and w.is_contiguous()) else w.to(torch.bfloat16).contiguous())
     if out is None:
         out = torch.empty(tuple(x.shape[:-1]) + (4 * H,), dtype=torch.bfloat16, device=x.device)
+    elif out.dtype != torch.bfloat16 or out.numel() != M * 4 * H or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous bfloat16 tensor of {M * 4 * H} elements")
     a = _lib.GatesArgs()
     a.M, a.NH, a.dh = M, num_heads, dh
     a.dtype = _lib.XS_BF16
@@ -352,6 +363,8 @@ def headwise_group_norm(y: torch.Tensor, weight: Optional[torch.Tensor] = None, 
         weight = weight.to(torch.bfloat16).contiguous()
     if out is None:
         out = torch.empty((B, T, NH * dh), dtype=torch.bfloat16, device=y.device)
+    elif out.dtype != torch.bfloat16 or out.numel() != B * T * NH * dh or not out.is_contiguous():
+        raise ValueError(f"out must be a contiguous bfloat16 tensor of {B * T * NH * dh} elements")
     a = _lib.NormArgs()
     a.B, a.T, a.NH, a.dh = B, T, NH, dh
     a.dtype = _lib.XS_BF16

@@ -222,19 +222,36 @@ class sLSTMLayer(nn.Module):
         return out
 
     def step(self, x: torch.Tensor, conv_state: Optional[tuple] = None, slstm_state: Optional[torch.Tensor] = None,
-             slstm_state_out: Optional[torch.Tensor] = None):
-        """One token (layer.py:92-121).  ``slstm_state_out`` is handed to the cell's ``step``."""
+             slstm_state_out: Optional[torch.Tensor] = None, conv_state_out: Optional[torch.Tensor] = None,
+             h_out: Optional[torch.Tensor] = None, h_prev: Optional[torch.Tensor] = None,
+             out: Optional[torch.Tensor] = None):
+        """One token (layer.py:92-121).  The optional buffers let a decode loop run without allocations:
+        ``slstm_state_out`` / ``h_out`` / ``h_prev`` are handed to the cell's ``step``; ``conv_state_out``
+        ([B,k,D]) receives the new convolution ring and ``out`` ([B,1,D]) the result - both only on the engine's
+        bfloat16 path (``_fused``), elsewhere fresh tensors are returned as usual."""
         B, S, _ = x.shape
-        if self.config.conv1d_kernel_size > 0 and self._fused(x):
-            ring = self.conv1d.advance(x, conv_state)  # [B,k,D]: the k-1 inputs before x, then x
+        fused = self._fused(x)
+        if self.config.conv1d_kernel_size > 0 and fused:
             conv = self.conv1d.conv
-            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, ring[:, :-1])
+            k = self.config.conv1d_kernel_size
+            prev = conv_state[0] if isinstance(conv_state, (tuple, list)) else conv_state
+            if prev is not None:
+                assert prev.shape[1] in (k, k - 1), f"conv state holds {prev.shape[1]} inputs, expected {k} or {k - 1}"
+                if prev.shape[1] == k:
+                    prev = prev[:, 1:]  # the oldest slot is dropped
+            ring = conv_state_out if conv_state_out is not None else torch.empty(B, k, x.shape[2], dtype=x.dtype, device=x.device)
+            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, prev, ring_out=ring)
             conv_state = (ring,)
         elif self.config.conv1d_kernel_size > 0:
             x_conv, conv_state = self.conv1d.step(x, conv_state=conv_state)
             x_conv = self.conv_act_fn(x_conv)
         else:
             x_conv = x
-        y, slstm_state = self.slstm_cell.step(self._gates(x, x_conv), slstm_state, state_out=slstm_state_out)
-        out = self._norm(self.dropout(y), B, S)
+        y, slstm_state = self.slstm_cell.step(self._gates(x, x_conv), slstm_state, state_out=slstm_state_out,
+                                              h_out=h_out, h_prev=h_prev)
+        y = self.dropout(y)
+        if fused and out is not None:
+            out = hipF.headwise_group_norm(y, self.group_norm.weight, self.group_norm.eps, out=out)
+        else:
+            out = self._norm(y, B, S)
         return out, {"conv_state": conv_state, "slstm_state": slstm_state}
