@@ -224,7 +224,7 @@ def bench_config4(device, iters=3):
     model = xLSTMLMHarness(HarnessConfig()).to(device).bfloat16().eval()
     idx = torch.randint(0, 50304, (B, T), device=device)
     mask = torch.from_numpy(geometric_reset_mask(4, B, T, 768)).to(device)
-    total, cells = [], []
+    total, cells, layers = [], [], []
     with torch.no_grad():
         for i in range(iters + 1):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -235,13 +235,82 @@ def bench_config4(device, iters=3):
             if i:
                 total.append(e0.elapsed_time(e1))
                 cells.append(list(model.cell_ms))
+                layers.append(list(model.layer_ms))
     cell_ms = np.median(np.array(cells), axis=0)
-    return {"workload": "config 4: 24-block xLSTM LM harness, sLSTM cells at blocks 3/11/19 on HIP, rest PyTorch-ROCm, "
+    layer_ms = np.median(np.array(layers), axis=0)
+    return {"workload": "config 4: 24-block xLSTM LM harness, sLSTM layers at blocks 3/11/19 on HIP (conv, gate projections, "
+                        "cell, group norm), rest PyTorch-ROCm, "
                         "B=8 T=2048 D=1024 NH=4 bf16, documents mean 768",
             "forward_ms": float(np.median(total)), "slstm_cell_ms": [float(c) for c in cell_ms],
+            "slstm_layer_ms": [float(c) for c in layer_ms], "cell_share_of_slstm_layer": float(cell_ms.sum() / layer_ms.sum()),
             "slstm_cells_share": float(cell_ms.sum() / np.median(total)),
             "slstm_tokens_per_s_per_cell": float(B * T / cell_ms.mean() * 1e3),
             "finite": bool(torch.isfinite(logits.float()).all())}
+
+
+def bench_layer(device, iters=10, decode_steps=512):
+    """The caller of the path: one sLSTM layer (conv + SiLU, gate projections, cell, group norm) at the layer shape of
+    BASELINE config 4 (B=8, T=2048, D=1024, NH=4, bf16, documents of mean length 768), once with the engine's kernels
+    around the cell and once with the PyTorch ops they replace; and one decode step of the layer at the shape of
+    config 3 (B=256, D=2048, NH=8) replayed from HIP graphs."""
+    import numpy as np
+    import torch
+
+    from tests._util import geometric_reset_mask
+    from xlstm_amd.decode import GraphedLayerDecoder
+    from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
+
+    def timed(fn, n):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / n
+
+    torch.manual_seed(0)
+    out = {}
+    B, T, D, NH = 8, 2048, 1024, 4
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=D, num_heads=NH, backend="hip", recurrent_weight_init="standard"))
+    layer = layer.to(device).bfloat16().eval()
+    x = torch.randn(B, T, D, device=device).bfloat16()
+    mask = torch.from_numpy(geometric_reset_mask(4, B, T, 768)).to(device)
+    with torch.no_grad():
+        res = {}
+        for name, fused in (("engine_ops", True), ("torch_ops", False)):
+            layer.fused_pre_ops = fused
+            res[name] = layer(x, reset_mask=mask).float()
+            out["forward_ms_" + name] = timed(lambda: layer(x, reset_mask=mask), iters)
+        layer.fused_pre_ops = True
+        wx = layer._gates(x, x)
+        out["cell_ms"] = timed(lambda: layer.slstm_cell(wx, reset_mask=mask), iters)
+        out["max_abs_difference_between_the_two"] = float((res["engine_ops"] - res["torch_ops"]).abs().max())
+    out["forward_workload"] = "one sLSTM layer, B=8 T=2048 D=1024 NH=4 bf16, documents mean 768"
+
+    B, D, NH = 256, 2048, 8
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=D, num_heads=NH, backend="hip", recurrent_weight_init="standard"))
+    layer = layer.to(device).bfloat16().eval()
+    layer.slstm_cell.keep_state_fp32 = True
+    xs = torch.randn(B, 64, D, device=device).bfloat16()
+    with torch.no_grad():
+        for name, fused in (("engine_ops", True), ("torch_ops", False)):
+            layer.fused_pre_ops = fused
+            dec = GraphedLayerDecoder(layer, B)
+            for t in range(8):
+                dec.step(xs[:, t:t + 1])
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for t in range(decode_steps):
+                dec.step(xs[:, t % 64:t % 64 + 1])
+            torch.cuda.synchronize()
+            out["decode_step_us_graphed_" + name] = (time.perf_counter() - t0) / decode_steps * 1e6
+            out["decode_finite"] = bool(torch.isfinite(dec.out.float()).all())
+    out["decode_workload"] = "one sLSTM layer decode step, B=256 D=2048 NH=8 bf16, two alternating HIP graphs"
+    return out
 
 
 def main():
@@ -256,6 +325,9 @@ def main():
                     help="also time the cell at BASELINE configs 1, 4 and 5 (adds an 'all_configs' object)")
     ap.add_argument("--config4", action="store_true",
                     help="also run BASELINE config 4: the 24-block LM harness, timing its three sLSTM cells")
+    ap.add_argument("--layer", action="store_true",
+                    help="also time one sLSTM layer around the cell (adds a 'layer' object); --layer-only: nothing else")
+    ap.add_argument("--layer-only", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -280,6 +352,9 @@ def main():
         return
     if args.decode_only:
         print(json.dumps({"decode": bench_decode(device)}))
+        return
+    if args.layer_only:
+        print(json.dumps({"layer": bench_layer(device)}))
         return
     B, T, NH, dh = 16, 2048, 4, 256
     H = NH * dh
@@ -345,6 +420,8 @@ def main():
         ]
     if args.config4:
         out["config4"] = bench_config4(device)
+    if args.layer:
+        out["layer"] = bench_layer(device)
     if not args.no_decode:
         out["decode"] = bench_decode(device)
     if not args.no_cpu_baseline:

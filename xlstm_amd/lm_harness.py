@@ -157,21 +157,28 @@ class xLSTMLMHarness(nn.Module):
         self.post_blocks_norm = LayerNorm(D)
         self.lm_head = nn.Linear(D, cfg.vocab_size, bias=False)
         self.cell_ms: List[float] = []
+        self.layer_ms: List[float] = []
+
+    def slstm_layers(self):
+        return [b.xlstm for i, b in enumerate(self.blocks) if i in self.cfg.slstm_at]
 
     def slstm_cells(self):
         return [b.xlstm.slstm_cell for i, b in enumerate(self.blocks) if i in self.cfg.slstm_at]
 
     def forward(self, idx: torch.Tensor, reset_mask: Optional[torch.Tensor] = None, time_cells: bool = False):
         """``idx`` [B,S] token ids.  With ``time_cells`` the sLSTM cell calls are bracketed by
-        events on the current stream; ``self.cell_ms`` then holds one time per sLSTM block."""
+        events on the current stream; ``self.cell_ms`` then holds one time per sLSTM block and
+        ``self.layer_ms`` the time of the sLSTM layer around it (conv, gate projections, cell, group norm)."""
         events = []
+        layer_events = []
         hooks = []
         if time_cells:
-            for cell in self.slstm_cells():
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                events.append((e0, e1))
-                hooks.append(cell.register_forward_pre_hook(lambda m, a, e=e0: e.record()))
-                hooks.append(cell.register_forward_hook(lambda m, a, o, e=e1: e.record()))
+            for mods, evs in ((self.slstm_cells(), events), (self.slstm_layers(), layer_events)):
+                for mod in mods:
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    evs.append((e0, e1))
+                    hooks.append(mod.register_forward_pre_hook(lambda m, a, e=e0: e.record()))
+                    hooks.append(mod.register_forward_hook(lambda m, a, o, e=e1: e.record()))
         x = self.token_embedding(idx)
         for i, block in enumerate(self.blocks):
             x = block(x, reset_mask=reset_mask) if i in self.cfg.slstm_at else block(x)
@@ -181,4 +188,5 @@ class xLSTMLMHarness(nn.Module):
         if time_cells:
             torch.cuda.synchronize()
             self.cell_ms = [e0.elapsed_time(e1) for e0, e1 in events]
+            self.layer_ms = [e0.elapsed_time(e1) for e0, e1 in layer_events]
         return logits
