@@ -290,6 +290,8 @@ def bench_layer(device, iters=10, decode_steps=512):
         out["cell_ms"] = timed(lambda: layer.slstm_cell(wx, reset_mask=mask), iters)
         out["max_abs_difference_between_the_two"] = float((res["engine_ops"] - res["torch_ops"]).abs().max())
     out["forward_workload"] = "one sLSTM layer, B=8 T=2048 D=1024 NH=4 bf16, documents mean 768"
+    if decode_steps <= 0:
+        return out
 
     B, D, NH = 256, 2048, 8
     layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=D, num_heads=NH, backend="hip", recurrent_weight_init="standard"))
@@ -328,6 +330,9 @@ def main():
     ap.add_argument("--layer", action="store_true",
                     help="also time one sLSTM layer around the cell (adds a 'layer' object); --layer-only: nothing else")
     ap.add_argument("--layer-only", action="store_true")
+    ap.add_argument("--layer-iters", type=int, default=10, help="timed forward calls of the layer leg")
+    ap.add_argument("--layer-decode-steps", type=int, default=512,
+                    help="graphed decode steps of the layer leg; 0 skips them (short counter runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -354,7 +359,7 @@ def main():
         print(json.dumps({"decode": bench_decode(device)}))
         return
     if args.layer_only:
-        print(json.dumps({"layer": bench_layer(device)}))
+        print(json.dumps({"layer": bench_layer(device, args.layer_iters, args.layer_decode_steps)}))
         return
     B, T, NH, dh = 16, 2048, 4, 256
     H = NH * dh
@@ -421,7 +426,7 @@ def main():
     if args.config4:
         out["config4"] = bench_config4(device)
     if args.layer:
-        out["layer"] = bench_layer(device)
+        out["layer"] = bench_layer(device, args.layer_iters, args.layer_decode_steps)
     if not args.no_decode:
         out["decode"] = bench_decode(device)
     if not args.no_cpu_baseline:
