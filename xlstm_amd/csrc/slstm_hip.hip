@@ -300,7 +300,7 @@ int run_conv(const xs_conv_args *a) {
       ((uintptr_t)a->weight % 16) || ((uintptr_t)a->bias % 16) || ((uintptr_t)a->out % 16))
     return fail(XS_ERR_ALIGN, "x and its strides, conv_state, weight, bias and out must be 16-byte aligned");
   const long long threads = (long long)a->B * a->T * (a->D / 8);
-  const long long blocks = (threads + 255) / 256;
+  const long long blocks = ((threads + 255) / 256 + 7) / 8 * 8;  // a multiple of 8: the kernel deals them out by XCD
   if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tokens for one launch");
   ConvParams p;
   p.x = (const uint16_t *)a->x; p.x_sb = a->x_stride_b; p.x_st = a->x_stride_t;

@@ -33,7 +33,10 @@ struct ConvParams {
 template <int KS>
 __global__ __launch_bounds__(256) void causal_conv_silu_kernel(ConvParams p) {
   const int pieces = p.D >> 3;
-  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+  // workgroup i runs on XCD i % 8: give every XCD one contiguous range of tokens (the grid is a multiple of 8),
+  // so that neighbouring tokens, which share all but one of their taps, find them in the same L2
+  const long long wg = (long long)(blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+  const long long idx = wg * 256 + threadIdx.x;
   if (idx >= (long long)p.B * p.T * pieces) return;
   const int piece = (int)(idx % pieces);
   const long long bt = idx / pieces;
