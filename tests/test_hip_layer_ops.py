@@ -201,3 +201,19 @@ def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
     assert max_err(st_f["slstm_state"].cpu().numpy(), st_p["slstm_state"].cpu().numpy()) <= 5e-2
     assert max_err(o_f.float().cpu().numpy(), o_p.float().cpu().numpy()) <= 5e-2
     assert torch.equal(st_f2["conv_state"][0], st_p2["conv_state"][0])
+
+
+def test_layer_under_autograd_keeps_the_pytorch_ops_and_backward_raises():
+    """The engine's kernels record no graph: with grad enabled the layer must not cut the graph silently."""
+    from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
+
+    torch.manual_seed(12)
+    layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=4, backend="hip")).to(DEV).bfloat16()
+    x = torch.randn(2, 6, 256, device=DEV).bfloat16()
+    with torch.no_grad():
+        assert layer._fused(x)
+    assert not layer._fused(x)  # parameters require grad and grad mode is on
+    out = layer(x)
+    assert out.requires_grad
+    with pytest.raises(RuntimeError):
+        out.float().sum().backward()

@@ -188,13 +188,19 @@ class sLSTMLayer(nn.Module):
 
     def _norm(self, y, B, S):
         """Group norm per head of the cell output [B,NH,S,DH] -> [B,S,D] (layer.py:159)."""
-        if (self.fused_pre_ops and y.is_cuda and y.dtype == torch.bfloat16 and y.shape[-1] % 4 == 0 and y.shape[-1] <= 1024
+        if (self._engine_ops_allowed(y) and y.shape[-1] % 4 == 0 and y.shape[-1] <= 1024
                 and (self.group_norm.weight is None or self.group_norm.weight.dtype == torch.bfloat16)):
             return hipF.headwise_group_norm(y, self.group_norm.weight, self.group_norm.eps)
         return self.group_norm(y).transpose(1, 2).reshape(B, S, -1)
 
+    def _engine_ops_allowed(self, t) -> bool:
+        # the engine's kernels record no autograd graph: under grad mode the PyTorch ops run, and a backward pass
+        # reaches the cell, which raises (inference engine)
+        return self.fused_pre_ops and t.is_cuda and t.dtype == torch.bfloat16 and not (
+            torch.is_grad_enabled() and (t.requires_grad or any(q.requires_grad for q in self.parameters())))
+
     def _fused(self, x) -> bool:
-        return (self.fused_pre_ops and self.fgate.weight.dtype == torch.bfloat16
+        return (self._engine_ops_allowed(x) and self.fgate.weight.dtype == torch.bfloat16
                 and hipF.fused_layer_ops_supported(x, self.config.num_heads, self.config.conv1d_kernel_size))
 
     def forward(self, x: torch.Tensor, conv_state: Optional[torch.Tensor] = None,
