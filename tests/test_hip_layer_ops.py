@@ -196,6 +196,15 @@ def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
         layer.fused_pre_ops = False
         plain, st_p = layer(x, reset_mask=mask, return_last_state=True)
         o_p, st_p2 = layer.step(x[:, :1], conv_state=st_p["conv_state"], slstm_state=st_p["slstm_state"])
+        # a forward continues from the ring a step returned (k inputs) and from a shorter state alike
+        layer.fused_pre_ops = True
+        a1 = layer(x[:, 1:9], conv_state=st_f2["conv_state"])
+        a2 = layer(x[:, 1:9], conv_state=st_f2["conv_state"][0][:, -2:])
+        layer.fused_pre_ops = False
+        b1 = layer(x[:, 1:9], conv_state=st_p2["conv_state"])
+        b2 = layer(x[:, 1:9], conv_state=st_p2["conv_state"][0][:, -2:])
+    assert max_err(a1.float().cpu().numpy(), b1.float().cpu().numpy()) <= 5e-2
+    assert max_err(a2.float().cpu().numpy(), b2.float().cpu().numpy()) <= 5e-2
     assert max_err(fused.float().cpu().numpy(), plain.float().cpu().numpy()) <= 5e-2  # two bf16 pipelines, group-normed
     assert torch.equal(st_f["conv_state"], st_p["conv_state"])
     assert max_err(st_f["slstm_state"].cpu().numpy(), st_p["slstm_state"].cpu().numpy()) <= 5e-2

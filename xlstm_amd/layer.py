@@ -207,9 +207,15 @@ class sLSTMLayer(nn.Module):
                 slstm_state: Optional[torch.Tensor] = None, return_last_state: bool = False,
                 reset_mask: Optional[torch.Tensor] = None, **kwargs):
         B, S, _ = x.shape
+        if isinstance(conv_state, (tuple, list)):  # the ring a step returned (conv.py:131-157): oldest input first
+            conv_state = conv_state[0]
         if self.config.conv1d_kernel_size > 0 and self._fused(x):
             conv = self.conv1d.conv
-            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, conv_state, reset_mask)
+            pad = self.conv1d.pad
+            taps = conv_state
+            if taps is not None and taps.shape[1] != pad:  # only the last k-1 inputs matter; missing ones are zeros
+                taps = taps[:, -pad:] if taps.shape[1] > pad else F.pad(taps, (0, 0, pad - taps.shape[1], 0))
+            x_conv = hipF.causal_conv_silu(x, conv.weight, conv.bias, taps, reset_mask)
             if return_last_state:  # the last k-1 inputs (conv.py:126-127)
                 x_all = x if conv_state is None else torch.cat([conv_state.to(x.dtype), x], dim=1)
                 conv_state = x_all[:, -self.conv1d.pad:]
