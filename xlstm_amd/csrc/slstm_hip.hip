@@ -61,23 +61,23 @@ inline size_t xbuf_elems(int B, int NH, int dh) {
 
 typedef void (*SeqKernel)(SeqParams);
 
-template <bool BF16, int NCH>
+template <bool BF16, int NCH, bool FULL>
 SeqKernel pick_mt(int MT) {
   switch (MT) {
-    case 1: return slstm_seq_kernel<BF16, NCH, 1>;
-    case 2: return slstm_seq_kernel<BF16, NCH, 2>;
-    case 4: return slstm_seq_kernel<BF16, NCH, 4>;
+    case 1: return slstm_seq_kernel<BF16, NCH, 1, FULL>;
+    case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL>;
+    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL>;
     default: return nullptr;
   }
 }
 
-template <bool BF16>
+template <bool BF16, bool FULL>
 SeqKernel pick_kernel(int nch, int MT) {
   switch (nch) {
-    case 1: return pick_mt<BF16, 1>(MT);
-    case 2: return pick_mt<BF16, 2>(MT);
-    case 4: return pick_mt<BF16, 4>(MT);
-    case 8: return pick_mt<BF16, 8>(MT);
+    case 1: return pick_mt<BF16, 1, FULL>(MT);
+    case 2: return pick_mt<BF16, 2, FULL>(MT);
+    case 4: return pick_mt<BF16, 4, FULL>(MT);
+    case 8: return pick_mt<BF16, 8, FULL>(MT);
     default: return nullptr;
   }
 }
@@ -234,11 +234,13 @@ int run_forward(const xs_slstm_args *a) {
   }
   const int rows_per_launch = rows_per_wg * max_groups_per_head;
 
-  SeqKernel kern = bf16 ? pick_kernel<true>(nch, MT) : pick_kernel<false>(nch, MT);
-  if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
-
   for (int b0 = 0; b0 < B; b0 += rows_per_launch) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
+    // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
+    const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
+    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT) : pick_kernel<true, false>(nch, MT))
+                          : (full ? pick_kernel<false, true>(nch, MT) : pick_kernel<false, false>(nch, MT));
+    if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NH * NBT;
     // grid shapes of the three placements the kernel knows: one XCD per group, two XCDs per group, spread

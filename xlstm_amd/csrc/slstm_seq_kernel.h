@@ -70,7 +70,12 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
                :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 
-template <bool BF16, int NCH, int MT>
+// FULL: the head dim fills the K range of the four waves exactly (dh == 16 * NCH * elements per chunk) and, with
+// more than one row tile, every batch row of every tile exists.  The per-chunk "is this chunk needed" masks of
+// the arrival test are then compiled out (with one row tile, lanes of rows that do not exist read zeros from
+// past the end of the buffer descriptor, which never look like the "not written yet" pattern).  That matters:
+// the compute waves are bound by the number of instructions between the arrival of h and the MFMAs.
+template <bool BF16, int NCH, int MT, bool FULL>
 __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
@@ -496,20 +501,20 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       const int arow = rowbase + mt * 16 + r16;
       bool need[NCH];
       uint32_t needmask[NCH];
-      const bool row_ok = arow < rend;
+      const bool row_ok = (FULL && MT > 1) ? true : arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
         if (!(MT > 1 && prefetched)) areg[c] = make_uint4(0, 0, 0, 0);
-        need[c] = row_ok && k0 < dh;
+        need[c] = FULL ? true : (row_ok && k0 < dh);
         needmask[c] = need[c] ? 0xFFFFFFFFu : 0u;  // (masks, not selects: the tests below stay straight-line code)
       }
       if (t == 0) {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
           const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-          if (need[c] && p.s0) {
+          if ((FULL ? row_ok : need[c]) && p.s0) {
             const float *src = p.s0 + (long long)arow * H + head * dh + k0;
             if (BF16) {
               const float4 lo = *reinterpret_cast<const float4 *>(src);
