@@ -501,6 +501,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       const int arow = rowbase + mt * 16 + r16;
       bool need[NCH];
       uint32_t needmask[NCH];
+      uint4 breg[NCH];     // one row tile: the second of the two polls in flight
       const bool row_ok = (FULL && MT > 1) ? true : arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
 #pragma unroll
@@ -510,6 +511,43 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         need[c] = FULL ? true : (row_ok && k0 < dh);
         needmask[c] = need[c] ? 0xFFFFFFFFu : 0u;  // (masks, not selects: the tests below stay straight-line code)
       }
+      // ---- 2. (defined here, used below) partial R.h over this wave's K slab, all four gates, from the operand
+      //      registers given; rows that start a document and chunks that are not needed count as zeros
+      f32x4 acc[4];
+      auto multiply = [&](uint4 (&op)[NCH]) {
+        // (a whole wave rarely has anything to clear: one uniform branch instead of 4 selects per chunk)
+        bool clear_any = row_reset;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) clear_any |= !need[c];
+        if (__builtin_amdgcn_ballot_w64(clear_any) != 0ull) {
+#pragma unroll
+          for (int c = 0; c < NCH; ++c)
+            if (row_reset || !need[c]) op[c] = make_uint4(0, 0, 0, 0);
+        }
+        XS_TICK(0);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          if (BF16) {
+            const bf16x8 av = __builtin_bit_cast(bf16x8, op[c]);
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+              acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, rreg[g][c]), acc[g], 0, 0, 0);
+          } else {
+            const uint32_t aw[4] = {op[c].x, op[c].y, op[c].z, op[c].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+#pragma unroll
+              for (int g = 0; g < 4; ++g) {
+                const uint32_t bw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
+                acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[g], 0, 0, 0);
+              }
+            }
+          }
+        }
+      };
+      bool multiplied = false;
       if (t == 0) {
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
@@ -525,6 +563,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
               areg[c] = *reinterpret_cast<const uint4 *>(src);
             }
           }
+        }
+        if (MT == 1) {
+          multiply(areg);
+          multiplied = true;
         }
       } else {
         if (kDeepPrefetch) {
@@ -545,9 +587,11 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           // and the skew between the four waves at the barrier.  Lanes whose batch row does not exist
           // ask for an offset past the descriptor's end: zeros, no memory traffic, so the doubled poll
           // rate stays far below what a compute unit can pull from the L2.  The decisions are
-          // wave-uniform (ballot) so that the waits keep exact counts.
+          // wave-uniform (ballot) so that the waits keep exact counts, and the MFMAs are issued right where
+          // a set is found complete, from that set's registers, while the other poll is still in flight
+          // (its registers are dead until the next step's polls overwrite them, in order): a single copy
+          // of the MFMAs behind the loop would have to wait for every outstanding load.
           const int xl = row_ok ? xlane : 0x7FFFFF00;
-          uint4 breg[NCH];
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
             areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
@@ -555,13 +599,17 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
             breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
+          uint32_t spins = 0;
           if (!aborted) {
-            uint32_t spins = 0;
             for (;;) {
               uint32_t ma = 0u;
 #pragma unroll
               for (int c = 0; c < NCH; ++c) ma = mark_join<BF16>(ma, chunk_mark<BF16>(areg[c]) & needmask[c]);
-              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(ma)) == 0ull) break;
+              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(ma)) == 0ull) {
+                multiply(areg);
+                multiplied = true;
+                break;
+              }
 #pragma unroll
               for (int c = 0; c < NCH; ++c)
                 areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
@@ -569,8 +617,10 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
               for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, chunk_mark<BF16>(breg[c]) & needmask[c]);
               if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mb)) == 0ull) {
-#pragma unroll
-                for (int c = 0; c < NCH; ++c) areg[c] = breg[c];
+                // (no copy into areg: the poll just re-issued into areg is still in flight, and a copy would
+                // have to wait for it - about half a round trip on the critical path of every step)
+                multiply(breg);
+                multiplied = true;
                 break;
               }
 #pragma unroll
@@ -609,9 +659,11 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
         // waits for ALL of its outstanding loads, the next tile's requests included)
         // first look at everything at once: one mark over all chunks this lane needs
         uint32_t mark = 0u;
+        if (MT != 1) {  // (with one row tile the loop above has seen a complete set, or given up)
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[c]) & needmask[c]);
-        if (!aborted && mark_has_sentinel<BF16>(mark)) {
+          for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[c]) & needmask[c]);
+        }
+        if (MT != 1 && !aborted && mark_has_sentinel<BF16>(mark)) {
           uint32_t spins = 0;
           for (;;) {
             bool any_bad = false;
@@ -647,39 +699,15 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #endif
         }
       }
-      // (a whole wave rarely has anything to clear: one uniform branch instead of 4 selects per chunk)
-      bool clear_any = row_reset;
+      if (MT == 1) {
+        // (every path above has multiplied, except a wait that ran out: nothing may refer to the poll registers
+        // behind the loop, or the compiler keeps copies of them alive across it and waits for the poll in flight)
+        if (!multiplied) {
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) clear_any |= !need[c];
-      if (__builtin_amdgcn_ballot_w64(clear_any) != 0ull) {
-#pragma unroll
-        for (int c = 0; c < NCH; ++c)
-          if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
-      }
-
-      // ---- 2. partial R.h over this wave's K slab, all four gates
-      XS_TICK(0);
-      f32x4 acc[4];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        if (BF16) {
-          const bf16x8 av = __builtin_bit_cast(bf16x8, areg[c]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, rreg[g][c]), acc[g], 0, 0, 0);
-        } else {
-          const uint32_t aw[4] = {areg[c].x, areg[c].y, areg[c].z, areg[c].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const uint32_t bw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
-              acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[g], 0, 0, 0);
-            }
-          }
+          for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
         }
+      } else if (!multiplied) {
+        multiply(areg);
       }
 
       if (kDeepPrefetch) {
