@@ -799,6 +799,17 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       hst[it & 3][tid] = y;
       if (kDrainerPublishes && lane == 0)
         __hip_atomic_store(&pubflag[wave], (uint32_t)it + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (MT == 1) {
+        // The poll that did not deliver is still in flight when its set's registers die.  Keeping both sets
+        // alive to the end of the iteration stops the compiler from handing those registers to the gating
+        // code, where the first write to one of them would have to wait for that poll (on the critical path);
+        // here, after the publication, it has long landed.
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+          asm volatile("" :: "v"(areg[c].x), "v"(areg[c].y), "v"(areg[c].z), "v"(areg[c].w));
+          asm volatile("" :: "v"(breg[c].x), "v"(breg[c].y), "v"(breg[c].z), "v"(breg[c].w));
+        }
+      }
       XS_TICK(4);
     }
   }
