@@ -64,7 +64,9 @@ struct CellState { float y, c, n, m; };
 // routines were (h within 5e-7, state within 5e-6 over 2048 steps; the float32 recurrence itself
 // sets that floor) at less than half the instructions, and gating is on the critical path of a step.
 __device__ __forceinline__ void slstm_pointwise(float iraw, float fraw, float zraw, float oraw, CellState &s) {
-  const float lfm = s.m + (fminf(fraw, 0.0f) - __logf(1.0f + __expf(-fabsf(fraw))));  // m + logsigmoid(f)
+  // m + logsigmoid(f).  The argument of the logarithm lies in (1, 2], so the bare v_log_f32 (a base-2 logarithm)
+  // serves: __logf would wrap it in a dozen instructions of range handling, all on the critical path of a step.
+  const float lfm = s.m + (fminf(fraw, 0.0f) - 0.69314718055994531f * __builtin_amdgcn_logf(1.0f + __expf(-fabsf(fraw))));
   const float mnew = (s.n == 0.0f) ? iraw : fmaxf(iraw, lfm);
   const float og = __builtin_amdgcn_rcpf(1.0f + __expf(-oraw));                      // sigmoid(o)
   const float ig = fminf(__expf(iraw - mnew), 1.0f);
