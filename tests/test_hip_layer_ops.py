@@ -226,3 +226,16 @@ def test_layer_under_autograd_keeps_the_pytorch_ops_and_backward_raises():
     assert out.requires_grad
     with pytest.raises(RuntimeError):
         out.float().sum().backward()
+
+
+def test_layer_ops_accept_empty_inputs():
+    from xlstm_amd import functional as hipF
+
+    w = torch.zeros(64, 4, dtype=torch.bfloat16, device=DEV)
+    assert tuple(hipF.causal_conv_silu(torch.zeros(2, 0, 64, dtype=torch.bfloat16, device=DEV), w).shape) == (2, 0, 64)
+    assert tuple(hipF.causal_conv_silu(torch.zeros(0, 5, 64, dtype=torch.bfloat16, device=DEV), w).shape) == (0, 5, 64)
+    ws = [torch.zeros(1, 64, 64, dtype=torch.bfloat16, device=DEV)] * 4
+    e = torch.zeros(0, 3, 64, dtype=torch.bfloat16, device=DEV)
+    assert tuple(hipF.headwise_gates(e, e, ws, 1).shape) == (0, 3, 256)
+    assert tuple(hipF.headwise_group_norm(torch.zeros(2, 1, 0, 64, dtype=torch.bfloat16, device=DEV)).shape) == (2, 0, 64)
+    torch.cuda.synchronize()
