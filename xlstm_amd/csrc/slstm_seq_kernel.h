@@ -54,7 +54,6 @@ struct SeqParams {
 // ---------------------------------------------------------------------------
 constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
 constexpr int kRing = 8;       // slots of the exchange ring
-constexpr int kPollStagger = 6;  // s_sleep units (64 cycles) between the two polls of a step (measured best of 2 .. 16)
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -75,7 +74,9 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
 // the arrival test are then compiled out (with one row tile, lanes of rows that do not exist read zeros from
 // past the end of the buffer descriptor, which never look like the "not written yet" pattern).  That matters:
 // the compute waves are bound by the number of instructions between the arrival of h and the MFMAs.
-template <bool BF16, int NCH, int MT, bool FULL>
+// STG (one row tile only): s_sleep units (64 cycles) between the two polls of a step, about half a poll round trip;
+// that grows with the number of workgroups that share an L2 (measured best: 3 at 16 workgroups per XCD, 6 at 32).
+template <bool BF16, int NCH, int MT, bool FULL, int STG>
 __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
@@ -582,7 +583,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
           for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
         } else if (MT == 1) {
-          // Two polls in flight, about half a round trip apart (kPollStagger), re-issued alternately:
+          // Two polls in flight, about half a round trip apart (STG, chosen by the host), re-issued alternately:
           // a poll returns every ~300 cycles instead of every ~600, which halves both the wait for h
           // and the skew between the four waves at the barrier.  Lanes whose batch row does not exist
           // ask for an offset past the descriptor's end: zeros, no memory traffic, so the doubled poll
@@ -595,7 +596,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
             areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
-          __builtin_amdgcn_s_sleep(kPollStagger);
+          __builtin_amdgcn_s_sleep(STG);
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
             breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
