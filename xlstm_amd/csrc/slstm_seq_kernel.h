@@ -24,6 +24,7 @@ struct SeqParams {
   int NBT;       // batch tiles (independent groups) per head
   int rows_per_wg;
   long long spin_limit;
+  int prefetch;  // 1: wave 6 pulls W.x of future steps into the L2 through the scalar cache (one row tile)
 };
 
 // ---------------------------------------------------------------------------
@@ -34,7 +35,7 @@ struct SeqParams {
 //         NCH*32 (bf16) or NCH*16 (fp32) input units, the four waves 4x that.
 //   MT  : 16-row batch tiles handled one after the other by a workgroup.
 //
-// Six waves per workgroup, one barrier per (step, tile) iteration shared by all:
+// Seven waves per workgroup, one barrier per (step, tile) iteration shared by all:
 //   waves 0-3  compute: poll h_{t-1}, MFMA, reduce through LDS, gating, publish h_t.
 //              Their vector-memory queue only ever holds L2-resident traffic (the
 //              exchange ring), because vector memory completes in order within a wave
@@ -43,6 +44,12 @@ struct SeqParams {
 //              into an LDS ring (kLookahead iterations in flight).
 //   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
 //              output tensor in HBM.
+//   wave 6     prefetcher (one row tile of at most 8 rows; ends at once otherwise): touches the W.x lines of
+//              the step kPrefetchAhead ahead with SCALAR loads.  A compute unit returns vector-memory data in
+//              order across its waves, so every feeder load that misses to HBM delays the polls issued behind
+//              it (measured: an L2 hit takes 200 cycles alone and 600 with another wave's misses in flight,
+//              unchanged at 210 when those misses go through the scalar cache).  With the lines already in the
+//              L2 the feeder's loads are short.
 //
 // Exchange ring: kRing slots, slot t % kRing holds h_t as [row tile][member][16 rows][16 units].
 // A word is either data or the "not written yet" pattern.  A workgroup re-arms its own
@@ -54,6 +61,7 @@ struct SeqParams {
 // ---------------------------------------------------------------------------
 constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
 constexpr int kRing = 8;       // slots of the exchange ring
+constexpr int kPrefetchAhead = 8;  // steps between the scalar-cache touch of a W.x line and the step that uses it
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
@@ -387,6 +395,44 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
       for (int i = 0; i < 2; ++i) dst[i] = dprof[i];
     }
 #endif
+    return;
+  }
+
+  // =========================================================================
+  // wave 6: prefetcher.  It takes part in every barrier (plain s_barrier: it has no LDS traffic of its own
+  // and must not wait for its loads there) and issues nothing but scalar loads whose results are never read:
+  // they all land in one scalar register that stays reserved for the whole loop.
+  // =========================================================================
+  if (wave == 6) {
+    if (MT != 1 || !p.prefetch) return;  // (a wave that has ended does not count for the barriers)
+    constexpr int LM = 128 / (16 * ESZ);  // members whose 16 units share one 128-byte line of W.x: 4 (bf16) / 2 (fp32)
+    const int nrows = rend - rowbase;
+    const long long row_bytes = 4ll * H * ESZ;
+    const long long cluster = ((long long)head * dh + (member / LM) * LM * 16) * ESZ;  // first byte of the shared line in a gate's block
+    const char *const wxb = reinterpret_cast<const char *>(p.wx);
+    uint32_t sink = 0;
+    __builtin_amdgcn_s_barrier();  // prologue barrier
+    for (int itp = 0; itp < NITpad; ++itp) {
+      const int tp = itp + kPrefetchAhead;
+      if (tp < p.T) {
+        for (int r = 0; r < nrows; ++r) {
+          const long long rowoff = ((long long)(rowbase + r) * p.wx_sb + (long long)tp * p.wx_st) * ESZ;
+          for (int g = member % LM; g < 4; g += LM) {  // the members that share a line split the gates between them
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+              long long o = (long long)g * H * ESZ + cluster + half * 64;
+              o = o < row_bytes - 4 ? o : row_bytes - 4;  // (a line of the last head may reach past the row)
+              const unsigned long long a = reinterpret_cast<unsigned long long>(wxb + rowoff + o);
+              const unsigned long long au = (unsigned long long)uniform((uint32_t)a) | ((unsigned long long)uniform((uint32_t)(a >> 32)) << 32);
+              asm volatile("s_load_dword %0, %1, 0x0" : "+s"(sink) : "s"(au));
+            }
+          }
+        }
+      }
+      __builtin_amdgcn_s_barrier();  // barrier #itp
+    }
+    __builtin_amdgcn_s_barrier();  // final barrier
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(sink));
     return;
   }
 
