@@ -267,7 +267,9 @@ int run_forward(const xs_slstm_args *a) {
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
     p.spin_limit = a->spin_limit;
-    p.prefetch = (MT == 1 && rows_per_wg <= 8) ? 1 : 0;
+    // the prefetch wave issues 2 (bf16) or 4 (fp32) scalar loads per batch row and step, and only about 15 of them
+    // can be in flight: with more than 16 per step it falls behind and holds up the barriers (measured 2x slower)
+    p.prefetch = (MT == 1 && rows_per_wg * (bf16 ? 2 : 4) <= 16) ? 1 : 0;
     // with four row tiles the polled tiles are staged in dynamic LDS: [2][4 waves][nch] KiB
     const size_t dyn_lds = MT >= 4 ? (size_t)nch * 8192 : 0;
     if (dyn_lds) {

@@ -44,7 +44,7 @@ struct SeqParams {
 //              into an LDS ring (kLookahead iterations in flight).
 //   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
 //              output tensor in HBM.
-//   wave 6     prefetcher (one row tile of at most 8 rows; ends at once otherwise): touches the W.x lines of
+//   wave 6     prefetcher (one row tile of few rows; ends at once otherwise): touches the W.x lines of
 //              the step kPrefetchAhead ahead with SCALAR loads.  A compute unit returns vector-memory data in
 //              order across its waves, so every feeder load that misses to HBM delays the polls issued behind
 //              it (measured: an L2 hit takes 200 cycles alone and 600 with another wave's misses in flight,
@@ -419,7 +419,7 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
           const long long rowoff = ((long long)(rowbase + r) * p.wx_sb + (long long)tp * p.wx_st) * ESZ;
           for (int g = member % LM; g < 4; g += LM) {  // the members that share a line split the gates between them
 #pragma unroll
-            for (int half = 0; half < 2; ++half) {
+            for (int half = 0; half < 2; ++half) {  // (a miss of the scalar cache brings 64 bytes into the L2, not the line)
               long long o = (long long)g * H * ESZ + cluster + half * 64;
               o = o < row_bytes - 4 ? o : row_bytes - 4;  // (a line of the last head may reach past the row)
               const unsigned long long a = reinterpret_cast<unsigned long long>(wxb + rowoff + o);
