@@ -9,7 +9,8 @@ namespace {
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kThreads = 448;           // 4 compute waves + feeder wave + drainer wave + prefetch wave
+constexpr int kThreads = 384;           // 4 compute waves + feeder wave + drainer wave (+ up to 2 prefetch waves)
+constexpr int kMaxPrefetchWaves = 2;
 constexpr int kTileStride = 20;         // floats between unit columns of a partial tile in LDS
 constexpr int kTileFloats = 16 * kTileStride;
 constexpr uint32_t kSentinel32 = 0xFFFFFFFFu;  // fp32 "not written yet"

@@ -267,16 +267,21 @@ int run_forward(const xs_slstm_args *a) {
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
     p.spin_limit = a->spin_limit;
-    // the prefetch wave issues 2 (bf16) or 4 (fp32) scalar loads per batch row and step, and only about 15 of them
-    // can be in flight: with more than 16 per step it falls behind and holds up the barriers (measured 2x slower)
-    p.prefetch = (MT == 1 && rows_per_wg * (bf16 ? 2 : 4) <= 16) ? 1 : 0;
+    // a prefetch wave issues 2 (bf16) or 4 (fp32) scalar loads per batch row of a tile; 8 per wave and iteration
+    // and 16 in all are what the scalar cache sustains, a tile that needs more goes without (prefetch waves that
+    // fall behind hold up the barriers: measured 2x slower)
+    {
+      const int rows_in_tile = rows_per_wg < 16 ? rows_per_wg : 16;
+      const int want = (rows_in_tile * (bf16 ? 2 : 4) + 7) / 8;
+      p.prefetch = want <= max_prefetch_waves(nch) ? want : 0;
+    }
     // with four row tiles the polled tiles are staged in dynamic LDS: [2][4 waves][nch] KiB
     const size_t dyn_lds = MT >= 4 ? (size_t)nch * 8192 : 0;
     if (dyn_lds) {
       const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), dyn_lds);
       if (rc != XS_OK) return rc;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads), dyn_lds, stream, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads + 64 * p.prefetch), dyn_lds, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
   }

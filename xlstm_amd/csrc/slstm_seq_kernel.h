@@ -24,7 +24,7 @@ struct SeqParams {
   int NBT;       // batch tiles (independent groups) per head
   int rows_per_wg;
   long long spin_limit;
-  int prefetch;  // 1: wave 6 pulls W.x of future steps into the L2 through the scalar cache (one row tile)
+  int prefetch;  // number of prefetch waves launched behind the six others (0 .. kMaxPrefetchWaves)
 };
 
 // ---------------------------------------------------------------------------
@@ -35,7 +35,7 @@ struct SeqParams {
 //         NCH*32 (bf16) or NCH*16 (fp32) input units, the four waves 4x that.
 //   MT  : 16-row batch tiles handled one after the other by a workgroup.
 //
-// Seven waves per workgroup, one barrier per (step, tile) iteration shared by all:
+// Six to ten waves per workgroup, one barrier per (step, tile) iteration shared by all:
 //   waves 0-3  compute: poll h_{t-1}, MFMA, reduce through LDS, gating, publish h_t.
 //              Their vector-memory queue only ever holds L2-resident traffic (the
 //              exchange ring), because vector memory completes in order within a wave
@@ -44,12 +44,15 @@ struct SeqParams {
 //              into an LDS ring (kLookahead iterations in flight).
 //   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
 //              output tensor in HBM.
-//   wave 6     prefetcher (one row tile of few rows; ends at once otherwise): touches the W.x lines of
-//              the step kPrefetchAhead ahead with SCALAR loads.  A compute unit returns vector-memory data in
-//              order across its waves, so every feeder load that misses to HBM delays the polls issued behind
-//              it (measured: an L2 hit takes 200 cycles alone and 600 with another wave's misses in flight,
-//              unchanged at 210 when those misses go through the scalar cache).  With the lines already in the
-//              L2 the feeder's loads are short.
+//   waves 6..  prefetchers (0 to 2 of them, chosen by the host): they touch the W.x lines of the step
+//              kPrefetchAhead ahead with SCALAR loads.  A compute unit returns vector-memory data in order across
+//              its waves, so every feeder load that misses to HBM delays the polls issued behind it (measured: an
+//              L2 hit takes 200 cycles alone and 600 with another wave's misses in flight, unchanged at 210 when
+//              those misses go through the scalar cache).  With the lines already in the L2 the feeder's loads
+//              are short.  A scalar miss brings 64 bytes and a wave keeps about 15 of them in flight, so a
+//              prefetch wave is given at most 8 loads per iteration, and the scalar cache serves about 16 per
+//              iteration in all (measured: two waves of 8 gain 18 %, four waves of 8 lose a factor of 2 because
+//              they hold up the barriers), so tiles of 16 rows go without.
 //
 // Exchange ring: kRing slots, slot t % kRing holds h_t as [row tile][member][16 rows][16 units].
 // A word is either data or the "not written yet" pattern.  A workgroup re-arms its own
@@ -61,6 +64,9 @@ struct SeqParams {
 // ---------------------------------------------------------------------------
 constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
 constexpr int kRing = 8;       // slots of the exchange ring
+// prefetch waves a kernel may be launched with (8 waves per workgroup = two per SIMD = 256 VGPRs each, which the
+// largest variants need)
+constexpr int max_prefetch_waves(int nch) { return nch >= 8 ? 1 : kMaxPrefetchWaves; }
 constexpr int kPrefetchAhead = 8;  // steps between the scalar-cache touch of a W.x line and the step that uses it
 
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
@@ -85,7 +91,7 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
 // STG (one row tile only): s_sleep units (64 cycles) between the two polls of a step, about half a poll round trip;
 // that grows with the number of workgroups that share an L2 (measured best: 3 at 16 workgroups per XCD, 6 at 32).
 template <bool BF16, int NCH, int MT, bool FULL, int STG>
-__global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
+__global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
   constexpr int ESZ = BF16 ? 2 : 4;
@@ -399,24 +405,27 @@ __global__ __launch_bounds__(kThreads) void slstm_seq_kernel(SeqParams p) {
   }
 
   // =========================================================================
-  // wave 6: prefetcher.  It takes part in every barrier (plain s_barrier: it has no LDS traffic of its own
-  // and must not wait for its loads there) and issues nothing but scalar loads whose results are never read:
-  // they all land in one scalar register that stays reserved for the whole loop.
+  // waves 6 and up: prefetchers.  They take part in every barrier (plain s_barrier: they have no LDS traffic of
+  // their own and must not wait for their loads there) and issue nothing but scalar loads whose results are never
+  // read: they all land in one scalar register that stays reserved for the whole loop.  Wave 6 + k takes the
+  // batch rows k, k + n, ... of a tile.
   // =========================================================================
-  if (wave == 6) {
-    if (MT != 1 || !p.prefetch) return;  // (a wave that has ended does not count for the barriers)
+  if (wave >= 6) {
+    const int pfi = (int)uniform((uint32_t)wave) - 6, npf = p.prefetch;  // (uniform: the loops below run on the scalar unit)
     constexpr int LM = 128 / (16 * ESZ);  // members whose 16 units share one 128-byte line of W.x: 4 (bf16) / 2 (fp32)
-    const int nrows = rend - rowbase;
     const long long row_bytes = 4ll * H * ESZ;
     const long long cluster = ((long long)head * dh + (member / LM) * LM * 16) * ESZ;  // first byte of the shared line in a gate's block
     const char *const wxb = reinterpret_cast<const char *>(p.wx);
     uint32_t sink = 0;
     __builtin_amdgcn_s_barrier();  // prologue barrier
     for (int itp = 0; itp < NITpad; ++itp) {
-      const int tp = itp + kPrefetchAhead;
+      const int itn = itp + kPrefetchAhead * MT;  // the iteration whose lines are touched now
+      const int tp = itn / MT;
+      const int row0 = rowbase + (itn - tp * MT) * 16;
+      const int nrows = rend - row0 < 16 ? rend - row0 : 16;
       if (tp < p.T) {
-        for (int r = 0; r < nrows; ++r) {
-          const long long rowoff = ((long long)(rowbase + r) * p.wx_sb + (long long)tp * p.wx_st) * ESZ;
+        for (int r = pfi; r < nrows; r += npf) {
+          const long long rowoff = ((long long)(row0 + r) * p.wx_sb + (long long)tp * p.wx_st) * ESZ;
           for (int g = member % LM; g < 4; g += LM) {  // the members that share a line split the gates between them
 #pragma unroll
             for (int half = 0; half < 2; ++half) {  // (a miss of the scalar cache brings 64 bytes into the L2, not the line)
