@@ -80,6 +80,8 @@ F32_CASES = [
     (40, 12, 1, 256, False, False),
     (2, 64, 2, 512, True, True),      # largest fp32 head
     (70, 6, 4, 512, False, True),     # four row tiles per workgroup (ragged), the drainer wave publishes
+    (50, 9, 8, 256, True, True),      # two row tiles (ragged): W.x is fetched in bursts of four iterations
+    (64, 1, 16, 128, False, False),   # two full row tiles, a single step: fewer iterations than one burst
 ]
 
 
@@ -106,6 +108,9 @@ BF16_CASES = [
     (100, 6, 8, 256, True, True),     # four row tiles inside one XCD, two row groups, ragged
     (40, 8, 4, 768, True, False),     # 48 members per head: 24 + 24 on an XCD pair
     (24, 8, 3, 1000, False, True),    # odd member count (spread placement), partial last member, two row tiles
+    (40, 21, 8, 256, True, True),     # two row tiles (ragged), W.x in bursts of eight iterations, 42 iterations
+    (64, 37, 8, 256, False, True),    # two full row tiles, bursts, 74 iterations
+    (64, 3, 4, 512, True, False),     # two full row tiles of a 512-wide head, fewer iterations than one burst
 ]
 
 

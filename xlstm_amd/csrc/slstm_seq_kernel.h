@@ -41,7 +41,7 @@ struct SeqParams {
 //              exchange ring), because vector memory completes in order within a wave
 //              and anything slower would sit in front of the latency-critical polls.
 //   wave 4     feeder: streams W.x and the reset flags of FUTURE iterations from HBM
-//              into an LDS ring (kLookahead iterations in flight).
+//              into an LDS ring (four iterations in flight; with two row tiles, bursts of eight).
 //   wave 5     drainer: writes h of PAST iterations from an LDS staging ring to the
 //              output tensor in HBM.
 //   waves 6..  prefetchers (0 to 2 of them, chosen by the host): they touch the W.x lines of the step
@@ -62,7 +62,6 @@ struct SeqParams {
 // a peer polling slot (t-2) % kRing for h_{t-2+kRing} has seen that publication, so it
 // can only ever read the pattern or the new data there, never the stale h_{t-2}.
 // ---------------------------------------------------------------------------
-constexpr int kLookahead = 4;  // iterations of W.x the feeder keeps in flight
 constexpr int kRing = 8;       // slots of the exchange ring
 // prefetch waves a kernel may be launched with (8 waves per workgroup = two per SIMD = 256 VGPRs each, which the
 // largest variants need)
@@ -192,7 +191,21 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const int rend = (rowbase + p.rows_per_wg < p.bend) ? rowbase + p.rows_per_wg : p.bend;
   const long long BH = (long long)p.B * H;
   const int NIT = p.T * MT;
-  const int NITpad = (NIT + kLookahead - 1) / kLookahead * kLookahead;  // barriers every wave executes
+  // How far ahead the feeder fetches W.x.  A compute unit returns vector-memory data in order across its waves, so
+  // while feeder loads that miss to HBM are in flight the polls of the compute waves wait behind them.
+  //   one row tile    a load per iteration, four iterations ahead (the prefetch waves keep those loads from missing
+  //                   where they can);
+  //   two row tiles   BURSTS of kBurst iterations, one burst ahead (a ring of two bursts in registers): the polls
+  //                   then wait behind W.x during one memory latency per burst instead of all the time;
+  //   four or more    as with one: those iterations are bound by their arithmetic, not by the polls (the time per
+  //                   step is the same with W.x in the Infinity Cache), and bursts measured 12 % slower there.
+  //                   With two row tiles of a 1024-wide head (NCH 8) the arithmetic dominates again (bursts 9 % slower).
+  // Measured with bursts: B 128 x dh 256 2.46 -> 2.11 us per step, B 64 x 8 heads x dh 256 2.64 -> 2.25, B 64 x dh 512
+  // 2.68 -> 2.42.  At which iteration of a burst the next one is requested makes no difference (0, 1, 4 tried).
+  constexpr bool kBursts = MT == 2 && NCH <= 4;
+  constexpr int kBurst = kBursts ? (BF16 ? 8 : 4) : 1;
+  constexpr int kFeedRing = kBursts ? 2 * kBurst : 4;
+  const int NITpad = (NIT + kFeedRing - 1) / kFeedRing * kFeedRing;  // barriers every wave executes
 
   // =========================================================================
   // wave 4: feeder.  Every iteration issues exactly WCH + 1 loads (addresses of
@@ -202,8 +215,8 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   if (wave == 4) {
     const int fb = lane & 15;  // batch row inside the tile
     const int fg = lane >> 4;  // gate
-    uint4 ring[kLookahead][WCH];
-    uint32_t fring[kLookahead];
+    uint4 ring[kFeedRing][WCH];
+    uint32_t fring[kFeedRing];
     const char *wxb = reinterpret_cast<const char *>(p.wx);
     const unsigned char *flagb = p.reset ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);
     const long long flag_sb = p.reset ? p.reset_sb : 0;
@@ -252,7 +265,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     };
 
 #pragma unroll
-    for (int u = 0; u < kLookahead; ++u) issue(u, ring[u], fring[u]);
+    for (int u = 0; u < (kBursts ? kBurst : kFeedRing); ++u) issue(u, ring[u], fring[u]);
     if (fg == 0) rfl[0][fb] = (rowbase + fb < rend) ? (fring[0] & flag_on) : 0u;
     lds_barrier();  // prologue barrier
 #ifdef XS_PROFILE
@@ -262,14 +275,27 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #else
 #define XS_FTICK(i) do { } while (0)
 #endif
-    for (int it0 = 0; it0 < NITpad; it0 += kLookahead) {
+    for (int it0 = 0; it0 < NITpad; it0 += kFeedRing) {
 #pragma unroll
-      for (int u = 0; u < kLookahead; ++u) {
+      for (int u = 0; u < kFeedRing; ++u) {
         const int it = it0 + u;
-        put(it, ring[u], fring[(u + 1) % kLookahead], it + 1);
-        XS_FTICK(0);
-        issue(it + kLookahead, ring[u], fring[u]);
-        XS_FTICK(1);
+        if constexpr (kBursts) {
+          if (u % kBurst == 0) {  // the burst behind the one that starts now; its registers held the burst before
+#pragma unroll
+            for (int v = 0; v < kBurst; ++v) {
+              const int slot = (u + kBurst + v) % kFeedRing;
+              issue(it + kBurst + v, ring[slot], fring[slot]);
+            }
+          }
+          XS_FTICK(1);
+          put(it, ring[u], fring[(u + 1) % kFeedRing], it + 1);
+          XS_FTICK(0);
+        } else {
+          put(it, ring[u], fring[(u + 1) % kFeedRing], it + 1);
+          XS_FTICK(0);
+          issue(it + kFeedRing, ring[u], fring[u]);
+          XS_FTICK(1);
+        }
         lds_barrier();  // barrier #it
         XS_FTICK(2);
       }
