@@ -175,22 +175,24 @@ int run_step(const xs_slstm_args *a) {
   // slab width in MFMA k-steps: the whole K range when it fits LDS (dh <= 256 bf16 / 128 fp32)
   const int slabch = nch == 1 ? 4 : (nch == 2 ? 8 : 2);
   const int nbuf = slabch >= 4 ? 1 : 2;
-  const size_t lds = (size_t)nbuf * (64 + 128) * (slabch * 64 + 16);
+  // one slab: eight waves in two roles (operands + MFMA / pointwise operands + gating), the sums of one row tile cross in 16 KiB of LDS
+  const bool split = slabch >= 4;
+  const size_t lds = (size_t)nbuf * (64 + 128) * (slabch * 64 + 16) + (split ? 4 * 256 * 16 : 0);
   typedef void (*StepKernel)(StepParams, int);
   StepKernel kern;
   const bool hint = full && bf16 && a->h_prev != nullptr;  // operand already in bf16 (h_out of the previous step)
   p.h_prev = hint ? a->h_prev : nullptr;
-#define XS_PICK(BF, SC) (full ? slstm_step_tile_kernel<BF, SC, true> : slstm_step_tile_kernel<BF, SC, false>)
-#define XS_PICK_HINT(SC) (hint ? slstm_step_tile_kernel<true, SC, true, true> : XS_PICK(true, SC))
-  if (bf16) kern = slabch == 4 ? XS_PICK_HINT(4) : (slabch == 8 ? XS_PICK_HINT(8) : XS_PICK_HINT(2));
-  else kern = slabch == 4 ? XS_PICK(false, 4) : (slabch == 8 ? XS_PICK(false, 8) : XS_PICK(false, 2));
+#define XS_PICK(BF, SC, SP) (full ? slstm_step_tile_kernel<BF, SC, true, false, SP> : slstm_step_tile_kernel<BF, SC, false, false, SP>)
+#define XS_PICK_HINT(SC, SP) (hint ? slstm_step_tile_kernel<true, SC, true, true, SP> : XS_PICK(true, SC, SP))
+  if (bf16) kern = slabch == 4 ? XS_PICK_HINT(4, true) : (slabch == 8 ? XS_PICK_HINT(8, true) : XS_PICK_HINT(2, false));
+  else kern = slabch == 4 ? XS_PICK(false, 4, true) : (slabch == 8 ? XS_PICK(false, 8, true) : XS_PICK(false, 2, false));
 #undef XS_PICK_HINT
 #undef XS_PICK
   if (lds > 64 * 1024) {  // the single-slab variant at dh = 256 needs 99 KiB of the 160 KiB of LDS
     const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
     if (rc != XS_OK) return rc;
   }
-  hipLaunchKernelGGL(kern, grid, dim3(256), lds, stream, p, nch_log2);
+  hipLaunchKernelGGL(kern, grid, dim3(split ? 512 : 256), lds, stream, p, nch_log2);
   const hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
   return XS_OK;

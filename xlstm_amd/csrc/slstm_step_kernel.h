@@ -65,9 +65,22 @@ __device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &he
 // HB (only with BF16 and FULL): the recurrent operand comes from StepParams::h_prev, a bf16 copy of
 // the y plane of s0 (the h_out of the previous step), instead of being converted from float32:
 // half the bytes of the most re-read operand (every unit tile of a row tile reads all of it).
-template <bool BF16, int SLABCH, bool FULL, bool HB = false>
-__global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
+// SPLIT (single-slab variants only): eight waves in two roles.  Waves 0-3 fetch and stage the operands, run the
+// MFMAs, ask for the pointwise operands (W.x, old state) of MFMA row tile 1 once every operand has landed, and
+// gate that tile; waves 4-7 fetch the pointwise operands of row tile 0, take its sums from the MFMA waves
+// through LDS and gate it.  With one role a wave that issues loads faster than the memory system takes them
+// stalls in the issue, so the MFMAs could not start before the last pointwise operand had been REQUESTED (5.9k
+// of a step's 13k cycles at B = 256, D = 2048) although their own operands had long arrived; and the gating
+// (bound by instruction issue and its waits) ran on one wave per SIMD.  What is not needed first must also be
+// ASKED FOR later, because everything in flight shares the memory system's queues: with all pointwise operands
+// requested up front by the gating waves the first K half is staged at 4.4-4.6k cycles instead of 2.9k.
+// Measured slower or equal: the gating waves fetching and staging the second K half (it then arrives later and
+// the MFMA waves wait for it), streaming loads for the once-read operands, a pause in front of the gating
+// waves' requests.
+template <bool BF16, int SLABCH, bool FULL, bool HB = false, bool SPLIT = false>
+__global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
   static_assert(!HB || (BF16 && FULL), "the bf16 operand hint is a steady-state bf16 path");
+  static_assert(!SPLIT || SLABCH >= 4, "two roles only with the whole K range in one slab");
   constexpr int HBYTES = HB ? 2 : 4;          // bytes per element of the recurrent operand as it is read
   constexpr int EPC = BF16 ? 8 : 4;
   constexpr int CHK = 4 * EPC;                // input units per MFMA k-step ("chunk")
@@ -81,8 +94,11 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   extern __shared__ __attribute__((aligned(16))) unsigned char step_lds[];
   unsigned char(*hbuf)[64 * RS] = reinterpret_cast<unsigned char(*)[64 * RS]>(step_lds);
   unsigned char(*rbuf)[128 * RS] = reinterpret_cast<unsigned char(*)[128 * RS]>(step_lds + NBUF * 64 * RS);
+  // SPLIT: the sums of MFMA row tile 0, [wave][gate][lane] x 16 bytes, behind the operand buffers
+  f32x4 *const totbuf = reinterpret_cast<f32x4 *>(step_lds + NBUF * (64 + 128) * RS);
 
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;
+  const bool gating_role = SPLIT && uniform((uint32_t)(threadIdx.x >> 8)) != 0u;  // scalar: the roles meet at barriers
   const int wave = tid >> 6;
   const int lane = tid & 63;
   const int q = lane >> 4;
@@ -97,7 +113,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   const int nch = 1 << nch_log2;              // chunks per K quarter (as in the sequence kernel)
   const int nslab = (4 * nch) / SLABCH;
 
-  if (blockIdx.x == 0 && tid < 16)
+  if (blockIdx.x == 0 && threadIdx.x < 16)
     reinterpret_cast<uint32_t *>(p.status)[tid] = tid == 5 ? 1u : 0u;  // a step never waits, so it never aborts; one launch
 
   const bool has_s0 = FULL || p.s0 != nullptr;
@@ -148,10 +164,12 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
               (FULL ? rpiece_of(j) * 16 : 0);
   }
   uint4 hring[kStepRing][HITEMS], rring[kStepRing][RITEMS];
-  auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS]) {
+  // phase < 0: the whole slab; otherwise the items of that K phase only (as in store_slab)
+  auto load_slab = [&](int sidx, uint4 (&hst)[HITEMS], uint4 (&rst)[RITEMS], int phase) {
     const int kbase = sidx * SLABK;
 #pragma unroll
     for (int ph = 0; ph < NSPLIT; ++ph) {
+      if (phase >= 0 && ph != phase) continue;
 #pragma unroll
       for (int j = ph * HIP; j < (ph + 1) * HIP; ++j) {
         if (HB) {
@@ -206,13 +224,16 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   };
 
 #ifdef XS_PROFILE
-  long long pstamp[6];
+  long long pstamp[10];
+  for (int i = 0; i < 10; ++i) pstamp[i] = 0;
   pstamp[0] = clock64();
   const long long pwall0 = wall_clock64();
 #endif
+  if (!gating_role) {
 #pragma unroll
-  for (int u = 0; u < kStepRing; ++u)
-    if (u < nslab) load_slab(u, hring[u], rring[u]);
+    for (int u = 0; u < kStepRing; ++u)
+      if (u < nslab) load_slab(u, hring[u], rring[u], -1);
+  }
 
   // ---- wave tiling 2 x 2: wave (wr, wu) owns rows 32*wr .. +31 (two MFMA row tiles, index ut below)
   // and units 16*wu .. +15 of all four gates, so a k-step reads 2 h and 4 R fragments from LDS for
@@ -225,38 +246,59 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   uint2 wxb[2][4];
   float4 wxf[2][4], bias4[4], c4[2], n4[2], m4[2];
   uint32_t pflag[2];
+  auto load_bias_and_flags = [&]() {
 #pragma unroll
-  for (int g = 0; g < 4; ++g)
-    bias4[g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
+    for (int g = 0; g < 4; ++g)
+      bias4[g] = *reinterpret_cast<const float4 *>(p.bias + ((long long)head * 4 + g) * dh + uac);
 #pragma unroll
-  for (int ut = 0; ut < 2; ++ut) {
-    const int brow = rowbase + 32 * wr + 16 * ut + r16;
-    const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
-    pflag[ut] = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
-      if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
-      else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
+    for (int ut = 0; ut < 2; ++ut) {
+      const int brow = rowbase + 32 * wr + 16 * ut + r16;
+      const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
+      pflag[ut] = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
     }
-    const long long so = (long long)browc * H + col;
-    c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
-    n4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 2 * BH + so : 0));
-    m4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 3 * BH + so : 0));
-  }
-
-  // ---- K loop
+  };
+  auto load_pointwise_operands = [&](int ut_lo, int ut_hi) {  // W.x and the old c, n, m of MFMA row tiles [ut_lo, ut_hi)
+#pragma unroll
+    for (int ut = 0; ut < 2; ++ut) {
+      if (ut < ut_lo || ut >= ut_hi) continue;
+      const int brow = rowbase + 32 * wr + 16 * ut + r16;
+      const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const long long o = (long long)browc * p.wx_sb + (long long)g * H + col;
+        if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
+        else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
+      }
+      const long long so = (long long)browc * H + col;
+      c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
+      n4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 2 * BH + so : 0));
+      m4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 3 * BH + so : 0));
+    }
+  };
   f32x4 acc[2][4], tot[2][4];
+  if (!SPLIT) { load_bias_and_flags(); load_pointwise_operands(0, 2); }
+
+  if (SPLIT && gating_role) {
+    load_bias_and_flags();
+    load_pointwise_operands(0, 1);
+    lds_barrier();  // first K half staged
+    lds_barrier();  // second K half staged
+    lds_barrier();  // sums of row tile 0 in LDS
+#pragma unroll
+    for (int g = 0; g < 4; ++g) tot[0][g] = totbuf[(wave * 4 + g) * 64 + lane];
+  } else {
+  // ---- K loop
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
     for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
 
+  if (SPLIT) load_bias_and_flags();
 #ifdef XS_PROFILE
   pstamp[1] = clock64();
 #endif
   store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
-  __syncthreads();
+  if (SPLIT) lds_barrier(); else __syncthreads();
 #ifdef XS_PROFILE
   pstamp[2] = clock64();
 #endif
@@ -267,8 +309,20 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
       if (w == 2) {
+#ifdef XS_PROFILE
+        asm volatile("" :: "v"(tot[0][0][0]), "v"(tot[1][3][3]));
+        pstamp[6] = clock64();
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        pstamp[7] = clock64();
+#endif
         store_slab(0, 0, hring[0], rring[0], 1);
-        __syncthreads();
+        if (SPLIT) lds_barrier(); else __syncthreads();
+        // every operand has landed: the requests for this role's share of the gating go out now and arrive
+        // behind the MFMAs of the second half
+        if (SPLIT) load_pointwise_operands(1, 2);
+#ifdef XS_PROFILE
+        pstamp[8] = clock64();
+#endif
       }
 #pragma unroll
       for (int cq = 0; cq < (NQ > 0 ? NQ : 1); ++cq) {
@@ -345,7 +399,7 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
           }
         }
         // slab sidx went to LDS one iteration ago: its ring entry takes the loads of slab sidx + kStepRing
-        if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u]);
+        if (sidx + kStepRing < nslab) load_slab(sidx + kStepRing, hring[u], rring[u], -1);
         if (sidx + 1 < nslab) {
           const int un = (u + 1) % kStepRing;
           store_slab(sidx + 1, (sidx + 1) & (NBUF - 1), hring[un], rring[un], -1);  // the other buffer was last read before the previous barrier
@@ -359,12 +413,30 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
 #ifdef XS_PROFILE
   asm volatile("" :: "v"(tot[0][0][0]), "v"(tot[1][3][3]));
   pstamp[3] = clock64();
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  pstamp[4] = clock64();
 #endif
-  // ---- gating
+  if (SPLIT) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) totbuf[(wave * 4 + g) * 64 + lane] = tot[0][g];
+    lds_barrier();  // sums of row tile 0 in LDS
+#ifdef XS_PROFILE
+    if (tid == 0 && blockIdx.x == 9) {
+      long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
+      for (int i = 0; i < 4; ++i) dst[i] = pstamp[i] - pstamp[0];
+      for (int i = 6; i < 10; ++i) dst[i] = pstamp[i] - pstamp[0];
+    }
+#endif
+  }
+  }  // MFMA role
+#ifdef XS_PROFILE
+  if (!SPLIT || gating_role) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    pstamp[4] = clock64();
+  }
+#endif
+  // ---- gating (SPLIT: row tile 0 by the gating role, row tile 1 by the MFMA role)
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
+    if (SPLIT && (ut == 0) != gating_role) continue;
     const int brow = rowbase + 32 * wr + 16 * ut + r16;
     const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag[ut] != 0u));
     const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
@@ -412,12 +484,12 @@ __global__ __launch_bounds__(256) void slstm_step_tile_kernel(StepParams p, int 
   }
 #ifdef XS_PROFILE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (tid == 0 && blockIdx.x == 9) {
+  if (tid == 0 && blockIdx.x == 9 && (!SPLIT || gating_role)) {
     pstamp[5] = clock64();
     long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
-    for (int i = 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
+    for (int i = SPLIT ? 4 : 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
   }
-  if (tid == 0) {
+  if (tid == 0 && (!SPLIT || gating_role)) {
     long long *wt = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 256);
     wt[2 * blockIdx.x] = pwall0;
     wt[2 * blockIdx.x + 1] = wall_clock64();
