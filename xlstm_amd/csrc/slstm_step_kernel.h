@@ -16,6 +16,13 @@ namespace {
 // four K quarters and the quarters are added in its order, so step-by-step decoding
 // reproduces a sequence call bit for bit.
 // ---------------------------------------------------------------------------
+// 16 bytes per lane from a buffer straight into LDS, lane i's bytes at lds_addr + 16 * i (see lds_direct_load_b128;
+// this one leaves the cache policy alone: operands, not polls)
+__device__ __forceinline__ void lds_direct_fetch_b128(u32x4_t rsrc, uint32_t lds_addr, int voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+
 struct StepParams {
   const void *wx;
   long long wx_sb;
@@ -66,17 +73,18 @@ __device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &he
 // the y plane of s0 (the h_out of the previous step), instead of being converted from float32:
 // half the bytes of the most re-read operand (every unit tile of a row tile reads all of it).
 // SPLIT (single-slab variants only): eight waves in two roles.  Waves 0-3 fetch and stage the operands, run the
-// MFMAs, ask for the pointwise operands (W.x, old state) of MFMA row tile 1 once every operand has landed, and
-// gate that tile; waves 4-7 fetch the pointwise operands of row tile 0, take its sums from the MFMA waves
-// through LDS and gate it.  With one role a wave that issues loads faster than the memory system takes them
-// stalls in the issue, so the MFMAs could not start before the last pointwise operand had been REQUESTED (5.9k
-// of a step's 13k cycles at B = 256, D = 2048) although their own operands had long arrived; and the gating
-// (bound by instruction issue and its waits) ran on one wave per SIMD.  What is not needed first must also be
-// ASKED FOR later, because everything in flight shares the memory system's queues: with all pointwise operands
-// requested up front by the gating waves the first K half is staged at 4.4-4.6k cycles instead of 2.9k.
+// MFMAs and gate MFMA row tile 1: they ask for its W.x right behind the operands (W.x comes from HBM unless the
+// previous kernel has just written it) and for its old state (which the previous step left in the Infinity Cache)
+// once every operand has landed.  Waves 4-7 fetch the pointwise operands of row tile 0, take its sums from the
+// MFMA waves through LDS and gate it.  With one role a wave that issues loads faster than the memory system
+// takes them stalls in the issue, so the MFMAs could not start before the last pointwise operand had been
+// REQUESTED (5.9k of a step's 13k cycles at B = 256, D = 2048) although their own operands had long arrived; and
+// the gating (bound by instruction issue and its waits) ran on one wave per SIMD.  What is not needed first must
+// also be ASKED FOR later, because everything in flight shares the memory system's queues: with all pointwise
+// operands requested up front by the gating waves the first K half is staged at 4.4-4.6k cycles instead of 2.9k.
 // Measured slower or equal: the gating waves fetching and staging the second K half (it then arrives later and
-// the MFMA waves wait for it), streaming loads for the once-read operands, a pause in front of the gating
-// waves' requests.
+// the MFMA waves wait for it), the gating waves fetching row tile 1's operands late and handing them over
+// through LDS, streaming loads for the once-read operands.
 template <bool BF16, int SLABCH, bool FULL, bool HB = false, bool SPLIT = false>
 __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
   static_assert(!HB || (BF16 && FULL), "the bf16 operand hint is a steady-state bf16 path");
@@ -95,7 +103,15 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
   unsigned char(*hbuf)[64 * RS] = reinterpret_cast<unsigned char(*)[64 * RS]>(step_lds);
   unsigned char(*rbuf)[128 * RS] = reinterpret_cast<unsigned char(*)[128 * RS]>(step_lds + NBUF * 64 * RS);
   // SPLIT: the sums of MFMA row tile 0, [wave][gate][lane] x 16 bytes, behind the operand buffers
-  f32x4 *const totbuf = reinterpret_cast<f32x4 *>(step_lds + NBUF * (64 + 128) * RS);
+  // DIRECT (the steady-state bf16 decode variant): the operands go from memory straight into LDS, no registers and
+  // no LDS writes in between.  Such a load fills 1 KiB of consecutive LDS, so the rows cannot be padded: each K
+  // half is an array of 256-byte rows (16 pieces of 16 bytes), and piece p of row r sits at position p ^ (r & 7),
+  // which keeps the MFMA loop's 16-byte reads (8 consecutive rows, one piece) free of bank conflicts.
+  constexpr bool DIRECT = SPLIT && HB && SLABCH == 8;
+  constexpr int kHalfH = 64 * 256, kHalfR = 128 * 256;  // bytes of one K half of h / of R
+  unsigned char *const hdir = step_lds;
+  unsigned char *const rdir = step_lds + 2 * kHalfH;
+  f32x4 *const totbuf = reinterpret_cast<f32x4 *>(step_lds + (DIRECT ? 2 * (kHalfH + kHalfR) : NBUF * (64 + 128) * RS));
 
   const int tid = threadIdx.x & 255;
   const bool gating_role = SPLIT && uniform((uint32_t)(threadIdx.x >> 8)) != 0u;  // scalar: the roles meet at barriers
@@ -229,17 +245,14 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
   pstamp[0] = clock64();
   const long long pwall0 = wall_clock64();
 #endif
-  if (!gating_role) {
-#pragma unroll
-    for (int u = 0; u < kStepRing; ++u)
-      if (u < nslab) load_slab(u, hring[u], rring[u], -1);
-  }
-
   // ---- wave tiling 2 x 2: wave (wr, wu) owns rows 32*wr .. +31 (two MFMA row tiles, index ut below)
   // and units 16*wu .. +15 of all four gates, so a k-step reads 2 h and 4 R fragments from LDS for
   // its 8 MFMAs.  Pointwise operands of this lane: batch rows rowbase + 32*wr + 16*ut + r16,
   // units a0 + 16*wu + 4q .. +3.
   const int wr = wave >> 1, wu = wave & 1;
+  // DIRECT: byte offset inside a 256-byte row of this lane's piece of k-step c of a K half: position (4c + q) ^ (row & 7),
+  // and the rows this lane reads (of h and of R) all have row & 7 == r16 & 7
+  const int swz[4] = {((0 + q) ^ (r16 & 7)) << 4, ((4 + q) ^ (r16 & 7)) << 4, ((8 + q) ^ (r16 & 7)) << 4, ((12 + q) ^ (r16 & 7)) << 4};
   const int ua = a0 + wu * 16 + 4 * q;
   const int uac = (FULL || ua < dh) ? ua : 0;
   const long long col = (long long)head * dh + uac;
@@ -257,7 +270,7 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
       pflag[ut] = FULL ? 0u : rsp[has_reset ? (long long)browc * p.reset_sb : 0];
     }
   };
-  auto load_pointwise_operands = [&](int ut_lo, int ut_hi) {  // W.x and the old c, n, m of MFMA row tiles [ut_lo, ut_hi)
+  auto load_wx = [&](int ut_lo, int ut_hi) {  // W.x of MFMA row tiles [ut_lo, ut_hi)
 #pragma unroll
     for (int ut = 0; ut < 2; ++ut) {
       if (ut < ut_lo || ut >= ut_hi) continue;
@@ -269,6 +282,14 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
         if (BF16) wxb[ut][g] = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.wx) + o);
         else wxf[ut][g] = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.wx) + o);
       }
+    }
+  };
+  auto load_state = [&](int ut_lo, int ut_hi) {  // the old c, n, m of MFMA row tiles [ut_lo, ut_hi)
+#pragma unroll
+    for (int ut = 0; ut < 2; ++ut) {
+      if (ut < ut_lo || ut >= ut_hi) continue;
+      const int brow = rowbase + 32 * wr + 16 * ut + r16;
+      const int browc = (FULL || brow < p.B) ? brow : p.B - 1;
       const long long so = (long long)browc * H + col;
       c4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? BH + so : 0));
       n4[ut] = *reinterpret_cast<const float4 *>(s0p + (has_s0 ? 2 * BH + so : 0));
@@ -276,28 +297,144 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
     }
   };
   f32x4 acc[2][4], tot[2][4];
-  if (!SPLIT) { load_bias_and_flags(); load_pointwise_operands(0, 2); }
+  // ---- gating of MFMA row tile ut, and its stores
+  auto gate_and_store = [&](int ut) {
+    const int brow = rowbase + 32 * wr + 16 * ut + r16;
+    const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag[ut] != 0u));
+    const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
+    const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
+    const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
+    float yv[4], cv[4], nv[4], mv[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float raw[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        float wxv;
+        if (BF16) {
+          const uint32_t wd = i < 2 ? wxb[ut][g].x : wxb[ut][g].y;
+          wxv = bf16_bits_to_float((i & 1) ? (wd >> 16) : (wd & 0xFFFFu));
+        } else {
+          const float wf[4] = {wxf[ut][g].x, wxf[ut][g].y, wxf[ut][g].z, wxf[ut][g].w};
+          wxv = wf[i];
+        }
+        const float bf[4] = {bias4[g].x, bias4[g].y, bias4[g].z, bias4[g].w};
+        raw[g] = (wxv + tot[ut][g][i]) + bf[i];
+      }
+      CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
+      slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
+      yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
+    }
+    if (FULL || (brow < p.B && ua < dh)) {
+      const long long o = (long long)brow * H + head * dh + ua;
+      // streaming stores: the lines leave the L2 while the kernel still runs instead of being
+      // written back when it ends (measured: 0.65 us per step at B = 256, D = 2048)
+      __builtin_nontemporal_store(f32x4{yv[0], yv[1], yv[2], yv[3]}, reinterpret_cast<f32x4 *>(p.s_out + o));
+      __builtin_nontemporal_store(f32x4{cv[0], cv[1], cv[2], cv[3]}, reinterpret_cast<f32x4 *>(p.s_out + BH + o));
+      __builtin_nontemporal_store(f32x4{nv[0], nv[1], nv[2], nv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 2 * BH + o));
+      __builtin_nontemporal_store(f32x4{mv[0], mv[1], mv[2], mv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 3 * BH + o));
+      if (BF16) {
+        uint2 hw;
+        hw.x = float_to_bf16_bits(yv[0]) | (float_to_bf16_bits(yv[1]) << 16);
+        hw.y = float_to_bf16_bits(yv[2]) | (float_to_bf16_bits(yv[3]) << 16);
+        // (h stays an ordinary store: as a streaming store its 8-byte pieces cost 0.8 us per step)
+        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = hw;
+      } else {
+        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.h_out) + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
+      }
+    }
+  };
+#ifdef XS_PROFILE
+  auto profile_end = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (tid == 0 && blockIdx.x == 9) {
+      pstamp[5] = clock64();
+      long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
+      for (int i = SPLIT ? 4 : 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
+    }
+    if (tid == 0) {
+      long long *wt = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 256);
+      wt[2 * blockIdx.x] = pwall0;
+      wt[2 * blockIdx.x + 1] = wall_clock64();
+    }
+  };
+#endif
 
   if (SPLIT && gating_role) {
+    // The compute unit returns vector-memory data in the order of the requests, across waves: a short pause lets
+    // the MFMA waves ask for their operands first (8 and 20 units of 64 cycles measured alike, 0 is 3 % slower).
+    __builtin_amdgcn_s_sleep(8);
     load_bias_and_flags();
-    load_pointwise_operands(0, 1);
+    load_wx(0, 1);
+    load_state(0, 1);
     lds_barrier();  // first K half staged
     lds_barrier();  // second K half staged
     lds_barrier();  // sums of row tile 0 in LDS
 #pragma unroll
     for (int g = 0; g < 4; ++g) tot[0][g] = totbuf[(wave * 4 + g) * 64 + lane];
+#ifdef XS_PROFILE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    pstamp[4] = clock64();
+#endif
+    gate_and_store(0);
+#ifdef XS_PROFILE
+    profile_end();
+#endif
+    return;  // (no path from here into the code below: the compiler's load bookkeeping of the two roles stays apart)
+  }
+  // ---- operands, K loop (SPLIT: the MFMA waves).  No load is issued before the roles part: where the two paths
+  // touch in the compiler's control-flow graph it waits for every load the other path might have in flight.
+  if (DIRECT) {
+    {
+      const unsigned long long hb = reinterpret_cast<unsigned long long>(p.h_prev), rb = reinterpret_cast<unsigned long long>(p.r);
+      const u32x4_t hrs = {uniform((uint32_t)hb), uniform((uint32_t)(hb >> 32) & 0xFFFFu), uniform((uint32_t)(BH * 2)), 0x00020000u};
+      const u32x4_t rrs = {uniform((uint32_t)rb), uniform((uint32_t)(rb >> 32) & 0xFFFFu), uniform((uint32_t)((long long)H * 4 * dh * 2)), 0x00020000u};
+      const uint32_t hl = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)hdir);
+      const uint32_t rl = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)rdir);
+      const int wv = (int)uniform((uint32_t)wave);
+      const int sub = lane >> 4, pos = lane & 15;  // a load covers 4 rows: row sub of them, position pos
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {  // h: 16 loads per half and workgroup
+          const int row = 4 * (wv * 4 + k) + sub;
+          const int voff = (int)(((long long)(rowbase + row) * H + head * dh) * 2) + (half * 16 + (pos ^ (row & 7))) * 16;
+          lds_direct_fetch_b128(hrs, uniform(hl + half * kHalfH + (wv * 4 + k) * 1024), voff);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {  // R: 32 loads per half and workgroup
+          const int colx = 4 * (wv * 8 + k) + sub;  // column of the workgroup's 128: gate colx / 32, unit colx % 32
+          const int voff = (int)(((long long)head * 4 * dh + (long long)(colx >> 5) * dh + a0 + (colx & 31)) * dh * 2) +
+                           (half * 16 + (pos ^ (colx & 7))) * 16;
+          lds_direct_fetch_b128(rrs, uniform(rl + half * kHalfR + (wv * 8 + k) * 1024), voff);
+        }
+      }
+    }
   } else {
-  // ---- K loop
+#pragma unroll
+    for (int u = 0; u < kStepRing; ++u)
+      if (u < nslab) load_slab(u, hring[u], rring[u], -1);
+  }
+
+  if (!SPLIT) { load_bias_and_flags(); load_wx(0, 2); load_state(0, 2); }
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
     for (int g = 0; g < 4; ++g) { acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; tot[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f}; }
 
-  if (SPLIT) load_bias_and_flags();
+  // W.x comes from HBM when the previous kernel did not just write it, the old state from the Infinity Cache: the
+  // requests for this role's W.x go out early, those for its state once every operand has landed
+  if (SPLIT) { load_bias_and_flags(); load_wx(1, 2); }
 #ifdef XS_PROFILE
   pstamp[1] = clock64();
 #endif
-  store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
+  if (DIRECT) {
+    // In flight, in this order: 12 + 12 operand loads, then the 4 bias and 4 W.x loads just above (the assembly
+    // statements keep them there; fewer would only make this wait longer): at most 20 left = the first K half is in LDS
+    asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+  } else {
+    store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
+  }
   if (SPLIT) lds_barrier(); else __syncthreads();
 #ifdef XS_PROFILE
   pstamp[2] = clock64();
@@ -315,11 +452,12 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         pstamp[7] = clock64();
 #endif
-        store_slab(0, 0, hring[0], rring[0], 1);
+        if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        else store_slab(0, 0, hring[0], rring[0], 1);
         if (SPLIT) lds_barrier(); else __syncthreads();
-        // every operand has landed: the requests for this role's share of the gating go out now and arrive
-        // behind the MFMAs of the second half
-        if (SPLIT) load_pointwise_operands(1, 2);
+        // every operand has landed: the requests for the state this role gates go out now and arrive behind the
+        // MFMAs of the second half
+        if (SPLIT) load_state(1, 2);
 #ifdef XS_PROFILE
         pstamp[8] = clock64();
 #endif
@@ -330,10 +468,12 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
         uint4 hv[2], rv[4];
 #pragma unroll
         for (int ut = 0; ut < 2; ++ut)
-          hv[ut] = *reinterpret_cast<const uint4 *>(&hbuf[0][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
+          hv[ut] = DIRECT ? *reinterpret_cast<const uint4 *>(hdir + (ch >> 2) * kHalfH + (32 * wr + 16 * ut + r16) * 256 + swz[ch & 3])
+                          : *reinterpret_cast<const uint4 *>(&hbuf[0][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-          rv[g] = *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
+          rv[g] = DIRECT ? *reinterpret_cast<const uint4 *>(rdir + (ch >> 2) * kHalfR + (g * 32 + wu * 16 + r16) * 256 + swz[ch & 3])
+                         : *reinterpret_cast<const uint4 *>(&rbuf[0][(g * 32 + wu * 16 + r16) * RS + ch * 64 + q * 16]);
 #pragma unroll
         for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
@@ -425,75 +565,17 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
       for (int i = 6; i < 10; ++i) dst[i] = pstamp[i] - pstamp[0];
     }
 #endif
-  }
-  }  // MFMA role
-#ifdef XS_PROFILE
-  if (!SPLIT || gating_role) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    pstamp[4] = clock64();
-  }
-#endif
-  // ---- gating (SPLIT: row tile 0 by the gating role, row tile 1 by the MFMA role)
-#pragma unroll
-  for (int ut = 0; ut < 2; ++ut) {
-    if (SPLIT && (ut == 0) != gating_role) continue;
-    const int brow = rowbase + 32 * wr + 16 * ut + r16;
-    const bool reset_row = !FULL && (!has_s0 || (has_reset && pflag[ut] != 0u));
-    const float cin[4] = {c4[ut].x, c4[ut].y, c4[ut].z, c4[ut].w};
-    const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
-    const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
-    float yv[4], cv[4], nv[4], mv[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float raw[4];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        float wxv;
-        if (BF16) {
-          const uint32_t wd = i < 2 ? wxb[ut][g].x : wxb[ut][g].y;
-          wxv = bf16_bits_to_float((i & 1) ? (wd >> 16) : (wd & 0xFFFFu));
-        } else {
-          const float wf[4] = {wxf[ut][g].x, wxf[ut][g].y, wxf[ut][g].z, wxf[ut][g].w};
-          wxv = wf[i];
-        }
-        const float bf[4] = {bias4[g].x, bias4[g].y, bias4[g].z, bias4[g].w};
-        raw[g] = (wxv + tot[ut][g][i]) + bf[i];
-      }
-      CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
-      slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
-      yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
-    }
-    if (FULL || (brow < p.B && ua < dh)) {
-      const long long o = (long long)brow * H + head * dh + ua;
-      // streaming stores: the lines leave the L2 while the kernel still runs instead of being
-      // written back when it ends (measured: 0.65 us per step at B = 256, D = 2048)
-      __builtin_nontemporal_store(f32x4{yv[0], yv[1], yv[2], yv[3]}, reinterpret_cast<f32x4 *>(p.s_out + o));
-      __builtin_nontemporal_store(f32x4{cv[0], cv[1], cv[2], cv[3]}, reinterpret_cast<f32x4 *>(p.s_out + BH + o));
-      __builtin_nontemporal_store(f32x4{nv[0], nv[1], nv[2], nv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 2 * BH + o));
-      __builtin_nontemporal_store(f32x4{mv[0], mv[1], mv[2], mv[3]}, reinterpret_cast<f32x4 *>(p.s_out + 3 * BH + o));
-      if (BF16) {
-        uint2 hw;
-        hw.x = float_to_bf16_bits(yv[0]) | (float_to_bf16_bits(yv[1]) << 16);
-        hw.y = float_to_bf16_bits(yv[2]) | (float_to_bf16_bits(yv[3]) << 16);
-        // (h stays an ordinary store: as a streaming store its 8-byte pieces cost 0.8 us per step)
-        *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.h_out) + o) = hw;
-      } else {
-        *reinterpret_cast<float4 *>(reinterpret_cast<float *>(p.h_out) + o) = make_float4(yv[0], yv[1], yv[2], yv[3]);
-      }
-    }
+    gate_and_store(1);
+    return;
   }
 #ifdef XS_PROFILE
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  if (tid == 0 && blockIdx.x == 9 && (!SPLIT || gating_role)) {
-    pstamp[5] = clock64();
-    long long *dst = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 64);
-    for (int i = SPLIT ? 4 : 0; i < 6; ++i) dst[i] = pstamp[i] - pstamp[0];
-  }
-  if (tid == 0 && (!SPLIT || gating_role)) {
-    long long *wt = reinterpret_cast<long long *>(reinterpret_cast<char *>(p.status) + 256);
-    wt[2 * blockIdx.x] = pwall0;
-    wt[2 * blockIdx.x + 1] = wall_clock64();
-  }
+  pstamp[4] = clock64();
+#endif
+  gate_and_store(0);
+  gate_and_store(1);
+#ifdef XS_PROFILE
+  profile_end();
 #endif
 }
 
