@@ -168,7 +168,7 @@ def bench_decode(device, steps=1024, prefill=128):
         "finite": bool(torch.isfinite(s_a).all()),
         "roofline": {"bound": "hbm", "achieved": nbytes / (best_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": nbytes / (best_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "slstm_step_tile_kernel<bf16,SLABCH=8,FULL,HB>", "algorithmic_bytes_per_launch": nbytes},
+                     "kernel": "slstm_step_tile_kernel<bf16,SLABCH=8,FULL,HB,SPLIT>", "algorithmic_bytes_per_launch": nbytes},
     }
 
 
