@@ -79,9 +79,12 @@ class GraphedLayerDecoder:
         self.slstm[self.cur].copy_(slstm_state)
         self.h[self.cur].copy_(self.slstm[self.cur][0:1])  # the step kernel's operand hint: y rounded to dtype
 
-    def step(self, x: torch.Tensor) -> torch.Tensor:
-        """``x`` [B,1,D] -> the layer's output for this token (a buffer that the next call overwrites)."""
-        self.x.copy_(x)
+    def step(self, x: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``x`` [B,1,D] -> the layer's output for this token (a buffer that the next call overwrites).
+        With ``x=None`` the token is taken from ``self.x``, where its producer has written it: one copy
+        kernel (and the gap in front of the graph) less per token."""
+        if x is not None and x.data_ptr() != self.x.data_ptr():
+            self.x.copy_(x)
         self.graphs[self.cur].replay()
         self.cur ^= 1
         return self.out
