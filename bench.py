@@ -28,6 +28,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "sLSTM fwd tokens/s @ D=1024 packed B16×T2048; decode step µs @ B=256"
+SERIAL_FLOOR_US = 1520 / 2350.0  # per timestep of the sequence kernel at config 2, see the roofline object
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 
 
@@ -419,7 +420,13 @@ def main():
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,STG=6>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_launch": nbytes, "us_per_timestep": kern_ms * 1e3 / T,
-                     "max_poll_rounds": status["max_spins"]},
+                     "max_poll_rounds": status["max_spins"],
+                     # The launch is a chain of T dependent steps.  Floor of one step of this decomposition, from
+                     # microbenchmarks on the same hardware: one publish -> poll hop inside an XCD (570 cycles), the
+                     # gating chain (650), MFMA + LDS reduction (250), one barrier (50) = 1,520 cycles at 2.35 GHz.
+                     "serial_floor_us_per_timestep": SERIAL_FLOOR_US,
+                     "frac_of_serial_floor": SERIAL_FLOOR_US / (kern_ms * 1e3 / T),
+                     "tflops": 8.0 * B * T * NH * dh * dh / (kern_ms * 1e-3) / 1e12},
     }
     traffic_file = os.path.join(ROOT, "profiles", "traffic_seq_cfg2.json")
     if os.path.exists(traffic_file):
