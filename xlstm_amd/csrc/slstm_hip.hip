@@ -62,22 +62,22 @@ inline size_t xbuf_elems(int B, int NH, int dh) {
 typedef void (*SeqKernel)(SeqParams);
 
 template <bool BF16, int NCH, bool FULL>
-SeqKernel pick_mt(int MT, bool long_stagger) {
+SeqKernel pick_mt(int MT) {
   switch (MT) {
-    case 1: return long_stagger ? slstm_seq_kernel<BF16, NCH, 1, FULL, 6> : slstm_seq_kernel<BF16, NCH, 1, FULL, 3>;
-    case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL, 6>;
-    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL, 6>;
+    case 1: return slstm_seq_kernel<BF16, NCH, 1, FULL>;
+    case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL>;
+    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL>;
     default: return nullptr;
   }
 }
 
 template <bool BF16, bool FULL>
-SeqKernel pick_kernel(int nch, int MT, bool long_stagger) {
+SeqKernel pick_kernel(int nch, int MT) {
   switch (nch) {
-    case 1: return pick_mt<BF16, 1, FULL>(MT, long_stagger);
-    case 2: return pick_mt<BF16, 2, FULL>(MT, long_stagger);
-    case 4: return pick_mt<BF16, 4, FULL>(MT, long_stagger);
-    case 8: return pick_mt<BF16, 8, FULL>(MT, long_stagger);
+    case 1: return pick_mt<BF16, 1, FULL>(MT);
+    case 2: return pick_mt<BF16, 2, FULL>(MT);
+    case 4: return pick_mt<BF16, 4, FULL>(MT);
+    case 8: return pick_mt<BF16, 8, FULL>(MT);
     default: return nullptr;
   }
 }
@@ -241,9 +241,8 @@ int run_forward(const xs_slstm_args *a) {
     // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
     const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
     const int NBT_ = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
-    const bool long_stagger = (long long)NH * NBT_ * G >= 24 * 8;  // 24 or more workgroups per XCD
-    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, long_stagger) : pick_kernel<true, false>(nch, MT, long_stagger))
-                          : (full ? pick_kernel<false, true>(nch, MT, long_stagger) : pick_kernel<false, false>(nch, MT, long_stagger));
+    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT) : pick_kernel<true, false>(nch, MT))
+                          : (full ? pick_kernel<false, true>(nch, MT) : pick_kernel<false, false>(nch, MT));
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NH * NBT;

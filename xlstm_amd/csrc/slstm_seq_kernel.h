@@ -35,7 +35,7 @@ struct SeqParams {
 //         NCH*32 (bf16) or NCH*16 (fp32) input units, the four waves 4x that.
 //   MT  : 16-row batch tiles handled one after the other by a workgroup.
 //
-// Six to ten waves per workgroup, one barrier per (step, tile) iteration shared by all:
+// Six to eight waves per workgroup, one barrier per (step, tile) iteration shared by all:
 //   waves 0-3  compute: poll h_{t-1}, MFMA, reduce through LDS, gating, publish h_t.
 //              Their vector-memory queue only ever holds L2-resident traffic (the
 //              exchange ring), because vector memory completes in order within a wave
@@ -87,9 +87,7 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
 // the arrival test are then compiled out (with one row tile, lanes of rows that do not exist read zeros from
 // past the end of the buffer descriptor, which never look like the "not written yet" pattern).  That matters:
 // the compute waves are bound by the number of instructions between the arrival of h and the MFMAs.
-// STG (one row tile only): s_sleep units (64 cycles) between the two polls of a step, about half a poll round trip;
-// that grows with the number of workgroups that share an L2 (measured best: 3 at 16 workgroups per XCD, 6 at 32).
-template <bool BF16, int NCH, int MT, bool FULL, int STG>
+template <bool BF16, int NCH, int MT, bool FULL>
 __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
@@ -583,9 +581,11 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       const int arow = rowbase + mt * 16 + r16;
       bool need[NCH];
       uint32_t needmask[NCH];
-      uint4 breg[NCH];     // one row tile: the second of the two polls in flight
       const bool row_ok = (FULL && MT > 1) ? true : arow < rend;
-      const bool row_reset = rfl[it & 3][r16] != 0u;  // a row that starts a document contributes R.0 = 0 exactly
+      // a row that starts a document contributes R.0 = 0 exactly.  (Fetching this flag behind the poll's issue, so that
+      // the poll goes out an LDS round trip earlier, measured 2.5 % SLOWER: an earlier poll more often comes back
+      // incomplete, and the next one is a full round trip away.)
+      const bool row_reset = rfl[it & 3][r16] != 0u;
 #pragma unroll
       for (int c = 0; c < NCH; ++c) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
@@ -664,23 +664,20 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #pragma unroll
           for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
         } else if (MT == 1) {
-          // Two polls in flight, about half a round trip apart (STG, chosen by the host), re-issued alternately:
-          // a poll returns every ~300 cycles instead of every ~600, which halves both the wait for h
-          // and the skew between the four waves at the barrier.  Lanes whose batch row does not exist
-          // ask for an offset past the descriptor's end: zeros, no memory traffic, so the doubled poll
-          // rate stays far below what a compute unit can pull from the L2.  The decisions are
-          // wave-uniform (ballot) so that the waits keep exact counts, and the MFMAs are issued right where
-          // a set is found complete, from that set's registers, while the other poll is still in flight
-          // (its registers are dead until the next step's polls overwrite them, in order): a single copy
-          // of the MFMAs behind the loop would have to wait for every outstanding load.
+          // ONE poll in flight, re-issued when it comes back incomplete.  With W.x out of the way of the polls
+          // (prefetch waves) a poll takes 200 to 300 cycles and finds everything in place in 92 % of the steps:
+          // the peers' h is in the L2 before this wave's own loop has come round.  A second poll half a round
+          // trip behind the first, which paid while polls took 600 cycles, then only costs: the compiler
+          // parks a wait for it behind the first MFMA (10 % of a step at config 2, and the time per step jumped
+          // by +-15 % with the distance between the two and with unrelated changes to the code).  A pause in front of
+          // the poll does not pay either (64 cycles: the same; 128: 2 % slower; 192: 6 % slower).
+          // Lanes whose batch row does not exist ask for an offset past the descriptor's end: zeros, no memory
+          // traffic.  The decision is wave-uniform (ballot) and the MFMAs are issued right where the set is
+          // found complete.
           const int xl = row_ok ? xlane : 0x7FFFFF00;
 #pragma unroll
           for (int c = 0; c < NCH; ++c)
             areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
-          __builtin_amdgcn_s_sleep(STG);
-#pragma unroll
-          for (int c = 0; c < NCH; ++c)
-            breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
           uint32_t spins = 0;
           if (!aborted) {
             for (;;) {
@@ -695,20 +692,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #pragma unroll
               for (int c = 0; c < NCH; ++c)
                 areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
-              uint32_t mb = 0u;
-#pragma unroll
-              for (int c = 0; c < NCH; ++c) mb = mark_join<BF16>(mb, chunk_mark<BF16>(breg[c]) & needmask[c]);
-              if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mb)) == 0ull) {
-                // (no copy into areg: the poll just re-issued into areg is still in flight, and a copy would
-                // have to wait for it - about half a round trip on the critical path of every step)
-                multiply(breg);
-                multiplied = true;
-                break;
-              }
-#pragma unroll
-              for (int c = 0; c < NCH; ++c)
-                breg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, xconst(c, mt), 16));
-              spins += 2;
+              spins += 1;
               if ((spins & 1023u) == 0u &&
                   __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
                 aborted = true;
@@ -882,15 +866,10 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       if (kDrainerPublishes && lane == 0)
         __hip_atomic_store(&pubflag[wave], (uint32_t)it + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (MT == 1) {
-        // The poll that did not deliver is still in flight when its set's registers die.  Keeping both sets
-        // alive to the end of the iteration stops the compiler from handing those registers to the gating
-        // code, where the first write to one of them would have to wait for that poll (on the critical path);
-        // here, after the publication, it has long landed.
+        // (the operand registers stay reserved to the end of the iteration: measured as fast or faster)
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
+        for (int c = 0; c < NCH; ++c)
           asm volatile("" :: "v"(areg[c].x), "v"(areg[c].y), "v"(areg[c].z), "v"(areg[c].w));
-          asm volatile("" :: "v"(breg[c].x), "v"(breg[c].y), "v"(breg[c].z), "v"(breg[c].w));
-        }
       }
       XS_TICK(4);
     }
