@@ -418,7 +418,7 @@ def main():
                    "tokens_per_step": B * T},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL>", "kernel_ms": kern_ms,
+                     "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,BURST=0>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_launch": nbytes, "us_per_timestep": kern_ms * 1e3 / T,
                      "max_poll_rounds": status["max_spins"],
                      # The launch is a chain of T dependent steps.  Floor of one step of this decomposition, from

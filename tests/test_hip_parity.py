@@ -82,6 +82,7 @@ F32_CASES = [
     (70, 6, 4, 512, False, True),     # four row tiles per workgroup (ragged), the drainer wave publishes
     (50, 9, 8, 256, True, True),      # two row tiles (ragged): W.x is fetched in bursts of four iterations
     (64, 1, 16, 128, False, False),   # two full row tiles, a single step: fewer iterations than one burst
+    (70, 5, 4, 128, True, True),      # one row tile of 16 rows (ragged batch): bursts with one tile
 ]
 
 
@@ -111,6 +112,8 @@ BF16_CASES = [
     (40, 21, 8, 256, True, True),     # two row tiles (ragged), W.x in bursts of eight iterations, 42 iterations
     (64, 37, 8, 256, False, True),    # two full row tiles, bursts, 74 iterations
     (64, 3, 4, 512, True, False),     # two full row tiles of a 512-wide head, fewer iterations than one burst
+    (32, 21, 4, 256, True, True),     # one row tile of 8 rows: prefetch waves and bursts together, 21 iterations
+    (50, 9, 4, 256, False, True),     # one row tile of 16 rows, ragged batch, bursts
 ]
 
 

@@ -62,22 +62,22 @@ inline size_t xbuf_elems(int B, int NH, int dh) {
 typedef void (*SeqKernel)(SeqParams);
 
 template <bool BF16, int NCH, bool FULL>
-SeqKernel pick_mt(int MT) {
+SeqKernel pick_mt(int MT, bool burst) {
   switch (MT) {
-    case 1: return slstm_seq_kernel<BF16, NCH, 1, FULL>;
-    case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL>;
-    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL>;
+    case 1: return (burst && NCH <= 4) ? slstm_seq_kernel<BF16, NCH, 1, FULL, NCH <= 4> : slstm_seq_kernel<BF16, NCH, 1, FULL, false>;
+    case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL, NCH <= 4>;
+    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL, false>;
     default: return nullptr;
   }
 }
 
 template <bool BF16, bool FULL>
-SeqKernel pick_kernel(int nch, int MT) {
+SeqKernel pick_kernel(int nch, int MT, bool burst) {
   switch (nch) {
-    case 1: return pick_mt<BF16, 1, FULL>(MT);
-    case 2: return pick_mt<BF16, 2, FULL>(MT);
-    case 4: return pick_mt<BF16, 4, FULL>(MT);
-    case 8: return pick_mt<BF16, 8, FULL>(MT);
+    case 1: return pick_mt<BF16, 1, FULL>(MT, burst);
+    case 2: return pick_mt<BF16, 2, FULL>(MT, burst);
+    case 4: return pick_mt<BF16, 4, FULL>(MT, burst);
+    case 8: return pick_mt<BF16, 8, FULL>(MT, burst);
     default: return nullptr;
   }
 }
@@ -241,8 +241,10 @@ int run_forward(const xs_slstm_args *a) {
     // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
     const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
     const int NBT_ = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
-    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT) : pick_kernel<true, false>(nch, MT))
-                          : (full ? pick_kernel<false, true>(nch, MT) : pick_kernel<false, false>(nch, MT));
+    // the feeder fetches W.x in bursts where the prefetch waves cannot cover it: row tiles of 8 rows or more
+    const bool burst = rows_per_wg >= 8;
+    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
+                          : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NH * NBT;

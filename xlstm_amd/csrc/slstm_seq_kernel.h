@@ -87,7 +87,9 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
 // the arrival test are then compiled out (with one row tile, lanes of rows that do not exist read zeros from
 // past the end of the buffer descriptor, which never look like the "not written yet" pattern).  That matters:
 // the compute waves are bound by the number of instructions between the arrival of h and the MFMAs.
-template <bool BF16, int NCH, int MT, bool FULL>
+// BURST: the feeder fetches W.x in bursts of several iterations (see there); the host asks for it with two row
+// tiles and with one row tile of 8 or 16 rows, for head dims up to 512 (bf16).
+template <bool BF16, int NCH, int MT, bool FULL, bool BURST>
 __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
@@ -191,16 +193,17 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const int NIT = p.T * MT;
   // How far ahead the feeder fetches W.x.  A compute unit returns vector-memory data in order across its waves, so
   // while feeder loads that miss to HBM are in flight the polls of the compute waves wait behind them.
-  //   one row tile    a load per iteration, four iterations ahead (the prefetch waves keep those loads from missing
-  //                   where they can);
-  //   two row tiles   BURSTS of kBurst iterations, one burst ahead (a ring of two bursts in registers): the polls
-  //                   then wait behind W.x during one memory latency per burst instead of all the time;
-  //   four or more    as with one: those iterations are bound by their arithmetic, not by the polls (the time per
-  //                   step is the same with W.x in the Infinity Cache), and bursts measured 12 % slower there.
-  //                   With two row tiles of a 1024-wide head (NCH 8) the arithmetic dominates again (bursts 9 % slower).
-  // Measured with bursts: B 128 x dh 256 2.46 -> 2.11 us per step, B 64 x 8 heads x dh 256 2.64 -> 2.25, B 64 x dh 512
-  // 2.68 -> 2.42.  At which iteration of a burst the next one is requested makes no difference (0, 1, 4 tried).
-  constexpr bool kBursts = MT == 2 && NCH <= 4;
+  //   plain   a load per iteration, four iterations ahead (with row tiles of 4 rows the prefetch waves keep those
+  //           loads from missing);
+  //   BURST   bursts of kBurst iterations, one burst ahead (a ring of two bursts in registers): the polls then wait
+  //           behind W.x during one memory latency per burst instead of all the time.
+  // Measured with bursts: two row tiles, B 128 x dh 256 2.46 -> 2.11 us per step, B 64 x 8 heads x dh 256 2.64 -> 2.25,
+  // B 64 x dh 512 2.68 -> 2.42; one row tile of 16 rows (B 64 x dh 256) 1.31 -> 1.20, of 8 rows (B 32, on top of the
+  // prefetch waves) 1.03 -> 0.96.  Not with row tiles of 4 rows, where the prefetch waves cover every line (config 2:
+  // 6 % slower), not with four row tiles (those iterations are bound by their arithmetic, the time per step is the
+  // same with W.x in the Infinity Cache; 12 % slower), not with a 1024-wide head (9 % slower).  At which iteration
+  // of a burst the next one is requested makes no difference (0, 1, 4 tried).
+  constexpr bool kBursts = BURST;
   constexpr int kBurst = kBursts ? (BF16 ? 8 : 4) : 1;
   constexpr int kFeedRing = kBursts ? 2 * kBurst : 4;
   const int NITpad = (NIT + kFeedRing - 1) / kFeedRing * kFeedRing;  // barriers every wave executes
