@@ -207,3 +207,27 @@ def test_status_reports_the_number_of_launches():
         torch.cuda.synchronize()
         st = F.read_status(ws)
         assert st["aborted"] == 0 and st["launches"] == want, st
+
+
+def test_fresh_rows_among_continued_rows_match_vanilla_rule_up_to_the_stabiliser():
+    """A supplied state whose rows are partly fresh (all zero) and partly
+    carried: vanilla's whole-tensor test (vanilla/slstm.py:24-28) then takes
+    m' = max(i, m + logsigmoid(f)) also for the fresh rows, the per-element
+    rule (slstm_pointwise.cu:79) m' = i.  That only moves the stabiliser:
+    h, c / n and m + log(n) are the same, and those are what is compared."""
+    B, T, NH, dh = 6, 24, 2, 32
+    wx, r_ext, b_ext, s0 = make_problem(77, B, T, NH, dh, with_state=True)
+    s0[:, ::2] = 0.0  # rows 0, 2, 4 start fresh
+    h_ref, s_ref = so.slstm_forward(wx, r_ext, b_ext, s0, None, n0_rule=so.N0_WHOLE_TENSOR)
+    print("case fresh-among-continued", wx.shape, flush=True)
+    h, s, status = _run_hip(wx, r_ext, b_ext, s0)
+    assert status["aborted"] == 0, status
+    assert max_err(h, h_ref) <= TOL_F32
+    assert max_err(s[0], s_ref[0]) <= TOL_F32
+    assert max_err(s[1] / s[2], s_ref[1] / s_ref[2]) <= TOL_F32
+    assert max_err(s[3] + np.log(s[2]), s_ref[3] + np.log(s_ref[2])) <= TOL_F32
+    # the rules do differ here: the stabiliser of a fresh row is not the vanilla one
+    h1, s1 = so.slstm_forward(wx[:, :1], r_ext, b_ext, s0, None, n0_rule=so.N0_WHOLE_TENSOR)
+    h2, s2 = so.slstm_forward(wx[:, :1], r_ext, b_ext, s0, None, n0_rule=so.N0_PER_ELEMENT)
+    assert np.abs(s1[3, ::2] - s2[3, ::2]).max() > 1e-3
+    assert max_err(h1, h2) <= 1e-12
