@@ -30,6 +30,8 @@ if ROOT not in sys.path:
 METRIC = "sLSTM fwd tokens/s @ D=1024 packed B16×T2048; decode step µs @ B=256"
 SERIAL_FLOOR_US = 1520 / 2350.0  # per timestep of the sequence kernel at config 2, see the roofline object
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
+CONFIG5_NAME = "config 5: B=64 T=4096 D=4096 NH=4 bf16, no resets"
 
 
 def algorithmic_bytes(B, T, NH, dh, wx_bytes, h_bytes, r_bytes, with_mask=True):
@@ -341,6 +343,9 @@ def main():
     ap.add_argument("--layer-iters", type=int, default=10, help="timed forward calls of the layer leg")
     ap.add_argument("--layer-decode-steps", type=int, default=512,
                     help="graphed decode steps of the layer leg; 0 skips them (short counter runs)")
+    ap.add_argument("--config5-only", action="store_true",
+                    help="only time the cell at BASELINE config 5 (B=64 T=4096 D=4096 NH=4 bf16), the shape bound by "
+                         "the bf16 MFMA roofline (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -365,6 +370,14 @@ def main():
         return
     if args.decode_only:
         print(json.dumps({"decode": bench_decode(device)}))
+        return
+    if args.config5_only:
+        c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=max(1, min(args.steps, 5)))
+        c5["roofline"] = {"bound": "mfma", "achieved": c5["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                          "frac": c5["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
+                          "kernel": "slstm_seq_kernel<bf16,NCH=8,MT=4,FULL,BURST=0>",
+                          "algorithmic_flops_per_launch": 8.0 * 64 * 4096 * 4096 * 1024}
+        print(json.dumps({"config5": c5}))
         return
     if args.layer_only:
         print(json.dumps({"layer": bench_layer(device, args.layer_iters, args.layer_decode_steps)}))
@@ -435,7 +448,7 @@ def main():
         out["all_configs"] = [
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),
             bench_config(device, "config 4 (one sLSTM cell): B=8 T=2048 D=1024 NH=4 bf16, documents mean 768", 8, 2048, 4, 256, True, 768),
-            bench_config(device, "config 5: B=64 T=4096 D=4096 NH=4 bf16, no resets", 64, 4096, 4, 1024, True, 0, iters=2),
+            bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=2),
         ]
     if args.config4:
         out["config4"] = bench_config4(device)
