@@ -734,19 +734,22 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         }
         if (MT != 1 && !aborted && mark_has_sentinel<BF16>(mark)) {
           uint32_t spins = 0;
-          for (;;) {
-            bool any_bad = false;
+          // The loop ENDS with the test of what it loaded.  The compiler lays a loop with lane-dependent exits out
+          // so that the wave leaves it at the bottom; with the reloads at the bottom it took the operand registers
+          // for possibly still being loaded behind the loop and put a wait for ALL outstanding loads (the next
+          // tile's requests included) in front of the MFMAs.  The two ways out on a failure leave before a reload.
+          bool bad[NCH];
+          bool any_bad;
+          auto test_chunks = [&]() {
+            any_bad = false;
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
-              if (need[c]) {
-                const bool bad = BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]);
-                if (bad) {
-                  any_bad = true;
-                  areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
-                }
-              }
+              bad[c] = need[c] && (BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]));
+              any_bad |= bad[c];
             }
-            if (!any_bad) break;
+          };
+          test_chunks();
+          while (any_bad) {
             ++spins;
             if ((spins & 1023u) == 0u &&
                 __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
@@ -761,6 +764,11 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
               }
               break;
             }
+#pragma unroll
+            for (int c = 0; c < NCH; ++c)
+              if (bad[c])
+                areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
+            test_chunks();
           }
           max_spins = spins > max_spins ? spins : max_spins;
 #ifdef XS_PROFILE
