@@ -27,7 +27,17 @@ def _cases(n, seed):
     return out
 
 
-@pytest.mark.parametrize("bf16,B,T,NH,dh,with_state,resets,seed", _cases(40, 2024) + _cases(16, 7))
+# more heads than the device holds at once (NH * ceil(dh/16) workgroups > 256 compute units): the heads are
+# independent, so the engine runs them in several launches
+_MANY_HEADS = [
+    (True, 5, 6, 32, 256, True, False, 11),    # 512 workgroups: two launches of 16 heads
+    (True, 40, 5, 24, 384, False, True, 12),   # 24 workgroups per head: 10 + 10 + 4 heads, three row chunks
+    (False, 3, 7, 40, 128, True, True, 13),    # fp32, 320 workgroups: 32 + 8 heads
+    (True, 70, 4, 6, 1024, False, False, 14),  # 64 workgroups per head: 4 + 2 heads, two XCDs per head
+]
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,with_state,resets,seed", _cases(40, 2024) + _cases(16, 7) + _MANY_HEADS)
 def test_random_shape_against_oracle_and_stepwise(bf16, B, T, NH, dh, with_state, resets, seed):
     from xlstm_amd import functional as F
 

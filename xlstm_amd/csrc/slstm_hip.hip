@@ -222,11 +222,18 @@ int run_forward(const xs_slstm_args *a) {
   const int G = (dh + 15) / 16;
   const int cus = device_cus();
   if (cus <= 0) return fail(XS_ERR_DEVICE, "cannot query the device");
-  if ((long long)NH * G > cus) return fail(XS_ERR_UNSUPPORTED, "NH * ceil(dh/16) = %lld workgroups exceed the %d compute units; they must all be resident", (long long)NH * G, cus);
+  if (G > cus) return fail(XS_ERR_UNSUPPORTED, "ceil(dh/16) = %d workgroups of one head exceed the %d compute units; they must all be resident", G, cus);
+
+  // Heads are independent (block-diagonal R): when the workgroups of all heads do not fit the device at once,
+  // the heads go in several launches, as many per launch as fit.
+  const int heads_per_launch = NH < cus / G ? NH : cus / G;
+  int launch_no = 0;
+  for (int head0 = 0; head0 < NH; head0 += heads_per_launch) {
+  const int NHL = head0 + heads_per_launch <= NH ? heads_per_launch : NH - head0;
 
   // batch tiling: the fewest rows per workgroup such that all groups of one launch are co-resident
   const int tiles = (B + 15) / 16;
-  const int max_groups_per_head = cus / (NH * G);  // >= 1
+  const int max_groups_per_head = cus / (NHL * G);  // >= 1
   int MT = 1;
   while (MT < 4 && (tiles + MT - 1) / MT > max_groups_per_head) MT *= 2;
   int rows_per_wg = 16 * MT;
@@ -247,7 +254,10 @@ int run_forward(const xs_slstm_args *a) {
                           : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
-    const int ngroups = NH * NBT;
+    const int ngroups = NHL * NBT;
+    if (launch_no++ > 0)  // the placement words of the previous launch must not pass for this one's
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(4), dim3(256), 0, stream,
+                         (uint32_t *)((char *)a->workspace + kStatusBytes), (size_t)kMaxWg, 0u);
     // grid shapes of the three placements the kernel knows: one XCD per group, two XCDs per group, spread
     const int grid = G <= 32 ? 8 * G * ((ngroups + 7) / 8)
                              : ((G <= 64 && G % 2 == 0) ? 8 * (G / 2) * ((ngroups + 3) / 4) : ngroups * G);
@@ -269,6 +279,7 @@ int run_forward(const xs_slstm_args *a) {
     p.xbuf = (char *)a->workspace + kHeaderBytes;
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
+    p.head0 = head0; p.NHL = NHL;
     p.spin_limit = a->spin_limit;
     // a prefetch wave issues 2 (bf16) or 4 (fp32) scalar loads per batch row of a tile; 8 per wave and iteration
     // and 16 in all are what the scalar cache sustains, a tile that needs more goes without (prefetch waves that
@@ -288,6 +299,7 @@ int run_forward(const xs_slstm_args *a) {
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
   }
+  }  // heads of one launch
   return XS_OK;
 }
 

@@ -22,6 +22,8 @@ struct SeqParams {
   int b0, bend;  // batch rows [b0, bend) handled by this launch
   int G;         // workgroups per head group
   int NBT;       // batch tiles (independent groups) per head
+  int head0;     // first head of this launch (more heads than fit the device at once go in several launches)
+  int NHL;       // heads of this launch
   int rows_per_wg;
   long long spin_limit;
   int prefetch;  // number of prefetch waves launched behind the six others (0 .. kMaxPrefetchWaves)
@@ -117,7 +119,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   // ---- role of this workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8,
   //      a head group takes consecutive slots of ONE XCD so its exchange stays in one L2)
   const int wg = blockIdx.x;
-  const int ngroups = p.NH * p.NBT;
+  const int ngroups = p.NHL * p.NBT;
   int gi, member;  // head group index, position inside the group
   const bool one_xcd_layout = p.G <= 32;
   if (one_xcd_layout) {
@@ -140,8 +142,8 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     member = wg - gi * p.G;
   }
   if (gi >= ngroups) return;
-  const int head = gi / p.NBT;
-  const int bt = gi - head * p.NBT;
+  const int head = p.head0 + gi / p.NBT;
+  const int bt = gi % p.NBT;
 
   const int tid = threadIdx.x;
   const int wave = tid >> 6;
