@@ -107,6 +107,13 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   // shared memory, [2][compute wave][NCH][lane] 16-byte pieces), because the load latency of a
   // freshly published tile (about 3000 to 5000 cycles) is longer than one iteration.
   constexpr bool kDeepPrefetch = kDrainerPublishes;
+  // Where in an iteration those requests are issued.  Four waves x NCH loads of 1 KiB each keep the compute unit's
+  // one address path busy for up to some 500 cycles, and a wave that issues into a full queue stalls.  Right behind
+  // the MFMAs (where the LDS slot has just been read) that stall sits in front of the partial sums and the barrier,
+  // on the critical path of all four waves; behind the gating it does not.  Measured, bf16: dh 1024 20.8 -> 17.2 ms
+  // (BASELINE config 5), dh 512 3.93 -> 3.50 us per step; dh 256 and the variants with a K tail 1 to 3 % slower,
+  // so those keep the early place.  A tile requested there still has a whole iteration to arrive.
+  constexpr bool kLateRequests = NCH >= 4 && FULL;
   extern __shared__ __attribute__((aligned(16))) unsigned char seq_dyn_lds[];
 
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
@@ -789,7 +796,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         multiply(areg);
       }
 
-      if (kDeepPrefetch) {
+      auto issue_requests = [&]() {
         // request the tile of iteration it + 2 (its LDS slot is the one just read); step 0 takes its
         // operand from s0.  A chunk past the last member reads zeros (the descriptor ends with the slot).
         const int nmt = (mt + 2) % MT;
@@ -801,6 +808,9 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #pragma unroll
           for (int c = 0; c < NCH; ++c) lds_direct_load_b128(rs, lds0 + (c << 10), xlane, xconst(c, nmt));
         }
+      };
+      if (kDeepPrefetch) {
+        if (!kLateRequests) issue_requests();
       } else if (MT > 1) {
         // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
         const int nmt = (mt + 1) % MT;
@@ -843,6 +853,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #ifdef XS_PROFILE
       asm volatile("" :: "v"(st[mt].y));
 #endif
+      if (kDeepPrefetch && kLateRequests) issue_requests();
       XS_TICK(3);
       // ---- 5. publish h_t to the peers, re-arm the words of h_{t-2}, stage h_t for the drainer
       float y = st[mt].y;
