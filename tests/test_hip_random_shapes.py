@@ -37,7 +37,18 @@ _MANY_HEADS = [
 ]
 
 
-@pytest.mark.parametrize("bf16,B,T,NH,dh,with_state,resets,seed", _cases(40, 2024) + _cases(16, 7) + _MANY_HEADS)
+# four row tiles per workgroup with a head dim that fills the K range exactly: the variants that request the tile
+# after next behind the gating (with document starts, carried state, a second launch of fewer rows)
+_FOUR_TILES = [
+    (True, 64, 9, 8, 512, True, True, 21),
+    (True, 128, 6, 4, 512, False, True, 22),
+    (True, 64, 7, 4, 1024, True, True, 23),
+    (False, 64, 5, 16, 256, False, True, 24),
+    (True, 96, 5, 8, 512, False, False, 25),
+]
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,with_state,resets,seed", _cases(40, 2024) + _cases(16, 7) + _MANY_HEADS + _FOUR_TILES)
 def test_random_shape_against_oracle_and_stepwise(bf16, B, T, NH, dh, with_state, resets, seed):
     from xlstm_amd import functional as F
 
