@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 5
+#define XS_ABI_VERSION 6
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -109,13 +109,15 @@ typedef struct xs_slstm_args {
 
 /* Status block at the start of the workspace, written by the kernels. */
 typedef struct xs_slstm_status {
-  uint32_t aborted;     /* 1 if a bounded wait ran out (results are invalid) */
+  uint32_t aborted;     /* 1 if a bounded wait ran out: the results are invalid, and every workgroup that finished after
+                           the give-up has overwritten its part of h_out and s_out with NaN */
   uint32_t abort_wg;    /* workgroup that gave up first */
   uint32_t abort_step;  /* timestep it was waiting for */
   uint32_t max_spins;   /* largest number of poll iterations any wait needed */
   uint32_t xcd_mixed;   /* number of head groups whose workgroups ran on more than one XCD */
   uint32_t launches;    /* kernel launches the call was split into */
-  uint32_t reserved[10];
+  uint32_t step_kernel; /* 1 if the call ran the single-token step kernel (xs_slstm_step, or xs_slstm_forward with T == 1) */
+  uint32_t reserved[9];
 } xs_slstm_status;
 
 /* Library / ABI identification.  Replaces nothing (the reference keys its JIT
@@ -135,6 +137,9 @@ size_t xs_slstm_workspace_bytes(int32_t B, int32_t T, int32_t NH, int32_t dh);
  * (xlstm/blocks/slstm/src/cuda/slstm.cc:53-135,
  *  xlstm/blocks/slstm/src/cuda/slstm_forward.cu:217-267) and the vanilla loop
  * (xlstm/blocks/slstm/src/vanilla/__init__.py:17-74).
+ * A call with T == 1 whose recurrent matrix is in the dtype of wx is what the
+ * reference's layer makes for every decoded token (xlstm/blocks/slstm/layer.py:113-115);
+ * it runs the step kernel of xs_slstm_step (same bits, status.step_kernel = 1).
  */
 int xs_slstm_forward(const xs_slstm_args *args);
 

@@ -136,3 +136,22 @@ def test_reference_checkpoint_layouts_convert_to_hip():
         reference_cell_params_to_hip(torch.from_numpy(z["r_cuda"]), torch.from_numpy(z["b_cuda"]), "vanilla", NH)
     with pytest.raises(ValueError):
         reference_cell_params_to_hip(torch.from_numpy(z["r_cuda"]), torch.from_numpy(z["b_cuda"]), "triton", NH)
+
+
+def test_cell_can_be_copied_and_pickled():
+    """copy.deepcopy / pickle of a cell (torch does it for EMA copies, DDP, checkpoints of whole modules): the
+    parameter proxies follow the copy, the per-cell runtime objects (workspaces, events, decode plan) do not."""
+    import copy
+    import pickle
+
+    import torch
+
+    from xlstm_amd.cell import sLSTMCell, sLSTMCellConfig
+
+    c = sLSTMCell(sLSTMCellConfig(hidden_size=64, num_heads=4, backend="hip", recurrent_weight_init="standard"),
+                  skip_backend_init=True)
+    for other in (copy.deepcopy(c), pickle.loads(pickle.dumps(c))):
+        assert other._rt is not c._rt and other.recurrent_kernel.module is other
+        assert torch.equal(other.recurrent_kernel[:], c.recurrent_kernel[:]) and torch.equal(other.bias[:], c.bias[:])
+        other.bias[0, 1] = torch.zeros(16)
+        assert not torch.equal(other.bias[:], c.bias[:])

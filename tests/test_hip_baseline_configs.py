@@ -70,25 +70,38 @@ def test_config2_and_config4_cell_packed_documents_full_size(B, mean_len, name):
 
 
 def test_config3_decode_full_width():
-    """B=256, D=2048 (8 x 256), bf16: 128-token prefill, then T=1 steps carrying the state."""
-    B, NH, dh, PRE, STEPS = 256, 8, 256, 128, 48
+    """B=256, D=2048 (8 x 256), bf16: 128-token prefill, then 1024 consecutive T=1 steps carrying the state,
+    as BASELINE states it."""
+    B, NH, dh, PRE, STEPS = 256, 8, 256, 128, 1024
     H = NH * dh
-    print("config 3", flush=True)
-    wx, r, b, _ = make_problem(103, B, PRE + STEPS, NH, dh, bf16=True)
+    print("config 3: building inputs on the device", flush=True)
+    g = torch.Generator(device=DEV).manual_seed(103)
+    wx_t = torch.empty(B, PRE + STEPS, 4 * H, dtype=torch.bfloat16, device=DEV)
+    for row in range(B):
+        wx_t[row] = torch.randn(PRE + STEPS, 4 * H, generator=g, device=DEV).bfloat16()
+    _, r, b, _ = make_problem(103, 1, 1, NH, dh)
     r_t, b_t = _params(r, b)
-    wx_t = torch.from_numpy(wx).to(DEV).bfloat16()
+    r_step = r_t.bfloat16()
+    print("config 3: prefill + 1024 steps", flush=True)
     h_pre, s = _hip(wx_t[:, :PRE], r_t, b_t)
-    hs = []
-    for t in range(PRE, PRE + STEPS):
-        h1, s = _hip(wx_t[:, t:t + 1], r_t, b_t, s, step=True)
-        hs.append(h1)
-    h_dec = torch.cat(hs)
+    from xlstm_amd import functional as F
+
+    ws = F.workspace_for(B, 1, NH, dh, wx_t.device)
+    h_dec = torch.empty(STEPS, B, H, dtype=torch.bfloat16, device=DEV)
+    s_a, s_b = s.clone(), torch.empty_like(s)
+    for t in range(STEPS):
+        F.slstm_forward(wx_t[:, PRE + t:PRE + t + 1], r_step, b_t, s_a, None, step=True, workspace=ws,
+                        h_out=h_dec[t:t + 1], s_out=s_b)
+        s_a, s_b = s_b, s_a
+    torch.cuda.synchronize()
+    assert F.read_status(ws)["step_kernel"] == 1
     # property at full size: decoding step by step == one sequence call, bit for bit
+    print("config 3: one sequence call over all 1152 tokens", flush=True)
     h_all, s_all = _hip(wx_t, r_t, b_t)
-    assert torch.equal(h_all[:PRE], h_pre) and torch.equal(h_all[PRE:], h_dec) and torch.equal(s_all, s)
+    assert torch.equal(h_all[:PRE], h_pre) and torch.equal(h_all[PRE:], h_dec) and torch.equal(s_all, s_a)
     # oracle on a few rows (rows are independent)
     rows = [0, 17, 255]
-    h_ref, s_ref = so.slstm_forward(wx[rows], r, b)
+    h_ref, s_ref = so.slstm_forward(wx_t[rows].float().cpu().numpy(), r, b)
     assert max_err(h_all[:, rows].float().cpu().numpy(), h_ref) <= 2e-2
     assert max_err(s_all[:, rows].cpu().numpy(), s_ref) <= 2e-2
     assert tuple(h_all.shape) == (PRE + STEPS, B, H)

@@ -90,6 +90,96 @@ def test_bf16_cell_with_reset_mask_and_step():
         assert torch.equal(s, st)
 
 
+@pytest.mark.parametrize("bf16", [True, False])
+def test_forward_with_one_token_is_the_decode_entry_and_runs_the_step_kernel(bf16):
+    """The reference's layer decodes by calling the cell's FORWARD with S = 1 (layer.py:113-115), never cell.step:
+    that call must reach the step kernel and reproduce one sequence call bit for bit."""
+    B, T, NH, dh = 6, 20, 4, 64
+    wx, r, b, s0 = make_problem(26, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=True)
+    reset = np.zeros((B, T), np.uint8); reset[2, 0] = 1; reset[4, 7] = 1; reset[0, [11, 12]] = 1
+    cell = _cell_from(r, b, dtype="bfloat16" if bf16 else "float32", output_shape="SBH")
+    cell.keep_state_fp32 = True
+    x = torch.from_numpy(wx).cuda()
+    x = x.bfloat16() if bf16 else x
+    m = torch.from_numpy(reset).cuda()
+    s0_t = torch.from_numpy(s0).cuda()
+    with torch.no_grad():
+        out, st = cell(x, s0_t, reset_mask=m)
+        assert cell.last_status()["step_kernel"] == 0 and cell.last_status()["launches"] == 1
+        # (a) the reference layer's way: slices of the input, the state handed from call to call, a mask kwarg
+        s = s0_t
+        for t in range(T):
+            o, s = cell(x[:, t:t + 1], s, reset_mask=m[:, t:t + 1])
+            assert cell.last_status()["step_kernel"] == 1, t
+            assert torch.equal(o[0], out[t]), t
+        assert torch.equal(s, st)
+        # (b) no mask, contiguous tokens, float32 state: the pre-validated plan; (c) no state at all
+        out_nm, st_nm = cell(x, s0_t)
+        s = s0_t
+        for t in range(T):
+            o, s = cell(x[:, t:t + 1].contiguous(), s)
+            assert cell.last_status()["step_kernel"] == 1
+            assert torch.equal(o[0], out_nm[t]), t
+        assert torch.equal(s, st_nm)
+        out_z, _ = cell(x)
+        o, _ = cell(x[:, :1])
+        assert cell.last_status()["step_kernel"] == 1 and torch.equal(o[0], out_z[0])
+    h_ref, s_ref = so.slstm_forward(wx, r, b, s0, reset)
+    tol = 2e-2 if bf16 else 1e-5
+    assert max_err(out.float().cpu().numpy(), h_ref) <= tol and max_err(st.cpu().numpy(), s_ref) <= tol
+
+
+def test_one_token_through_the_c_abi_forward_entry_runs_the_step_kernel():
+    """xs_slstm_forward itself hands a T == 1 call to the step kernel when R is in the operand type."""
+    from tests._util import r_ext_to_kernel
+    from xlstm_amd import functional as F
+
+    B, NH, dh = 70, 2, 128
+    wx, r, b, s0 = make_problem(27, B, 1, NH, dh, bf16=True, with_state=True)
+    x = torch.from_numpy(wx).cuda().bfloat16()
+    r_t = r_ext_to_kernel(torch.from_numpy(r)).cuda()
+    b_t, s0_t = torch.from_numpy(b).cuda(), torch.from_numpy(s0).cuda()
+    ws = F.workspace_for(B, 1, NH, dh, x.device)
+    h_f, s_f = F.slstm_forward(x, r_t.bfloat16(), b_t, s0_t, None, workspace=ws)           # forward entry, bf16 R
+    assert F.read_status(ws)["step_kernel"] == 1
+    h_s, s_s = F.slstm_forward(x, r_t.bfloat16(), b_t, s0_t, None, workspace=ws, step=True)  # step entry
+    assert torch.equal(h_f, h_s) and torch.equal(s_f, s_s)
+    h_q, s_q = F.slstm_forward(x, r_t, b_t, s0_t, None, workspace=ws)                      # float32 R: the sequence kernel
+    assert F.read_status(ws)["step_kernel"] == 0
+    assert torch.equal(h_f, h_q) and torch.equal(s_f, s_q)
+
+
+@pytest.mark.parametrize("backend", ["vanilla", "cuda"])
+def test_reference_checkpoint_runs_through_the_hip_cell(backend):
+    """Parameters as the reference's vanilla / cuda cells store them (tests/golden/ckpt_layouts.npz, written from
+    those classes) -> reference_state_dict_to_hip -> load_state_dict -> HIP forward, against the oracle run on the
+    external views the fixture holds."""
+    from xlstm_amd.cell import reference_state_dict_to_hip, sLSTMCell, sLSTMCellConfig
+
+    z = np.load(os.path.join(GOLDEN, "ckpt_layouts.npz"))
+    NH = int(z["num_heads"])
+    r_ext, b_ext = z["r_ext"], z["b_ext"]
+    dh = r_ext.shape[1]
+    cell = sLSTMCell(sLSTMCellConfig(hidden_size=NH * dh, num_heads=NH, backend="hip", dtype="float32", output_shape="SBH"))
+    sd = {"_recurrent_kernel_": torch.from_numpy(z[f"r_{backend}"]), "_bias_": torch.from_numpy(z[f"b_{backend}"])}
+    cell.load_state_dict(reference_state_dict_to_hip(sd, backend, NH))
+    cell = cell.to("cuda:0").eval()
+    B, T = 3, 17
+    wx, _, _, s0 = make_problem(28, B, T, NH, dh, with_state=True)
+    h_ref, s_ref = so.slstm_forward(wx, r_ext, b_ext, s0)
+    with torch.no_grad():
+        out, st = cell(torch.from_numpy(wx).cuda(), torch.from_numpy(s0).cuda())
+    assert max_err(out.cpu().numpy(), h_ref) <= 1e-5 and max_err(st.cpu().numpy(), s_ref) <= 1e-5
+    assert np.abs(r_ext).max() > 0 and np.abs(h_ref).max() > 1e-2  # (the fixture's R is not the zeros init)
+
+
+def test_forward_clipval_is_refused_not_ignored():
+    from xlstm_amd.cell import sLSTMCell, sLSTMCellConfig
+
+    with pytest.raises(NotImplementedError, match="forward_clipval"):
+        sLSTMCell(sLSTMCellConfig(hidden_size=64, num_heads=4, backend="hip", forward_clipval=1.0))
+
+
 def test_float16_input_is_computed_in_float32_and_rounded_back():
     B, T, NH, dh = 2, 5, 2, 16
     wx, r, b, _ = make_problem(23, B, T, NH, dh, rscale=3.0)

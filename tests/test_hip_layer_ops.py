@@ -203,9 +203,22 @@ def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
         layer.fused_pre_ops = False
         b1 = layer(x[:, 1:9], conv_state=st_p2["conv_state"])
         b2 = layer(x[:, 1:9], conv_state=st_p2["conv_state"][0][:, -2:])
+        # the same layer in float32 (bf16-rounded parameters, PyTorch ops, float32 cell kernel): the yardstick
+        import copy
+
+        ref_layer = copy.deepcopy(layer).float()
+        ref_layer.fused_pre_ops = False
+        ref32 = ref_layer(x.float(), reset_mask=mask)
+    # The engine's layer path against the float32 layer at the bf16 bar.  The PyTorch bf16 path rounds after every op
+    # (conv, SiLU, each projection) and is itself up to that far from float32, so the two bf16 pipelines are compared
+    # with each other at the sum of the two bars, after the group norm has divided by a head's spread.
+    e_fused = max_err(fused.float().cpu().numpy(), ref32.cpu().numpy())
+    e_plain = max_err(plain.float().cpu().numpy(), ref32.cpu().numpy())
+    print("layer vs float32 layer: engine ops %.3e, torch ops %.3e" % (e_fused, e_plain), flush=True)
+    assert e_fused <= 2e-2
+    assert max_err(fused.float().cpu().numpy(), plain.float().cpu().numpy()) <= 2e-2 + max(e_plain, 2e-2)
     assert max_err(a1.float().cpu().numpy(), b1.float().cpu().numpy()) <= 5e-2
     assert max_err(a2.float().cpu().numpy(), b2.float().cpu().numpy()) <= 5e-2
-    assert max_err(fused.float().cpu().numpy(), plain.float().cpu().numpy()) <= 5e-2  # two bf16 pipelines, group-normed
     assert torch.equal(st_f["conv_state"], st_p["conv_state"])
     assert max_err(st_f["slstm_state"].cpu().numpy(), st_p["slstm_state"].cpu().numpy()) <= 5e-2
     assert max_err(o_f.float().cpu().numpy(), o_p.float().cpu().numpy()) <= 5e-2

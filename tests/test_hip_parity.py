@@ -172,23 +172,126 @@ def test_empty_sequence_returns_initial_state():
     np.testing.assert_array_equal(s, np.zeros_like(s0))
 
 
+def _assert_flagged_or_right(h, s, status, h_ref, s_ref):
+    """A call whose bounded wait ran out says so twice: in the status block and by NaN in every output a workgroup
+    wrote after the give-up (at least the final state of the workgroup that gave up).  A call that never had to
+    wait longer than the bound is simply right."""
+    if status["aborted"]:
+        assert not np.isfinite(s).all(), "aborted call left a plausible final state"
+        assert not np.isfinite(h).all(), "aborted call left a plausible h"
+    else:
+        assert max_err(h, h_ref) <= TOL_BF16 and max_err(s, s_ref) <= TOL_BF16
+
+
 def test_spin_limit_runs_out_is_reported_not_hung():
     """Error path forced from the host: a one-iteration bound on the waits
-    between compute units.  The kernel must finish and flag the call."""
+    between compute units.  The kernel must finish, flag the call and poison its outputs."""
     wx, r, b, _ = make_problem(16, 16, 64, 4, 256, bf16=True)
+    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
     h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
     assert status["aborted"] in (0, 1)
     if status["aborted"]:
         assert status["abort_step"] >= 1
+    _assert_flagged_or_right(h, s, status, h_ref, s_ref)
     # four row tiles per workgroup: the drainer wave's wait for the compute waves is bounded the same way
     wx, r, b, _ = make_problem(17, 64, 6, 4, 1024, bf16=True)
+    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
     h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
     assert status["aborted"] in (0, 1)
+    _assert_flagged_or_right(h, s, status, h_ref, s_ref)
     # and the next call on the same device is unaffected
     h2, s2, status2 = _run_hip(wx, r, b, bf16=True)
     assert status2["aborted"] == 0
-    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
     assert max_err(h2, h_ref) <= TOL_BF16
+
+
+def test_cell_raises_for_an_aborted_call_at_the_next_host_contact():
+    """The cell copies the status word of every sequence call to pinned memory behind the kernel; a call that gave
+    up surfaces as EngineError from check_status() (or from the cell's next call)."""
+    from xlstm_amd import functional as F
+    from xlstm_amd.cell import sLSTMCell, sLSTMCellConfig
+
+    wx, r, b, _ = make_problem(16, 16, 64, 4, 256, bf16=True)
+    cell = sLSTMCell(sLSTMCellConfig(hidden_size=1024, num_heads=4, backend="hip", output_shape="SBH"))
+    cell.recurrent_kernel[:] = torch.from_numpy(r)
+    cell.bias[:] = torch.from_numpy(b)
+    cell = cell.to("cuda:0").eval()
+    x = torch.from_numpy(wx).cuda().bfloat16()
+    with torch.no_grad():
+        out, st = cell(x)
+        cell.check_status()  # a normal call: nothing to report
+        assert cell.last_status()["aborted"] == 0 and bool(torch.isfinite(st.float()).all())
+        # the same call with a one-poll bound, through the cell's own workspace and watch
+        ws = cell._workspace(16, x.device)
+        h, s = F.slstm_forward(x, cell._recurrent_kernel_.detach(), cell._bias_.detach().view(4, 4, 256), None, None,
+                               workspace=ws, spin_limit=1)
+        cell._watch(ws)
+        torch.cuda.synchronize()
+        if F.read_status(ws)["aborted"]:
+            assert not bool(torch.isfinite(s).all())
+            with pytest.raises(F.EngineError, match="gave up waiting"):
+                cell.check_status()
+        else:
+            cell.check_status()
+        out2, st2 = cell(x)  # the cell keeps working
+        cell.check_status()
+        assert torch.equal(out2, out) and torch.equal(st2, st)
+
+
+MASKED_START_CASES = [
+    # bf16, B, T, NH, dh: a supplied state AND a mask whose first column is mixed 0 / 1
+    (False, 6, 9, 2, 64),      # one row tile of 4 rows ... 8 rows
+    (False, 40, 5, 4, 128),    # 16-row tiles, ragged
+    (False, 70, 4, 4, 512),    # four row tiles (the drainer publishes), fp32
+    (True, 16, 12, 4, 256),    # BASELINE config 2's variant
+    (True, 50, 6, 8, 256),     # two row tiles
+    (True, 70, 5, 4, 1024),    # four row tiles, groups over two XCDs
+    (True, 5, 7, 3, 40),       # K tail
+]
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh", MASKED_START_CASES)
+def test_mask_at_the_first_step_overrides_the_supplied_state(bf16, B, T, NH, dh):
+    """mask[b, 0] = 1 makes row b ignore the state it was given (the row starts a document), rows with
+    mask[b, 0] = 0 continue from it: sequence kernel and step kernel against the oracle, and the masked rows
+    bit for bit against the same call without a state."""
+    print("case masked start", bf16, B, T, NH, dh, flush=True)
+    wx, r, b, s0 = make_problem(31, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=True)
+    reset = geometric_reset_mask(9, B, T, max(2, T // 2))
+    reset[:, 0] = (np.arange(B) % 3 != 1).astype(np.uint8)  # rows 1, 4, 7, ... continue from s0
+    tol = TOL_BF16 if bf16 else TOL_F32
+    h_ref, s_ref = so.slstm_forward(wx, r, b, s0, reset)
+    h, s, status = _run_hip(wx, r, b, s0, reset, bf16=bf16)
+    _check(h, s, h_ref, s_ref, tol, status)
+    # the state really matters for the rows that keep it, and not at all for the others
+    h_z, s_z, _ = _run_hip(wx, r, b, None, reset, bf16=bf16)
+    fresh = reset[:, 0] != 0
+    np.testing.assert_array_equal(h[:, fresh], h_z[:, fresh])
+    np.testing.assert_array_equal(s[:, fresh], s_z[:, fresh])
+    assert np.abs(h[0][~fresh] - h_z[0][~fresh]).max() > 1e-3
+    # the step kernel, one token at a time, with the same first-column mask
+    st = s0
+    for t in range(min(T, 3)):
+        ht, st, status = _run_hip(wx[:, t:t + 1], r, b, st, reset[:, t:t + 1], bf16=bf16, step=True)
+        assert status["step_kernel"] == 1
+        np.testing.assert_array_equal(ht[0], h[t])
+    h1_ref, s1_ref = so.slstm_forward(wx[:, :1], r, b, s0, reset[:, :1])
+    h1, s1, _ = _run_hip(wx[:, :1], r, b, s0, reset[:, :1], bf16=bf16, step=True)
+    assert max_err(h1, h1_ref) <= tol and max_err(s1, s1_ref) <= tol
+
+
+def test_head_groups_are_sized_per_xcd():
+    """24 workgroups per head group (dh 384): an XCD of 32 compute units holds ONE such group, so 10 heads go in
+    two launches of at most 8 groups.  Sized per device (256 / 24 = 10 groups) two XCDs would get 48 workgroups
+    and the late group's members would spin until the early ones finish.  A few hundred steps, no long waits."""
+    B, T, NH, dh = 4, 300, 10, 384
+    print("case per-XCD sizing", B, T, NH, dh, flush=True)
+    wx, r, b, _ = make_problem(41, B, T, NH, dh, bf16=True)
+    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
+    h, s, status = _run_hip(wx, r, b, bf16=True)
+    _check(h, s, h_ref, s_ref, TOL_BF16, status)
+    assert status["launches"] == 2, status
+    assert status["max_spins"] < 20000, status  # (a starved group would need millions of polls per step)
 
 
 def test_status_reports_the_number_of_launches():

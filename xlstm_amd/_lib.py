@@ -13,7 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 EXPORTS = (
     "xs_abi_version",
@@ -108,7 +108,8 @@ class SlstmStatus(ctypes.Structure):
     _fields_ = [
         ("aborted", ctypes.c_uint32), ("abort_wg", ctypes.c_uint32), ("abort_step", ctypes.c_uint32),
         ("max_spins", ctypes.c_uint32), ("xcd_mixed", ctypes.c_uint32), ("launches", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32 * 10),
+        ("step_kernel", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32 * 9),
     ]
 
 

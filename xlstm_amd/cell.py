@@ -17,7 +17,10 @@ What differs, on purpose:
   * the stabiliser uses the native kernel's per-element ``n == 0`` rule
     (slstm_pointwise.cu:79), which equals the vanilla rule for every state the
     cell itself can produce;
-  * forward only: the hip backend is an inference engine, ``backward`` raises.
+  * forward only: the hip backend is an inference engine, ``backward`` raises;
+  * a call with S == 1 -- what the reference's ``sLSTMLayer.step`` makes for every decoded
+    token (layer.py:113-115) -- runs the single-token step kernel, bit-identical to the same
+    step inside a longer call.
 """
 from __future__ import annotations
 
@@ -78,6 +81,9 @@ class ParameterProxy:
         return self.internal_to_external(self._param().grad)
 
     def __getattr__(self, name: str):
+        # (only reached for names the proxy itself lacks; while a copy is being rebuilt it has no fields yet)
+        if name in ("module", "parameter_name") or (name.startswith("__") and name.endswith("__")):
+            raise AttributeError(name)
         return getattr(getattr(self.module, self.parameter_name), name)
 
 
@@ -177,6 +183,24 @@ class _ForwardOnly(torch.autograd.Function):
         )
 
 
+class _Runtime:
+    """What a cell keeps between calls and must not travel with it: workspaces, pinned status words and events of
+    calls in flight, the cached bf16 copy of R, the decode plan.  A copied or unpickled cell starts with none."""
+
+    def __init__(self):
+        self.workspaces = {}
+        self.status_ring = None
+        self.last_workspace = None
+        self.r_bf16 = None
+        self.step_plan = None
+
+    def __deepcopy__(self, memo):
+        return _Runtime()
+
+    def __reduce__(self):
+        return (_Runtime, ())
+
+
 class sLSTMCell_hip(nn.Module):
     """The cell on the MI355X engine.
 
@@ -206,8 +230,14 @@ class sLSTMCell_hip(nn.Module):
         self._bias_ = nn.Parameter(torch.zeros(4 * NH * dh, dtype=torch.float32))
         self.bias = ParameterProxy(self, "_bias", self._bias_int2ext, self._bias_ext2int)
         self.config.internal_input_shape = "SBGNH"  # the kernel reads the external (gate, head, unit) order in place
+        if self.config.forward_clipval is not None:
+            # the reference's native kernel clips y to +-clipval when built with it (slstm_pointwise.cu:107-110);
+            # the hip kernels have no such path, and ignoring the setting would change results silently
+            raise NotImplementedError("sLSTMCell backend 'hip' does not implement forward_clipval; leave it None")
         # optional: keep the carried state in float32 instead of the input dtype
         self.keep_state_fp32 = False
+        # workspaces of the sequence kernel, one per (device, stream), the status words of calls in flight, caches
+        self._rt = _Runtime()
         self.reset_parameters()
         if not skip_backend_init:
             from . import _lib
@@ -325,16 +355,87 @@ class sLSTMCell_hip(nn.Module):
         """bf16 copy of R for decoding, refreshed when the parameter changes."""
         p = self._recurrent_kernel_
         key = (p.data_ptr(), p._version, p.device)
-        cache = getattr(self, "_r_bf16_cache", None)
+        cache = self._rt.r_bf16
         if cache is None or cache[0] != key:
             cache = (key, p.detach().to(torch.bfloat16).contiguous())
-            object.__setattr__(self, "_r_bf16_cache", cache)
+            self._rt.r_bf16 = cache
         return cache[1]
+
+    # ------------------------------------------------------------------ status of calls in flight
+    _STATUS_SLOTS = 16
+
+    def _workspace(self, B: int, device) -> torch.Tensor:
+        """The cell's workspace for calls on the current stream of ``device`` (calls on one stream run one after the
+        other, so they can share it; calls on different streams may overlap and get one each)."""
+        stream = torch.cuda.current_stream(device).cuda_stream
+        NH, dh = self.config.num_heads, self.head_dim
+        need = F_hip._lib.load().xs_slstm_workspace_bytes(B, 1, NH, dh)
+        key = (device, stream)
+        ws = self._rt.workspaces.get(key)
+        if ws is None or ws.numel() < need:
+            ws = torch.empty(need, dtype=torch.uint8, device=device)
+            self._rt.workspaces[key] = ws
+        return ws
+
+    def _watch(self, workspace: torch.Tensor) -> None:
+        """Queues a copy of the call's ``aborted`` word to pinned host memory behind the kernel and looks at the
+        words of earlier calls that have arrived: a sequence call whose wait between compute units ran out
+        (its outputs are NaN by then) raises here, at the next call, or in :meth:`check_status`."""
+        if torch.cuda.is_current_stream_capturing():
+            return
+        ring = self._rt.status_ring
+        if ring is None:
+            ring = {"host": torch.zeros(self._STATUS_SLOTS, dtype=torch.int32).pin_memory(),
+                    "events": [None] * self._STATUS_SLOTS, "next": 0}
+            self._rt.status_ring = ring
+        self._poll_status(block=False)
+        i = ring["next"]
+        if ring["events"][i] is not None:  # the ring is full of calls still running: wait for the oldest
+            ring["events"][i].synchronize()
+            self._poll_status(block=False)
+        ring["host"][i:i + 1].copy_(workspace[:4].view(torch.int32), non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        ring["events"][i] = ev
+        ring["next"] = (i + 1) % self._STATUS_SLOTS
+
+    def _poll_status(self, block: bool) -> None:
+        ring = self._rt.status_ring
+        if ring is None:
+            return
+        bad = False
+        for i, ev in enumerate(ring["events"]):
+            if ev is None:
+                continue
+            if block:
+                ev.synchronize()
+            elif not ev.query():
+                continue
+            ring["events"][i] = None
+            bad |= int(ring["host"][i]) != 0
+        if bad:
+            raise F_hip.EngineError(
+                "an earlier sLSTM sequence call on the hip backend gave up waiting for some of its compute units "
+                "(they were held by other work on the GPU); its outputs were set to NaN"
+            )
+
+    def check_status(self) -> None:
+        """Waits for this cell's calls in flight and raises ``EngineError`` if one of them was aborted."""
+        self._poll_status(block=True)
+
+    def last_status(self) -> dict:
+        """The status block of this cell's most recent call (synchronises): ``aborted``, ``launches``,
+        ``step_kernel`` (1 when the call ran the single-token kernel), ``max_spins``, ..."""
+        ws = self._rt.last_workspace
+        if ws is None:
+            raise RuntimeError("the cell has not been called yet")
+        return F_hip.read_status(ws)
 
     def _run(self, input, state, reset_mask, step: bool, state_out=None):
         self._check_input(input)
         x = self._input_bs(input)
         B = x.shape[0]
+        step = step or x.shape[1] == 1  # one token: the step kernel (the reference layer decodes through forward)
         self._check_state(B, state)
         in_dtype = input.dtype
         if in_dtype == torch.float16:  # no fp16 kernels: compute in float32, round the results back
@@ -344,6 +445,7 @@ class sLSTMCell_hip(nn.Module):
         r = self._recurrent_kernel_.detach()
         if step and x.dtype == torch.bfloat16:
             r = self._bf16_recurrent_kernel()  # the step kernel reads R every token: keep it in the operand type
+        ws = self._workspace(B, x.device) if x.is_cuda else None
         h, s = F_hip.slstm_forward(
             x,
             r,
@@ -352,7 +454,11 @@ class sLSTMCell_hip(nn.Module):
             reset_mask,
             step=step,
             s_out=state_out,
+            workspace=ws,
         )
+        self._rt.last_workspace = ws
+        if not step and x.shape[1] > 1:
+            self._watch(ws)
         if torch.is_grad_enabled() and (
             input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
         ):
@@ -368,6 +474,10 @@ class sLSTMCell_hip(nn.Module):
         """``input`` [B,S,4H] (or [S,B,4H] for input_shape 'SBGNH'), optional ``state`` [4,B,H],
         optional ``reset_mask`` [B,S].  Returns ``(output, state)`` like cell.py:496-506."""
         del lengths  # unused, as in the reference
+        if input.dim() == 3 and input.shape[1 if self.config.input_shape == "BSGNH" else 0] == 1:
+            fast = self._step_fast(input, state, reset_mask, None)
+            if fast is not None:
+                return fast
         return self._run(input, state, reset_mask, step=False)
 
     def step(self, input: torch.Tensor, state: Optional[torch.Tensor] = None, reset_mask=None,
@@ -407,11 +517,11 @@ class sLSTMCell_hip(nn.Module):
         self._check_state(B, state)
         r, b = self._recurrent_kernel_, self._bias_
         key = (B, input.dtype, input.device, r.data_ptr(), r._version, b.data_ptr(), b._version)
-        cached = getattr(self, "_step_plan_cache", None)
+        cached = self._rt.step_plan
         if cached is None or cached[0] != key:
             plan = F_hip.StepPlan(B, r.detach(), b.detach().view(self.config.num_heads, 4, self.head_dim), wx_dtype=input.dtype)
             cached = (key, plan)
-            object.__setattr__(self, "_step_plan_cache", cached)
+            self._rt.step_plan = cached
         H = self.config.hidden_size
         h = h_out if h_out is not None else torch.empty((1, B, H), dtype=input.dtype, device=input.device)
         if h.dtype != input.dtype or h.numel() != B * H or not h.is_contiguous():
@@ -419,6 +529,7 @@ class sLSTMCell_hip(nn.Module):
         s_out = state_out if state_out is not None else torch.empty((4, B, H), dtype=torch.float32, device=input.device)
         with torch.cuda.device(input.device):
             cached[1](input, state, s_out, h, h_prev=h_prev)
+        self._rt.last_workspace = cached[1].workspace
         return self._permute_output(h), (s_out if self.keep_state_fp32 else s_out.to(input.dtype))
 
 

@@ -16,6 +16,8 @@ constexpr int kTileFloats = 16 * kTileStride;
 constexpr uint32_t kSentinel32 = 0xFFFFFFFFu;  // fp32 "not written yet"
 constexpr uint32_t kSentinel16 = 0xFFFFu;      // bf16 "not written yet"
 constexpr long long kDefaultSpinLimit = 1ll << 22;
+// what the outputs of a call hold after one of its bounded waits ran out (a quiet NaN; as bf16 it is 0x7FC0)
+constexpr float kPoison = __builtin_bit_cast(float, 0x7FC00000u);
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
 

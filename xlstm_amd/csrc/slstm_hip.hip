@@ -24,7 +24,6 @@
 #include <string.h>
 
 #include <mutex>
-#include <vector>
 
 #include "xlstm_amd.h"
 
@@ -82,7 +81,7 @@ SeqKernel pick_kernel(int nch, int MT, bool burst) {
   }
 }
 
-int validate(const xs_slstm_args *a, bool step) {
+int validate(const xs_slstm_args *a, bool step, bool own_scratch = false) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
   if (step && a->T != 1) return fail(XS_ERR_SHAPE, "xs_slstm_step needs T == 1, got %d", a->T);
@@ -113,9 +112,11 @@ int validate(const xs_slstm_args *a, bool step) {
       ((uintptr_t)a->h_prev % al))
     return fail(XS_ERR_ALIGN, "r, h_out, s0, s_out and h_prev must be 16-byte aligned");
   if (a->h_prev && !a->s0) return fail(XS_ERR_NULL, "h_prev is a copy of the y plane of s0: s0 is required with it");
-  if (!a->workspace || a->workspace_bytes < xs_slstm_workspace_bytes(a->B, a->T, a->NH, a->dh))
-    return fail(XS_ERR_WORKSPACE, "workspace missing or smaller than xs_slstm_workspace_bytes()");
-  if ((uintptr_t)a->workspace % 256) return fail(XS_ERR_ALIGN, "workspace must be 256-byte aligned");
+  if (!own_scratch) {  // (the entry point with a scratch array of its own checks what the launches really need)
+    if (!a->workspace || a->workspace_bytes < xs_slstm_workspace_bytes(a->B, a->T, a->NH, a->dh))
+      return fail(XS_ERR_WORKSPACE, "workspace missing or smaller than xs_slstm_workspace_bytes()");
+    if ((uintptr_t)a->workspace % 256) return fail(XS_ERR_ALIGN, "workspace must be 256-byte aligned");
+  }
   return XS_OK;
 }
 
@@ -133,15 +134,16 @@ int device_cus() {
 int ensure_dynamic_lds(const void *kernel, size_t bytes) {
   struct Done { const void *kernel; int device; size_t bytes; };
   static std::mutex mu;
-  static std::vector<Done> done;
+  static Done done[256];  // (a fixed table: nothing on the launch path allocates, host memory included)
+  static int ndone = 0;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) return fail(XS_ERR_DEVICE, "cannot query the current device");
   std::lock_guard<std::mutex> lock(mu);
-  for (const Done &d : done)
-    if (d.kernel == kernel && d.device == dev && d.bytes >= bytes) return XS_OK;
+  for (int i = 0; i < ndone; ++i)
+    if (done[i].kernel == kernel && done[i].device == dev && done[i].bytes >= bytes) return XS_OK;
   const hipError_t ea = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
   if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(ea));
-  done.push_back(Done{kernel, dev, bytes});
+  if (ndone < 256) done[ndone++] = Done{kernel, dev, bytes};  // (a full table only means the attribute is set again next time)
   return XS_OK;
 }
 
@@ -198,17 +200,22 @@ int run_step(const xs_slstm_args *a) {
   return XS_OK;
 }
 
-int run_forward(const xs_slstm_args *a) {
+// need != nullptr: launch nothing, only report the bytes of workspace the launches of this call touch
+int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   hipStream_t stream = (hipStream_t)a->stream;
   const int B = a->B, T = a->T, NH = a->NH, dh = a->dh;
   const long long H = (long long)NH * dh;
   const bool bf16 = a->wx_dtype == XS_BF16;
+  const bool dry = need != nullptr;
+  if (dry) *need = kHeaderBytes;
 
   // status block + per-workgroup placement words start clean
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(4), dim3(256), 0, stream, (uint32_t *)a->workspace,
-                     (kStatusBytes + (size_t)kMaxWg * 4) / 4, 0u);
+  if (!dry)
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(4), dim3(256), 0, stream, (uint32_t *)a->workspace,
+                       (kStatusBytes + (size_t)kMaxWg * 4) / 4, 0u);
   if (B == 0) return XS_OK;
   if (T == 0) {
+    if (dry) return XS_OK;
     const size_t n = (size_t)4 * B * H;
     hipLaunchKernelGGL(copy_state_kernel, dim3(256), dim3(256), 0, stream, a->s0, a->s_out, n);
     return hipGetLastError() == hipSuccess ? XS_OK : fail(XS_ERR_LAUNCH, "state copy launch failed");
@@ -224,16 +231,27 @@ int run_forward(const xs_slstm_args *a) {
   if (cus <= 0) return fail(XS_ERR_DEVICE, "cannot query the device");
   if (G > cus) return fail(XS_ERR_UNSUPPORTED, "ceil(dh/16) = %d workgroups of one head exceed the %d compute units; they must all be resident", G, cus);
 
-  // Heads are independent (block-diagonal R): when the workgroups of all heads do not fit the device at once,
-  // the heads go in several launches, as many per launch as fit.
-  const int heads_per_launch = NH < cus / G ? NH : cus / G;
+  // Every workgroup of a head group waits for the others, so all groups of a launch must be resident at once, and
+  // the placement deals groups out per XCD: a group of up to 32 workgroups sits on ONE XCD, a larger even one on
+  // an XCD pair, anything else is spread over the device.  What a launch may hold is therefore counted per XCD
+  // (one workgroup per compute unit), not per device: with 24 workgroups per group an XCD of 32 compute units
+  // holds one group, not 32 * 8 / 24 of the device's.
+  const int cus_per_xcd = cus / 8 > 0 ? cus / 8 : 1;
+  int capacity;  // head groups per launch
+  if (G <= 32) capacity = 8 * (cus_per_xcd / G);
+  else if (G <= 64 && G % 2 == 0) capacity = 4 * ((2 * cus_per_xcd) / G);
+  else capacity = cus / G;
+  if (capacity < 1) return fail(XS_ERR_DEVICE, "a head group of %d workgroups does not fit the %d compute units of this device's XCDs", G, cus);
+  // Heads are independent (block-diagonal R): when the groups of all heads do not fit at once, the heads go in
+  // several launches, as many per launch as fit.
+  const int heads_per_launch = NH < capacity ? NH : capacity;
   int launch_no = 0;
   for (int head0 = 0; head0 < NH; head0 += heads_per_launch) {
   const int NHL = head0 + heads_per_launch <= NH ? heads_per_launch : NH - head0;
 
   // batch tiling: the fewest rows per workgroup such that all groups of one launch are co-resident
   const int tiles = (B + 15) / 16;
-  const int max_groups_per_head = cus / (NHL * G);  // >= 1
+  const int max_groups_per_head = capacity / NHL;  // >= 1
   int MT = 1;
   while (MT < 4 && (tiles + MT - 1) / MT > max_groups_per_head) MT *= 2;
   int rows_per_wg = 16 * MT;
@@ -247,7 +265,6 @@ int run_forward(const xs_slstm_args *a) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
     // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
     const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
-    const int NBT_ = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     // the feeder fetches W.x in bursts where the prefetch waves cannot cover it: row tiles of 8 rows or more
     const bool burst = rows_per_wg >= 8;
     SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
@@ -255,6 +272,11 @@ int run_forward(const xs_slstm_args *a) {
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NHL * NBT;
+    if (dry) {
+      const size_t ring = (size_t)kRing * ngroups * G * 16 * MT * 16 * (bf16 ? 2 : 4);
+      if (kHeaderBytes + ring > *need) *need = kHeaderBytes + ring;
+      continue;
+    }
     if (launch_no++ > 0)  // the placement words of the previous launch must not pass for this one's
       hipLaunchKernelGGL(fill_u32_kernel, dim3(4), dim3(256), 0, stream,
                          (uint32_t *)((char *)a->workspace + kStatusBytes), (size_t)kMaxWg, 0u);
@@ -452,6 +474,8 @@ int xs_slstm_forward(const xs_slstm_args *args) {
   g_err[0] = 0;
   const int rc = validate(args, false);
   if (rc != XS_OK) return rc;
+  // one token: the tiled step kernel (no waits between compute units, bit-identical to the sequence kernel)
+  if (args->T == 1 && args->B > 0 && args->r_dtype == args->wx_dtype) return run_step(args);
   return run_forward(args);
 }
 

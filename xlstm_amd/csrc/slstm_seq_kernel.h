@@ -330,11 +330,12 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     const int drow = lane >> 2;   // batch row inside the tile
     const int dq = lane & 3;      // which 4 of the 16 units
     bool dcross = false;
-    auto drain = [&](int it, bool publish) {
+    auto drain = [&](int it, bool publish, bool poison = false) {
       const int t = it / MT;
       const int mt = it - t * MT;
       const int brow = rowbase + mt * 16 + drow;
-      const f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
+      f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
+      if (poison) v = f32x4{kPoison, kPoison, kPoison, kPoison};
       if (kDrainerPublishes && publish) {
         // h_t of this tile goes to the exchange ring from here, and the words of h_{t-2} are re-armed,
         // so the compute waves wait on nothing but their polls.  Every lane stores: words outside
@@ -431,6 +432,12 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     lds_barrier();  // final barrier
     for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it, false);
     }
+    // A bounded wait ran out somewhere: whatever this workgroup computed from then on is built on operands that
+    // never arrived.  A caller that does not read the status block must not mistake it for a result, so the
+    // workgroup's part of h_out becomes NaN (the compute waves do the same to s_out).  Any workgroup that consumed
+    // such operands did so after the flag was raised, and looks at the flag here, later still.
+    if (__hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
+      for (int it = 0; it < NIT; ++it) drain(it, false, true);
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
@@ -907,12 +914,14 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   }
 #endif
 
-  // ---- final state
+  // ---- final state (NaN when a bounded wait ran out anywhere in the call: see the drainer)
+  const bool poisoned = __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int brow = rowbase + mt * 16 + pb;
     if (unit_ok && brow < rend) {
       const long long o = (long long)brow * H + col;
+      if (poisoned) st[mt] = CellState{kPoison, kPoison, kPoison, kPoison};
       p.s_out[o] = st[mt].y; p.s_out[BH + o] = st[mt].c; p.s_out[2 * BH + o] = st[mt].n; p.s_out[3 * BH + o] = st[mt].m;
     }
   }

@@ -130,7 +130,7 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
   const int nslab = (4 * nch) / SLABCH;
 
   if (blockIdx.x == 0 && threadIdx.x < 16)
-    reinterpret_cast<uint32_t *>(p.status)[tid] = tid == 5 ? 1u : 0u;  // a step never waits, so it never aborts; one launch
+    reinterpret_cast<uint32_t *>(p.status)[tid] = (tid == 5 || tid == 6) ? 1u : 0u;  // a step never waits, so it never aborts; one launch; step_kernel = 1
 
   const bool has_s0 = FULL || p.s0 != nullptr;
   const bool has_reset = !FULL && p.reset != nullptr;
@@ -385,6 +385,11 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
   // ---- operands, K loop (SPLIT: the MFMA waves).  No load is issued before the roles part: where the two paths
   // touch in the compiler's control-flow graph it waits for every load the other path might have in flight.
   if (DIRECT) {
+    // Every load between the first hand-issued operand request and the hand-written wait for the first K half is
+    // hand-issued too, so that wait's count is a constant of this file, not of what the compiler emits: the
+    // compiler's own loads of this role (the bias) go out BEFORE the requests (the assembly statements clobber
+    // memory, so the compiler moves no load across them), W.x goes out behind them as assembly.
+    load_bias_and_flags();
     {
       const unsigned long long hb = reinterpret_cast<unsigned long long>(p.h_prev), rb = reinterpret_cast<unsigned long long>(p.r);
       const u32x4_t hrs = {uniform((uint32_t)hb), uniform((uint32_t)(hb >> 32) & 0xFFFFu), uniform((uint32_t)(BH * 2)), 0x00020000u};
@@ -424,14 +429,27 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
 
   // W.x comes from HBM when the previous kernel did not just write it, the old state from the Infinity Cache: the
   // requests for this role's W.x go out early, those for its state once every operand has landed
-  if (SPLIT) { load_bias_and_flags(); load_wx(1, 2); }
+  if (DIRECT) {
+    // W.x of this role's row tile (4 gates x 4 units of one row per lane): hand-issued, see above.  The compiler takes
+    // the registers for written when the statement has been issued; they are read behind the wait for all loads in
+    // front of the second K half, which names them as operands so that nothing that reads them moves above it.
+    const int brow = rowbase + 32 * wr + 16 + r16;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const uint16_t *src = reinterpret_cast<const uint16_t *>(p.wx) + ((long long)brow * p.wx_sb + (long long)g * H + col);
+      asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(wxb[1][g]) : "v"(src) : "memory");
+    }
+  } else if (SPLIT) {
+    load_bias_and_flags();
+    load_wx(1, 2);
+  }
 #ifdef XS_PROFILE
   pstamp[1] = clock64();
 #endif
   if (DIRECT) {
-    // In flight, in this order: 12 + 12 operand loads, then the 4 bias and 4 W.x loads just above (the assembly
-    // statements keep them there; fewer would only make this wait longer): at most 20 left = the first K half is in LDS
-    asm volatile("s_waitcnt vmcnt(20)" ::: "memory");
+    // In flight behind the first K half's 12 requests, all hand-issued: 12 requests of the second half and 4 of W.x.
+    // At most 16 left = the first K half is in LDS.
+    asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   } else {
     store_slab(0, 0, hring[0], rring[0], SLABCH >= 4 ? 0 : -1);
   }
@@ -452,7 +470,8 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         pstamp[7] = clock64();
 #endif
-        if (DIRECT) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (DIRECT)  // the second K half and the hand-issued W.x
+          asm volatile("s_waitcnt vmcnt(0)" : "+v"(wxb[1][0]), "+v"(wxb[1][1]), "+v"(wxb[1][2]), "+v"(wxb[1][3]) :: "memory");
         else store_slab(0, 0, hring[0], rring[0], 1);
         if (SPLIT) lds_barrier(); else __syncthreads();
         // every operand has landed: the requests for the state this role gates go out now and arrive behind the

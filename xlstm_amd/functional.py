@@ -167,6 +167,9 @@ class StepPlan:
 
     The caller keeps the plan's contract: tensors on the plan's device, which is the current one,
     the dtypes and shapes given at construction, contiguous, ``s_out`` not overlapping ``s_in``.
+    A plan is NOT re-entrant: every call rewrites the one argument block the plan owns, so a plan
+    belongs to one host thread at a time (calls from one thread onto different streams are fine,
+    the block is read before the call returns).
     """
 
     def __init__(self, B: int, r: torch.Tensor, bias: torch.Tensor, wx_dtype: torch.dtype = torch.bfloat16,
