@@ -144,6 +144,21 @@ size_t xs_slstm_workspace_bytes(int32_t B, int32_t T, int32_t NH, int32_t dh);
 int xs_slstm_forward(const xs_slstm_args *args);
 
 /*
+ * xs_slstm_forward for callers that cannot allocate device memory or pass a workspace (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference.
+ * Same arguments and results as xs_slstm_forward, except that args->workspace and args->workspace_bytes are
+ * ignored: the status block, the placement words and the exchange ring live in an array of
+ * XS_STATIC_SCRATCH_BYTES that is part of the library's device image (each GPU the library runs on holds it
+ * until the process ends).  It calls no allocator, host or device.  4 MiB + 64 KiB hold every bfloat16 call on a
+ * device of 256 compute units; a call whose launches need more (float32 with four row tiles per workgroup on all
+ * compute units, e.g. B >= 128 at NH 4 x dh 512: 8 MiB) returns XS_ERR_WORKSPACE before anything is launched.  All calls on one GPU share its array: calls that overlap in
+ * time on one GPU race (give each stream its own workspace through xs_slstm_forward instead); what must start
+ * clean is cleared by fill kernels at the start of every call.  The status block is not reachable by the caller.
+ */
+#define XS_STATIC_SCRATCH_BYTES ((4u << 20) + (64u << 10))
+int xs_slstm_forward_static(const xs_slstm_args *args);
+
+/*
  * Single-token decode step (T must be 1): state in, state out, no waits
  * between compute units; bit-identical to the same step inside a sequence
  * call.  The recurrent matrix must be in the dtype of wx (keep a bf16 copy

@@ -13,6 +13,7 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
+STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
 ABI_VERSION = 6
 
 EXPORTS = (
@@ -21,6 +22,7 @@ EXPORTS = (
     "xs_slstm_workspace_bytes",
     "xs_slstm_forward",
     "xs_slstm_step",
+    "xs_slstm_forward_static",
     "xs_causal_conv_silu",
     "xs_headwise_gates",
     "xs_headwise_group_norm",
@@ -133,7 +135,7 @@ def load() -> ctypes.CDLL:
     lib.xs_last_error.argtypes = []
     lib.xs_slstm_workspace_bytes.restype = ctypes.c_size_t
     lib.xs_slstm_workspace_bytes.argtypes = [ctypes.c_int32] * 4
-    for name in ("xs_slstm_forward", "xs_slstm_step"):
+    for name in ("xs_slstm_forward", "xs_slstm_step", "xs_slstm_forward_static"):
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmArgs)]

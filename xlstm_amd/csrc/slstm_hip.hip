@@ -32,6 +32,13 @@
 #include "slstm_step_kernel.h"
 #include "slstm_layer_kernels.h"
 
+// ---------------------------------------------------------------------------
+// Scratch of the entry point that allocates nothing (xs_slstm_forward_static): status block, placement words and
+// exchange ring in an array that every GPU the library runs on holds until the process ends.  In host code the
+// array's name is only a stand-in: the device address comes from hipGetSymbolAddress, once per device.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[XS_STATIC_SCRATCH_BYTES];
+
 namespace {
 
 // ---------------------------------------------------------------------------
@@ -457,6 +464,26 @@ int run_group_norm(const xs_norm_args *a) {
   return XS_OK;
 }
 
+// host side of the static scratch array: its device address, per device
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void *g_scratch_ptr[kMaxDevices] = {};
+
+int static_scratch(void **out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return fail(XS_ERR_DEVICE, "cannot query the current device");
+  if (dev < 0 || dev >= kMaxDevices) return fail(XS_ERR_DEVICE, "device %d beyond the %d this entry point keeps scratch for", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));  // this device's copy of the array
+    if (e != hipSuccess || !ptr) return fail(XS_ERR_DEVICE, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return XS_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -477,6 +504,24 @@ int xs_slstm_forward(const xs_slstm_args *args) {
   // one token: the tiled step kernel (no waits between compute units, bit-identical to the sequence kernel)
   if (args->T == 1 && args->B > 0 && args->r_dtype == args->wx_dtype) return run_step(args);
   return run_forward(args);
+}
+
+int xs_slstm_forward_static(const xs_slstm_args *args) {
+  g_err[0] = 0;
+  int rc = validate(args, false, true);
+  if (rc != XS_OK) return rc;
+  xs_slstm_args a = *args;
+  rc = static_scratch(&a.workspace);
+  if (rc != XS_OK) return rc;
+  a.workspace_bytes = XS_STATIC_SCRATCH_BYTES;
+  if (a.T == 1 && a.B > 0 && a.r_dtype == a.wx_dtype) return run_step(&a);  // (touches the status block only)
+  size_t need = 0;
+  rc = run_forward(&a, &need);  // what the launches of this call would touch; launches nothing
+  if (rc != XS_OK) return rc;
+  if (need > (size_t)XS_STATIC_SCRATCH_BYTES)
+    return fail(XS_ERR_WORKSPACE, "this call needs %zu bytes of scratch, the static array holds %zu: use xs_slstm_forward with a workspace",
+                need, (size_t)XS_STATIC_SCRATCH_BYTES);
+  return run_forward(&a);
 }
 
 int xs_slstm_step(const xs_slstm_args *args) {
