@@ -171,7 +171,8 @@ def bench_decode(device, steps=1024, prefill=128):
         "finite": bool(torch.isfinite(s_a).all()),
         "roofline": {"bound": "hbm", "achieved": nbytes / (best_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": nbytes / (best_us * 1e-6) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
-                     "kernel": "slstm_step_tile_kernel<bf16,SLABCH=8,FULL,HB,SPLIT>", "algorithmic_bytes_per_launch": nbytes},
+                     "kernel": "slstm_step_pipe_kernel<NK=8>", "algorithmic_bytes_per_launch": nbytes,
+                     "traffic_source": "profiles/traffic_step_cfg3.json (rocprofv3 counters of a separate run, not of this one)"},
     }
 
 
@@ -444,6 +445,7 @@ def main():
     traffic_file = os.path.join(ROOT, "profiles", "traffic_seq_cfg2.json")
     if os.path.exists(traffic_file):
         out["roofline"]["traffic"] = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
+        out["roofline"]["traffic_source"] = "profiles/traffic_seq_cfg2.json (rocprofv3 counters of a separate run, not of this one)"
     if args.all_configs:
         out["all_configs"] = [
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),

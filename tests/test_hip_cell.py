@@ -269,3 +269,41 @@ def test_bf16_operand_hint_gives_the_same_bits():
             prev = h[t & 1]
             torch.cuda.synchronize()
             assert torch.equal(prev, h_ref) and torch.equal(a, ref), (B, NH, dh, t)
+
+
+@pytest.mark.parametrize("B,NH,dh", [(256, 8, 256), (64, 4, 128), (128, 2, 256)])
+def test_operand_hint_chain_back_to_back_with_different_inputs(B, NH, dh):
+    """The kernels that take the previous h in bf16 place their operands in LDS themselves (hand-issued loads, hand-counted
+    waits, no markers that would expose a piece that has not landed).  A chain of steps with very different inputs is
+    launched back to back, nothing in between (every compute unit starts a step with the previous step's operands
+    still in its LDS), and compared bit for bit with the same chain through the kernel without the hint, run
+    afterwards.  BASELINE config 3's shape first."""
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    torch.manual_seed(7)
+    H = NH * dh
+    STEPS = 6
+    r = ((torch.rand(NH, 4 * dh, dh, device=dev) - 0.5) * 0.3).bfloat16()
+    bias = torch.randn(NH, 4, dh, device=dev)
+    scale = torch.tensor([1.0, -3.0, 0.1, 5.0, -0.5, 2.0], device=dev).view(STEPS, 1, 1, 1)
+    wx = (torch.randn(STEPS, B, 1, 4 * H, device=dev) * scale).bfloat16()
+    s = torch.randn(4, B, H, device=dev)
+    s[2] = s[2].abs() + 0.5
+    plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16)
+    print("case hint chain", B, NH, dh, flush=True)
+    # the chain with the hint: state and h buffers alternate, all outputs kept
+    states = [s.clone()] + [torch.empty_like(s) for _ in range(STEPS)]
+    hs = [torch.empty(1, B, H, dtype=torch.bfloat16, device=dev) for _ in range(STEPS + 1)]
+    hs[0].copy_(s[0].bfloat16().view(1, B, H))  # the bf16 copy of the first state's y plane
+    for t in range(STEPS):
+        plan(wx[t], states[t], states[t + 1], hs[t + 1], h_prev=hs[t])
+    torch.cuda.synchronize()
+    assert F.read_status(plan.workspace)["step_kernel"] == 1
+    # the same chain without it
+    ref = s.clone()
+    for t in range(STEPS):
+        h_ref, ref = F.slstm_forward(wx[t], r, bias, ref, None, step=True)
+        assert torch.equal(hs[t + 1], h_ref), t
+        assert torch.equal(states[t + 1], ref), t
+

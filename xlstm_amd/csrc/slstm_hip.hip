@@ -30,6 +30,7 @@
 #include "slstm_device_common.h"
 #include "slstm_seq_kernel.h"
 #include "slstm_step_kernel.h"
+#include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
 
 // ---------------------------------------------------------------------------
@@ -191,6 +192,18 @@ int run_step(const xs_slstm_args *a) {
   StepKernel kern;
   const bool hint = full && bf16 && a->h_prev != nullptr;  // operand already in bf16 (h_out of the previous step)
   p.h_prev = hint ? a->h_prev : nullptr;
+  // the steady state of bf16 decoding with the previous h at hand, head dim 256: the pipelined kernel (row tiles move
+  // through fetch, MFMA, gating and store one behind the other); its buffer offsets are 31-bit
+  if (hint && dh == 256 && 63ll * a->wx_stride_b * 2 + 4ll * NH * dh * 2 < (1ll << 31) && 4ll * B * NH * dh * 4 < (1ll << 31)) {
+    const size_t plds = (size_t)2 * 64 * 256 + 3 * 64 * 128 + 4 * 64 * 64 + 2 * 128 * 256 + 64;  // h, c/n/m, W.x, R (later the sums), counters
+    void (*pk)(StepParams) = slstm_step_pipe_kernel<8>;
+    const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(pk), plds);
+    if (rc != XS_OK) return rc;
+    hipLaunchKernelGGL(pk, grid, dim3(kStepPipeThreads), plds, stream, p);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
+    return XS_OK;
+  }
 #define XS_PICK(BF, SC, SP) (full ? slstm_step_tile_kernel<BF, SC, true, false, SP> : slstm_step_tile_kernel<BF, SC, false, false, SP>)
 #define XS_PICK_HINT(SC, SP) (hint ? slstm_step_tile_kernel<true, SC, true, true, SP> : XS_PICK(true, SC, SP))
   if (bf16) kern = slabch == 4 ? XS_PICK_HINT(4, true) : (slabch == 8 ? XS_PICK_HINT(8, true) : XS_PICK_HINT(2, false));
