@@ -214,6 +214,24 @@ def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
             "aborted": F.read_status(ws)["aborted"]}
 
 
+def bench_small_batch(device, T=1024):
+    """The sequence kernel at the batch sizes where an MFMA row tile is mostly padding: B = 1, 2, 4 at head dims 128
+    and 256 (4 heads), bf16 and fp32, plus the reference test's shape (B 1, 4 heads of 16, one step:
+    tests/test_slstm_cell_vanilla_vs_cuda.py:12-40).  Run once with the shipped library (MFMA contraction) and once
+    with a library built with -DXS_SMALL_BATCH_FMA (XLSTM_AMD_LIB=...) to compare the two contractions."""
+    rows = []
+    for bf16 in (True, False):
+        for dh in (128, 256):
+            if not bf16 and dh == 256:
+                continue  # (a float32 head of 256 is not a whole K range of the small variants)
+            for B in (1, 2, 4):
+                r = bench_config(device, f"B={B} T={T} NH=4 dh={dh} {'bf16' if bf16 else 'fp32'}", B, T, 4, dh, bf16, 0, iters=5)
+                rows.append({k: r[k] for k in ("workload", "ms", "us_per_timestep", "aborted")})
+    r = bench_config(device, "reference test shape: B=1 T=1 NH=4 dh=16 fp32 (one step)", 1, 1, 4, 16, False, 0, iters=20)
+    rows.append({"workload": r["workload"], "us_per_call": r["ms"] * 1e3})
+    return {"library": os.environ.get("XLSTM_AMD_LIB", "xlstm_amd/lib/libxlstm_amd.so"), "rows": rows}
+
+
 def bench_config4(device, iters=3):
     """BASELINE config 4: 24 blocks (sLSTM at 3, 11, 19), D=1024, 4 heads, vocab 50304, bf16, B=8, T=2048,
     packed documents of mean length 768.  Only the sLSTM cells run on the HIP engine."""
@@ -347,6 +365,8 @@ def main():
     ap.add_argument("--config5-only", action="store_true",
                     help="only time the cell at BASELINE config 5 (B=64 T=4096 D=4096 NH=4 bf16), the shape bound by "
                          "the bf16 MFMA roofline (profiling runs)")
+    ap.add_argument("--small-batch-only", action="store_true",
+                    help="only time the sequence kernel at B = 1, 2, 4 (head dims 128 and 256) and the reference test's shape")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -371,6 +391,9 @@ def main():
         return
     if args.decode_only:
         print(json.dumps({"decode": bench_decode(device)}))
+        return
+    if args.small_batch_only:
+        print(json.dumps({"small_batch": bench_small_batch(device)}))
         return
     if args.config5_only:
         c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=max(1, min(args.steps, 5)))
@@ -451,6 +474,7 @@ def main():
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),
             bench_config(device, "config 4 (one sLSTM cell): B=8 T=2048 D=1024 NH=4 bf16, documents mean 768", 8, 2048, 4, 256, True, 768),
             bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=2),
+            bench_config(device, "reference test shape: B=1 T=1 NH=4 dh=16 fp32 (one step, the step kernel)", 1, 1, 4, 16, False, 0, iters=20),
         ]
     if args.config4:
         out["config4"] = bench_config4(device)

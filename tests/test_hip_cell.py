@@ -307,3 +307,25 @@ def test_operand_hint_chain_back_to_back_with_different_inputs(B, NH, dh):
         assert torch.equal(hs[t + 1], h_ref), t
         assert torch.equal(states[t + 1], ref), t
 
+
+def test_cell_forward_decode_loop_uses_the_previous_h_when_the_state_comes_back_untouched():
+    """A decode loop through cell.forward with the float32 state kept (cell.keep_state_fp32): from the second token
+    on the cell hands the step kernel the h of the previous call (the bf16 copy of the state's y plane).  Same bits
+    as a sequence call; a state that was modified in between is not trusted."""
+    B, T, NH, dh = 64, 8, 2, 256
+    wx, r, b, s0 = make_problem(29, B, T, NH, dh, bf16=True, with_state=True)
+    cell = _cell_from(r, b, dtype="bfloat16", output_shape="SBH")
+    cell.keep_state_fp32 = True
+    x = torch.from_numpy(wx).cuda().bfloat16()
+    with torch.no_grad():
+        out, st = cell(x, torch.from_numpy(s0).cuda())
+        s = torch.from_numpy(s0).cuda()
+        for t in range(T):
+            if t == 5:
+                s.mul_(1.0)  # an in-place touch: the cell must fall back to reading y from the state
+            o, s = cell(x[:, t:t + 1].contiguous(), s)
+            assert torch.equal(o[0], out[t]), t
+            used_hint = cell._rt.step_plan[1]._args.h_prev is not None
+            assert used_hint == (t not in (0, 5)), (t, used_hint)
+        assert torch.equal(s, st)
+

@@ -25,10 +25,14 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = False) -> str:
+def build(verbose: bool = False, extra_flags=(), out: str = LIB) -> str:
+    """Builds the engine.  ``extra_flags`` / ``out`` are for the two measurement builds the kernels know about:
+    ``-DXS_PROFILE`` (per-phase cycle stamps, read back by ``bench.py --phase-profile``) and
+    ``-DXS_SMALL_BATCH_FMA`` (the FMA contraction for row tiles of 4 rows); from the command line:
+    ``python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so``."""
     hipcc = os.environ.get("HIPCC", "hipcc")
-    os.makedirs(os.path.dirname(LIB), exist_ok=True)
-    cmd = [hipcc, *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *SOURCES]
+    os.makedirs(os.path.dirname(out), exist_ok=True)
+    cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, "-I", os.path.join(ROOT, "include"), "-o", out, *SOURCES]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -37,9 +41,15 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
     if verbose and out.strip():
         print(out)
-    return LIB
+    return out
 
 
 if __name__ == "__main__":
-    print(build(verbose=True))
+    argv = sys.argv[1:]
+    target = LIB
+    if "-o" in argv:
+        i = argv.index("-o")
+        target = os.path.abspath(argv[i + 1])
+        del argv[i:i + 2]
+    print(build(verbose=True, extra_flags=tuple(argv), out=target))
     sys.exit(0)

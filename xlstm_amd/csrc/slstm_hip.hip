@@ -289,6 +289,13 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
     const bool burst = rows_per_wg >= 8;
     SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
                           : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
+#ifdef XS_SMALL_BATCH_FMA
+    // the measured alternative for small batches (see the kernel): only in a library built for that measurement
+    if (MT == 1 && rows_per_wg == 4 && nch <= 2 && full) {
+      if (bf16) kern = nch == 1 ? slstm_seq_kernel<true, 1, 1, true, false, true> : slstm_seq_kernel<true, 2, 1, true, false, true>;
+      else kern = nch == 1 ? slstm_seq_kernel<false, 1, 1, true, false, true> : slstm_seq_kernel<false, 2, 1, true, false, true>;
+    }
+#endif
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NHL * NBT;

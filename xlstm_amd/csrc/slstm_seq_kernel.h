@@ -91,8 +91,15 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
 // the compute waves are bound by the number of instructions between the arrival of h and the MFMAs.
 // BURST: the feeder fetches W.x in bursts of several iterations (see there); the host asks for it with two row
 // tiles and with one row tile of 8 or 16 rows, for head dims up to 512 (bf16).
-template <bool BF16, int NCH, int MT, bool FULL, bool BURST>
+// FMAC: the contraction of a row tile of at most 4 rows with FMA instructions and a reduction across the wave instead
+// of MFMA (the alternative for small batches; measured, slower at every batch size, so the host never picks it
+// unless the library is built with XS_SMALL_BATCH_FMA for that measurement).  Each lane multiplies its 8 (bf16) or
+// 4 (fp32) inputs of every real row - fetched from the lane that holds them - into its own column's weights, and
+// the four lane groups' partial sums over K are added with two cross-lane steps.  The sums are formed in a different
+// order than the MFMA forms them, so the bits differ from the MFMA path (and from the decode kernel).
+template <bool BF16, int NCH, int MT, bool FULL, bool BURST, bool FMAC = false>
 __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
+  static_assert(!FMAC || MT == 1, "the FMA contraction is for one row tile of at most 4 rows");
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
   constexpr int ESZ = BF16 ? 2 : 4;
@@ -628,6 +635,54 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         XS_TICK(0);
 #pragma unroll
         for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+        if constexpr (FMAC) {
+          float sum[4][4];  // [gate][row]: this lane's column, this lane group's slice of K
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sum[g][r] = 0.0f;
+#pragma unroll
+          for (int c = 0; c < NCH; ++c) {
+            float w[4][EPC];  // the weights of this lane's column
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const uint32_t rw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (BF16) { w[g][2 * e] = bf16_bits_to_float(rw[e] & 0xFFFFu); w[g][2 * e + 1] = __uint_as_float(rw[e] & 0xFFFF0000u); }
+                else w[g][e] = __uint_as_float(rw[e]);
+              }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              if (r >= rend - rowbase) break;  // (wave-uniform: only the rows that exist cost anything)
+              // the inputs of row r for this lane group's slice of K sit in lane 16 q + r
+              const uint32_t hw[4] = {(uint32_t)__shfl((int)op[c].x, (lane & 48) + r), (uint32_t)__shfl((int)op[c].y, (lane & 48) + r),
+                                      (uint32_t)__shfl((int)op[c].z, (lane & 48) + r), (uint32_t)__shfl((int)op[c].w, (lane & 48) + r)};
+              float hx[EPC];
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                if (BF16) { hx[2 * e] = bf16_bits_to_float(hw[e] & 0xFFFFu); hx[2 * e + 1] = __uint_as_float(hw[e] & 0xFFFF0000u); }
+                else hx[e] = __uint_as_float(hw[e]);
+              }
+#pragma unroll
+              for (int g = 0; g < 4; ++g)
+#pragma unroll
+                for (int e = 0; e < EPC; ++e) sum[g][r] = fmaf(hx[e], w[g][e], sum[g][r]);
+            }
+          }
+          // add the four lane groups' slices; the result tile keeps the MFMA's layout (rows 4q .. 4q+3 of column r16)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              float v = sum[g][r];
+              v += __shfl_xor(v, 16);
+              v += __shfl_xor(v, 32);
+              acc[g][r] = q == 0 ? v : 0.0f;
+            }
+          return;
+        }
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
           if (BF16) {
