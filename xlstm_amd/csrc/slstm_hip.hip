@@ -29,6 +29,7 @@
 
 #include "slstm_device_common.h"
 #include "slstm_seq_kernel.h"
+#include "slstm_seq_roles_kernel.h"
 #include "slstm_step_kernel.h"
 #include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
@@ -74,6 +75,17 @@ SeqKernel pick_mt(int MT, bool burst) {
     case 1: return (burst && NCH <= 4) ? slstm_seq_kernel<BF16, NCH, 1, FULL, NCH <= 4> : slstm_seq_kernel<BF16, NCH, 1, FULL, false>;
     case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL, NCH <= 4>;
     case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL, false>;
+    default: return nullptr;
+  }
+}
+
+template <bool BF16, bool FULL>
+SeqKernel pick_roles_kernel(int nch) {
+  switch (nch) {
+    case 1: return slstm_seq_roles_kernel<BF16, 1, FULL>;
+    case 2: return slstm_seq_roles_kernel<BF16, 2, FULL>;
+    case 4: return slstm_seq_roles_kernel<BF16, 4, FULL>;
+    case 8: return slstm_seq_roles_kernel<BF16, 8, FULL>;
     default: return nullptr;
   }
 }
@@ -296,6 +308,11 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
       else kern = nch == 1 ? slstm_seq_kernel<false, 1, 1, true, false, true> : slstm_seq_kernel<false, 2, 1, true, false, true>;
     }
 #endif
+    // four row tiles per workgroup: the kernel with MFMA waves and gating waves
+    const bool roles = MT == 4 && !getenv("XS_NO_ROLES");
+    if (roles)
+      kern = bf16 ? (full ? pick_roles_kernel<true, true>(nch) : pick_roles_kernel<true, false>(nch))
+                  : (full ? pick_roles_kernel<false, true>(nch) : pick_roles_kernel<false, false>(nch));
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NHL * NBT;
@@ -344,7 +361,7 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
       const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), dyn_lds);
       if (rc != XS_OK) return rc;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(kThreads + 64 * p.prefetch), dyn_lds, stream, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(roles ? kRolesThreads : kThreads + 64 * p.prefetch), dyn_lds, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
   }

@@ -84,6 +84,64 @@ __device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_
                :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
 }
 
+// ---- role of a workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8; a head group takes consecutive slots of
+//      ONE XCD so its exchange stays in one L2): head group index and position inside the group
+__device__ __forceinline__ void seq_place(const SeqParams &p, int wg, int &gi, int &member) {
+  if (p.G <= 32) {
+    const int xcd = wg & 7;
+    const int local = wg >> 3;
+    const int slot = local / p.G;
+    member = local - slot * p.G;
+    gi = slot * 8 + xcd;
+  } else if (p.G <= 64 && (p.G & 1) == 0) {
+    // two XCDs per group (workgroup i runs on XCD i % 8): members 0 .. G/2-1 on the even XCD of a
+    // pair, the rest on the odd one, so that half of a member's polls stay inside its own L2
+    const int xcd = wg & 7;
+    const int local = wg >> 3;
+    const int half = p.G >> 1;
+    const int slot = local / half;
+    member = (xcd & 1) * half + (local - slot * half);
+    gi = slot * 4 + (xcd >> 1);
+  } else {  // larger groups are spread over all XCDs
+    gi = wg / p.G;
+    member = wg - gi * p.G;
+  }
+}
+
+// ---- placement handshake (one thread of the workgroup): do all members of this head group share one XCD (one L2)?
+//      If so h is published with plain stores (they land in that L2); otherwise with device-scope stores that are
+//      written through to memory.  Returns 1 for "more than one XCD".
+__device__ __forceinline__ uint32_t seq_handshake(const SeqParams &p, int wg, int gi, long long spin_limit) {
+  const bool one_xcd_layout = p.G <= 32;
+  if (wg == 0) atomicAdd(&p.status->launches, 1u);  // a long batch is run as several launches of row chunks
+  const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
+  __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
+                     __HIP_MEMORY_SCOPE_AGENT);
+  uint32_t cross = one_xcd_layout ? 0u : 1u;
+  if (one_xcd_layout) {
+    const int xcd = wg & 7;
+    const int slot = (wg >> 3) / p.G;
+    for (int j = 0; j < p.G; ++j) {
+      const int peer = ((slot * p.G + j) << 3) | xcd;
+      uint32_t w = 0;
+      long long spins = 0;
+      while (((w = __hip_atomic_load(&p.wg_xcc[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & 0x80000000u) == 0u) {
+        if (++spins >= spin_limit) {  // a peer never started: the grid is not co-resident
+          if (atomicExch(&p.status->aborted, 1u) == 0u) {
+            p.status->abort_wg = (uint32_t)wg;
+            p.status->abort_step = 0xFFFFFFFFu;
+          }
+          cross = 1u;
+          break;
+        }
+      }
+      if ((w & 0xFu) != my_xcc) cross = 1u;
+    }
+    if (cross) atomicAdd(&p.status->xcd_mixed, 1u);
+  }
+  return cross;
+}
+
 // FULL: the head dim fills the K range of the four waves exactly (dh == 16 * NCH * elements per chunk) and, with
 // more than one row tile, every batch row of every tile exists.  The per-chunk "is this chunk needed" masks of
 // the arrival test are then compiled out (with one row tile, lanes of rows that do not exist read zeros from
@@ -130,31 +188,11 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   __shared__ uint32_t cross_s;
   __shared__ uint32_t pubflag[4];               // [compute wave] iterations whose h is staged in hst
 
-  // ---- role of this workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8,
-  //      a head group takes consecutive slots of ONE XCD so its exchange stays in one L2)
+  // ---- role of this workgroup
   const int wg = blockIdx.x;
   const int ngroups = p.NHL * p.NBT;
   int gi, member;  // head group index, position inside the group
-  const bool one_xcd_layout = p.G <= 32;
-  if (one_xcd_layout) {
-    const int xcd = wg & 7;
-    const int local = wg >> 3;
-    const int slot = local / p.G;
-    member = local - slot * p.G;
-    gi = slot * 8 + xcd;
-  } else if (p.G <= 64 && (p.G & 1) == 0) {
-    // two XCDs per group (workgroup i runs on XCD i % 8): members 0 .. G/2-1 on the even XCD of a
-    // pair, the rest on the odd one, so that half of a member's polls stay inside its own L2
-    const int xcd = wg & 7;
-    const int local = wg >> 3;
-    const int half = p.G >> 1;
-    const int slot = local / half;
-    member = (xcd & 1) * half + (local - slot * half);
-    gi = slot * 4 + (xcd >> 1);
-  } else {  // larger groups are spread over all XCDs
-    gi = wg / p.G;
-    member = wg - gi * p.G;
-  }
+  seq_place(p, wg, gi, member);
   if (gi >= ngroups) return;
   const int head = p.head0 + gi / p.NBT;
   const int bt = gi % p.NBT;
@@ -164,38 +202,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const int lane = tid & 63;
   const long long spin_limit = p.spin_limit > 0 ? p.spin_limit : kDefaultSpinLimit;
 
-  // ---- placement handshake: do all members of this head group share one XCD (one L2)?
-  //      If so h is published with plain stores (they land in that L2); otherwise with
-  //      device-scope stores that are written through to memory.
-  if (tid == 0) {
-    if (wg == 0) atomicAdd(&p.status->launches, 1u);  // a long batch is run as several launches of row chunks
-    const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
-    __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
-                       __HIP_MEMORY_SCOPE_AGENT);
-    uint32_t cross = one_xcd_layout ? 0u : 1u;
-    if (one_xcd_layout) {
-      const int xcd = wg & 7;
-      const int slot = (wg >> 3) / p.G;
-      for (int j = 0; j < p.G; ++j) {
-        const int peer = ((slot * p.G + j) << 3) | xcd;
-        uint32_t w = 0;
-        long long spins = 0;
-        while (((w = __hip_atomic_load(&p.wg_xcc[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) & 0x80000000u) == 0u) {
-          if (++spins >= spin_limit) {  // a peer never started: the grid is not co-resident
-            if (atomicExch(&p.status->aborted, 1u) == 0u) {
-              p.status->abort_wg = (uint32_t)wg;
-              p.status->abort_step = 0xFFFFFFFFu;
-            }
-            cross = 1u;
-            break;
-          }
-        }
-        if ((w & 0xFu) != my_xcc) cross = 1u;
-      }
-      if (cross) atomicAdd(&p.status->xcd_mixed, 1u);
-    }
-    cross_s = cross;
-  }
+  if (tid == 0) cross_s = seq_handshake(p, wg, gi, spin_limit);
   if (tid < 4) pubflag[tid] = 0u;
 
   const int dh = p.dh;
