@@ -399,7 +399,7 @@ def main():
         c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=max(1, min(args.steps, 5)))
         c5["roofline"] = {"bound": "mfma", "achieved": c5["tflops"], "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                           "frac": c5["tflops"] / MFMA_BF16_PEAK_TFLOPS, "traffic": None,
-                          "kernel": "slstm_seq_kernel<bf16,NCH=8,MT=4,FULL,BURST=0>",
+                          "kernel": "slstm_seq_roles_kernel<bf16,NCH=8,FULL>",
                           "algorithmic_flops_per_launch": 8.0 * 64 * 4096 * 4096 * 1024}
         print(json.dumps({"config5": c5}))
         return

@@ -74,7 +74,6 @@ SeqKernel pick_mt(int MT, bool burst) {
   switch (MT) {
     case 1: return (burst && NCH <= 4) ? slstm_seq_kernel<BF16, NCH, 1, FULL, NCH <= 4> : slstm_seq_kernel<BF16, NCH, 1, FULL, false>;
     case 2: return slstm_seq_kernel<BF16, NCH, 2, FULL, NCH <= 4>;
-    case 4: return slstm_seq_kernel<BF16, NCH, 4, FULL, false>;
     default: return nullptr;
   }
 }
@@ -299,8 +298,16 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
     const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
     // the feeder fetches W.x in bursts where the prefetch waves cannot cover it: row tiles of 8 rows or more
     const bool burst = rows_per_wg >= 8;
-    SeqKernel kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
-                          : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
+    // four row tiles per workgroup: the kernel with MFMA waves and gating waves; one or two: the kernel in which
+    // every compute wave does both
+    const bool roles = MT == 4;
+    SeqKernel kern;
+    if (roles)
+      kern = bf16 ? (full ? pick_roles_kernel<true, true>(nch) : pick_roles_kernel<true, false>(nch))
+                  : (full ? pick_roles_kernel<false, true>(nch) : pick_roles_kernel<false, false>(nch));
+    else
+      kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
+                  : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
 #ifdef XS_SMALL_BATCH_FMA
     // the measured alternative for small batches (see the kernel): only in a library built for that measurement
     if (MT == 1 && rows_per_wg == 4 && nch <= 2 && full) {
@@ -308,11 +315,6 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
       else kern = nch == 1 ? slstm_seq_kernel<false, 1, 1, true, false, true> : slstm_seq_kernel<false, 2, 1, true, false, true>;
     }
 #endif
-    // four row tiles per workgroup: the kernel with MFMA waves and gating waves
-    const bool roles = MT == 4 && !getenv("XS_NO_ROLES");
-    if (roles)
-      kern = bf16 ? (full ? pick_roles_kernel<true, true>(nch) : pick_roles_kernel<true, false>(nch))
-                  : (full ? pick_roles_kernel<false, true>(nch) : pick_roles_kernel<false, false>(nch));
     if (!kern) return fail(XS_ERR_UNSUPPORTED, "no kernel for nch=%d MT=%d", nch, MT);
     const int NBT = (bend - b0 + rows_per_wg - 1) / rows_per_wg;
     const int ngroups = NHL * NBT;
@@ -355,13 +357,7 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
       const int want = (rows_in_tile * (bf16 ? 2 : 4) + 7) / 8;
       p.prefetch = want <= max_prefetch_waves(nch) ? want : 0;
     }
-    // with four row tiles the polled tiles are staged in dynamic LDS: [2][4 waves][nch] KiB
-    const size_t dyn_lds = MT >= 4 ? (size_t)nch * 8192 : 0;
-    if (dyn_lds) {
-      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), dyn_lds);
-      if (rc != XS_OK) return rc;
-    }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(roles ? kRolesThreads : kThreads + 64 * p.prefetch), dyn_lds, stream, p);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(roles ? kRolesThreads : kThreads + 64 * p.prefetch), 0, stream, p);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "sequence kernel launch failed: %s", hipGetErrorString(e));
   }

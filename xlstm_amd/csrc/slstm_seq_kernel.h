@@ -75,15 +75,6 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint32_t uniform(uint32_t v) { return __builtin_amdgcn_readfirstlane(v); }
 
-// 16 bytes per lane from a buffer straight into LDS (no registers): lane i's bytes land at
-// lds_addr + 16 * i.  Issued as inline assembly on purpose: the compiler then knows nothing of
-// these loads, and the waits for them are written by hand with exact counts (s_waitcnt vmcnt).
-// rsrc and lds_addr must be wave-uniform values (see uniform()).
-__device__ __forceinline__ void lds_direct_load_b128(u32x4_t rsrc, uint32_t lds_addr, int voffset, int soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen sc1 lds"
-               :: "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset) : "memory", "m0");
-}
-
 // ---- role of a workgroup (XCD-aware: workgroup i is dispatched to XCD i % 8; a head group takes consecutive slots of
 //      ONE XCD so its exchange stays in one L2): head group index and position inside the group
 __device__ __forceinline__ void seq_place(const SeqParams &p, int wg, int &gi, int &member) {
@@ -163,30 +154,13 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int WCH = 16 / EPC;          // 16-byte chunks holding the 16 units of one (row, gate)
   constexpr int ROWS = 16 * MT;          // batch rows of a workgroup
-  // With four row tiles a tile is polled by the peers three iterations after it was computed, so
-  // it can leave through the drainer wave (two iterations late) and the compute waves issue no
-  // stores at all: their waits for poll data then never include a store acknowledgement (loads
-  // and stores share one counter and complete out of order with each other).
-  constexpr bool kDrainerPublishes = MT >= 4;
-  // ... and the polls of a tile are then issued TWO iterations ahead, straight into LDS (dynamic
-  // shared memory, [2][compute wave][NCH][lane] 16-byte pieces), because the load latency of a
-  // freshly published tile (about 3000 to 5000 cycles) is longer than one iteration.
-  constexpr bool kDeepPrefetch = kDrainerPublishes;
-  // Where in an iteration those requests are issued.  Four waves x NCH loads of 1 KiB each keep the compute unit's
-  // one address path busy for up to some 500 cycles, and a wave that issues into a full queue stalls.  Right behind
-  // the MFMAs (where the LDS slot has just been read) that stall sits in front of the partial sums and the barrier,
-  // on the critical path of all four waves; behind the gating it does not.  Measured, bf16: dh 1024 20.8 -> 17.2 ms
-  // (BASELINE config 5), dh 512 3.93 -> 3.50 us per step; dh 256 and the variants with a K tail 1 to 3 % slower,
-  // so those keep the early place.  A tile requested there still has a whole iteration to arrive.
-  constexpr bool kLateRequests = NCH >= 4 && FULL;
-  extern __shared__ __attribute__((aligned(16))) unsigned char seq_dyn_lds[];
+  static_assert(MT == 1 || MT == 2, "workgroups of four row tiles run slstm_seq_roles_kernel");
 
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
   __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
   __shared__ float hst[4][256];                 // [slot][row*16 + unit]             h on its way to HBM
   __shared__ uint32_t rfl[4][16];               // [slot][row]                       reset flags
   __shared__ uint32_t cross_s;
-  __shared__ uint32_t pubflag[4];               // [compute wave] iterations whose h is staged in hst
 
   // ---- role of this workgroup
   const int wg = blockIdx.x;
@@ -203,7 +177,6 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const long long spin_limit = p.spin_limit > 0 ? p.spin_limit : kDefaultSpinLimit;
 
   if (tid == 0) cross_s = seq_handshake(p, wg, gi, spin_limit);
-  if (tid < 4) pubflag[tid] = 0u;
 
   const int dh = p.dh;
   const int H = p.NH * dh;
@@ -337,49 +310,16 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   // =========================================================================
   // wave 5: drainer.  h of iteration it is staged in LDS by the compute waves
   // between barriers #it and #it+1; it is written to HBM two iterations later
-  // (with four row tiles: as soon as it is staged, together with the publication
-  // of the tile in the exchange ring).
   // =========================================================================
   if (wave == 5) {
     const int drow = lane >> 2;   // batch row inside the tile
     const int dq = lane & 3;      // which 4 of the 16 units
-    bool dcross = false;
-    auto drain = [&](int it, bool publish, bool poison = false) {
+    auto drain = [&](int it, bool poison = false) {
       const int t = it / MT;
       const int mt = it - t * MT;
       const int brow = rowbase + mt * 16 + drow;
       f32x4 v = *reinterpret_cast<const f32x4 *>(&hst[it & 3][drow * 16 + dq * 4]);
       if (poison) v = f32x4{kPoison, kPoison, kPoison, kPoison};
-      if (kDrainerPublishes && publish) {
-        // h_t of this tile goes to the exchange ring from here, and the words of h_{t-2} are re-armed,
-        // so the compute waves wait on nothing but their polls.  Every lane stores: words outside
-        // the batch or the head belong to this member's block and are never polled.
-        constexpr int TB = 16 * 16 * ESZ;  // one member's tile; a ring slot is [row tile][member][16 rows][16 units]
-        const int xsl = p.G * MT * TB;
-        char *const blk = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xsl + ((long long)mt * p.G + member) * TB +
-                          (drow * 16 + dq * 4) * ESZ;
-        unsigned long long *cur = reinterpret_cast<unsigned long long *>(blk + (t % kRing) * xsl);
-        unsigned long long *old = reinterpret_cast<unsigned long long *>(blk + ((t + kRing - 2) % kRing) * xsl);
-        unsigned long long w0, w1 = 0;
-        if (BF16) {
-          w0 = (unsigned long long)(float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16)) |
-               ((unsigned long long)(float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16)) << 32);
-        } else {
-          w0 = (unsigned long long)__float_as_uint(v[0]) | ((unsigned long long)__float_as_uint(v[1]) << 32);
-          w1 = (unsigned long long)__float_as_uint(v[2]) | ((unsigned long long)__float_as_uint(v[3]) << 32);
-        }
-        if (dcross) {
-          __hip_atomic_store(cur, w0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (!BF16) __hip_atomic_store(cur + 1, w1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(old, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (!BF16) __hip_atomic_store(old + 1, ~0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-          cur[0] = w0;
-          if (!BF16) cur[1] = w1;
-          old[0] = ~0ull;
-          if (!BF16) old[1] = ~0ull;
-        }
-      }
       if (brow < rend && a0 + dq * 4 < dh) {
         const long long o = (long long)t * BH + (long long)brow * H + head * dh + a0 + dq * 4;
         if (BF16) {
@@ -393,48 +333,12 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       }
     };
     lds_barrier();  // prologue barrier
-    dcross = cross_s != 0u;
 #ifdef XS_PROFILE
     long long dprof[2] = {0, 0};
     long long dt = clock64();
 #endif
-    if (kDrainerPublishes) {
-      // iteration j leaves as soon as the four compute waves have staged it (they raise their
-      // counters after the LDS write): the peers fetch a tile two iterations before they use it
-      bool gave_up = false;
-      for (int j = 0; j < NITpad; ++j) {
-        lds_barrier();  // barrier #j
-#ifdef XS_PROFILE
-        { const long long now_ = clock64(); dprof[1] += now_ - dt; dt = now_; }
-#endif
-        if (j < NIT) {
-          long long spins = 0;
-          while (!gave_up) {
-            const uint32_t want = (uint32_t)j + 1u;
-            const uint32_t f0 = __hip_atomic_load(&pubflag[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            const uint32_t f1 = __hip_atomic_load(&pubflag[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            const uint32_t f2 = __hip_atomic_load(&pubflag[2], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            const uint32_t f3 = __hip_atomic_load(&pubflag[3], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (f0 >= want && f1 >= want && f2 >= want && f3 >= want) break;
-            __builtin_amdgcn_s_sleep(1);
-            if (++spins >= spin_limit) {  // cannot happen while the compute waves run; never wait forever
-              gave_up = true;
-              if (lane == 0 && atomicExch(&p.status->aborted, 1u) == 0u) {
-                p.status->abort_wg = (uint32_t)wg;
-                p.status->abort_step = (uint32_t)(j / MT);
-              }
-            }
-          }
-          drain(j, true);
-        }
-#ifdef XS_PROFILE
-        { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
-#endif
-      }
-      lds_barrier();  // final barrier
-    } else {
     for (int j = 0; j < NITpad; ++j) {
-      if (j >= 2 && j - 2 < NIT) drain(j - 2, true);
+      if (j >= 2 && j - 2 < NIT) drain(j - 2);
 #ifdef XS_PROFILE
       { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
 #endif
@@ -444,14 +348,13 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #endif
     }
     lds_barrier();  // final barrier
-    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it, false);
-    }
+    for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it);
     // A bounded wait ran out somewhere: whatever this workgroup computed from then on is built on operands that
     // never arrived.  A caller that does not read the status block must not mistake it for a result, so the
     // workgroup's part of h_out becomes NaN (the compute waves do the same to s_out).  Any workgroup that consumed
     // such operands did so after the flag was raised, and looks at the flag here, later still.
     if (__hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u)
-      for (int it = 0; it < NIT; ++it) drain(it, false, true);
+      for (int it = 0; it < NIT; ++it) drain(it, true);
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
@@ -590,8 +493,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   //   MT == 2  the polls of the NEXT (t, mt) iteration are issued right after the MFMAs of the
   //            current one have consumed the operand registers (the peers published that tile one
   //            iteration ago);
-  //   MT == 4  the tile of iteration it + 2 is requested straight into LDS (kDeepPrefetch).
-  // The completion test, the re-arm and their order are the same in all three.
+  // The completion test, the re-arm and their order are the same in both.
   uint4 areg[NCH];
   bool prefetched = false;
   // poll address of chunk c of row tile mt = per-lane part (one register) + a compile-time constant:
@@ -599,7 +501,6 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const int xlane = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
   const int xtile_stride = p.G * XTILE;
   auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
-  auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
     // (the descriptor ends with the slot: a chunk past the last member reads zeros)
@@ -732,19 +633,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
           multiplied = true;
         }
       } else {
-        if (kDeepPrefetch) {
-          // this tile was requested two iterations ago; the only younger requests are the NCH of the next tile
-#ifdef XS_PROFILE
-          const long long w0_ = clock64();
-#endif
-          if (it + 1 < NIT) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NCH) : "memory");
-          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#ifdef XS_PROFILE
-          prof[7] += clock64() - w0_;
-#endif
-#pragma unroll
-          for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
-        } else if (MT == 1) {
+        if (MT == 1) {
           // ONE poll in flight, re-issued when it comes back incomplete.  With W.x out of the way of the polls
           // (prefetch waves) a poll takes 200 to 300 cycles and finds everything in place in 92 % of the steps:
           // the peers' h is in the L2 before this wave's own loop has come round.  A second poll half a round
@@ -802,8 +691,6 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
               areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
           }
         }
-        // (tiles fetched ahead through LDS are checked once outside the loop: inside it the wave
-        // waits for ALL of its outstanding loads, the next tile's requests included)
         // first look at everything at once: one mark over all chunks this lane needs
         uint32_t mark = 0u;
         if (MT != 1) {  // (with one row tile the loop above has seen a complete set, or given up)
@@ -865,22 +752,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         multiply(areg);
       }
 
-      auto issue_requests = [&]() {
-        // request the tile of iteration it + 2 (its LDS slot is the one just read); step 0 takes its
-        // operand from s0.  A chunk past the last member reads zeros (the descriptor ends with the slot).
-        const int nmt = (mt + 2) % MT;
-        const int nt = t + (mt + 2 >= MT ? 1 : 0);
-        if (nt >= 1 && nt < p.T) {
-          const unsigned long long sb = reinterpret_cast<unsigned long long>(xbase + ((nt + kRing - 1) % kRing) * xslot);
-          const u32x4_t rs = {uniform((uint32_t)sb), uniform((uint32_t)(sb >> 32) & 0xFFFFu), uniform((uint32_t)xslot), 0x00020000u};
-          const uint32_t lds0 = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(it, 0)));
-#pragma unroll
-          for (int c = 0; c < NCH; ++c) lds_direct_load_b128(rs, lds0 + (c << 10), xlane, xconst(c, nmt));
-        }
-      };
-      if (kDeepPrefetch) {
-        if (!kLateRequests) issue_requests();
-      } else if (MT > 1) {
+      if (MT > 1) {
         // early polls of the next iteration's tile (see above); step 0 takes its operand from s0
         const int nmt = (mt + 1) % MT;
         const int nt = t + (mt + 1 == MT ? 1 : 0);
@@ -922,42 +794,36 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #ifdef XS_PROFILE
       asm volatile("" :: "v"(st[mt].y));
 #endif
-      if (kDeepPrefetch && kLateRequests) issue_requests();
       XS_TICK(3);
       // ---- 5. publish h_t to the peers, re-arm the words of h_{t-2}, stage h_t for the drainer
       float y = st[mt].y;
       if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
-      // (With four row tiles the drainer wave publishes: see there.)  Every lane stores, every
-      // iteration: lanes outside the batch or the head write words of their own block that nobody
-      // polls, and the re-arm of steps 0 and 1 hits slots that still hold the pattern.
-      if (!kDrainerPublishes) {
-        const long long xo = ((long long)mt * p.G + member) * (XTILE / ESZ) + pb * 16 + pa;
-        if (BF16) {
-          const uint16_t v = (uint16_t)float_to_bf16_bits(y);
-          uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
-          uint16_t *old = reinterpret_cast<uint16_t *>(hold) + xo;
-          if (cross) {
-            __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          } else {
-            *dst = v;
-            *old = (uint16_t)kSentinel16;
-          }
+      // Every lane stores, every iteration: lanes outside the batch or the head write words of their own
+      // block that nobody polls, and the re-arm of steps 0 and 1 hits slots that still hold the pattern.
+      const long long xo = ((long long)mt * p.G + member) * (XTILE / ESZ) + pb * 16 + pa;
+      if (BF16) {
+        const uint16_t v = (uint16_t)float_to_bf16_bits(y);
+        uint16_t *dst = reinterpret_cast<uint16_t *>(hcur) + xo;
+        uint16_t *old = reinterpret_cast<uint16_t *>(hold) + xo;
+        if (cross) {
+          __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(old, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         } else {
-          float *dst = reinterpret_cast<float *>(hcur) + xo;
-          float *old = reinterpret_cast<float *>(hold) + xo;
-          if (cross) {
-            __hip_atomic_store(dst, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          } else {
-            *dst = y;
-            *old = __uint_as_float(kSentinel32);
-          }
+          *dst = v;
+          *old = (uint16_t)kSentinel16;
+        }
+      } else {
+        float *dst = reinterpret_cast<float *>(hcur) + xo;
+        float *old = reinterpret_cast<float *>(hold) + xo;
+        if (cross) {
+          __hip_atomic_store(dst, y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(old, __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          *dst = y;
+          *old = __uint_as_float(kSentinel32);
         }
       }
       hst[it & 3][tid] = y;
-      if (kDrainerPublishes && lane == 0)
-        __hip_atomic_store(&pubflag[wave], (uint32_t)it + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (MT == 1) {
         // (the operand registers stay reserved to the end of the iteration: measured as fast or faster)
 #pragma unroll

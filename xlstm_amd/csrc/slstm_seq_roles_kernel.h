@@ -11,9 +11,11 @@ namespace {
 // the time.  Here the chain is cut in two and the halves of consecutive iterations run side by side, two waves per
 // SIMD:
 //
-//   waves 0-3  MFMA waves (K quarter = wave; their 64 columns of R in registers).  Per iteration: the operand tile
-//              (requested one iteration ahead straight into LDS) out of LDS, arrival test, 32 MFMAs, partial sums to
-//              LDS, barrier, request for the tile after next.  No stores, no W.x, no gating.
+//   waves 0-3  MFMA waves (K quarter = wave; their 64 columns of R in registers).  A wave fetches its piece of the next
+//              operand tile one iteration ahead straight into a second set of registers: ordinary loads that the
+//              compiler tracks, issued right behind the wait for the current tile, so that this wait (the only one
+//              in these waves, which issue no stores) never covers them.  Per iteration: arrival test, 32 MFMAs,
+//              partial sums to LDS, barrier.  No W.x, no gating, no LDS round trip for the operands.
 //   waves 4-7  gating waves (rows 4 (wave - 4) .. + 3 of every tile, one element per lane).  Per iteration: barrier,
 //              partial sums out of LDS, exponential gating, h to the exchange ring and to the output tensor.  They
 //              fetch their own W.x and reset flags straight from memory into a ring of registers, eight iterations
@@ -27,13 +29,14 @@ constexpr int kRolesThreads = 512;
 template <bool BF16, int NCH, bool FULL>
 __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParams p) {
   constexpr int MT = 4;
+  constexpr int NMW = 4;                 // MFMA waves
+  constexpr int CPW = NCH;               // 16-byte chunks of an operand row per lane and MFMA wave
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
-  constexpr int KW = NCH * 4 * EPC;      // input units per MFMA wave
+  constexpr int KW = CPW * 4 * EPC;      // input units per MFMA wave
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int D = 8;                   // iterations the gating waves fetch W.x ahead (a ring of registers)
-  extern __shared__ __attribute__((aligned(16))) unsigned char seq_dyn_lds[];  // [2][MFMA wave][NCH] KiB: operand tiles
+  __shared__ float part[2][NMW][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
 
-  __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
   __shared__ uint32_t rfl[4][16];               // [slot][row] reset flags, written two iterations ahead by the gating waves
   __shared__ uint32_t cross_s;
 
@@ -60,13 +63,13 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
   constexpr int XTILE = 16 * 16 * ESZ;               // bytes one member publishes per row tile
   const int xslot = p.G * MT * XTILE;                // bytes one group publishes per step
   char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
-  if (wave < 4) __builtin_amdgcn_s_setprio(3);
+  if (wave < NMW) __builtin_amdgcn_s_setprio(3);
 
-  if (wave >= 4) {
+  if (wave >= NMW) {
     // =====================================================================
     // gating waves
     // =====================================================================
-    const int pel = (wave - 4) * 64 + lane;  // element inside a tile: row * 16 + unit
+    const int pel = (wave - NMW) * 64 + lane;  // element inside a tile: row * 16 + unit
     const int pa = pel & 15, pb = pel >> 4;
     const int ua = a0 + pa;
     const bool unit_ok = ua < dh;
@@ -205,8 +208,8 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
       }
     }
 #ifdef XS_PROFILE
-    if (lane == 0 && member == 0 && gi == 0 && wave == 4) {
-      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 4 * 8;
+    if (lane == 0 && member == 0 && gi == 0 && wave == NMW) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
       for (int i = 0; i < 4; ++i) dst[i] = gprof[i];
     }
 #endif
@@ -238,13 +241,13 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
   const int q = lane >> 4;     // lane group: which 16-byte chunk of a 4-chunk K slab
   const int r16 = lane & 15;   // MFMA row (A) / column (B, C)
   // ---- R slice -> registers (once).  B operand: column n = unit a0 + r16 of gate g, K chunk c of this wave / lane group.
-  uint4 rreg[4][NCH];
+  uint4 rreg[4][CPW];
   {
     const int a = a0 + r16;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
+      for (int c = 0; c < CPW; ++c) {
         const int k0 = wave * KW + c * 4 * EPC + q * EPC;
         uint4 v = make_uint4(0, 0, 0, 0);
         if (a < dh && k0 < dh) {
@@ -267,37 +270,40 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
     }
   }
   // (R has landed before the first hand-issued request goes out: the counts below are of hand-issued loads only)
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#pragma unroll
+  for (int g = 0; g < 4; ++g)
+#pragma unroll
+    for (int c = 0; c < CPW; ++c)
+      asm volatile("s_waitcnt vmcnt(0)" : "+v"(rreg[g][c].x), "+v"(rreg[g][c].y), "+v"(rreg[g][c].z), "+v"(rreg[g][c].w) :: "memory");
   bool aborted = false;
   uint32_t max_spins = 0;
   lds_barrier();  // prologue barrier: the reset flags of iterations 0 and 1 and the placement verdict are in LDS
 
   // poll address of chunk c of row tile mt = per-lane part + a compile-time constant: unit k of row r of row tile mt
-  // lives at [mt][member k/16][r][k%16]
-  const int xlane = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
+  // lives at [mt][member k/16][r][k%16].  Lanes whose batch row does not exist ask for an offset past the descriptor's
+  // end: zeros, no memory traffic.
+  const int xlane_ok = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
   const int xtile_stride = p.G * XTILE;
   auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
-  auto dma_slot = [&](int itx, int c) { return seq_dyn_lds + ((((itx & 1) * 4 + wave) * NCH + c) << 10); };
-  // request the tile of iteration itr into the LDS slot itr & 1; step 0 takes its operand from s0.  A chunk past the
-  // last member reads zeros (the descriptor ends with the slot).
-  auto issue_requests = [&](int itr) {
-    const int nt = itr / MT, nmt = itr - nt * MT;
-    if (nt >= 1 && nt < p.T) {
-      const unsigned long long sb = reinterpret_cast<unsigned long long>(xbase + ((nt + kRing - 1) % kRing) * xslot);
-      const u32x4_t rs = {uniform((uint32_t)sb), uniform((uint32_t)(sb >> 32) & 0xFFFFu), uniform((uint32_t)xslot), 0x00020000u};
-      const uint32_t lds0 = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dma_slot(itr, 0)));
+  uint4 aset[2][CPW];  // the operand tile being consumed and the one on its way
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) lds_direct_load_b128(rs, lds0 + (c << 10), xlane, xconst(c, nmt));
-    }
+  for (int s_ = 0; s_ < 2; ++s_)
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) aset[s_][c] = make_uint4(0, 0, 0, 0);
+  // requests the piece of iteration itr's tile this wave multiplies; step 0 takes its operand from s0.
+  // A chunk past the last member reads zeros (the descriptor ends with the slot).
+  auto ring_rsrc = [&](int t_) {
+    return __builtin_amdgcn_make_buffer_rsrc(xbase + ((t_ + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
   };
-  // requests in flight: always exactly those of the tile after the one being consumed (or none)
-  bool next_requested = false;
-  {
-    // tile 1 (iteration 1) before the loop when it comes from the ring; tile 0 of step 0 comes from s0
-    const int nt = 1 / MT;
-    next_requested = nt >= 1 && nt < p.T && 1 < NIT;
-    if (next_requested) issue_requests(1);
-  }
+  auto request = [&](int itr, uint4 (&dst)[CPW]) -> bool {
+    const int nt = itr / MT, nmt = itr - nt * MT;
+    if (!(itr < NIT && nt >= 1)) return false;
+    const __amdgpu_buffer_rsrc_t rs = ring_rsrc(nt);
+    const int xl = (FULL || rowbase + nmt * 16 + r16 < rend) ? xlane_ok : 0x7FFFFF00;
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) dst[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, xl, xconst(c, nmt), 16));
+    return true;
+  };
 #ifdef XS_PROFILE
   long long mprof[6] = {0, 0, 0, 0, 0, 0};
   long long mt_ = clock64();
@@ -305,75 +311,64 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
 #else
 #define XS_MTICK(i) do { } while (0)
 #endif
+  bool next_requested = false;
   int it = 0;
   for (int t = 0; t < p.T; ++t) {
-    const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(
-        xbase + ((t + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt, ++it) {
+      uint4 (&cur)[CPW] = aset[mt & 1];   // (it & 1 == mt & 1)
+      uint4 (&nxt)[CPW] = aset[(mt + 1) & 1];
       // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
       const int arow = rowbase + mt * 16 + r16;
       const bool row_ok = FULL ? true : arow < rend;
       const bool row_reset = rfl[it & 3][r16] != 0u;
-      bool need[NCH];
-      uint4 areg[NCH];
+      bool need[CPW];
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
-        const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-        areg[c] = make_uint4(0, 0, 0, 0);
-        need[c] = FULL ? true : (row_ok && k0 < dh);
-      }
+      for (int c = 0; c < CPW; ++c) need[c] = FULL ? true : (row_ok && wave * KW + c * 4 * EPC + q * EPC < dh);
       XS_MTICK(0);
-      // the tile after this one goes out first: its requests are the only ones younger than this tile's
       const bool this_requested = next_requested;
-      {
-        const int itn = it + 1, nt = itn / MT;
-        next_requested = itn < NIT && nt >= 1 && nt < p.T;
-        if (next_requested) issue_requests(itn);
-      }
-      XS_MTICK(1);
-      if (t == 0) {
+      if (!this_requested) {  // step 0: the operand comes from the initial state (or is zero)
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
+        for (int c = 0; c < CPW; ++c) {
           const int k0 = wave * KW + c * 4 * EPC + q * EPC;
+          uint4 v = make_uint4(0, 0, 0, 0);
           if (need[c] && p.s0) {
             const float *src = p.s0 + (long long)arow * H + head * dh + k0;
             if (BF16) {
               const float4 lo = *reinterpret_cast<const float4 *>(src);
               const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
-              areg[c].x = pack_bf16x2(lo.x, lo.y); areg[c].y = pack_bf16x2(lo.z, lo.w);
-              areg[c].z = pack_bf16x2(hi.x, hi.y); areg[c].w = pack_bf16x2(hi.z, hi.w);
+              v.x = pack_bf16x2(lo.x, lo.y); v.y = pack_bf16x2(lo.z, lo.w);
+              v.z = pack_bf16x2(hi.x, hi.y); v.w = pack_bf16x2(hi.z, hi.w);
             } else {
-              areg[c] = *reinterpret_cast<const uint4 *>(src);
+              v = *reinterpret_cast<const uint4 *>(src);
             }
           }
+          cur[c] = v;
         }
-      } else {
-        (void)this_requested;  // (t >= 1: always requested, one iteration ago)
-        if (next_requested) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(NCH) : "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        XS_MTICK(2);
+      }
+      // this tile's piece, requested one iteration ago, has to be here now (the compiler's wait: nothing younger is in flight) ...
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) areg[c] = *reinterpret_cast<const uint4 *>(dma_slot(it, c) + lane * 16);
+      for (int c = 0; c < CPW; ++c) asm volatile("" : "+v"(cur[c].x), "+v"(cur[c].y), "+v"(cur[c].z), "+v"(cur[c].w));
+      XS_MTICK(2);
+      // ... and the next tile's goes out
+      next_requested = request(it + 1, nxt);
+      XS_MTICK(1);
+      if (this_requested) {
         // one look at everything at once: one mark over all chunks this lane needs
-        uint32_t mark = 0u;
+        auto any_missing = [&]() {
+          uint32_t mark = 0u;
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[c]) & (need[c] ? 0xFFFFFFFFu : 0u));
-        if (!aborted && mark_has_sentinel<BF16>(mark)) {
-          // the tile had not been published completely when it was requested: the ordinary bounded register poll
+          for (int c = 0; c < CPW; ++c)
+            mark = mark_join<BF16>(mark, chunk_mark<BF16>(cur[c]) & (need[c] ? 0xFFFFFFFFu : 0u));
+          return __builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mark)) != 0ull;
+        };
+        if (!aborted && any_missing()) {
+          // the tile had not been published completely when it was requested: poll it again, bounded (behind the next
+          // tile's requests, which are waited for with it)
           uint32_t spins = 0;
-          bool bad[NCH];
-          bool any_bad;
-          auto test_chunks = [&]() {
-            any_bad = false;
-#pragma unroll
-            for (int c = 0; c < NCH; ++c) {
-              bad[c] = need[c] && (BF16 ? chunk_has_sentinel_bf16(areg[c]) : chunk_has_sentinel_f32(areg[c]));
-              any_bad |= bad[c];
-            }
-          };
-          test_chunks();
-          while (any_bad) {
+          const __amdgpu_buffer_rsrc_t rs = ring_rsrc(t);
+          const int xl = row_ok ? xlane_ok : 0x7FFFFF00;
+          for (;;) {
             ++spins;
             if ((spins & 1023u) == 0u &&
                 __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
@@ -389,34 +384,22 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
               break;
             }
 #pragma unroll
-            for (int c = 0; c < NCH; ++c)
-              if (bad[c])
-                areg[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xlane, xconst(c, mt), 16));
-            test_chunks();
+            for (int c = 0; c < CPW; ++c) cur[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, xl, xconst(c, mt), 16));
+            if (!any_missing()) break;
           }
           max_spins = spins > max_spins ? spins : max_spins;
         }
       }
       // ---- 2. partial R.h over this wave's K slab; rows that start a document and chunks that are not needed count as zeros
-      {
-        bool clear_any = row_reset;
+      uint4 areg[CPW];
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) clear_any |= !need[c];
-        if (__builtin_amdgcn_ballot_w64(clear_any) != 0ull) {
-#pragma unroll
-          for (int c = 0; c < NCH; ++c)
-            if (row_reset || !need[c]) areg[c] = make_uint4(0, 0, 0, 0);
-        }
-      }
-#ifdef XS_PROFILE
-      asm volatile("" : "+v"(areg[0].x), "+v"(areg[NCH - 1].w));
-#endif
+      for (int c = 0; c < CPW; ++c) areg[c] = (row_reset || !need[c]) ? make_uint4(0, 0, 0, 0) : cur[c];
       XS_MTICK(3);
       f32x4 acc[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int c = 0; c < NCH; ++c) {
+      for (int c = 0; c < CPW; ++c) {
         if (BF16) {
           const bf16x8 av = __builtin_bit_cast(bf16x8, areg[c]);
 #pragma unroll
@@ -445,7 +428,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
     }
   }
 #ifdef XS_PROFILE
-  if (lane == 0 && member == 0 && gi == 0) {
+  if (lane == 0 && member == 0 && gi == 0 && wave < 4) {
     long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + wave * 8;
     for (int i = 0; i < 6; ++i) dst[i] = mprof[i];
   }
