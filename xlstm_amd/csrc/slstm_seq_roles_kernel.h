@@ -2,6 +2,8 @@
 // Included by slstm_hip.hip only, after slstm_seq_kernel.h (same parameters, same exchange ring, same bits).
 #pragma once
 
+#include <type_traits>
+
 namespace {
 
 // With four row tiles per workgroup a tile is needed by the peers again only four iterations after it was computed, so
@@ -15,12 +17,19 @@ namespace {
 //              operand tile one iteration ahead straight into a second set of registers: ordinary loads that the
 //              compiler tracks, issued right behind the wait for the current tile, so that this wait (the only one
 //              in these waves, which issue no stores) never covers them.  Per iteration: arrival test, 32 MFMAs,
-//              partial sums to LDS, barrier.  No W.x, no gating, no LDS round trip for the operands.
+//              partial sums to LDS, barrier.  No W.x, no gating, no reset flags (a row that starts a document has
+//              its sums discarded by the gating waves: the same +0 as a zero operand row gives).
 //   waves 4-7  gating waves (rows 4 (wave - 4) .. + 3 of every tile, one element per lane).  Per iteration: barrier,
 //              partial sums out of LDS, exponential gating, h to the exchange ring and to the output tensor.  They
 //              fetch their own W.x and reset flags straight from memory into a ring of registers, eight iterations
 //              ahead, with hand-issued loads and hand-counted waits (loads and stores share one counter, and a wait
 //              the compiler places would be a wait for everything).  There is no feeder and no drainer wave.
+//
+// Measured and dropped: the same MFMA loop written by hand, with the loads of the tile TWO iterations on placed between
+// the MFMA groups of the current one (exact hand-counted waits, the texture path busy while the matrix cores work).
+// Bit-identical, and slower everywhere (head dim 1024: 5.4 against 3.5 us per step; 512: 2.8 against 2.5; 256: 5.0
+// against 4.5): twice the operand bytes in flight per compute unit only lengthen the queue that every memory
+// instruction of the compute unit, the gating waves' included, waits in.
 //
 // Barrier #it means "the partial sums of iteration it are in LDS"; the gating waves reach it when they are done with
 // iteration it - 1.  The sums are formed in the same order as everywhere else: the same bits.
@@ -37,7 +46,6 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
   constexpr int D = 8;                   // iterations the gating waves fetch W.x ahead (a ring of registers)
   __shared__ float part[2][NMW][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
 
-  __shared__ uint32_t rfl[4][16];               // [slot][row] reset flags, written two iterations ahead by the gating waves
   __shared__ uint32_t cross_s;
 
   const int wg = blockIdx.x;
@@ -115,23 +123,33 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
       const unsigned char *sf = flagb + (long long)browc * flag_sb + (p.reset ? t : 0);
       asm volatile("global_load_ubyte %0, %1, off" : "=v"(flag) : "v"(sf) : "memory");
     };
+    if (!FULL) {
 #pragma unroll
-    for (int u = 0; u < D; ++u) issue(u, wxr[u], flr[u]);
-    // the flags of iterations 0 and 1 go to LDS before the first barrier (the MFMA waves clear the operand rows of
-    // documents that start); from then on the flag of iteration it + 2 is written during iteration it
-    asm volatile("s_waitcnt vmcnt(%[cnt])" : "+v"(flr[0]), "+v"(flr[1]) : [cnt] "n"(5 * (D - 2)) : "memory");
-    if (pa == 0) {
-      rfl[0][pb] = (rowbase + pb < rend) ? (flr[0] & flag_on) : 0u;
-      rfl[1][pb] = (NIT > 1 && rowbase + 16 + pb < rend) ? (flr[1] & flag_on) : 0u;
+      for (int u = 0; u < D; ++u) issue(u, wxr[u], flr[u]);
     }
-    lds_barrier();  // prologue barrier
-    const bool cross = cross_s != 0u;
+    if (!FULL) lds_barrier();  // prologue barrier (the other loop has its own)
+    bool cross = false;
+    if (!FULL) cross = cross_s != 0u;
 
-    auto gate_tile = [&](int it, int mt, const uint32_t (&wxv)[4], uint32_t flag, uint32_t flag_ahead) {
+#ifdef XS_PROFILE
+    long long gprof[6] = {0, 0, 0, 0, 0, 0};
+    long long gt_ = clock64();
+#define XS_GTICK(i) do { const long long now_ = clock64(); gprof[i] += now_ - gt_; gt_ = now_; } while (0)
+#else
+#define XS_GTICK(i) do { } while (0)
+#endif
+    const __amdgpu_buffer_rsrc_t ring_rs = __builtin_amdgcn_make_buffer_rsrc(xbase, 0, kRing * xslot, 0x00020000);
+    const int lane_ring = member * XTILE + (pb * 16 + pa) * ESZ;
+    const uint32_t lane_h = (uint32_t)((pb * H + pa) * ESZ);
+    char *const h_member = reinterpret_cast<char *>(p.h_out) + (long long)(head * dh + a0) * ESZ;
+    auto gate_tile = [&](int it, int mt, const uint32_t (&wxv)[4], uint32_t flag) {
       const int t = it / MT;
       const int buf = it & 1;
       const int brow = rowbase + mt * 16 + pb;
-      const bool row_ok = brow < rend;
+      const bool row_ok = FULL ? true : brow < rend;
+      const bool lane_ok = FULL ? true : (row_ok && unit_ok);
+      // a row that starts a document: zero state, and R.h counts as the +0 a zero operand row gives
+      const bool restart = row_ok && (flag & flag_on) != 0u;
       float raw[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -140,53 +158,188 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
         ry += part[buf][1][g][pa * kTileStride + pb];
         ry += part[buf][2][g][pa * kTileStride + pb];
         ry += part[buf][3][g][pa * kTileStride + pb];
+        if (restart) ry = 0.0f;
         float wx = BF16 ? bf16_bits_to_float(wxv[g]) : __uint_as_float(wxv[g]);
-        if (!row_ok || !unit_ok) wx = 0.0f;
+        if (!lane_ok) wx = 0.0f;
         raw[g] = (wx + ry) + bias_g[g];
       }
-      if (row_ok && (flag & flag_on) != 0u) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+      if (restart) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+#ifdef XS_PROFILE
+      asm volatile("" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
+      XS_GTICK(4);
+#endif
       slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
+#ifdef XS_PROFILE
+      asm volatile("" : "+v"(st[mt].y));
+      XS_GTICK(5);
+#endif
       // ---- publish h_t to the peers, re-arm the words of h_{t-2}, write h_t to the output tensor.  Every lane stores to
       //      the ring (lanes outside the batch or the head write words of their own block that nobody polls).
       float y = st[mt].y;
       if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
-      char *const blk = xbase + ((long long)mt * p.G + member) * XTILE + (pb * 16 + pa) * ESZ;
-      char *const cur = blk + (t % kRing) * xslot;
-      char *const old = blk + ((t + kRing - 2) % kRing) * xslot;
+      const int tile_off = mt * p.G * XTILE;
+      const int off_cur = (t % kRing) * xslot + tile_off;              // (uniform: scalar offsets of the stores)
+      const int off_old = ((t + kRing - 2) % kRing) * xslot + tile_off;
+      char *const hdst = h_member + ((long long)t * BH + (long long)(rowbase + mt * 16) * H) * ESZ + lane_h;
       if (BF16) {
         const uint16_t v = (uint16_t)float_to_bf16_bits(y);
-        if (cross) {
-          __hip_atomic_store(reinterpret_cast<uint16_t *>(cur), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(reinterpret_cast<uint16_t *>(old), (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (cross) {  // (groups that span two L2s publish past them)
+          __builtin_amdgcn_raw_buffer_store_b16(v, ring_rs, lane_ring, off_cur, 16);
+          __builtin_amdgcn_raw_buffer_store_b16((uint16_t)kSentinel16, ring_rs, lane_ring, off_old, 16);
         } else {
-          *reinterpret_cast<uint16_t *>(cur) = v;
-          *reinterpret_cast<uint16_t *>(old) = (uint16_t)kSentinel16;
+          __builtin_amdgcn_raw_buffer_store_b16(v, ring_rs, lane_ring, off_cur, 0);
+          __builtin_amdgcn_raw_buffer_store_b16((uint16_t)kSentinel16, ring_rs, lane_ring, off_old, 0);
         }
-        if (row_ok && unit_ok)
-          reinterpret_cast<uint16_t *>(p.h_out)[(long long)t * BH + (long long)brow * H + col] = v;
+        if (lane_ok) *reinterpret_cast<uint16_t *>(hdst) = v;
       } else {
         if (cross) {
-          __hip_atomic_store(reinterpret_cast<float *>(cur), y, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          __hip_atomic_store(reinterpret_cast<float *>(old), __uint_as_float(kSentinel32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), ring_rs, lane_ring, off_cur, 16);
+          __builtin_amdgcn_raw_buffer_store_b32(kSentinel32, ring_rs, lane_ring, off_old, 16);
         } else {
-          *reinterpret_cast<float *>(cur) = y;
-          *reinterpret_cast<float *>(old) = __uint_as_float(kSentinel32);
+          __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), ring_rs, lane_ring, off_cur, 0);
+          __builtin_amdgcn_raw_buffer_store_b32(kSentinel32, ring_rs, lane_ring, off_old, 0);
         }
-        if (row_ok && unit_ok)
-          reinterpret_cast<float *>(p.h_out)[(long long)t * BH + (long long)brow * H + col] = y;
+        if (lane_ok) *reinterpret_cast<float *>(hdst) = y;
       }
-      // the reset flags of iteration it + 2 for the MFMA waves
-      const int it2 = it + 2, t2 = it2 / MT, mt2 = it2 - t2 * MT;
-      if (pa == 0) rfl[it2 & 3][pb] = (it2 < NIT && rowbase + mt2 * 16 + pb < rend) ? (flag_ahead & flag_on) : 0u;
     };
 
+    if constexpr (FULL) {
+      // ---- Every row and unit exists.  An address is then a per-lane 32-bit offset, set up once, on top of a base
+      //      that the scalar unit steps, and W.x of an iteration takes ONE load per wave: lane l fetches units
+      //      4 (l & 3) .. + 3 of gate (l >> 2) & 3 for row l >> 4 of the wave's four rows.  The pieces go through a
+      //      private corner of LDS to the lanes that gate them (same wave: no barrier, LDS keeps a wave's order).
+      constexpr int WB = 4 * ESZ;                 // bytes a lane fetches
+      constexpr int NW = WB / 4;                  // ... in registers
+      typedef uint32_t wxq_t __attribute__((ext_vector_type(NW)));
+      typedef typename std::conditional<BF16, uint16_t, uint32_t>::type wxe_t;
+      __shared__ __attribute__((aligned(16))) wxe_t wxt[4][16][16];  // [gating wave][row * 4 + gate][unit]
+      const int gw = wave - NMW;
+      const uint32_t lane_wxq =
+          (uint32_t)(((long long)(4 * gw + (lane >> 4)) * p.wx_sb + (long long)((lane >> 2) & 3) * H + 4 * (lane & 3)) * ESZ);
+      const uint32_t lane_flagq = (uint32_t)((long long)pb * flag_sb);
+      const char *const wx_member = wxb + (long long)(head * dh + a0) * ESZ;
+      wxq_t wxq[D];
+      uint32_t flq[D];
+      // the bases of the D / MT steps an outer round fetches for (clamped to the last step: what the rounds past the
+      // end fetch is never looked at), as offsets the scalar unit adds per iteration
+      long long pf_wx[D / MT], pf_flag[D / MT];
+      auto set_prefetch_steps = [&](int tfirst) {
+#pragma unroll
+        for (int d = 0; d < D / MT; ++d) {
+          const int tp = tfirst + d < p.T ? tfirst + d : p.T - 1;
+          pf_wx[d] = (long long)tp * p.wx_st * ESZ;
+          pf_flag[d] = p.reset ? tp : 0;
+        }
+      };
+      auto fetch = [&](int u, wxq_t &dst, uint32_t &flag) {  // iteration (round, u): step u / MT of the round, row tile u % MT
+        const int mt = u % MT;
+        const char *src = wx_member + (long long)(rowbase + mt * 16) * p.wx_sb * ESZ + pf_wx[u / MT];
+        const unsigned char *sf = flagb + (long long)(rowbase + mt * 16) * flag_sb + pf_flag[u / MT];
+        // One statement: the bases are in scalar registers before it starts, and the wait states in front keep a base
+        // that the compiler has just moved there with a vector instruction (a reload of a spilled scalar) from being
+        // read too early; the compiler does not look for that inside a statement like this.
+        if (BF16)
+          asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %2, %3\n\tglobal_load_ubyte %1, %4, %5"
+                       : "=&v"(dst), "=&v"(flag) : "v"(lane_wxq), "s"(src), "v"(lane_flagq), "s"(sf) : "memory");
+        else
+          asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %2, %3\n\tglobal_load_ubyte %1, %4, %5"
+                       : "=&v"(dst), "=&v"(flag) : "v"(lane_wxq), "s"(src), "v"(lane_flagq), "s"(sf) : "memory");
+      };
+      set_prefetch_steps(0);
+#pragma unroll
+      for (int u = 0; u < D; ++u) fetch(u, wxq[u], flq[u]);
+      lds_barrier();  // prologue barrier
+      const bool cross_xcd = cross_s != 0u;
+      const int lane_ring = member * XTILE + (pb * 16 + pa) * ESZ;
+      const uint32_t lane_h = (uint32_t)((pb * H + pa) * ESZ);
+      char *const h_member = reinterpret_cast<char *>(p.h_out) + (long long)(head * dh + a0) * ESZ;
+      const __amdgpu_buffer_rsrc_t ring = __builtin_amdgcn_make_buffer_rsrc(xbase, 0, kRing * xslot, 0x00020000);
+      // (two copies of the loop: calls without a mask run the one without the selects)
+      auto gating_loop = [&](auto mask_c) {
+        constexpr bool MASK = decltype(mask_c)::value;
+        for (int it0 = 0; it0 < NIT; it0 += D) {
+          const int t0 = it0 / MT;
+          set_prefetch_steps(t0 + D / MT);
+#pragma unroll
+          for (int u = 0; u < D; ++u) {
+            if (it0 + u >= NIT) break;  // (uniform)
+            const int mt = u % MT;
+            const int t = t0 + u / MT;
+            const int buf = u & 1;  // (D is even: the parity of the iteration)
+            // Before the barrier, while the MFMA waves still work on this iteration: W.x through the LDS corner.
+            // The loads of this iteration have landed when no more than the loads of the D - 1 iterations behind it are
+            // outstanding (the stores in between count as well, so this waits for a little more: operations that are
+            // several iterations old).
+            asm volatile("s_waitcnt vmcnt(%[cnt])" : "+v"(wxq[u]), "+v"(flq[u]) : [cnt] "n"(2 * (D - 1)) : "memory");
+            XS_GTICK(1);
+            *reinterpret_cast<wxq_t *>(&wxt[gw][lane >> 2][4 * (lane & 3)]) = wxq[u];
+            float wxf[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const uint32_t wxbits = wxt[gw][(lane >> 4) * 4 + g][pa];
+              wxf[g] = BF16 ? bf16_bits_to_float(wxbits) : __uint_as_float(wxbits);
+            }
+            const bool restart = MASK && (flq[u] & flag_on) != 0u;
+            asm volatile("" : "+v"(wxf[0]), "+v"(wxf[1]), "+v"(wxf[2]), "+v"(wxf[3]));  // (here, not behind the barrier)
+            XS_GTICK(3);
+            lds_barrier();  // barrier #it: the partial sums of iteration it are in LDS
+            XS_GTICK(0);
+            float raw[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
+              float ry = part[buf][0][g][pa * kTileStride + pb];
+              ry += part[buf][1][g][pa * kTileStride + pb];
+              ry += part[buf][2][g][pa * kTileStride + pb];
+              ry += part[buf][3][g][pa * kTileStride + pb];
+              if (MASK && restart) ry = 0.0f;  // a row that starts a document: R.h counts as the +0 a zero operand row gives
+              raw[g] = (wxf[g] + ry) + bias_g[g];
+            }
+            if (MASK && restart) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
 #ifdef XS_PROFILE
-    long long gprof[4] = {0, 0, 0, 0};
-    long long gt_ = clock64();
-#define XS_GTICK(i) do { const long long now_ = clock64(); gprof[i] += now_ - gt_; gt_ = now_; } while (0)
-#else
-#define XS_GTICK(i) do { } while (0)
+            asm volatile("" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
+            XS_GTICK(4);
 #endif
+            slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
+#ifdef XS_PROFILE
+            asm volatile("" : "+v"(st[mt].y));
+            XS_GTICK(5);
+#endif
+            // ---- publish h_t to the peers, re-arm the words of h_{t-2}, write h_t to the output tensor
+            float y = st[mt].y;
+            if (!BF16 && y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
+            const int tile_off = mt * p.G * XTILE;
+            const int off_cur = (t % kRing) * xslot + tile_off;
+            const int off_old = ((t + kRing - 2) % kRing) * xslot + tile_off;
+            char *const hdst = h_member + ((long long)t * BH + (long long)(rowbase + mt * 16) * H) * ESZ;
+            if (BF16) {
+              const uint16_t v = (uint16_t)float_to_bf16_bits(y);
+              if (cross_xcd) {  // (groups that span two L2s publish past them)
+                __builtin_amdgcn_raw_buffer_store_b16(v, ring, lane_ring, off_cur, 16);
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)kSentinel16, ring, lane_ring, off_old, 16);
+              } else {
+                __builtin_amdgcn_raw_buffer_store_b16(v, ring, lane_ring, off_cur, 0);
+                __builtin_amdgcn_raw_buffer_store_b16((uint16_t)kSentinel16, ring, lane_ring, off_old, 0);
+              }
+              *reinterpret_cast<uint16_t *>(hdst + lane_h) = v;
+            } else {
+              if (cross_xcd) {
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), ring, lane_ring, off_cur, 16);
+                __builtin_amdgcn_raw_buffer_store_b32(kSentinel32, ring, lane_ring, off_old, 16);
+              } else {
+                __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(y), ring, lane_ring, off_cur, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(kSentinel32, ring, lane_ring, off_old, 0);
+              }
+              *reinterpret_cast<float *>(hdst + lane_h) = y;
+            }
+            XS_GTICK(2);
+            fetch(u, wxq[u], flq[u]);
+          }
+        }
+      };
+      if (p.reset != nullptr) gating_loop(std::integral_constant<bool, true>{});
+      else gating_loop(std::integral_constant<bool, false>{});
+    } else
     for (int it0 = 0; it0 < NIT; it0 += D) {
 #pragma unroll
       for (int u = 0; u < D; ++u) {
@@ -195,14 +348,14 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
         XS_GTICK(3);
         lds_barrier();  // barrier #it: the partial sums of iteration it are in LDS
         XS_GTICK(0);
-        // The loads of the iterations up to it + 2 have landed when at most those of the 5 iterations behind are
-        // outstanding (stores of the last iteration may be waited for as well; they are a whole iteration old).
-        const int u2 = (u + 2) % D;
+        // The loads of iteration it have landed when no more than the loads of the D - 1 iterations behind it are
+        // outstanding (the stores in between count as well, so this waits for a little more: operations that are
+        // five iterations old).
         asm volatile("s_waitcnt vmcnt(%[cnt])"
-                     : "+v"(wxr[u][0]), "+v"(wxr[u][1]), "+v"(wxr[u][2]), "+v"(wxr[u][3]), "+v"(flr[u]), "+v"(flr[u2])
-                     : [cnt] "n"(5 * (D - 3)) : "memory");
+                     : "+v"(wxr[u][0]), "+v"(wxr[u][1]), "+v"(wxr[u][2]), "+v"(wxr[u][3]), "+v"(flr[u])
+                     : [cnt] "n"(5 * (D - 1)) : "memory");
         XS_GTICK(1);
-        gate_tile(it, u % MT, wxr[u], flr[u], flr[u2]);
+        gate_tile(it, u % MT, wxr[u], flr[u]);
         XS_GTICK(2);
         issue(it + D, wxr[u], flr[u]);
       }
@@ -210,7 +363,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0 && wave == NMW) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
-      for (int i = 0; i < 4; ++i) dst[i] = gprof[i];
+      for (int i = 0; i < 6; ++i) dst[i] = gprof[i];
     }
 #endif
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -277,33 +430,13 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
       asm volatile("s_waitcnt vmcnt(0)" : "+v"(rreg[g][c].x), "+v"(rreg[g][c].y), "+v"(rreg[g][c].z), "+v"(rreg[g][c].w) :: "memory");
   bool aborted = false;
   uint32_t max_spins = 0;
-  lds_barrier();  // prologue barrier: the reset flags of iterations 0 and 1 and the placement verdict are in LDS
+  lds_barrier();  // prologue barrier: the placement verdict is in LDS
 
-  // poll address of chunk c of row tile mt = per-lane part + a compile-time constant: unit k of row r of row tile mt
-  // lives at [mt][member k/16][r][k%16].  Lanes whose batch row does not exist ask for an offset past the descriptor's
-  // end: zeros, no memory traffic.
+  // poll address of chunk c of row tile mt = per-lane part + a constant: unit k of row r of row tile mt lives at
+  // [mt][member k/16][r][k%16] of a ring slot
   const int xlane_ok = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
   const int xtile_stride = p.G * XTILE;
   auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
-  uint4 aset[2][CPW];  // the operand tile being consumed and the one on its way
-#pragma unroll
-  for (int s_ = 0; s_ < 2; ++s_)
-#pragma unroll
-    for (int c = 0; c < CPW; ++c) aset[s_][c] = make_uint4(0, 0, 0, 0);
-  // requests the piece of iteration itr's tile this wave multiplies; step 0 takes its operand from s0.
-  // A chunk past the last member reads zeros (the descriptor ends with the slot).
-  auto ring_rsrc = [&](int t_) {
-    return __builtin_amdgcn_make_buffer_rsrc(xbase + ((t_ + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
-  };
-  auto request = [&](int itr, uint4 (&dst)[CPW]) -> bool {
-    const int nt = itr / MT, nmt = itr - nt * MT;
-    if (!(itr < NIT && nt >= 1)) return false;
-    const __amdgpu_buffer_rsrc_t rs = ring_rsrc(nt);
-    const int xl = (FULL || rowbase + nmt * 16 + r16 < rend) ? xlane_ok : 0x7FFFFF00;
-#pragma unroll
-    for (int c = 0; c < CPW; ++c) dst[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, xl, xconst(c, nmt), 16));
-    return true;
-  };
 #ifdef XS_PROFILE
   long long mprof[6] = {0, 0, 0, 0, 0, 0};
   long long mt_ = clock64();
@@ -311,49 +444,104 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
 #else
 #define XS_MTICK(i) do { } while (0)
 #endif
-  bool next_requested = false;
-  int it = 0;
-  for (int t = 0; t < p.T; ++t) {
+
+  // ---- partial R.h over this wave's K slab -> LDS (C layout: lane holds unit column r16, batch rows 4q..4q+3), barrier #it
+  auto multiply_and_hand_over = [&](int it, const uint4 (&areg)[CPW]) {
+    f32x4 acc[4];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt, ++it) {
-      uint4 (&cur)[CPW] = aset[mt & 1];   // (it & 1 == mt & 1)
-      uint4 (&nxt)[CPW] = aset[(mt + 1) & 1];
-      // ---- 1. A operand: h_{t-1} of batch row (rowbase + mt*16 + r16), this wave's K slab
-      const int arow = rowbase + mt * 16 + r16;
-      const bool row_ok = FULL ? true : arow < rend;
-      const bool row_reset = rfl[it & 3][r16] != 0u;
-      bool need[CPW];
+    for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-      for (int c = 0; c < CPW; ++c) need[c] = FULL ? true : (row_ok && wave * KW + c * 4 * EPC + q * EPC < dh);
-      XS_MTICK(0);
-      const bool this_requested = next_requested;
-      if (!this_requested) {  // step 0: the operand comes from the initial state (or is zero)
+    for (int c = 0; c < CPW; ++c) {
+      if (BF16) {
+        const bf16x8 av = __builtin_bit_cast(bf16x8, areg[c]);
 #pragma unroll
-        for (int c = 0; c < CPW; ++c) {
-          const int k0 = wave * KW + c * 4 * EPC + q * EPC;
-          uint4 v = make_uint4(0, 0, 0, 0);
-          if (need[c] && p.s0) {
-            const float *src = p.s0 + (long long)arow * H + head * dh + k0;
-            if (BF16) {
-              const float4 lo = *reinterpret_cast<const float4 *>(src);
-              const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
-              v.x = pack_bf16x2(lo.x, lo.y); v.y = pack_bf16x2(lo.z, lo.w);
-              v.z = pack_bf16x2(hi.x, hi.y); v.w = pack_bf16x2(hi.z, hi.w);
-            } else {
-              v = *reinterpret_cast<const uint4 *>(src);
-            }
+        for (int g = 0; g < 4; ++g)
+          acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, rreg[g][c]), acc[g], 0, 0, 0);
+      } else {
+        const uint32_t aw[4] = {areg[c].x, areg[c].y, areg[c].z, areg[c].w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const uint32_t bw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[g], 0, 0, 0);
           }
-          cur[c] = v;
         }
       }
-      // this tile's piece, requested one iteration ago, has to be here now (the compiler's wait: nothing younger is in flight) ...
+    }
+    XS_MTICK(3);
+    const int buf = it & 1;
 #pragma unroll
-      for (int c = 0; c < CPW; ++c) asm volatile("" : "+v"(cur[c].x), "+v"(cur[c].y), "+v"(cur[c].z), "+v"(cur[c].w));
-      XS_MTICK(2);
-      // ... and the next tile's goes out
-      next_requested = request(it + 1, nxt);
-      XS_MTICK(1);
-      if (this_requested) {
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<f32x4 *>(&part[buf][wave][g][r16 * kTileStride + 4 * q]) = acc[g];
+    XS_MTICK(4);
+    lds_barrier();  // barrier #it
+    XS_MTICK(5);
+  };
+  auto row_exists = [&](int mt) { return FULL ? true : rowbase + mt * 16 + r16 < rend; };
+  auto chunk_needed = [&](int mt, int c) { return FULL ? true : (row_exists(mt) && wave * KW + c * 4 * EPC + q * EPC < dh); };
+
+  // ---- step 0: the operand comes from the initial state (or is zero)
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    uint4 areg[CPW];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+      const int k0 = wave * KW + c * 4 * EPC + q * EPC;
+      uint4 v = make_uint4(0, 0, 0, 0);
+      if (chunk_needed(mt, c) && p.s0) {
+        const float *src = p.s0 + (long long)(rowbase + mt * 16 + r16) * H + head * dh + k0;
+        if (BF16) {
+          const float4 lo = *reinterpret_cast<const float4 *>(src);
+          const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
+          v.x = pack_bf16x2(lo.x, lo.y); v.y = pack_bf16x2(lo.z, lo.w);
+          v.z = pack_bf16x2(hi.x, hi.y); v.w = pack_bf16x2(hi.z, hi.w);
+        } else {
+          v = *reinterpret_cast<const uint4 *>(src);
+        }
+      }
+      areg[c] = v;
+    }
+    multiply_and_hand_over(mt, areg);
+  }
+
+  if (p.T > 1) {
+    // ---- steps 1 .. T-1: a wave fetches its piece of the next tile one iteration ahead into a
+    //      second set of registers, right behind the wait for the current tile, so that this wait (the only one in these
+    //      waves, which issue no stores) never covers the new loads.
+    //      Lanes whose batch row does not exist ask for an offset past the descriptor's end: zeros, no memory traffic;
+    //      a chunk past the last member reads zeros as well (the descriptor ends with the slot).
+    auto ring_rsrc = [&](int t_) {  // the slot that holds h_{t_ - 1}
+      return __builtin_amdgcn_make_buffer_rsrc(xbase + ((t_ + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
+    };
+    uint4 aset[2][CPW];
+    auto request = [&](int itr, uint4 (&dst)[CPW]) {
+      if (itr >= NIT) return;
+      const int nt = itr / MT, nmt = itr - nt * MT;
+      const __amdgpu_buffer_rsrc_t rs = ring_rsrc(nt);
+      const int xl = row_exists(nmt) ? xlane_ok : 0x7FFFFF00;
+#pragma unroll
+      for (int c = 0; c < CPW; ++c) dst[c] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, xl, xconst(c, nmt), 16));
+    };
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) aset[1][c] = make_uint4(0, 0, 0, 0);
+    request(MT, aset[0]);
+    int it = MT;
+    for (int t = 1; t < p.T; ++t) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt, ++it) {
+        uint4 (&cur)[CPW] = aset[mt & 1];   // (it & 1 == mt & 1)
+        uint4 (&nxt)[CPW] = aset[(mt + 1) & 1];
+        bool need[CPW];
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) need[c] = chunk_needed(mt, c);
+        XS_MTICK(0);
+        // this tile's piece, requested one iteration ago, has to be here now (the compiler's wait: nothing younger is in flight) ...
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) asm volatile("" : "+v"(cur[c].x), "+v"(cur[c].y), "+v"(cur[c].z), "+v"(cur[c].w));
+        XS_MTICK(1);
+        // ... and the next tile's goes out
+        request(it + 1, nxt);
         // one look at everything at once: one mark over all chunks this lane needs
         auto any_missing = [&]() {
           uint32_t mark = 0u;
@@ -367,7 +555,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
           // tile's requests, which are waited for with it)
           uint32_t spins = 0;
           const __amdgpu_buffer_rsrc_t rs = ring_rsrc(t);
-          const int xl = row_ok ? xlane_ok : 0x7FFFFF00;
+          const int xl = row_exists(mt) ? xlane_ok : 0x7FFFFF00;
           for (;;) {
             ++spins;
             if ((spins & 1023u) == 0u &&
@@ -389,42 +577,12 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
           }
           max_spins = spins > max_spins ? spins : max_spins;
         }
+        uint4 areg[CPW];
+#pragma unroll
+        for (int c = 0; c < CPW; ++c) areg[c] = need[c] ? cur[c] : make_uint4(0, 0, 0, 0);
+        XS_MTICK(2);
+        multiply_and_hand_over(it, areg);
       }
-      // ---- 2. partial R.h over this wave's K slab; rows that start a document and chunks that are not needed count as zeros
-      uint4 areg[CPW];
-#pragma unroll
-      for (int c = 0; c < CPW; ++c) areg[c] = (row_reset || !need[c]) ? make_uint4(0, 0, 0, 0) : cur[c];
-      XS_MTICK(3);
-      f32x4 acc[4];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) acc[g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int c = 0; c < CPW; ++c) {
-        if (BF16) {
-          const bf16x8 av = __builtin_bit_cast(bf16x8, areg[c]);
-#pragma unroll
-          for (int g = 0; g < 4; ++g)
-            acc[g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, __builtin_bit_cast(bf16x8, rreg[g][c]), acc[g], 0, 0, 0);
-        } else {
-          const uint32_t aw[4] = {areg[c].x, areg[c].y, areg[c].z, areg[c].w};
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-              const uint32_t bw[4] = {rreg[g][c].x, rreg[g][c].y, rreg[g][c].z, rreg[g][c].w};
-              acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[g], 0, 0, 0);
-            }
-          }
-        }
-      }
-      // ---- 3. partial tiles -> LDS.  C layout: lane holds unit column r16, batch rows 4q..4q+3
-      const int buf = it & 1;
-#pragma unroll
-      for (int g = 0; g < 4; ++g)
-        *reinterpret_cast<f32x4 *>(&part[buf][wave][g][r16 * kTileStride + 4 * q]) = acc[g];
-      XS_MTICK(4);
-      lds_barrier();  // barrier #it
-      XS_MTICK(5);
     }
   }
 #ifdef XS_PROFILE
