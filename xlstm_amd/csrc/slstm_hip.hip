@@ -295,12 +295,15 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   for (int b0 = 0; b0 < B; b0 += rows_per_launch) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
     // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
-    // (and, for the kernel of four row tiles, per-lane offsets inside a row tile that fit 31 bits: its gating waves
-    // address W.x, the mask and h_out as a scalar base plus a 32-bit offset)
-    const long long esz = bf16 ? 2 : 4;
-    const bool small_offsets = 16ll * a->wx_stride_b * esz < (1ll << 31) && 16ll * a->reset_stride_b < (1ll << 31) &&
-                               16ll * NH * dh * esz < (1ll << 31);
-    const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0) && (MT < 4 || small_offsets);
+    const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
+    // (the gating waves of the kernel of four row tiles address W.x, the mask and h_out as a scalar base plus a 32-bit
+    // offset per lane inside four rows / one row tile)
+    if (MT == 4) {
+      const long long esz = bf16 ? 2 : 4;
+      if (4ll * a->wx_stride_b * esz + 4ll * NH * dh * esz >= 0xFFFFFF00ll || (a->reset && 4ll * a->reset_stride_b >= 0xFFFFFF00ll) ||
+          16ll * NH * dh * esz >= (1ll << 31))
+        return fail(XS_ERR_UNSUPPORTED, "row strides of wx / reset too large (four rows must span less than 4 GiB)");
+    }
     // the feeder fetches W.x in bursts where the prefetch waves cannot cover it: row tiles of 8 rows or more
     const bool burst = rows_per_wg >= 8;
     // four row tiles per workgroup: the kernel with MFMA waves and gating waves; one or two: the kernel in which
