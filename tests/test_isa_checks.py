@@ -1,0 +1,78 @@
+"""The two checks of xlstm_amd/isa_check.py: on small listings that show what they look for, and on the assembly the
+compiler really makes of the kernels (no GPU needed: hipcc cross-compiles)."""
+import os
+
+from xlstm_amd import isa_check
+
+HAZARD = """
+_Z6kernelv:
+	v_readlane_b32 s44, v83, 26
+	v_mul_lo_u32 v62, v65, s0
+	v_readlane_b32 s45, v83, 27
+	;;#ASMSTART
+	global_load_ubyte v68, v62, s[44:45]
+	;;#ASMEND
+	s_endpgm
+"""
+
+HAZARD_FIXED = HAZARD.replace("\tglobal_load_ubyte", "\ts_nop 4\n\tglobal_load_ubyte")
+
+COPY_IN_FLIGHT = """
+_Z6kernelv:
+	;;#ASMSTART
+	global_load_dwordx2 v[4:5], v60, s[2:3]
+	;;#ASMEND
+	v_mov_b64_e32 v[26:27], v[4:5]
+	;;#ASMSTART
+	s_waitcnt vmcnt(0)
+	;;#ASMEND
+	ds_write_b64 v67, v[26:27]
+	s_endpgm
+"""
+
+COPY_AFTER_WAIT = """
+_Z6kernelv:
+	;;#ASMSTART
+	global_load_dwordx2 v[4:5], v60, s[2:3]
+	;;#ASMEND
+	;;#ASMSTART
+	global_load_dwordx2 v[6:7], v60, s[2:3]
+	;;#ASMEND
+	;;#ASMSTART
+	s_waitcnt vmcnt(1)
+	;;#ASMEND
+	v_mov_b64_e32 v[26:27], v[4:5]
+	s_endpgm
+"""
+
+TO_LDS = """
+_Z6kernelv:
+	;;#ASMSTART
+	s_nop 4
+	s_mov_b32 m0, s35
+	s_nop 0
+	buffer_load_dwordx4 v39, s[12:15], 0 offen lds
+	;;#ASMEND
+	v_mov_b32_e32 v39, 0
+	s_endpgm
+"""
+
+
+def test_a_freshly_written_scalar_register_read_by_hand_issued_memory_instruction_is_found():
+    assert len(isa_check.scalar_read_hazards(HAZARD)) == 2  # s44 (3 wait states behind) and s45 (1 behind)
+    assert isa_check.scalar_read_hazards(HAZARD_FIXED) == []
+
+
+def test_a_copy_of_a_register_with_a_hand_issued_load_in_flight_is_found():
+    assert len(isa_check.inflight_register_uses(COPY_IN_FLIGHT)) == 1
+    # vmcnt(1) with one younger load: the first load has landed, the second has not
+    assert isa_check.inflight_register_uses(COPY_AFTER_WAIT) == []
+    assert len(isa_check.inflight_register_uses(COPY_AFTER_WAIT.replace("v[26:27], v[4:5]", "v[26:27], v[6:7]"))) == 1
+    # a load that goes straight to LDS has no destination register (v39 is its address)
+    assert isa_check.inflight_register_uses(TO_LDS) == []
+
+
+def test_the_kernels_as_compiled_have_neither(tmp_path):
+    listing = isa_check.emit_assembly(os.path.join(tmp_path, "device.s"))
+    assert listing.count("ASMSTART") > 50  # (the listing really is the kernels')
+    assert isa_check.check(listing) == []

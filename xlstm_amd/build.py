@@ -26,8 +26,8 @@ HIPCC_FLAGS = [
 
 
 def build(verbose: bool = False, extra_flags=(), out: str = LIB) -> str:
-    """Builds the engine.  ``extra_flags`` / ``out`` are for the two measurement builds the kernels know about:
-    ``-DXS_PROFILE`` (per-phase cycle stamps, read back by ``bench.py --phase-profile``) and
+    """Builds the engine and returns the path of the library.  ``extra_flags`` / ``out`` are for the two measurement
+    builds the kernels know about: ``-DXS_PROFILE`` (per-phase cycle stamps, read back by ``bench.py --phase-profile``) and
     ``-DXS_SMALL_BATCH_FMA`` (the FMA contraction for row tiles of 4 rows); from the command line:
     ``python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so``."""
     hipcc = os.environ.get("HIPCC", "hipcc")
@@ -36,11 +36,11 @@ def build(verbose: bool = False, extra_flags=(), out: str = LIB) -> str:
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+    log = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{out}")
-    if verbose and out.strip():
-        print(out)
+        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{log}")
+    if verbose and log.strip():
+        print(log)
     return out
 
 
