@@ -28,7 +28,6 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 METRIC = "sLSTM fwd tokens/s @ D=1024 packed B16×T2048; decode step µs @ B=256"
-SERIAL_FLOOR_US = 1520 / 2350.0  # per timestep of the sequence kernel at config 2, see the roofline object
 HBM_PEAK_GBS = 8000.0  # MI355X published HBM3E bandwidth
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X published dense bf16 MFMA rate
 CONFIG5_NAME = "config 5: B=64 T=4096 D=4096 NH=4 bf16, no resets"
@@ -232,6 +231,73 @@ def bench_small_batch(device, T=1024):
     return {"library": os.environ.get("XLSTM_AMD_LIB", "xlstm_amd/lib/libxlstm_amd.so"), "rows": rows}
 
 
+PROFILE_LIB = os.path.join(ROOT, "xlstm_amd", "lib", "libxlstm_amd_profile.so")
+
+
+def phase_profile(device):
+    """Per-phase cycle table of the sequence kernels, from the cycle stamps of the measurement build of the library
+    (``-DXS_PROFILE``: every wave of workgroup 0 sums the cycles between fixed points of its loop).  The stamps cost
+    time themselves (a step of config 2 takes about a quarter longer than in the product build), so the table says where
+    a step's time goes, not how long a step takes."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    def run(B, T, NH, dh, mean_doc):
+        H = NH * dh
+        wx_c, r_ext_c, bias_c, mask_c = make_inputs(B, T, NH, dh, mean_doc, torch.device("cpu"))
+        wx = wx_c.to(device)
+        r = r_ext_c.permute(0, 2, 3, 1).reshape(NH, 4 * dh, dh).contiguous().to(device)
+        bias = bias_c.to(device)
+        mask = mask_c.to(device) if mean_doc else None
+        ws = F.workspace_for(B, T, NH, dh, device)
+        h = torch.empty(T, B, H, dtype=torch.bfloat16, device=device)
+        s = torch.empty(4, B, H, dtype=torch.float32, device=device)
+        ms = []
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            F.slstm_forward(wx, r, bias, None, mask, workspace=ws, h_out=h, s_out=s)
+            e1.record()
+            torch.cuda.synchronize()
+            ms.append(e0.elapsed_time(e1))
+        if F.read_status(ws)["aborted"]:
+            sys.exit("bench.py: the engine flagged the run as aborted")
+        return F.read_phase_stamps(ws).double(), sorted(ms)[1]
+
+    out = {}
+    # config 2: slstm_seq_kernel, one row tile of 4 rows; per timestep
+    T = 2048
+    st, ms = run(16, T, 4, 256, 512)
+    names = ["poll (request to complete operand)", "mfma + partial sums to LDS", "barrier", "LDS sum + gating",
+             "publish + stage h", "loop top"]
+    out["config 2 (slstm_seq_kernel<bf16,NCH=2,MT=1,FULL>), cycles per timestep, workgroup 0"] = {
+        "ms_per_call_with_stamps": ms,
+        "compute waves 0-3": {n: [round(float(st[w][i] / T)) for w in range(4)] for i, n in enumerate(names)},
+        "compute waves: sum": [round(float(st[w][:6].sum() / T)) for w in range(4)],
+        "compute waves: polls repeated per step": [round(float(st[w][6] / T), 2) for w in range(4)],
+        "feeder wave": {"W.x into LDS": round(float(st[4][0] / T)), "issue": round(float(st[4][1] / T)),
+                        "barrier": round(float(st[4][2] / T))},
+        "drainer wave": {"h to HBM": round(float(st[5][0] / T)), "barrier": round(float(st[5][1] / T))},
+    }
+    # config 5 at a quarter of its length and config 3's prefill: slstm_seq_roles_kernel; per tile iteration (4 per step)
+    for label, (B, T, NH, dh) in (("config 5, T = 1024 (slstm_seq_roles_kernel<bf16,NCH=8,FULL>)", (64, 1024, 4, 1024)),
+                                  ("config 3 prefill, T = 128 (slstm_seq_roles_kernel<bf16,NCH=2,FULL>)", (256, 128, 8, 256))):
+        st, ms = run(B, T, NH, dh, 0)
+        n = 4.0 * T
+        mnames = ["loop top", "wait for the operand tile", "request next tile + arrival test", "mfma", "partial sums to LDS", "barrier"]
+        out[label + ", cycles per tile iteration, workgroup 0"] = {
+            "ms_per_call_with_stamps": ms,
+            "MFMA waves 0-3": {nm: [round(float(st[w][i] / n)) for w in range(4)] for i, nm in enumerate(mnames)},
+            "MFMA waves: sum": [round(float(st[w][:6].sum() / n)) for w in range(4)],
+            "gating wave 4": {"barrier": round(float(st[5][0] / n)), "partial sums out of LDS + sums": round(float(st[5][4] / n)),
+                              "gating": round(float(st[5][5] / n)), "3 stores + fetch": round(float(st[5][2] / n)),
+                              "W.x of the next iteration out of the ring": round(float(st[5][1] / n)),
+                              "loop top": round(float(st[5][3] / n)), "sum": round(float(st[5][:6].sum() / n))},
+        }
+    return out
+
+
 def bench_config4(device, iters=3):
     """BASELINE config 4: 24 blocks (sLSTM at 3, 11, 19), D=1024, 4 heads, vocab 50304, bf16, B=8, T=2048,
     packed documents of mean length 768.  Only the sLSTM cells run on the HIP engine."""
@@ -367,12 +433,21 @@ def main():
                          "the bf16 MFMA roofline (profiling runs)")
     ap.add_argument("--small-batch-only", action="store_true",
                     help="only time the sequence kernel at B = 1, 2, 4 (head dims 128 and 256) and the reference test's shape")
+    ap.add_argument("--phase-profile", action="store_true",
+                    help="per-phase cycle tables of the sequence kernels from the measurement build of the library "
+                         "(python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures ONE GPU; the path shards over batch rows / heads without "
                  "communication, and no multi-GPU figure is produced (run with --gpus 1)")
+
+    if args.phase_profile:  # (before the package loads its library)
+        if not os.path.exists(PROFILE_LIB):
+            sys.exit(f"bench.py --phase-profile needs {PROFILE_LIB}: "
+                     "python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so")
+        os.environ["XLSTM_AMD_LIB"] = PROFILE_LIB
 
     import torch
 
@@ -381,6 +456,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (the hip backend has no CPU path)")
     device = torch.device("cuda:0")
+    if args.phase_profile:
+        print(json.dumps({"phase_profile": phase_profile(device)}, indent=1))
+        return
     if args.copy_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device=device)  # 1 GiB read + 1 GiB written per copy
         dst = torch.empty_like(src)
@@ -458,11 +536,6 @@ def main():
                      "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,BURST=0>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_launch": nbytes, "us_per_timestep": kern_ms * 1e3 / T,
                      "max_poll_rounds": status["max_spins"],
-                     # The launch is a chain of T dependent steps.  Floor of one step of this decomposition, from
-                     # microbenchmarks on the same hardware: one publish -> poll hop inside an XCD (570 cycles), the
-                     # gating chain (650), MFMA + LDS reduction (250), one barrier (50) = 1,520 cycles at 2.35 GHz.
-                     "serial_floor_us_per_timestep": SERIAL_FLOOR_US,
-                     "frac_of_serial_floor": SERIAL_FLOOR_US / (kern_ms * 1e3 / T),
                      "tflops": 8.0 * B * T * NH * dh * dh / (kern_ms * 1e-3) / 1e12},
     }
     traffic_file = os.path.join(ROOT, "profiles", "traffic_seq_cfg2.json")

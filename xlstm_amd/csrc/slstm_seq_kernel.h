@@ -65,6 +65,9 @@ struct SeqParams {
 // can only ever read the pattern or the new data there, never the stale h_{t-2}.
 // ---------------------------------------------------------------------------
 constexpr int kRing = 8;       // slots of the exchange ring
+// Measurement builds (-DXS_PROFILE): the waves of workgroup 0 leave their per-phase cycle sums in the last 128 of the
+// 4096 placement words of the workspace header, 8 counters of 8 bytes per wave slot.
+constexpr int kStampWord = 4096 - 128;
 // prefetch waves a kernel may be launched with (8 waves per workgroup = two per SIMD = 256 VGPRs each, which the
 // largest variants need)
 constexpr int max_prefetch_waves(int nch) { return nch >= 8 ? 1 : kMaxPrefetchWaves; }
@@ -300,7 +303,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     lds_barrier();  // final barrier
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
-      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 4 * 8;
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + 4 * 8;
       for (int i = 0; i < 3; ++i) dst[i] = fprof[i];
     }
 #endif
@@ -357,7 +360,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       for (int it = 0; it < NIT; ++it) drain(it, true);
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0) {
-      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + 5 * 8;
       for (int i = 0; i < 2; ++i) dst[i] = dprof[i];
     }
 #endif
@@ -837,7 +840,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   lds_barrier();                                     // final barrier
 #ifdef XS_PROFILE
   if (lane == 0 && member == 0 && gi == 0) {
-    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + wave * 8;
+    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + wave * 8;
     for (int i = 0; i < 8; ++i) dst[i] = prof[i];
   }
 #endif

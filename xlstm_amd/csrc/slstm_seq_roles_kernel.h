@@ -26,11 +26,16 @@ namespace {
 //              counter, and a wait the compiler places would be a wait for everything).  There is no feeder and no
 //              drainer wave.
 //
-// Measured and dropped: the same MFMA loop written by hand, with the loads of the tile TWO iterations on placed between
-// the MFMA groups of the current one (exact hand-counted waits, the texture path busy while the matrix cores work).
-// Bit-identical, and slower everywhere (head dim 1024: 5.4 against 3.5 us per step; 512: 2.8 against 2.5; 256: 5.0
-// against 4.5): twice the operand bytes in flight per compute unit only lengthen the queue that every memory
-// instruction of the compute unit, the gating waves' included, waits in.
+// Measured and dropped (all bit-identical; us per step at head dim 1024 / 512 / 256 against 3.5 / 2.5 / 4.4 as it is):
+//  - the MFMA loop written by hand with exact waits, the loads of the tile TWO iterations on between the MFMA groups of
+//    the current one: 5.4 / 2.8 / 5.0 (a tile is asked for before all peers have published it, and every miss costs
+//    a full round trip);
+//  - the same with the loads of the NEXT tile in two halves, four at the top and four between the first MFMA groups
+//    (head dim 1024 only): 3.7.  The MFMA waves get shorter, the gating waves longer by as much: their memory
+//    instructions then always find the compute unit's one texture path busy;
+//  - the gating waves' stores and fetch moved up behind the barrier, under the latency of the partial sums: 5.5 / 3.0 /
+//    5.1, for the same reason (that is when the MFMA waves issue their requests);
+//  - a ring of 16 slots instead of 8 (twice as long for the stores to complete before a wait counts them): no change.
 //
 // Barrier #it means "the partial sums of iteration it are in LDS"; the gating waves reach it when they are done with
 // iteration it - 1.  The sums are formed in the same order as everywhere else: the same bits.
@@ -44,7 +49,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = CPW * 4 * EPC;      // input units per MFMA wave
   constexpr int ESZ = BF16 ? 2 : 4;
-  constexpr int D = 8;                   // iterations the gating waves fetch W.x ahead (a ring of registers)
+  constexpr int D = 8;                   // iterations the gating waves fetch W.x ahead (slots of their rings in LDS)
   __shared__ float part[2][NMW][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
 
   __shared__ uint32_t cross_s;
@@ -292,7 +297,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
     else gating_loop(std::integral_constant<bool, false>{});
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0 && wave == NMW) {
-      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + 5 * 8;
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + 5 * 8;
       for (int i = 0; i < 6; ++i) dst[i] = gprof[i];
     }
 #endif
@@ -517,7 +522,7 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
   }
 #ifdef XS_PROFILE
   if (lane == 0 && member == 0 && gi == 0 && wave < 4) {
-    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + 4096 - 128) + wave * 8;
+    long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + wave * 8;
     for (int i = 0; i < 6; ++i) dst[i] = mprof[i];
   }
 #endif

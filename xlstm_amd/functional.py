@@ -42,6 +42,14 @@ def read_status(workspace: torch.Tensor) -> dict:
     return {k: getattr(st, k) for k, _ in _lib.SlstmStatus._fields_ if k != "reserved"}
 
 
+def read_phase_stamps(workspace: torch.Tensor) -> torch.Tensor:
+    """Per-phase cycle sums that a library built with ``-DXS_PROFILE`` leaves behind a sequence call: ``[6, 8]`` int64,
+    one row per wave slot of workgroup 0 (which waves and phases: see ``bench.py --phase-profile``).  The product
+    library writes nothing there."""
+    off = 256 + 4 * (4096 - 128)
+    return workspace[off: off + 6 * 8 * 8].cpu().view(torch.int64).view(6, 8)
+
+
 def read_placement(workspace: torch.Tensor, max_wg: int = 4096) -> torch.Tensor:
     """Per-workgroup placement words written by the sequence kernel:
     bit 31 = workgroup was active, bits [30:8] head group, bits [3:0] XCD id."""
