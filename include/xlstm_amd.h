@@ -117,7 +117,9 @@ typedef struct xs_slstm_status {
   uint32_t xcd_mixed;   /* number of head groups whose workgroups ran on more than one XCD */
   uint32_t launches;    /* kernel launches the call was split into */
   uint32_t step_kernel; /* 1 if the call ran the single-token step kernel (xs_slstm_step, or xs_slstm_forward with T == 1) */
-  uint32_t reserved[9];
+  uint32_t rows_per_workgroup; /* sequence kernels: batch rows a workgroup handles (4, 8, 16, 32 = two row tiles, 64 = four
+                                  row tiles: the kernel with MFMA waves and gating waves), of the last launch; 0 after a step */
+  uint32_t reserved[8];
 } xs_slstm_status;
 
 /* Library / ABI identification.  Replaces nothing (the reference keys its JIT

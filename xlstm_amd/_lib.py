@@ -110,8 +110,8 @@ class SlstmStatus(ctypes.Structure):
     _fields_ = [
         ("aborted", ctypes.c_uint32), ("abort_wg", ctypes.c_uint32), ("abort_step", ctypes.c_uint32),
         ("max_spins", ctypes.c_uint32), ("xcd_mixed", ctypes.c_uint32), ("launches", ctypes.c_uint32),
-        ("step_kernel", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32 * 9),
+        ("step_kernel", ctypes.c_uint32), ("rows_per_workgroup", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32 * 8),
     ]
 
 

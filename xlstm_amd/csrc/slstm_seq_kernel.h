@@ -107,7 +107,10 @@ __device__ __forceinline__ void seq_place(const SeqParams &p, int wg, int &gi, i
 //      written through to memory.  Returns 1 for "more than one XCD".
 __device__ __forceinline__ uint32_t seq_handshake(const SeqParams &p, int wg, int gi, long long spin_limit) {
   const bool one_xcd_layout = p.G <= 32;
-  if (wg == 0) atomicAdd(&p.status->launches, 1u);  // a long batch is run as several launches of row chunks
+  if (wg == 0) {
+    atomicAdd(&p.status->launches, 1u);  // a long batch is run as several launches of row chunks
+    p.status->rows_per_workgroup = (uint32_t)p.rows_per_wg;
+  }
   const uint32_t my_xcc = __builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu;  // XCC_ID, bits [3:0]
   __hip_atomic_store(&p.wg_xcc[wg], 0x80000000u | ((uint32_t)gi << 8) | my_xcc, __ATOMIC_RELAXED,
                      __HIP_MEMORY_SCOPE_AGENT);
