@@ -107,86 +107,12 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
     for (int mt = 0; mt < MT; ++mt)
       asm volatile("" : "+v"(st[mt].y), "+v"(st[mt].c), "+v"(st[mt].n), "+v"(st[mt].m));
 
-    // ---- W.x and the reset flags travel from memory STRAIGHT INTO LDS (no registers), D - 1 iterations ahead, into a
-    //      ring of D slots per gating wave.  Nothing of a load in flight is visible to the compiler, so it cannot move or
-    //      copy a destination that has not landed, and the waits are counted by hand: exactly one load (two with a mask)
-    //      per iteration, loads and stores share one counter, and a wait the compiler places would be a wait for
-    //      everything.  A 16-byte load per lane: the wave's 16 (row, gate) pieces of 16 units land as
-    //      [row * 4 + gate][unit], which is how the lanes that gate them read them back.  Rows and units that do not
-    //      exist ask for an offset past the end of the buffer descriptor: zeros, no memory access.
-    constexpr int UPL = 16 / ESZ;                 // units a lane fetches (8 bf16 / 4 fp32)
-    constexpr int LPP = 16 / UPL;                 // lanes per piece
-    typedef typename std::conditional<BF16, uint16_t, uint32_t>::type wxe_t;
-    __shared__ __attribute__((aligned(16))) wxe_t wxring[4][D][16][16];  // [gating wave][slot][row * 4 + gate][unit]
-    __shared__ uint32_t flring[4][D][64];                                  // [gating wave][slot][lane]: the row's flag byte
     const int gw = wave - NMW;
-    constexpr uint32_t kPastEnd = 0xFFFFFF00u;    // (= the descriptors' size)
     const bool has_mask = p.reset != nullptr;
     const long long flag_sb = has_mask ? p.reset_sb : 0;
-    const int dl_piece = lane / LPP, dl_part = lane % LPP;
-    const bool dl_active = lane < 16 * LPP;       // (bf16: the lower half of the wave fetches)
-    uint32_t voff_wx[MT], voff_flag[MT];
     bool lane_ok[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-      const int row0 = rowbase + mt * 16 + 4 * gw;  // first row of this wave in the tile
-      const bool piece_ok = row0 + (dl_piece >> 2) < rend && a0 + dl_part * UPL < dh;
-      voff_wx[mt] = piece_ok ? (uint32_t)(((long long)(dl_piece >> 2) * p.wx_sb + (long long)(dl_piece & 3) * H + dl_part * UPL) * ESZ)
-                             : kPastEnd;
-      voff_flag[mt] = row0 + (lane >> 4) < rend ? (uint32_t)((long long)(lane >> 4) * flag_sb) : kPastEnd;
-      lane_ok[mt] = FULL ? true : (unit_ok && rowbase + mt * 16 + pb < rend);
-    }
-    const char *const wx_wave = reinterpret_cast<const char *>(p.wx) + (long long)(head * dh + a0) * ESZ;
-    // The offsets of the D / MT steps a round of D iterations fetches for (clamped to the last step: what the rounds
-    // past the end fetch is never looked at), kept as offsets that the scalar unit adds per iteration.
-    constexpr int NPF = D / MT;
-    long long pf_wx[NPF], pf_flag[NPF];
-    auto set_prefetch_steps = [&](int tfirst) {
-#pragma unroll
-      for (int d = 0; d < NPF; ++d) {
-        const int tp = tfirst + d < p.T ? tfirst + d : p.T - 1;
-        pf_wx[d] = (long long)tp * p.wx_st * ESZ;
-        pf_flag[d] = tp;
-      }
-    };
-    auto descriptor = [&](const void *base) {  // raw bytes from base, kPastEnd of them
-      const unsigned long long a = reinterpret_cast<unsigned long long>(base);
-      return u32x4_t{uniform((uint32_t)a), uniform((uint32_t)(a >> 32) & 0xFFFFu), kPastEnd, 0x00020000u};
-    };
-    // (The wait states in front: the descriptor may sit in scalar registers that the compiler has just written with a
-    // vector instruction, e.g. the reload of a spilled scalar, and it does not look for that hazard inside a statement
-    // like this.  M0 = the LDS address of lane 0's bytes.)
-    auto fetch = [&](auto mask_c, int mt, int d, int slot) {  // row tile mt of step pf[d] -> ring slot
-      const uint32_t vw = voff_wx[mt], vf = voff_flag[mt];
-      const long long step_flag = pf_flag[d];
-      const char *src = wx_wave + (long long)(rowbase + mt * 16 + 4 * gw) * p.wx_sb * ESZ + pf_wx[d];
-      const u32x4_t rs = descriptor(src);
-      const uint32_t lds = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) wxe_t *)&wxring[gw][slot][0][0]));
-      if (dl_active)
-        asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                     :: "s"(lds), "v"(vw), "s"(rs) : "memory", "m0");
-      if (decltype(mask_c)::value) {
-        const unsigned char *sf = p.reset + (long long)(rowbase + mt * 16 + 4 * gw) * flag_sb + step_flag;
-        const u32x4_t fs = descriptor(sf);
-        const uint32_t fl = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) uint32_t *)&flring[gw][slot][0]));
-        asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ubyte %1, %2, 0 offen lds"
-                     :: "s"(fl), "v"(vf), "s"(fs) : "memory", "m0");
-      }
-    };
-    // W.x of the iteration in a ring slot -> the lanes that gate it.  Its loads have landed when no more than the loads
-    // of the D - 1 iterations fetched behind it are outstanding (the stores in between count as well, so this waits for
-    // a little more: operations that are several iterations old).
-    auto stage = [&](auto mask_c, int slot, float (&wxf)[4], uint32_t &flag) {
-      constexpr bool MASK = decltype(mask_c)::value;
-      asm volatile("s_waitcnt vmcnt(%[cnt])" :: [cnt] "n"((MASK ? 2 : 1) * (D - 1)) : "memory");
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const uint32_t wxbits = wxring[gw][slot][(lane >> 4) * 4 + g][pa];
-        wxf[g] = BF16 ? bf16_bits_to_float(wxbits) : __uint_as_float(wxbits);
-      }
-      flag = MASK ? (flring[gw][slot][lane] & 0xFFu) : 0u;
-      asm volatile("" : "+v"(wxf[0]), "+v"(wxf[1]), "+v"(wxf[2]), "+v"(wxf[3]), "+v"(flag));  // (here, not where they are used)
-    };
+    for (int mt = 0; mt < MT; ++mt) lane_ok[mt] = FULL ? true : (unit_ok && rowbase + mt * 16 + pb < rend);
 #ifdef XS_PROFILE
     long long gprof[6] = {0, 0, 0, 0, 0, 0};
     long long gt_ = clock64();
@@ -226,75 +152,275 @@ __global__ __launch_bounds__(kRolesThreads) void slstm_seq_roles_kernel(SeqParam
         if (lane_ok[mt]) *reinterpret_cast<uint32_t *>(hdst + lane_h) = hbits;
       }
     };
-    // Per iteration: barrier #it, the partial sums out of LDS, the gating, the tile's three stores, the fetch for
-    // iteration it + D into the ring slot just freed, and W.x of iteration it + 1 out of the ring, so that nothing of it
-    // is left to do behind the next barrier.  The memory instructions come late in the iteration on purpose: right behind
-    // the barrier the MFMA waves issue their requests for the next operand tile, and memory instructions of both kinds
-    // queue in the one texture path of the compute unit (measured: with the stores and the fetch of the previous tile
-    // moved up behind the barrier, 2.4 -> 3.0 us per step at head dim 512 and 3.5 -> 5.5 at 1024).
-    // (Two copies of the loop: calls without a mask run the one without the flag loads and the selects.)
-    auto gating_loop = [&](auto mask_c) {
-      constexpr bool MASK = decltype(mask_c)::value;
+    if constexpr (FULL) {
+      // ---- Every row and unit exists (the common case, and the fast one).  W.x of an iteration takes ONE load per wave,
+      //      D iterations ahead, into a ring of registers: lane l fetches units 4 (l & 3) .. + 3 of gate (l >> 2) & 3 for
+      //      row l >> 4 of the wave's four rows, as a 32-bit offset on top of a base that the scalar unit steps.  When
+      //      they are needed the pieces go through a private corner of LDS to the lanes that gate them (same wave: no
+      //      barrier, LDS keeps a wave's order).  The loads are hand-issued and the waits hand-counted (two loads per
+      //      iteration; loads and stores share one counter, and a wait the compiler places would be a wait for
+      //      everything).  The compiler does not know that a ring register is in flight between the load and the wait:
+      //      it must not copy or reuse one in between, and xlstm_amd/isa_check.py checks the compiled code for exactly
+      //      that.  (The rings in LDS of the loop for ragged tiles below have no such condition; here they cost 15 %
+      //      at config 5's full length, 16.4 against 13.9 ms, and nothing at half of it.)
+      constexpr int WB = 4 * ESZ;                 // bytes a lane fetches
+      typedef uint32_t wxq_t __attribute__((ext_vector_type(WB / 4)));
+      typedef typename std::conditional<BF16, uint16_t, uint32_t>::type wxe_t;
+      __shared__ __attribute__((aligned(16))) wxe_t wxt[4][16][16];  // [gating wave][row * 4 + gate][unit]
+      const uint32_t lane_wxq =
+          (uint32_t)(((long long)(lane >> 4) * p.wx_sb + (long long)((lane >> 2) & 3) * H + 4 * (lane & 3)) * ESZ);
+      const uint32_t lane_flagq = (uint32_t)((long long)(lane >> 4) * flag_sb);
+      const char *const wx_wave = reinterpret_cast<const char *>(p.wx) + (long long)(head * dh + a0) * ESZ;
+      const unsigned char *const flagb = has_mask ? p.reset : reinterpret_cast<const unsigned char *>(p.wx);
+      wxq_t wxq[D];
+      uint32_t flq[D];
+      // the offsets of the D / MT steps a round of D iterations fetches for (clamped to the last step: what the rounds
+      // past the end fetch is never looked at), kept as offsets that the scalar unit adds per iteration
+      long long pf_wx[D / MT], pf_flag[D / MT];
+      auto set_prefetch_steps = [&](int tfirst) {
+#pragma unroll
+        for (int d = 0; d < D / MT; ++d) {
+          const int tp = tfirst + d < p.T ? tfirst + d : p.T - 1;
+          pf_wx[d] = (long long)tp * p.wx_st * ESZ;
+          pf_flag[d] = has_mask ? tp : 0;
+        }
+      };
+      auto fetch = [&](int u, wxq_t &dst, uint32_t &flag) {  // iteration (round, u): step u / MT of the round, row tile u % MT
+        const int mt = u % MT;
+        const char *src = wx_wave + (long long)(rowbase + mt * 16 + 4 * gw) * p.wx_sb * ESZ + pf_wx[u / MT];
+        const unsigned char *sf = flagb + (long long)(rowbase + mt * 16 + 4 * gw) * flag_sb + pf_flag[u / MT];
+        // One statement: the bases are in scalar registers before it starts, and the wait states in front keep a base
+        // that the compiler has just moved there with a vector instruction (a reload of a spilled scalar) from being
+        // read too early; the compiler does not look for that inside a statement like this.
+        if (BF16)
+          asm volatile("s_nop 4\n\tglobal_load_dwordx2 %0, %2, %3\n\tglobal_load_ubyte %1, %4, %5"
+                       : "=&v"(dst), "=&v"(flag) : "v"(lane_wxq), "s"(src), "v"(lane_flagq), "s"(sf) : "memory");
+        else
+          asm volatile("s_nop 4\n\tglobal_load_dwordx4 %0, %2, %3\n\tglobal_load_ubyte %1, %4, %5"
+                       : "=&v"(dst), "=&v"(flag) : "v"(lane_wxq), "s"(src), "v"(lane_flagq), "s"(sf) : "memory");
+      };
       set_prefetch_steps(0);
 #pragma unroll
-      for (int j = 0; j < D; ++j) fetch(mask_c, j % MT, j / MT, j);
-      float wxf[4];
-      uint32_t flag_now;
-      stage(mask_c, 0, wxf, flag_now);
+      for (int u = 0; u < D; ++u) fetch(u, wxq[u], flq[u]);
       lds_barrier();  // prologue barrier
       cross_xcd = cross_s != 0u;
-      for (int it0 = 0; it0 < NIT; it0 += D) {
-        const int t0 = it0 / MT;
-        set_prefetch_steps(t0 + D / MT);
+      // (everything fetched so far has landed before the loop is entered: whatever the compiler does to the ring
+      // registers at the loop's entry, it does to landed data)
 #pragma unroll
-        for (int u = 0; u < D; ++u) {
-          if (it0 + u >= NIT) break;  // (uniform)
-          const int mt = u % MT;
-          const int buf = u & 1;  // (D is even: the parity of the iteration)
-          XS_GTICK(3);
-          lds_barrier();  // barrier #it: the partial sums of iteration it are in LDS
-          XS_GTICK(0);
-          // a row that starts a document: zero state, and R.h counts as the +0 a zero operand row gives
-          const bool restart = MASK && flag_now != 0u;
-          float raw[4];
+      for (int u = 0; u < D; ++u) asm volatile("s_waitcnt vmcnt(0)" : "+v"(wxq[u]), "+v"(flq[u]) :: "memory");
+      // (two copies of the loop: calls without a mask run the one without the selects)
+      auto gating_loop = [&](auto mask_c) {
+        constexpr bool MASK = decltype(mask_c)::value;
+        for (int it0 = 0; it0 < NIT; it0 += D) {
+          const int t0 = it0 / MT;
+          set_prefetch_steps(t0 + D / MT);
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
-            float ry = part[buf][0][g][pa * kTileStride + pb];
-            ry += part[buf][1][g][pa * kTileStride + pb];
-            ry += part[buf][2][g][pa * kTileStride + pb];
-            ry += part[buf][3][g][pa * kTileStride + pb];
-            if (MASK && restart) ry = 0.0f;
-            raw[g] = (wxf[g] + ry) + bias_g[g];
-          }
-          if (MASK && restart) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+          for (int u = 0; u < D; ++u) {
+            if (it0 + u >= NIT) break;  // (uniform)
+            const int mt = u % MT;
+            const int buf = u & 1;  // (D is even: the parity of the iteration)
+            // Before the barrier, while the MFMA waves still work on this iteration: W.x through the LDS corner.
+            // The loads of this iteration have landed when no more than the loads of the D - 1 iterations behind it are
+            // outstanding (the stores in between count as well, so this waits for a little more: operations that are
+            // several iterations old).
+            asm volatile("s_waitcnt vmcnt(%[cnt])" : "+v"(wxq[u]), "+v"(flq[u]) : [cnt] "n"(2 * (D - 1)) : "memory");
+            XS_GTICK(1);
+            *reinterpret_cast<wxq_t *>(&wxt[gw][lane >> 2][4 * (lane & 3)]) = wxq[u];
+            float wxf[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              const uint32_t wxbits = wxt[gw][(lane >> 4) * 4 + g][pa];
+              wxf[g] = BF16 ? bf16_bits_to_float(wxbits) : __uint_as_float(wxbits);
+            }
+            // a row that starts a document: zero state, and R.h counts as the +0 a zero operand row gives
+            const bool restart = MASK && (flq[u] & 0xFFu) != 0u;
+            asm volatile("" : "+v"(wxf[0]), "+v"(wxf[1]), "+v"(wxf[2]), "+v"(wxf[3]));  // (here, not behind the barrier)
+            XS_GTICK(3);
+            lds_barrier();  // barrier #it: the partial sums of iteration it are in LDS
+            XS_GTICK(0);
+            float raw[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
+              float ry = part[buf][0][g][pa * kTileStride + pb];
+              ry += part[buf][1][g][pa * kTileStride + pb];
+              ry += part[buf][2][g][pa * kTileStride + pb];
+              ry += part[buf][3][g][pa * kTileStride + pb];
+              if (MASK && restart) ry = 0.0f;
+              raw[g] = (wxf[g] + ry) + bias_g[g];
+            }
+            if (MASK && restart) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
 #ifdef XS_PROFILE
-          asm volatile("" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
-          XS_GTICK(4);
+            asm volatile("" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
+            XS_GTICK(4);
 #endif
-          slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
-          float y = st[mt].y;
-          uint32_t hbits;
-          if (BF16) {
-            hbits = float_to_bf16_bits(y);
-          } else {
-            if (y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
-            hbits = __float_as_uint(y);
-          }
+            slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
+            float y = st[mt].y;
+            uint32_t hbits;
+            if (BF16) {
+              hbits = float_to_bf16_bits(y);
+            } else {
+              if (y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
+              hbits = __float_as_uint(y);
+            }
 #ifdef XS_PROFILE
-          asm volatile("" : "+v"(hbits));
-          XS_GTICK(5);
+            asm volatile("" : "+v"(hbits));
+            XS_GTICK(5);
 #endif
-          store_tile(t0 + u / MT, mt, hbits);
-          fetch(mask_c, mt, u / MT, u);  // iteration it + D, into the slot of this one
-          XS_GTICK(2);
-          stage(mask_c, (u + 1) % D, wxf, flag_now);
-          XS_GTICK(1);
+            store_tile(t0 + u / MT, mt, hbits);
+            XS_GTICK(2);
+            fetch(u, wxq[u], flq[u]);  // iteration it + D, into the slot of this one
+          }
         }
+      };
+      if (has_mask) gating_loop(std::integral_constant<bool, true>{});
+      else gating_loop(std::integral_constant<bool, false>{});
+    } else {
+      // ---- W.x and the reset flags travel from memory STRAIGHT INTO LDS (no registers), D - 1 iterations ahead, into a
+      //      ring of D slots per gating wave.  Nothing of a load in flight is visible to the compiler, so it cannot move or
+      //      copy a destination that has not landed, and the waits are counted by hand: exactly one load (two with a mask)
+      //      per iteration, loads and stores share one counter, and a wait the compiler places would be a wait for
+      //      everything.  A 16-byte load per lane: the wave's 16 (row, gate) pieces of 16 units land as
+      //      [row * 4 + gate][unit], which is how the lanes that gate them read them back.  Rows and units that do not
+      //      exist ask for an offset past the end of the buffer descriptor: zeros, no memory access.
+      constexpr int UPL = 16 / ESZ;                 // units a lane fetches (8 bf16 / 4 fp32)
+      constexpr int LPP = 16 / UPL;                 // lanes per piece
+      typedef typename std::conditional<BF16, uint16_t, uint32_t>::type wxe_t;
+      __shared__ __attribute__((aligned(16))) wxe_t wxring[4][D][16][16];  // [gating wave][slot][row * 4 + gate][unit]
+      __shared__ uint32_t flring[4][D][64];                                  // [gating wave][slot][lane]: the row's flag byte
+      constexpr uint32_t kPastEnd = 0xFFFFFF00u;    // (= the descriptors' size)
+      const int dl_piece = lane / LPP, dl_part = lane % LPP;
+      const bool dl_active = lane < 16 * LPP;       // (bf16: the lower half of the wave fetches)
+      uint32_t voff_wx[MT], voff_flag[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int row0 = rowbase + mt * 16 + 4 * gw;  // first row of this wave in the tile
+        const bool piece_ok = row0 + (dl_piece >> 2) < rend && a0 + dl_part * UPL < dh;
+        voff_wx[mt] = piece_ok ? (uint32_t)(((long long)(dl_piece >> 2) * p.wx_sb + (long long)(dl_piece & 3) * H + dl_part * UPL) * ESZ)
+                               : kPastEnd;
+        voff_flag[mt] = row0 + (lane >> 4) < rend ? (uint32_t)((long long)(lane >> 4) * flag_sb) : kPastEnd;
       }
-    };
-    if (has_mask) gating_loop(std::integral_constant<bool, true>{});
-    else gating_loop(std::integral_constant<bool, false>{});
+      const char *const wx_wave = reinterpret_cast<const char *>(p.wx) + (long long)(head * dh + a0) * ESZ;
+      // The offsets of the D / MT steps a round of D iterations fetches for (clamped to the last step: what the rounds
+      // past the end fetch is never looked at), kept as offsets that the scalar unit adds per iteration.
+      constexpr int NPF = D / MT;
+      long long pf_wx[NPF], pf_flag[NPF];
+      auto set_prefetch_steps = [&](int tfirst) {
+#pragma unroll
+        for (int d = 0; d < NPF; ++d) {
+          const int tp = tfirst + d < p.T ? tfirst + d : p.T - 1;
+          pf_wx[d] = (long long)tp * p.wx_st * ESZ;
+          pf_flag[d] = tp;
+        }
+      };
+      auto descriptor = [&](const void *base) {  // raw bytes from base, kPastEnd of them
+        const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+        return u32x4_t{uniform((uint32_t)a), uniform((uint32_t)(a >> 32) & 0xFFFFu), kPastEnd, 0x00020000u};
+      };
+      // (The wait states in front: the descriptor may sit in scalar registers that the compiler has just written with a
+      // vector instruction, e.g. the reload of a spilled scalar, and it does not look for that hazard inside a statement
+      // like this.  M0 = the LDS address of lane 0's bytes.)
+      auto fetch = [&](auto mask_c, int mt, int d, int slot) {  // row tile mt of step pf[d] -> ring slot
+        const uint32_t vw = voff_wx[mt], vf = voff_flag[mt];
+        const long long step_flag = pf_flag[d];
+        const char *src = wx_wave + (long long)(rowbase + mt * 16 + 4 * gw) * p.wx_sb * ESZ + pf_wx[d];
+        const u32x4_t rs = descriptor(src);
+        const uint32_t lds = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) wxe_t *)&wxring[gw][slot][0][0]));
+        if (dl_active)
+          asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                       :: "s"(lds), "v"(vw), "s"(rs) : "memory", "m0");
+        if (decltype(mask_c)::value) {
+          const unsigned char *sf = p.reset + (long long)(rowbase + mt * 16 + 4 * gw) * flag_sb + step_flag;
+          const u32x4_t fs = descriptor(sf);
+          const uint32_t fl = uniform((uint32_t)(unsigned long long)((__attribute__((address_space(3))) uint32_t *)&flring[gw][slot][0]));
+          asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ubyte %1, %2, 0 offen lds"
+                       :: "s"(fl), "v"(vf), "s"(fs) : "memory", "m0");
+        }
+      };
+      // W.x of the iteration in a ring slot -> the lanes that gate it.  Its loads have landed when no more than the loads
+      // of the D - 1 iterations fetched behind it are outstanding (the stores in between count as well, so this waits for
+      // a little more: operations that are several iterations old).
+      auto stage = [&](auto mask_c, int slot, float (&wxf)[4], uint32_t &flag) {
+        constexpr bool MASK = decltype(mask_c)::value;
+        asm volatile("s_waitcnt vmcnt(%[cnt])" :: [cnt] "n"((MASK ? 2 : 1) * (D - 1)) : "memory");
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint32_t wxbits = wxring[gw][slot][(lane >> 4) * 4 + g][pa];
+          wxf[g] = BF16 ? bf16_bits_to_float(wxbits) : __uint_as_float(wxbits);
+        }
+        flag = MASK ? (flring[gw][slot][lane] & 0xFFu) : 0u;
+        asm volatile("" : "+v"(wxf[0]), "+v"(wxf[1]), "+v"(wxf[2]), "+v"(wxf[3]), "+v"(flag));  // (here, not where they are used)
+      };
+      // Per iteration: barrier #it, the partial sums out of LDS, the gating, the tile's three stores, the fetch for
+      // iteration it + D into the ring slot just freed, and W.x of iteration it + 1 out of the ring, so that nothing of it
+      // is left to do behind the next barrier.  The memory instructions come late in the iteration on purpose: right behind
+      // the barrier the MFMA waves issue their requests for the next operand tile, and memory instructions of both kinds
+      // queue in the one texture path of the compute unit (measured: with the stores and the fetch of the previous tile
+      // moved up behind the barrier, 2.4 -> 3.0 us per step at head dim 512 and 3.5 -> 5.5 at 1024).
+      // (Two copies of the loop: calls without a mask run the one without the flag loads and the selects.)
+      auto gating_loop = [&](auto mask_c) {
+        constexpr bool MASK = decltype(mask_c)::value;
+        set_prefetch_steps(0);
+#pragma unroll
+        for (int j = 0; j < D; ++j) fetch(mask_c, j % MT, j / MT, j);
+        float wxf[4];
+        uint32_t flag_now;
+        stage(mask_c, 0, wxf, flag_now);
+        lds_barrier();  // prologue barrier
+        cross_xcd = cross_s != 0u;
+        for (int it0 = 0; it0 < NIT; it0 += D) {
+          const int t0 = it0 / MT;
+          set_prefetch_steps(t0 + D / MT);
+#pragma unroll
+          for (int u = 0; u < D; ++u) {
+            if (it0 + u >= NIT) break;  // (uniform)
+            const int mt = u % MT;
+            const int buf = u & 1;  // (D is even: the parity of the iteration)
+            XS_GTICK(3);
+            lds_barrier();  // barrier #it: the partial sums of iteration it are in LDS
+            XS_GTICK(0);
+            // a row that starts a document: zero state, and R.h counts as the +0 a zero operand row gives
+            const bool restart = MASK && flag_now != 0u;
+            float raw[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              // fixed summation order: wave 0 + wave 1 + wave 2 + wave 3
+              float ry = part[buf][0][g][pa * kTileStride + pb];
+              ry += part[buf][1][g][pa * kTileStride + pb];
+              ry += part[buf][2][g][pa * kTileStride + pb];
+              ry += part[buf][3][g][pa * kTileStride + pb];
+              if (MASK && restart) ry = 0.0f;
+              raw[g] = (wxf[g] + ry) + bias_g[g];
+            }
+            if (MASK && restart) st[mt] = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+#ifdef XS_PROFILE
+            asm volatile("" : "+v"(raw[0]), "+v"(raw[1]), "+v"(raw[2]), "+v"(raw[3]));
+            XS_GTICK(4);
+#endif
+            slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st[mt]);
+            float y = st[mt].y;
+            uint32_t hbits;
+            if (BF16) {
+              hbits = float_to_bf16_bits(y);
+            } else {
+              if (y != y) y = __uint_as_float(0x7FC00000u);  // keep the "not written yet" NaN pattern unique
+              hbits = __float_as_uint(y);
+            }
+#ifdef XS_PROFILE
+            asm volatile("" : "+v"(hbits));
+            XS_GTICK(5);
+#endif
+            store_tile(t0 + u / MT, mt, hbits);
+            fetch(mask_c, mt, u / MT, u);  // iteration it + D, into the slot of this one
+            XS_GTICK(2);
+            stage(mask_c, (u + 1) % D, wxf, flag_now);
+            XS_GTICK(1);
+          }
+        }
+      };
+      if (has_mask) gating_loop(std::integral_constant<bool, true>{});
+      else gating_loop(std::integral_constant<bool, false>{});
+    }
 #ifdef XS_PROFILE
     if (lane == 0 && member == 0 && gi == 0 && wave == NMW) {
       long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + 5 * 8;

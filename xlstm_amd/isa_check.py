@@ -116,6 +116,9 @@ def inflight_register_uses(listing: str) -> list:
             continue
         if not _is_code(ins):
             continue
+        if not in_asm and (ins.startswith("s_branch") or ins.startswith("s_endpgm")):
+            inflight = []  # (what follows in the listing is not what runs next)
+            continue
         if ins.startswith("s_waitcnt"):
             m = re.search(r"vmcnt\((\d+)\)", ins)
             if m:
