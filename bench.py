@@ -291,9 +291,11 @@ def phase_profile(device):
             "MFMA waves 0-3": {nm: [round(float(st[w][i] / n)) for w in range(4)] for i, nm in enumerate(mnames)},
             "MFMA waves: sum": [round(float(st[w][:6].sum() / n)) for w in range(4)],
             "gating wave 4": {"barrier": round(float(st[5][0] / n)), "partial sums out of LDS + sums": round(float(st[5][4] / n)),
-                              "gating": round(float(st[5][5] / n)), "3 stores + fetch": round(float(st[5][2] / n)),
-                              "W.x of the next iteration out of the ring": round(float(st[5][1] / n)),
-                              "loop top": round(float(st[5][3] / n)), "sum": round(float(st[5][:6].sum() / n))},
+                              "gating": round(float(st[5][5] / n)), "3 stores": round(float(st[5][2] / n)),
+                              "fetch of W.x D iterations ahead + loop top + wait for this iteration's W.x":
+                                  round(float(st[5][1] / n)),
+                              "W.x through the LDS corner": round(float(st[5][3] / n)),
+                              "sum": round(float(st[5][:6].sum() / n))},
         }
     return out
 
