@@ -35,7 +35,21 @@ namespace {
 //    instructions then always find the compute unit's one texture path busy;
 //  - the gating waves' stores and fetch moved up behind the barrier, under the latency of the partial sums: 5.5 / 3.0 /
 //    5.1, for the same reason (that is when the MFMA waves issue their requests);
-//  - a ring of 16 slots instead of 8 (twice as long for the stores to complete before a wait counts them): no change.
+//  - a ring of 16 slots instead of 8 (twice as long for the stores to complete before a wait counts them): no change;
+//  - the MFMA waves asking for the next tile at different times (wave w behind the first w/4 of its MFMAs, so that the
+//    requests of one wave leave while the other three multiply): 3.45 against 3.38; in two groups: 3.50.  The late waves
+//    then wait for the arrival instead (a request takes 1,200 cycles and more to come back from the other XCD);
+//  - no barrier in the loop (counters in LDS hand the sums over and the buffers back, one buffer per row tile) and the
+//    gating by ONE wave per row tile, four elements per lane (the sums are then 16-byte reads and W.x needs no
+//    staging), or by TWO waves per row tile, two elements per lane: the same bits, the gating waves busy a fifth of the
+//    time - and 5.0 to 5.3 us per step.  Timestamps of one workgroup and per-workgroup sums of all 256 showed why: h of
+//    a tile is stored 1,400 to 2,000 cycles behind the sums instead of 1,000 (one wave gates two or four elements),
+//    which is too late for the request that the MFMA waves issue one iteration ahead; every request then finds
+//    unwritten words and is repeated, a repeat costs a round trip inside the wave that should multiply, and all
+//    workgroups alike wait 1,900 cycles per iteration for their operand.  The step is a loop - MFMAs, sums through LDS,
+//    gating, store, the way to the other XCD, request, arrival test - that a tile's h goes round once, about 7,000 cycles,
+//    and four tiles are in flight: the roles as they are finish just early enough for the requests to be valid;
+//  - the two XCDs of a head group chosen as (i, i + 2) or (i, i + 4) instead of (i, i + 1): 3.37 and 3.30 against 3.34.
 //
 // Barrier #it means "the partial sums of iteration it are in LDS"; the gating waves reach it when they are done with
 // iteration it - 1.  The sums are formed in the same order as everywhere else: the same bits.
