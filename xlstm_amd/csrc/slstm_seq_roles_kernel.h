@@ -49,7 +49,7 @@ namespace {
 //    workgroups alike wait 1,900 cycles per iteration for their operand.  The step is a loop - MFMAs, sums through LDS,
 //    gating, store, the way to the other XCD, request, arrival test - that a tile's h goes round once, about 7,000 cycles,
 //    and four tiles are in flight: the roles as they are finish just early enough for the requests to be valid;
-//  - the two XCDs of a head group chosen as (i, i + 2) or (i, i + 4) instead of (i, i + 1): 3.37 and 3.30 against 3.34.
+//  - (the two XCDs of a head group are (i, i + 4): 3.30 against 3.34 with (i, i + 1) and 3.37 with (i, i + 2).)
 //
 // Barrier #it means "the partial sums of iteration it are in LDS"; the gating waves reach it when they are done with
 // iteration it - 1.  The sums are formed in the same order as everywhere else: the same bits.
