@@ -66,3 +66,33 @@ def test_four_row_tiles_packed_documents_equal_separate_calls(bf16, B, NH, dh):
     np.testing.assert_array_equal(h[:cut], ha)
     np.testing.assert_array_equal(h[cut:], hb)
     np.testing.assert_array_equal(s, sb)
+
+
+def test_rows_a_gigabyte_apart_fall_back_to_two_row_tiles():
+    """The kernel of four row tiles addresses four rows with 32-bit lane offsets.  A W.x whose rows lie a gigabyte apart
+    (a view into a larger buffer) runs through the kernel of two row tiles in more launches instead: same results."""
+    from xlstm_amd import functional as F
+    from tests._util import r_ext_to_kernel
+
+    bf16, B, T, NH, dh = True, 33, 3, 8, 512
+    H = NH * dh
+    print("case rows a gigabyte apart", B, T, NH, dh, flush=True)
+    wx, r, b, _ = make_problem(79, B, T, NH, dh, rscale=2.0, bf16=bf16)
+    h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
+    dev = torch.device("cuda:0")
+    stride = 1 << 29  # elements: 1 GiB of bf16 per row
+    try:
+        buf = torch.empty(B * stride, dtype=torch.bfloat16, device=dev)
+    except RuntimeError as e:  # (a box without 33 GiB to spare)
+        pytest.skip(f"cannot allocate the spread-out buffer: {e}")
+    wx_t = buf.as_strided((B, T, 4 * H), (stride, 4 * H, 1))
+    wx_t.copy_(torch.from_numpy(wx).to(dev))
+    ws = F.workspace_for(B, T, NH, dh, dev)
+    h, s = F.slstm_forward(wx_t, r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev), None, None, workspace=ws)
+    torch.cuda.synchronize()
+    status = F.read_status(ws)
+    assert status["rows_per_workgroup"] == 32 and status["launches"] == 2, status
+    _check(h.float().cpu().numpy(), s.cpu().numpy(), h_ref, s_ref, TOL_BF16, status)
+    # and the same call on a contiguous W.x takes the kernel of four row tiles
+    _, _, st4 = _run_hip(wx, r, b, None, None, bf16=bf16)
+    assert st4["rows_per_workgroup"] == 64, st4

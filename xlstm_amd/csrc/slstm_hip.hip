@@ -285,6 +285,15 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   const int max_groups_per_head = capacity / NHL;  // >= 1
   int MT = 1;
   while (MT < 4 && (tiles + MT - 1) / MT > max_groups_per_head) MT *= 2;
+  {
+    // The gating waves of the kernel of four row tiles address W.x, the mask and h_out as a scalar base plus a 32-bit
+    // offset per lane inside four rows / one row tile.  Where four rows span more than that (sequences of a gigabyte
+    // per row), the batch goes through the kernel of two row tiles in more launches instead.
+    const long long esz = bf16 ? 2 : 4;
+    const bool offsets_fit = 4ll * a->wx_stride_b * esz + 4ll * NH * dh * esz < 0xFFFFFF00ll &&
+                             (!a->reset || 4ll * a->reset_stride_b < 0xFFFFFF00ll) && 16ll * NH * dh * esz < (1ll << 31);
+    if (MT == 4 && !offsets_fit) MT = 2;
+  }
   int rows_per_wg = 16 * MT;
   if (MT == 1) {  // spare compute units: smaller row tiles, smaller exchanges
     for (int r = 4; r < 16; r *= 2)
@@ -296,14 +305,6 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
     const int bend = b0 + rows_per_launch < B ? b0 + rows_per_launch : B;
     // the variant without per-chunk masks: no K tail and, with several row tiles, no missing rows in this launch
     const bool full = dh == nch * 16 * epc && (MT == 1 || (bend - b0) % rows_per_wg == 0);
-    // (the gating waves of the kernel of four row tiles address W.x, the mask and h_out as a scalar base plus a 32-bit
-    // offset per lane inside four rows / one row tile)
-    if (MT == 4) {
-      const long long esz = bf16 ? 2 : 4;
-      if (4ll * a->wx_stride_b * esz + 4ll * NH * dh * esz >= 0xFFFFFF00ll || (a->reset && 4ll * a->reset_stride_b >= 0xFFFFFF00ll) ||
-          16ll * NH * dh * esz >= (1ll << 31))
-        return fail(XS_ERR_UNSUPPORTED, "row strides of wx / reset too large (four rows must span less than 4 GiB)");
-    }
     // the feeder fetches W.x in bursts where the prefetch waves cannot cover it: row tiles of 8 rows or more
     const bool burst = rows_per_wg >= 8;
     // four row tiles per workgroup: the kernel with MFMA waves and gating waves; one or two: the kernel in which
