@@ -52,7 +52,8 @@ namespace {
 //  - the arrival test left to the hardware (the MFMAs run on what arrived; an unwritten word is a NaN and makes the sums of
 //    its batch row NaNs; the words are looked at only then): the same bits, 400 cycles less in the MFMA waves - and 4.03
 //    against 3.33 (2.69 against 2.47 at head dim 512).  Waves that come round sooner ask sooner, find the tile
-//    unwritten more often, and then multiply twice: the pace of the loop is the peers' h, not the waves' work;
+//    unwritten more often, and then multiply twice: the pace of the loop is the peers' h, not the waves' work.  With
+//    the request moved behind a quarter, half, three quarters, all of the MFMAs: 4.05, 3.92, 3.80, 3.57;
 //  - (the two XCDs of a head group are (i, i + 4): 3.30 against 3.34 with (i, i + 1) and 3.37 with (i, i + 2).)
 //
 // Barrier #it means "the partial sums of iteration it are in LDS"; the gating waves reach it when they are done with
