@@ -111,16 +111,24 @@ def bench_decode(device, steps=1024, prefill=128):
     # eager loop: one xs_slstm_step call per token from Python through a StepPlan (arguments validated once)
     plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16, workspace=ws)
     stream = torch.cuda.current_stream().cuda_stream
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    t0 = time.perf_counter()
-    e0.record()
-    for t in range(steps):
-        plan(wx_dec[t], s_a, s_b, h2[t & 1], stream, h2[(t + 1) & 1] if t else None)
-        s_a, s_b = s_b, s_a
-    e1.record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    gpu_us = e0.elapsed_time(e1) * 1e3 / steps
+    # (three passes over the same 1024 steps from the same state, the median pass is reported: one pass is at the mercy
+    # of whatever else the box does in those 7 ms)
+    walls, gpus = [], []
+    for rep in range(3):
+        s_a.copy_(state)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        for t in range(steps):
+            plan(wx_dec[t], s_a, s_b, h2[t & 1], stream, h2[(t + 1) & 1] if t else None)
+            s_a, s_b = s_b, s_a
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+        gpus.append(e0.elapsed_time(e1) * 1e3 / steps)
+    wall = sorted(walls)[1]
+    gpu_us = sorted(gpus)[1]
     nbytes = algorithmic_bytes(B, 1, NH, dh, 2, 2, 2, with_mask=False) + 4 * B * H * 4  # state is read AND written
     eager_state = s_a.clone()
 
@@ -165,7 +173,8 @@ def bench_decode(device, steps=1024, prefill=128):
         traffic = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
     return {
         "workload": f"decode B={B} D={H} NH={NH}, {steps} consecutive T=1 steps after a {prefill}-token prefill",
-        "us_per_step": wall * 1e6 / steps, "gpu_us_per_step": gpu_us, "graph_us_per_step": graph_us,
+        "us_per_step": wall * 1e6 / steps, "gpu_us_per_step": gpu_us, "gpu_us_per_step_passes": gpus,
+        "graph_us_per_step": graph_us,
         "graph_equals_eager": graph_ok, "steps": steps,
         "finite": bool(torch.isfinite(s_a).all()),
         "roofline": {"bound": "hbm", "achieved": nbytes / (best_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
