@@ -7,7 +7,8 @@
 namespace {
 
 // With four row tiles per workgroup a tile is needed by the peers again only four iterations after it was computed, so
-// nothing in an iteration waits for another compute unit: an iteration is throughput, not latency.  The kernel with
+// an iteration does not wait for another compute unit as long as a tile's h gets round in less than four iterations
+// (across two XCDs it just does; see the measurements at the end of this comment).  The kernel with
 // the common roles (slstm_seq_kernel, MT = 4) still runs it as ONE chain per SIMD - operand tile out of LDS, 32
 // MFMAs, partial sums through LDS, barrier, gating with 9 transcendentals, staging - and the MFMA pipe idles 80 % of
 // the time.  Here the chain is cut in two and the halves of consecutive iterations run side by side, two waves per
