@@ -26,8 +26,8 @@ N0_WHOLE_TENSOR = 1  # vanilla rule, vanilla/slstm.py:25
 
 def build(force: bool = False) -> str:
     """Compile the oracle with gcc; returns the path of the shared object."""
-    src = os.path.join(_HERE, "slstm_oracle.c")
-    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < os.path.getmtime(src):
+    srcs = [os.path.join(_HERE, f) for f in ("slstm_oracle.c", "slstm_oracle_backward.c")]
+    if force or not os.path.exists(_SO) or os.path.getmtime(_SO) < max(os.path.getmtime(f) for f in srcs):
         subprocess.run(["make", "-C", _HERE, "-B" if force else "-s"], check=True,
                        stdout=subprocess.DEVNULL)
     return _SO
@@ -36,13 +36,15 @@ def build(force: bool = False) -> str:
 def _lib():
     global _LIB
     if _LIB is None:
-        if not os.path.exists(_SO):
-            build()
+        build()  # (no-op when the library is newer than its sources)
         lib = ctypes.CDLL(_SO)
         for name in ("slstm_oracle_forward_f64", "slstm_oracle_forward_f32"):
             fn = getattr(lib, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5
+        if hasattr(lib, "slstm_oracle_backward_f64"):  # (a library built before the backward oracle existed has none)
+            lib.slstm_oracle_backward_f64.restype = ctypes.c_int
+            lib.slstm_oracle_backward_f64.argtypes = [ctypes.c_void_p] * 11 + [ctypes.c_int] * 5
         _LIB = lib
     return _LIB
 
@@ -108,3 +110,24 @@ def slstm_forward_per_document(wx, r_ext, b_ext, reset, dtype=np.float64):
             h[lo:hi, b] = hd[:, 0]
             s[:, b] = sd[:, 0]
     return h, s
+
+
+def slstm_backward(wx, r_ext, b_ext, s0, reset, d_h, d_s_final=None, n0_rule=N0_PER_ELEMENT):
+    """Gradients of a loss with d loss / d h_out = ``d_h`` [T,B,H] (and d loss / d final state = ``d_s_final`` [4,B,H])
+    with respect to W.x [B,T,4H], R_ext [NH,dh,4,dh], b_ext [NH,4,dh] and the initial state [4,B,H], in float64, by
+    the rule of the reference's native kernel: the stabiliser m is a constant (slstm_pointwise.cu:118-196)."""
+    lib = _lib()
+    B, T = wx.shape[0], wx.shape[1]
+    NH, dh = r_ext.shape[0], r_ext.shape[1]
+    H = NH * dh
+    f64 = lambda a: None if a is None else np.ascontiguousarray(a, dtype=np.float64)
+    wx_, r_, b_, s0_, dh_, dsf_ = f64(wx), f64(r_ext), f64(b_ext), f64(s0), f64(d_h), f64(d_s_final)
+    rs_ = None if reset is None else np.ascontiguousarray(reset, dtype=np.uint8)
+    assert wx_.shape == (B, T, 4 * H) and dh_.shape == (T, B, H)
+    d_wx = np.zeros((B, T, 4 * H)); d_r = np.zeros((NH, dh, 4, dh)); d_b = np.zeros((NH, 4, dh)); d_s0 = np.zeros((4, B, H))
+    ptr = lambda a: None if a is None else a.ctypes.data_as(ctypes.c_void_p)
+    rc = lib.slstm_oracle_backward_f64(ptr(wx_), ptr(r_), ptr(b_), ptr(s0_), ptr(rs_), ptr(dh_), ptr(dsf_), ptr(d_wx),
+                                       ptr(d_r), ptr(d_b), ptr(d_s0), B, T, NH, dh, n0_rule)
+    if rc != 0:
+        raise MemoryError("slstm_oracle_backward_f64 failed")
+    return d_wx, d_r, d_b, d_s0
