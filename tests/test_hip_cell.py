@@ -23,7 +23,7 @@ def _cell_from(r_ext, b_ext, **kw):
     return cell.to("cuda:0").eval()
 
 
-@pytest.mark.parametrize("path", sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_"))), ids=lambda p: os.path.basename(p)[:-4])
+@pytest.mark.parametrize("path", sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_", "bwd_"))), ids=lambda p: os.path.basename(p)[:-4])
 def test_cell_reproduces_reference_vanilla_outputs(path):
     """Same inputs, same external parameters, same (output[B,NH,S,dh], state[4,B,H]) as the
     reference's vanilla cell wrote into tests/golden/."""

@@ -48,7 +48,7 @@ def _check(h, s, h_ref, s_ref, tol, status):
     assert es <= tol, f"state error {es:.3e} > {tol}"
 
 
-@pytest.mark.parametrize("path", sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_"))), ids=lambda p: os.path.basename(p)[:-4])
+@pytest.mark.parametrize("path", sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_", "bwd_"))), ids=lambda p: os.path.basename(p)[:-4])
 def test_reference_golden_vectors_f32(path):
     """The reference's own vanilla outputs (written by tests/golden/make_golden.py)."""
     z = np.load(path)

@@ -15,7 +15,7 @@ GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
 
 
 def _cases():
-    return sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_")))
+    return sorted(p for p in glob.glob(os.path.join(GOLDEN, "*.npz")) if not os.path.basename(p).startswith(("layer_", "ckpt_", "bwd_")))
 
 
 def _bnsh(h, NH):
