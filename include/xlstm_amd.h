@@ -245,6 +245,49 @@ typedef struct xs_norm_args {
 
 int xs_headwise_group_norm(const xs_norm_args *args);
 
+/*
+ * Backward pass of the cell (training), by the rule of the reference's native kernel: the stabiliser m is a
+ * constant of the differentiation (xlstm/blocks/slstm/src/cuda/slstm_pointwise.cu:118-196).  Two calls replace the
+ * reference's per-timestep launches (slstm_backward.cu:291-319) and the state history and gate cache its forward
+ * writes for them (slstm.cc:79-108); the forward entry points above store nothing for training.
+ *
+ * xs_slstm_backward_prepare  walks forward in time over raw = wx + ry + bias, where ry[t,b,h,g,a] =
+ *   sum_d y_{t-1}[b,h,d] * r[h][g*dh+a][d] is given for all steps at once (one batched GEMM over the outputs of the
+ *   forward call, shifted by one step, rows that start a document zeroed), and writes nine float32 coefficients per
+ *   step and element into coef [T,B,9,H].
+ * xs_slstm_backward          one launch for all T steps, reverse in time: d_wx [B,T,4,NH,dh] (float32, the gradient
+ *   with respect to the raw gates: the gradient of wx, and with the outputs what the gradients of R and the bias are
+ *   sums of, slstm_backward.cu:381-386, 52-108) and d_s0 [4,B,H] (the m part is zero).
+ *
+ * dtype is the type of wx, d_h and r_t (XS_F32 or XS_BF16).  r_t is R transposed - element (input unit d, gate
+ * unit k = g*dh + a) of head h is the reference's external view recurrent_kernel[h][d][g][a] (cell.py:234-242) -
+ * tiled as MFMA operands: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC] with EPC = 16 bytes of elements (8 bf16, 4 f32)
+ * and KC = 4*EPC, so that what the 64 lanes of a wave load for one k-step is 1 KiB in a row.  Head dims: 64, 128, 256.
+ * The caller owns every buffer; both calls only enqueue kernels on `stream`.
+ */
+typedef struct xs_slstm_bwd_args {
+  int32_t B, T, NH, dh;
+  int32_t dtype;
+  const void *wx;            /* [B,T,4,NH,dh], strides in elements, innermost 4*H contiguous (prepare) */
+  int64_t wx_stride_b, wx_stride_t;
+  const float *ry;           /* [T,B,NH,4,dh] (prepare) */
+  const float *bias;         /* [NH,4,dh] (prepare) */
+  const float *s0;           /* [4,B,H] or NULL (prepare) */
+  const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */
+  int64_t reset_stride_b;
+  float *coef;               /* [T,B,9,H]: written by prepare, read by backward */
+  const void *d_h;           /* [T,B,H]: gradient with respect to h_out (backward) */
+  const float *d_s_final;    /* [4,B,H] or NULL: gradient with respect to the final state; y, c, n are used (backward) */
+  const void *r_t;           /* (backward) */
+  float *d_wx;               /* [B,T,4,NH,dh], strides in elements (backward) */
+  int64_t d_wx_stride_b, d_wx_stride_t;
+  float *d_s0;               /* [4,B,H] (backward) */
+  void *stream;
+} xs_slstm_bwd_args;
+
+int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);
+int xs_slstm_backward(const xs_slstm_bwd_args *args);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,123 @@
+"""GPU parity of the backward pass (xs_slstm_backward_prepare + xs_slstm_backward, through ``functional.slstm_backward``
+and through the cell's autograd) against the float64 backward oracle, which the reference's own autograd gradients pin
+(tests/test_oracle_backward.py).  Tolerances: float32 1e-5, bfloat16 2e-2, relative to the largest entry of a gradient
+(at least 1), the bars of the forward tests."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import slstm_oracle as so
+from tests._util import geometric_reset_mask, make_problem, r_ext_to_kernel
+
+pytestmark = pytest.mark.gpu
+
+
+def _rel(a, g):
+    return float(np.abs(a - g).max() / max(1.0, np.abs(g).max()))
+
+
+CASES = [
+    # bf16, B, T, NH, dh, masked + state
+    (False, 3, 7, 2, 64, False),
+    (False, 5, 9, 2, 64, True),
+    (False, 20, 6, 2, 128, True),     # two row tiles, the second ragged
+    (False, 4, 12, 4, 256, True),
+    (False, 1, 1, 1, 64, False),      # one step
+    (False, 33, 40, 2, 128, True),
+    (True, 5, 9, 2, 64, True),
+    (True, 16, 10, 4, 256, True),     # config 2's cell, a few steps
+    (True, 40, 33, 8, 128, True),
+    (True, 8, 64, 4, 256, False),
+]
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES)
+def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked):
+    from xlstm_amd import functional as F
+
+    print("case backward", bf16, B, T, NH, dh, masked, flush=True)
+    H = NH * dh
+    wx, r, b, s0 = make_problem(91, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=masked)
+    reset = geometric_reset_mask(7, B, T, max(2, T // 2)) if masked else None
+    if reset is not None:
+        reset[0, 0] = 0  # one row that uses the supplied state
+    rng = np.random.default_rng(92)
+    d_h = rng.standard_normal((T, B, H)).astype(np.float32)
+    d_sf = rng.standard_normal((4, B, H)).astype(np.float32)
+    d_sf[3] = 0.0
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev)
+    if bf16:
+        wx_t = wx_t.bfloat16()
+        d_h = torch.from_numpy(d_h).bfloat16().float().numpy()
+        r = torch.from_numpy(r).bfloat16().float().numpy()  # the forward rounds R to bf16; give the oracle the same R
+    r_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev)
+    b_t = torch.from_numpy(b).to(dev)
+    s0_t = torch.from_numpy(s0).to(dev) if s0 is not None else None
+    m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
+    h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
+    d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), torch.from_numpy(d_sf).to(dev))
+    torch.cuda.synchronize()
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
+    o_r_k = r_ext_to_kernel(torch.from_numpy(o_r)).numpy()
+    tol = 2e-2 if bf16 else 1e-5
+    errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), o_r_k), d_b=_rel(d_b.cpu().numpy(), o_b),
+                d_s0=_rel(d_s0.cpu().numpy(), o_s0))
+    print(errs, flush=True)
+    assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
+
+
+def test_packed_rows_have_the_gradients_of_their_documents():
+    """A reset cuts the recurrence: the gradients of a packed batch are those of the two halves run alone."""
+    from xlstm_amd import functional as F
+
+    B, T, NH, dh, cut = 6, 11, 2, 64, 5
+    H = NH * dh
+    wx, r, b, _ = make_problem(93, B, T, NH, dh, rscale=2.0)
+    dev = torch.device("cuda:0")
+    wx_t, r_t, b_t = torch.from_numpy(wx).to(dev), r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    mask = torch.zeros(B, T, dtype=torch.uint8, device=dev)
+    mask[:, 0] = 1
+    mask[:, cut] = 1
+    d_h = torch.randn(T, B, H, generator=torch.Generator().manual_seed(5)).to(dev)
+    h, _ = F.slstm_forward(wx_t, r_t, b_t, None, mask)
+    whole = F.slstm_backward(wx_t, r_t, b_t, None, mask, h, d_h)
+    parts = []
+    for lo, hi in ((0, cut), (cut, T)):
+        hp, _ = F.slstm_forward(wx_t[:, lo:hi], r_t, b_t)
+        parts.append(F.slstm_backward(wx_t[:, lo:hi], r_t, b_t, None, None, hp, d_h[lo:hi].contiguous()))
+    assert torch.equal(whole[0][:, :cut], parts[0][0]) and torch.equal(whole[0][:, cut:], parts[1][0])
+    torch.testing.assert_close(whole[1], parts[0][1] + parts[1][1], rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(whole[2], parts[0][2] + parts[1][2], rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", 1e-5), ("bfloat16", 2e-2)])
+def test_cell_autograd_matches_the_oracle(dtype, tol):
+    """loss.backward() through ``sLSTMCell(backend="hip")``: gradients of the input, the parameters (in the reference's
+    external views) and the initial state for a loss that is a linear form of the output in its public BNSH layout."""
+    from tests.test_hip_cell import _cell_from
+
+    B, T, NH, dh = 3, 8, 2, 64
+    H = NH * dh
+    bf16 = dtype == "bfloat16"
+    wx, r, b, s0 = make_problem(94, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=True)
+    if bf16:
+        r = torch.from_numpy(r).bfloat16().float().numpy()
+        s0 = torch.from_numpy(s0).bfloat16().float().numpy()
+    cell = _cell_from(r, b, dtype=dtype).train()
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    x = torch.from_numpy(wx).cuda().to(tdt).requires_grad_(True)
+    st = torch.from_numpy(s0).cuda().to(tdt).requires_grad_(True)
+    out, _ = cell(x, st)                                   # [B, NH, T, dh]
+    w = torch.randn(out.shape, generator=torch.Generator().manual_seed(6)).cuda()
+    if bf16:
+        w = w.bfloat16().float()
+    (out.float() * w).sum().backward()
+    d_h = w.permute(2, 0, 1, 3).reshape(T, B, H).cpu().numpy()
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, None, d_h, None)
+    d_r_ext = cell._recurrent_kernel_int2ext(cell._recurrent_kernel_.grad).float().cpu().numpy()
+    d_b_ext = cell._bias_int2ext(cell._bias_.grad).float().cpu().numpy()
+    errs = dict(d_wx=_rel(x.grad.float().cpu().numpy(), o_wx), d_r=_rel(d_r_ext, o_r), d_b=_rel(d_b_ext, o_b),
+                d_s0=_rel(st.grad.float().cpu().numpy()[:3], o_s0[:3]))
+    print(errs, flush=True)
+    assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs

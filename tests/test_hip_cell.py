@@ -192,12 +192,12 @@ def test_float16_input_is_computed_in_float32_and_rounded_back():
     assert max_err(out.float().cpu().numpy(), h_ref) <= 1e-3
 
 
-def test_backward_raises_forward_only():
+def test_backward_raises_for_head_dims_without_backward_kernels():
     wx, r, b, _ = make_problem(24, 1, 2, 1, 16)
     cell = _cell_from(r, b, dtype="float32").train()
     x = torch.from_numpy(wx).cuda().requires_grad_(True)
     out, _ = cell(x)
-    with pytest.raises(RuntimeError, match="forward/inference only"):
+    with pytest.raises(RuntimeError, match="backward pass for head dims"):
         out.sum().backward()
 
 

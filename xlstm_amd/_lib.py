@@ -52,6 +52,30 @@ class SlstmArgs(ctypes.Structure):
     ]
 
 
+class SlstmBwdArgs(ctypes.Structure):
+    """Mirror of ``xs_slstm_bwd_args``."""
+
+    _fields_ = [
+        ("B", ctypes.c_int32), ("T", ctypes.c_int32), ("NH", ctypes.c_int32), ("dh", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("wx", ctypes.c_void_p),
+        ("wx_stride_b", ctypes.c_int64), ("wx_stride_t", ctypes.c_int64),
+        ("ry", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("s0", ctypes.c_void_p),
+        ("reset", ctypes.c_void_p),
+        ("reset_stride_b", ctypes.c_int64),
+        ("coef", ctypes.c_void_p),
+        ("d_h", ctypes.c_void_p),
+        ("d_s_final", ctypes.c_void_p),
+        ("r_t", ctypes.c_void_p),
+        ("d_wx", ctypes.c_void_p),
+        ("d_wx_stride_b", ctypes.c_int64), ("d_wx_stride_t", ctypes.c_int64),
+        ("d_s0", ctypes.c_void_p),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
 class ConvArgs(ctypes.Structure):
     """Mirror of ``xs_conv_args``."""
 
@@ -139,6 +163,9 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmArgs)]
+    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.POINTER(SlstmBwdArgs)]
     lib.xs_causal_conv_silu.restype = ctypes.c_int
     lib.xs_causal_conv_silu.argtypes = [ctypes.POINTER(ConvArgs)]
     lib.xs_headwise_gates.restype = ctypes.c_int

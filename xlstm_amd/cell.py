@@ -168,9 +168,12 @@ class sLSTMCellConfig:
         self.num_states = rnn_function_registry[self.function]["states"]
 
 
+BACKWARD_HEAD_DIMS = (64, 128, 256)  # what xs_slstm_backward covers
+
+
 class _ForwardOnly(torch.autograd.Function):
-    """Identity on (h, state) whose backward raises: the hip backend has no BPTT kernels
-    (the reference's are slstm_backward.cu, out of this engine's scope)."""
+    """Identity on (h, state) whose backward raises: for the head dims the backward kernels of the hip backend do
+    not cover, a backward pass fails loudly instead of silently yielding no gradient."""
 
     @staticmethod
     def forward(ctx, h, s, *deps):
@@ -179,8 +182,33 @@ class _ForwardOnly(torch.autograd.Function):
     @staticmethod
     def backward(ctx, *grads):
         raise RuntimeError(
-            "sLSTMCell backend 'hip' is forward/inference only; use the reference's 'cuda' or 'vanilla' backend to train"
+            f"sLSTMCell backend 'hip' has a backward pass for head dims {BACKWARD_HEAD_DIMS} only; "
+            "use the reference's 'cuda' or 'vanilla' backend to train this shape"
         )
+
+
+class _CellFunction(torch.autograd.Function):
+    """Joins the results of a forward call of the engine to the autograd graph.  The backward runs the engine's two
+    backward kernels (``functional.slstm_backward``): the gradient by the rule of the reference's native kernel
+    (``slstm_pointwise.cu:118-196``; what ``sLSTMFunc.backward`` returns, ``slstm.cc:137-304``).  ``h`` and ``s`` are
+    what the forward call returned for ``x, r, bias, state, mask``; nothing else is stored for the backward."""
+
+    @staticmethod
+    def forward(ctx, x, r, bias, state, h, s, mask, num_heads):
+        ctx.save_for_backward(x, r, bias, h, *(() if state is None else (state,)))
+        ctx.mask, ctx.num_heads = mask, num_heads
+        return h.view_as(h), s.view_as(s)
+
+    @staticmethod
+    def backward(ctx, d_h, d_s):
+        x, r, bias, h = ctx.saved_tensors[:4]
+        state = ctx.saved_tensors[4] if len(ctx.saved_tensors) > 4 else None
+        NH, dh = ctx.num_heads, r.shape[2]
+        d_wx, d_r, d_bias, d_s0 = F_hip.slstm_backward(
+            x.detach(), r.detach(), bias.detach().view(NH, 4, dh), None if state is None else state.detach(), ctx.mask,
+            h, d_h, d_s)
+        return (d_wx.to(x.dtype), d_r.to(r.dtype), d_bias.reshape(bias.shape).to(bias.dtype),
+                None if state is None else d_s0.to(state.dtype), None, None, None, None)
 
 
 class _Runtime:
@@ -462,10 +490,13 @@ class sLSTMCell_hip(nn.Module):
             self._watch(ws)
         if torch.is_grad_enabled() and (
             input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
+            or (state is not None and state.requires_grad)
         ):
-            # forward-only engine: the results join the autograd graph only so that a
-            # backward pass through them fails loudly instead of silently yielding no gradient
-            h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
+            if self.head_dim in BACKWARD_HEAD_DIMS and x.is_cuda:
+                h, s = _CellFunction.apply(x, self._recurrent_kernel_, self._bias_, state, h, s, reset_mask,
+                                           self.config.num_heads)
+            else:
+                h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
         output = self._permute_output(h)
         if torch.is_autocast_enabled():
             return output, s

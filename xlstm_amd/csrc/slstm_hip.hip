@@ -33,6 +33,7 @@
 #include "slstm_step_kernel.h"
 #include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
+#include "slstm_backward_kernels.h"
 
 // ---------------------------------------------------------------------------
 // Scratch of the entry point that allocates nothing (xs_slstm_forward_static): status block, placement words and
@@ -374,6 +375,59 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   return XS_OK;
 }
 
+// ---- backward pass: the forward walk that leaves the coefficients, and the reverse-time kernel
+int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
+  if (a->dtype != XS_F32 && a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
+  if (a->dh != 64 && a->dh != 128 && a->dh != 256) return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256)", a->dh);
+  if (a->B == 0 || a->T == 0) return XS_OK;
+  const bool bf16 = a->dtype == XS_BF16;
+  const long long H = (long long)a->NH * a->dh;
+  if (!a->coef) return fail(XS_ERR_NULL, "coef is required");
+  if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
+  hipStream_t stream = (hipStream_t)a->stream;
+  if (prepare) {
+    if (!a->wx || !a->ry || !a->bias) return fail(XS_ERR_NULL, "wx, ry and bias are required");
+    if (a->wx_stride_t < 4 * H || (a->B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");
+    BwdPrepParams p;
+    p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
+    p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
+    p.ry = a->ry; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
+    const long long blocks = ((long long)a->B * H + 255) / 256;
+    if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
+    hipLaunchKernelGGL(bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+  } else {
+    if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
+    if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");
+    if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
+    BwdParams p;
+    p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
+    p.coef = a->coef; p.d_h = a->d_h; p.d_s_final = a->d_s_final; p.r_t = a->r_t;
+    p.reset = a->reset; p.reset_sb = a->reset_stride_b;
+    p.d_wx = a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t; p.d_s0 = a->d_s0;
+    void (*kern)(BwdParams) = nullptr;
+    int waves = 0;
+#ifndef XS_BWD_NB256
+#define XS_BWD_NB256 2
+#endif
+    if (a->dh == 64) { kern = bf16 ? slstm_bwd_kernel<true, 1, 4> : slstm_bwd_kernel<false, 1, 4>; waves = 4; }
+    else if (a->dh == 128) { kern = bf16 ? slstm_bwd_kernel<true, 1, 8> : slstm_bwd_kernel<false, 1, 8>; waves = 8; }
+    else { kern = bf16 ? slstm_bwd_kernel<true, XS_BWD_NB256, 16 / XS_BWD_NB256> : slstm_bwd_kernel<false, XS_BWD_NB256, 16 / XS_BWD_NB256>; waves = 16 / XS_BWD_NB256; }
+    const int esz = bf16 ? 2 : 4;
+    const size_t lds = (size_t)16 * (4 * a->dh + 16 / esz) * esz;  // the delta tile
+    if (lds > 64 * 1024) {
+      const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel: %zu bytes of LDS refused: %s", lds, hipGetErrorString(ea));
+    }
+    const long long blocks = (long long)a->NH * ((a->B + 15) / 16);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(waves * 64), lds, stream, p);
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 int run_conv(const xs_conv_args *a) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->D <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d D=%d", a->B, a->T, a->D);
@@ -571,6 +625,16 @@ int xs_slstm_step(const xs_slstm_args *args) {
   const int rc = validate(args, true);
   if (rc != XS_OK) return rc;
   return run_step(args);
+}
+
+int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args) {
+  g_err[0] = 0;
+  return run_backward(args, true);
+}
+
+int xs_slstm_backward(const xs_slstm_bwd_args *args) {
+  g_err[0] = 0;
+  return run_backward(args, false);
 }
 
 int xs_causal_conv_silu(const xs_conv_args *args) {

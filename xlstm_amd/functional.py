@@ -42,6 +42,100 @@ def read_status(workspace: torch.Tensor) -> dict:
     return {k: getattr(st, k) for k, _ in _lib.SlstmStatus._fields_ if k != "reserved"}
 
 
+def slstm_backward(
+    wx: torch.Tensor,
+    r: torch.Tensor,
+    bias: torch.Tensor,
+    s0: Optional[torch.Tensor],
+    reset_mask: Optional[torch.Tensor],
+    h_out: torch.Tensor,
+    d_h: torch.Tensor,
+    d_s_final: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
+    differentiation, ``slstm_pointwise.cu:118-196``).
+
+    ``wx, r, bias, s0, reset_mask`` are the arguments of the forward call, ``h_out[S,B,H]`` what it returned, ``d_h`` the
+    gradient with respect to ``h_out`` and ``d_s_final[4,B,H]`` (optional) with respect to the final state.  Returns
+    ``(d_wx[B,S,4H] float32, d_r[NH,4*dh,dh], d_bias[NH,4,dh], d_s0[4,B,H])``.
+
+    Two kernels of the engine (``xs_slstm_backward_prepare``, ``xs_slstm_backward``) around three plain library GEMMs and
+    a reduction: ``R.h_{t-1}`` for all steps at once in front, and the gradients of R and the bias, which are sums over
+    all steps of products of the gate deltas with the outputs, behind.
+    """
+    lib = _lib.load()
+    _require_cuda("wx", wx)
+    NH, dh = int(r.shape[0]), int(r.shape[2])
+    H = NH * dh
+    B, T = int(wx.shape[0]), int(wx.shape[1])
+    if wx.dtype not in _DTYPE_CODE:
+        raise TypeError(f"wx dtype {wx.dtype} not supported by the hip backend (float32 or bfloat16)")
+    bf16 = wx.dtype == torch.bfloat16
+    dev = wx.device
+    if tuple(h_out.shape) != (T, B, H) or tuple(d_h.shape) != (T, B, H):
+        raise ValueError(f"h_out and d_h must be [S, B, H] = {(T, B, H)}")
+    if wx.stride(2) != 1 or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H):
+        wx = wx.contiguous()
+    bias = bias.to(torch.float32).contiguous()
+    if s0 is not None:
+        s0 = s0.to(torch.float32).contiguous()
+    if reset_mask is not None:
+        reset_mask = (reset_mask != 0).to(torch.uint8).contiguous()
+    # the operand of every step as the forward saw it: y_{t-1} (the initial y in front), rows that start a document zero,
+    # rounded like the forward's operands
+    y_prev = torch.empty((T, B, H), dtype=torch.float32, device=dev)
+    y_prev[0] = s0[0] if s0 is not None else 0.0
+    if T > 1:
+        y_prev[1:] = h_out[:-1]
+    if reset_mask is not None:
+        y_prev.masked_fill_(reset_mask.t().bool().unsqueeze(-1), 0.0)
+    r32 = r.to(torch.float32)
+    if bf16:
+        y_prev = y_prev.bfloat16().float()
+        r32 = r32.bfloat16().float()
+    yp = y_prev.view(T * B, NH, dh).transpose(0, 1)                      # [NH, T*B, dh]
+    ry = torch.bmm(yp, r32.transpose(1, 2)).transpose(0, 1).contiguous()  # [T*B, NH, 4*dh] = [T,B,NH,4,dh]
+    coef = torch.empty((T, B, 9, H), dtype=torch.float32, device=dev)
+    d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
+    d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
+    # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
+    epc = 8 if bf16 else 4
+    r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
+           .reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).permute(0, 1, 3, 4, 2, 5).contiguous())
+    d_h = d_h.to(wx.dtype).contiguous()
+    if d_s_final is not None:
+        d_s_final = d_s_final.to(torch.float32).contiguous()
+
+    a = _lib.SlstmBwdArgs()
+    a.B, a.T, a.NH, a.dh = B, T, NH, dh
+    a.dtype = _DTYPE_CODE[wx.dtype]
+    a.wx = wx.data_ptr()
+    a.wx_stride_b, a.wx_stride_t = wx.stride(0), wx.stride(1)
+    a.ry = ry.data_ptr()
+    a.bias = bias.data_ptr()
+    a.s0 = s0.data_ptr() if s0 is not None else None
+    a.reset = reset_mask.data_ptr() if reset_mask is not None else None
+    a.reset_stride_b = reset_mask.stride(0) if reset_mask is not None else 0
+    a.coef = coef.data_ptr()
+    a.d_h = d_h.data_ptr()
+    a.d_s_final = d_s_final.data_ptr() if d_s_final is not None else None
+    a.r_t = r_t.data_ptr()
+    a.d_wx = d_wx.data_ptr()
+    a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
+    a.d_s0 = d_s0.data_ptr()
+    a.stream = torch.cuda.current_stream(dev).cuda_stream
+    with torch.cuda.device(dev):
+        for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
+            rc = fn(ctypes.byref(a))
+            if rc != 0:
+                raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+    # d R[h][g dh + a][d] = sum over steps and rows of delta[b,t,g,h,a] * y_{t-1}[b,h,d]; d bias = sum of delta
+    dl = d_wx.view(B, T, 4, NH, dh).permute(3, 2, 4, 1, 0).reshape(NH, 4 * dh, T * B)  # [NH, 4*dh, (t, b)]
+    d_r = torch.bmm(dl, yp)                                                            # [NH, 4*dh, dh]
+    d_bias = d_wx.view(B * T, 4, NH, dh).sum(0).transpose(0, 1).contiguous()
+    return d_wx, d_r, d_bias, d_s0
+
+
 def read_phase_stamps(workspace: torch.Tensor) -> torch.Tensor:
     """Per-phase cycle sums that a library built with ``-DXS_PROFILE`` leaves behind a sequence call: ``[6, 8]`` int64,
     one row per wave slot of workgroup 0 (which waves and phases: see ``bench.py --phase-profile``).  The product
