@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 6
+#define XS_ABI_VERSION 7
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };

@@ -32,6 +32,19 @@ def test_abi_version_and_struct_mirror():
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
+    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8  # 5 int32 (+4 padding), then 17 8-byte fields
+
+
+def test_backward_argument_errors_without_touching_the_gpu():
+    lib = _lib.load()
+    assert lib.xs_slstm_backward(None) == -1 and lib.xs_slstm_backward_prepare(None) == -1
+    a = _lib.SlstmBwdArgs()
+    a.B, a.T, a.NH, a.dh, a.dtype = 2, 3, 2, 48, _lib.XS_F32
+    assert lib.xs_slstm_backward(ctypes.byref(a)) == -5 and b"head dim 48" in lib.xs_last_error()
+    a.dh = 64
+    assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -1  # coef missing
+    a.dtype = 5
+    assert lib.xs_slstm_backward(ctypes.byref(a)) == -3
 
 
 def test_argument_errors_without_touching_the_gpu():

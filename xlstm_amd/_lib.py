@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 
 XS_F32, XS_BF16 = 0, 1
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 EXPORTS = (
     "xs_abi_version",
@@ -23,6 +23,8 @@ EXPORTS = (
     "xs_slstm_forward",
     "xs_slstm_step",
     "xs_slstm_forward_static",
+    "xs_slstm_backward_prepare",
+    "xs_slstm_backward",
     "xs_causal_conv_silu",
     "xs_headwise_gates",
     "xs_headwise_group_norm",
