@@ -184,6 +184,49 @@ def bench_decode(device, steps=1024, prefill=128):
     }
 
 
+def bench_backward(device, iters=3):
+    """The backward pass at BASELINE config 2 (B=16, T=2048, D=1024, NH=4, bf16, packed documents): the whole call
+    (three library GEMMs and a reduction around the engine's two kernels) and the two kernels by HIP events."""
+    import numpy as np
+    import torch
+
+    from tests._util import geometric_reset_mask
+    from xlstm_amd import functional as F
+
+    B, T, NH, dh = 16, 2048, 4, 256
+    H = NH * dh
+    torch.manual_seed(0)
+    wx = torch.randn(B, T, 4 * H, device=device).bfloat16()
+    r = (torch.rand(NH, 4 * dh, dh, device=device) * 2 - 1) / np.sqrt(H)
+    bias = torch.zeros(NH, 4, dh, device=device)
+    bias[:, 1] = torch.linspace(3, 6, dh, device=device)
+    mask = torch.from_numpy(geometric_reset_mask(0, B, T, 512)).to(device)
+    h, _ = F.slstm_forward(wx, r, bias, None, mask)
+    d_h = torch.randn(T, B, H, device=device).bfloat16()
+    total, prep, rev = [], [], []
+    for i in range(iters + 1):
+        tm = {}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = F.slstm_backward(wx, r, bias, None, mask, h, d_h, timings=tm)
+        torch.cuda.synchronize()
+        if i:
+            total.append((time.perf_counter() - t0) * 1e3)
+            ev = tm["events"]
+            prep.append(ev[0].elapsed_time(ev[1]))
+            rev.append(ev[1].elapsed_time(ev[2]))
+    rev_ms = float(np.median(rev))
+    # what the reverse kernel has to move per step and element: nine coefficients and the four gate deltas in float32,
+    # the output gradient in bf16; R transposed once
+    nbytes = (9 * 4 + 4 * 4 + 2) * B * T * H + NH * 4 * dh * dh * 2
+    return {"workload": "backward pass at config 2: B=16 T=2048 D=1024 NH=4 bf16, documents mean 512",
+            "ms": float(np.median(total)), "prepare_kernel_ms": float(np.median(prep)), "reverse_kernel_ms": rev_ms,
+            "tokens_per_s": B * T / (float(np.median(total)) * 1e-3), "finite": bool(torch.isfinite(out[0]).all()),
+            "roofline": {"bound": "hbm", "achieved": nbytes / (rev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": nbytes / (rev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                         "kernel": "slstm_bwd_kernel<bf16,NB=2,NW=8>", "algorithmic_bytes_per_launch": nbytes}}
+
+
 def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
     """Times one forward call of the cell at another BASELINE shape (median of `iters`)."""
     import numpy as np
@@ -444,6 +487,8 @@ def main():
                          "the bf16 MFMA roofline (profiling runs)")
     ap.add_argument("--small-batch-only", action="store_true",
                     help="only time the sequence kernel at B = 1, 2, 4 (head dims 128 and 256) and the reference test's shape")
+    ap.add_argument("--backward-only", action="store_true",
+                    help="only time the backward pass at config 2 (its own JSON line)")
     ap.add_argument("--phase-profile", action="store_true",
                     help="per-phase cycle tables of the sequence kernels from the measurement build of the library "
                          "(python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so)")
@@ -483,6 +528,9 @@ def main():
         return
     if args.small_batch_only:
         print(json.dumps({"small_batch": bench_small_batch(device)}))
+        return
+    if args.backward_only:
+        print(json.dumps({"backward": bench_backward(device, iters=max(1, min(args.steps, 5)))}))
         return
     if args.config5_only:
         c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=max(1, min(args.steps, 5)))
@@ -560,6 +608,7 @@ def main():
             bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=2),
             bench_config(device, "reference test shape: B=1 T=1 NH=4 dh=16 fp32 (one step, the step kernel)", 1, 1, 4, 16, False, 0, iters=20),
         ]
+        out["backward"] = bench_backward(device)
     if args.config4:
         out["config4"] = bench_config4(device)
     if args.layer:

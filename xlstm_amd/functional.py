@@ -51,6 +51,7 @@ def slstm_backward(
     h_out: torch.Tensor,
     d_h: torch.Tensor,
     d_s_final: Optional[torch.Tensor] = None,
+    timings: Optional[dict] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -61,7 +62,8 @@ def slstm_backward(
 
     Two kernels of the engine (``xs_slstm_backward_prepare``, ``xs_slstm_backward``) around three plain library GEMMs and
     a reduction: ``R.h_{t-1}`` for all steps at once in front, and the gradients of R and the bias, which are sums over
-    all steps of products of the gate deltas with the outputs, behind.
+    all steps of products of the gate deltas with the outputs, behind.  ``timings`` (a dict) receives three events around
+    the two kernels.
     """
     lib = _lib.load()
     _require_cuda("wx", wx)
@@ -124,11 +126,19 @@ def slstm_backward(
     a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
     a.d_s0 = d_s0.data_ptr()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
+    marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
+            if timings is not None:
+                marks.append(torch.cuda.Event(enable_timing=True))
+                marks[-1].record()
             rc = fn(ctypes.byref(a))
             if rc != 0:
                 raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+        if timings is not None:
+            marks.append(torch.cuda.Event(enable_timing=True))
+            marks[-1].record()
+            timings["events"] = marks  # prepare = [0] -> [1], reverse kernel = [1] -> [2]
     # d R[h][g dh + a][d] = sum over steps and rows of delta[b,t,g,h,a] * y_{t-1}[b,h,d]; d bias = sum of delta
     dl = d_wx.view(B, T, 4, NH, dh).permute(3, 2, 4, 1, 0).reshape(NH, 4 * dh, T * B)  # [NH, 4*dh, (t, b)]
     d_r = torch.bmm(dl, yp)                                                            # [NH, 4*dh, dh]
