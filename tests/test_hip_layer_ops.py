@@ -225,20 +225,26 @@ def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
     assert torch.equal(st_f2["conv_state"][0], st_p2["conv_state"][0])
 
 
-def test_layer_under_autograd_keeps_the_pytorch_ops_and_backward_raises():
-    """The engine's kernels record no graph: with grad enabled the layer must not cut the graph silently."""
+def test_layer_under_autograd_keeps_the_pytorch_ops_and_trains_through_the_cell():
+    """The engine's layer kernels record no graph: with grad enabled the layer keeps its PyTorch ops around the cell,
+    and the cell's own backward kernels carry the gradient (head dims 64, 128, 256); other head dims raise."""
     from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
 
     torch.manual_seed(12)
     layer = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=4, backend="hip")).to(DEV).bfloat16()
-    x = torch.randn(2, 6, 256, device=DEV).bfloat16()
+    x = torch.randn(2, 6, 256, device=DEV).bfloat16().requires_grad_(True)
     with torch.no_grad():
         assert layer._fused(x)
     assert not layer._fused(x)  # parameters require grad and grad mode is on
     out = layer(x)
     assert out.requires_grad
-    with pytest.raises(RuntimeError):
-        out.float().sum().backward()
+    out.float().sum().backward()
+    grads = [p.grad for p in layer.parameters()]
+    assert all(g is not None and torch.isfinite(g.float()).all() for g in grads)
+    assert x.grad is not None and torch.isfinite(x.grad.float()).all() and x.grad.float().abs().max() > 0
+    small = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=8, backend="hip")).to(DEV).bfloat16()  # head dim 32
+    with pytest.raises(RuntimeError, match="backward pass for head dims"):
+        small(x.detach()).float().sum().backward()
 
 
 def test_layer_ops_accept_empty_inputs():
