@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 7
+#define XS_ABI_VERSION 8
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -283,6 +283,16 @@ typedef struct xs_slstm_bwd_args {
   int64_t d_wx_stride_b, d_wx_stride_t;
   float *d_s0;               /* [4,B,H] (backward) */
   void *stream;
+  /* backward, optional: a head spread over dh/64 compute units (head dims 128, 256; 512 in bf16).  With split != 0,
+   * r_t is tiled per workgroup slice, [NH][dh/64][dh/16][KS/KC][KC/EPC][16][EPC] over the KS = 256 gate units
+   * k = g*64 + (a % 64) of the 64 hidden units a of a slice; exchange is a float32 buffer of
+   * 2 * NH * ceil(B/16) * (dh/64) * 16 * dh elements, counters 2 * NH * ceil(B/16) + 1 words that are ZERO when the call
+   * starts (the last one is set when a bounded wait between the compute units of a head ran out: d_s0 is NaN then).
+   * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once. */
+  int32_t split;
+  void *exchange;
+  uint32_t *counters;
+  int64_t spin_limit;        /* 0 = default */
 } xs_slstm_bwd_args;
 
 int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);

@@ -32,7 +32,7 @@ def test_abi_version_and_struct_mirror():
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
-    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8  # 5 int32 (+4 padding), then 17 8-byte fields
+    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8  # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more
 
 
 def test_backward_argument_errors_without_touching_the_gpu():

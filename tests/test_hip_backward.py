@@ -31,11 +31,24 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES)
-def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked):
+# what the kernel that spreads a head over dh / 64 compute units adds: head dim 512 (bf16), many row tiles
+SPLIT_CASES = [
+    (True, 9, 7, 2, 512, True),
+    (True, 100, 5, 2, 256, True),
+    (False, 50, 6, 4, 128, True),
+]
+
+
+@pytest.mark.parametrize("split", [False, True], ids=["one-unit", "split"])
+@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES + SPLIT_CASES)
+def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, split):
     from xlstm_amd import functional as F
 
-    print("case backward", bf16, B, T, NH, dh, masked, flush=True)
+    if split and dh == 64:
+        pytest.skip("head dim 64 is one workgroup's worth: no split")
+    if not split and dh == 512:
+        pytest.skip("head dim 512 has the split kernel only")
+    print("case backward", bf16, B, T, NH, dh, masked, split, flush=True)
     H = NH * dh
     wx, r, b, s0 = make_problem(91, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=masked)
     reset = geometric_reset_mask(7, B, T, max(2, T // 2)) if masked else None
@@ -56,7 +69,8 @@ def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked):
     s0_t = torch.from_numpy(s0).to(dev) if s0 is not None else None
     m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
-    d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), torch.from_numpy(d_sf).to(dev))
+    d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), torch.from_numpy(d_sf).to(dev),
+                                            split_override=split)
     torch.cuda.synchronize()
     o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
     o_r_k = r_ext_to_kernel(torch.from_numpy(o_r)).numpy()

@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 
 XS_F32, XS_BF16 = 0, 1
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 EXPORTS = (
     "xs_abi_version",
@@ -75,6 +75,10 @@ class SlstmBwdArgs(ctypes.Structure):
         ("d_wx_stride_b", ctypes.c_int64), ("d_wx_stride_t", ctypes.c_int64),
         ("d_s0", ctypes.c_void_p),
         ("stream", ctypes.c_void_p),
+        ("split", ctypes.c_int32),
+        ("exchange", ctypes.c_void_p),
+        ("counters", ctypes.c_void_p),
+        ("spin_limit", ctypes.c_int64),
     ]
 
 

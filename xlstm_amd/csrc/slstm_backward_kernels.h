@@ -259,4 +259,205 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The reverse pass with a head SPREAD OVER S = dh / 64 workgroups (compute units), the forward's idea turned round:
+// workgroup s of a (head, 16-row tile) group owns 64 hidden units.  Its slice of R transposed - the 256 gate units of
+// its own 64 units by all dh input units, 128 KiB in bf16 at head dim 256 - stays in the registers of its eight waves
+// for the whole call, its MFMAs need only the gate deltas of its OWN units, and what travels per step is a
+// reduce-scatter of partial sums: every workgroup writes its 16 x dh partial result, waits for the S - 1 others of its
+// group (one arrival counter per step parity, two buffers: a workgroup that is a step ahead writes the other one), and
+// adds up, in the order of the workgroups, the S partial sums of its own 64 columns.  Nothing is read from memory per
+// step but the coefficients of the workgroup's own 16 x 64 elements.
+//
+// All workgroups of a group run on one XCD (workgroup i is dispatched to XCD i % 8) and must be resident at once; the
+// host launches at most as many as there are compute units.  Waits are bounded: when one runs out the call's abort
+// word is set, every workgroup stops waiting, and the gradient of the initial state is overwritten with NaN.
+struct BwdSplitParams {
+  int B, T, NH, dh;
+  const float *coef;
+  const void *d_h;
+  const float *d_s_final;
+  const void *r_ts;          // R transposed per workgroup slice, tiled as MFMA fragments:
+                             // [NH][S][dh / 16][KSTEPS][64 lanes][16 bytes], k = g 64 + (unit % 64) inside a slice
+  const uint8_t *reset;
+  long long reset_sb;
+  float *d_wx;
+  long long d_wx_sb, d_wx_st;
+  float *d_s0;
+  float *xch;                // [2][groups][S][16][dh] partial sums
+  unsigned int *cnt;         // [groups][2] arrival counters, then one abort word; zero at the start of a call
+  long long spin_limit;
+};
+
+template <bool BF16, int NB>  // eight waves, NB 16-column blocks each: dh = 128 NB, S = 2 NB workgroups per group
+__global__ __launch_bounds__(512) void slstm_bwd_split_kernel(BwdSplitParams p) {
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int EPC = 16 / ESZ;
+  constexpr int dh = NB * 128;
+  constexpr int UW = 64;                      // hidden units of a workgroup
+  constexpr int S = dh / UW;
+  constexpr int KS = 4 * UW;                  // gate units of a workgroup: its share of K
+  constexpr int KSTEPS = KS / (4 * EPC);
+  constexpr int LDK = KS + EPC;
+  __shared__ __attribute__((aligned(16))) char tile[16 * LDK * ESZ];
+  __shared__ int gave_up;
+  const int H = p.NH * dh;
+  const long long BH = (long long)p.B * H;
+  const int ngroups = p.NH * ((p.B + 15) / 16);
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int group = (local / S) * 8 + xcd, s = local % S;
+  if (group >= ngroups) return;
+  const int head = group % p.NH;
+  const int row0 = (group / p.NH) * 16;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
+  unsigned int *const abort_word = p.cnt + 2 * ngroups;
+  if (tid == 0) gave_up = 0;
+  // ---- this workgroup's slice of R transposed -> registers, once
+  uint4 bq[KSTEPS][NB];
+  {
+    const char *base = reinterpret_cast<const char *>(p.r_ts) + ((long long)(head * S + s) * (dh / 16) * KSTEPS * 64 << 4);
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+        bq[ks][nb] = *reinterpret_cast<const uint4 *>(base + ((((long long)(wave * NB + nb) * KSTEPS + ks) * 64 + lane) << 4));
+  }
+  // ---- the thread's two elements: row prow, units s 64 + 2 pu, + 1 of the head
+  const int prow = tid >> 5, pu = (tid & 31) * 2;
+  const int row = row0 + prow;
+  const bool there = row < p.B;
+  const long long ecol = (long long)head * dh + s * UW + pu;
+  float dy[2] = {0.0f, 0.0f}, dc[2] = {0.0f, 0.0f}, dn[2] = {0.0f, 0.0f};
+  if (there && p.d_s_final) {
+    const long long o = (long long)row * H + ecol;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) { dy[e] = p.d_s_final[o + e]; dc[e] = p.d_s_final[BH + o + e]; dn[e] = p.d_s_final[2 * BH + o + e]; }
+  }
+  __syncthreads();
+  // the step's inputs of the thread's elements, fetched one step ahead (while the workgroup waits for its peers)
+  f32x2 c9[9], dh2;
+  bool restart = false;
+  auto fetch_step = [&](int t) {
+    if (!there) return;
+    restart = p.reset && p.reset[(long long)row * p.reset_sb + t];
+    const long long e = (long long)t * p.B + row;
+    const float *cf = p.coef + e * 9 * H + ecol;
+#pragma unroll
+    for (int j = 0; j < 9; ++j) c9[j] = *reinterpret_cast<const f32x2 *>(cf + (long long)j * H);
+    if (BF16) {
+      const uint32_t w = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(p.d_h) + e * H + ecol);
+      dh2 = f32x2{__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u)};
+    } else {
+      dh2 = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(p.d_h) + e * H + ecol);
+    }
+  };
+  fetch_step(p.T - 1);
+  for (int t = p.T - 1; t >= 0; --t) {
+    const int n = p.T - 1 - t, par = n & 1;
+    // ---- the gradient of the step for the thread's elements; gate deltas to d_wx and, as the A operand, to LDS
+    float delta[4][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}, {0.0f, 0.0f}, {0.0f, 0.0f}};
+    const bool restart_now = restart;
+    if (there) {
+      const float dh_in[2] = {dh2[0], dh2[1]};
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const float dyt = dh_in[k] + dy[k];
+        const float dct = dc[k] + dyt * c9[0][k];
+        const float dnt = dn[k] - dyt * c9[1][k];
+        delta[0][k] = c9[2][k] * dct + c9[3][k] * dnt;
+        delta[1][k] = c9[4][k] * dct + c9[5][k] * dnt;
+        delta[2][k] = c9[6][k] * dct;
+        delta[3][k] = c9[7][k] * dyt;
+        dc[k] = restart_now ? 0.0f : c9[8][k] * dct;  // (a row that starts a document at t took nothing from the step before)
+        dn[k] = restart_now ? 0.0f : c9[8][k] * dnt;
+      }
+      float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
+    }
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int k = g * UW + pu;
+      if (BF16) *reinterpret_cast<uint32_t *>(tile + ((long long)prow * LDK + k) * 2) = pack_bf16x2(delta[g][0], delta[g][1]);
+      else *reinterpret_cast<f32x2 *>(tile + ((long long)prow * LDK + k) * 4) = f32x2{delta[g][0], delta[g][1]};
+    }
+    __syncthreads();
+    // ---- this workgroup's share of what reaches y_{t-1}: delta [16 x KS] . R^T slice [KS x dh], 16 NB columns per wave
+    f32x4 acc[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const uint4 av = *reinterpret_cast<const uint4 *>(tile + ((long long)r16 * LDK + ks * 4 * EPC + q * EPC) * ESZ);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) {
+        const uint4 bv = bq[ks][nb];
+        if (BF16) {
+          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc[nb], 0, 0, 0);
+        } else {
+          const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[nb], 0, 0, 0);
+        }
+      }
+    }
+    // ---- partial sums out (past the first-level cache: the peers read them), then the group's arrival counter
+    float *const mine = p.xch + ((((long long)par * ngroups + group) * S + s) * 16) * dh;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        __hip_atomic_store(mine + (long long)(4 * q + i) * dh + (wave * NB + nb) * 16 + r16, acc[nb][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    // The stores above are device-scope stores: acknowledged means visible to every compute unit.  Waiting for the
+    // acknowledgements and then for the workgroup's other waves orders them in front of the counter without a fence
+    // (a device-scope fence writes back and invalidates caches: two of them cost more than the rest of the step).
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (t > 0) fetch_step(t - 1);  // (behind the wait for the acknowledgements, which would be a wait for these loads too)
+    __syncthreads();  // (every wave's partial sums are out; the tile may be written again)
+    if (tid == 0) {
+      unsigned int *const counter = p.cnt + 2 * group + par;
+      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned int want = (unsigned int)S * (unsigned int)((n >> 1) + 1);
+      if (!gave_up) {
+        long long spins = 0;
+        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+          if (++spins > p.spin_limit || ((spins & 255) == 0 && __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+            __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            gave_up = 1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(1);
+        }
+      }
+    }
+    __syncthreads();
+    // ---- the S partial sums of the thread's two columns, in the order of the workgroups (device-scope loads: not from
+    //      the first-level cache, which may still hold what the buffer held two steps ago)
+    {
+      const float *src = p.xch + ((((long long)par * ngroups + group) * S) * 16 + prow) * dh + s * UW + pu;
+      float sum0 = 0.0f, sum1 = 0.0f;
+#pragma unroll
+      for (int peer = 0; peer < S; ++peer) {
+        sum0 += __hip_atomic_load(src + (long long)peer * 16 * dh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        sum1 += __hip_atomic_load(src + (long long)peer * 16 * dh + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      dy[0] = restart_now ? 0.0f : sum0;
+      dy[1] = restart_now ? 0.0f : sum1;
+    }
+  }
+  // ---- gradient w.r.t. the initial state (the stabiliser's part is zero by the rule; NaN all over when a wait ran out)
+  if (there) {
+    const bool poisoned = gave_up || __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const long long o = (long long)row * H + ecol;
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      p.d_s0[o + e] = poisoned ? kPoison : dy[e];
+      p.d_s0[BH + o + e] = poisoned ? kPoison : dc[e];
+      p.d_s0[2 * BH + o + e] = poisoned ? kPoison : dn[e];
+      p.d_s0[3 * BH + o + e] = 0.0f;
+    }
+  }
+}
+
 }  // namespace

@@ -380,7 +380,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
   if (a->dtype != XS_F32 && a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
-  if (a->dh != 64 && a->dh != 128 && a->dh != 256) return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256)", a->dh);
+  if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && a->dtype == XS_BF16 && (prepare || a->split)))
+    return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256; 512 in bf16 over several compute units)", a->dh);
   if (a->B == 0 || a->T == 0) return XS_OK;
   const bool bf16 = a->dtype == XS_BF16;
   const long long H = (long long)a->NH * a->dh;
@@ -401,6 +402,30 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
     if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");
     if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
+    if (a->split) {
+      if (a->dh != 128 && a->dh != 256 && !(a->dh == 512 && bf16))
+        return fail(XS_ERR_UNSUPPORTED, "backward pass over several compute units per head: head dim %d not supported", a->dh);
+      if (!a->exchange || !a->counters) return fail(XS_ERR_NULL, "exchange and counters are required with split");
+      const int S = a->dh / 64;
+      const long long ngroups = (long long)a->NH * ((a->B + 15) / 16);
+      const long long grid = (ngroups + 7) / 8 * 8 * S;
+      if (grid > device_cus()) return fail(XS_ERR_DEVICE, "%lld workgroups of the split backward pass do not fit %d compute units at once", grid, device_cus());
+      BwdSplitParams q;
+      q.B = a->B; q.T = a->T; q.NH = a->NH; q.dh = a->dh;
+      q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
+      q.reset = a->reset; q.reset_sb = a->reset_stride_b;
+      q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+      q.xch = (float *)a->exchange; q.cnt = a->counters;
+      q.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+      void (*ks)(BwdSplitParams) = nullptr;
+      if (a->dh == 128) ks = bf16 ? slstm_bwd_split_kernel<true, 1> : slstm_bwd_split_kernel<false, 1>;
+      else if (a->dh == 256) ks = bf16 ? slstm_bwd_split_kernel<true, 2> : slstm_bwd_split_kernel<false, 2>;
+      else ks = slstm_bwd_split_kernel<true, 4>;
+      hipLaunchKernelGGL(ks, dim3((unsigned)grid), dim3(512), 0, stream, q);
+      const hipError_t es = hipGetLastError();
+      if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
+      return XS_OK;
+    }
     BwdParams p;
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.coef = a->coef; p.d_h = a->d_h; p.d_s_final = a->d_s_final; p.r_t = a->r_t;

@@ -42,6 +42,16 @@ def read_status(workspace: torch.Tensor) -> dict:
     return {k: getattr(st, k) for k, _ in _lib.SlstmStatus._fields_ if k != "reserved"}
 
 
+_CU_COUNT = {}
+
+
+def _compute_units(dev) -> int:
+    idx = dev.index if dev.index is not None else torch.cuda.current_device()
+    if idx not in _CU_COUNT:
+        _CU_COUNT[idx] = torch.cuda.get_device_properties(idx).multi_processor_count
+    return _CU_COUNT[idx]
+
+
 def slstm_backward(
     wx: torch.Tensor,
     r: torch.Tensor,
@@ -52,6 +62,7 @@ def slstm_backward(
     d_h: torch.Tensor,
     d_s_final: Optional[torch.Tensor] = None,
     timings: Optional[dict] = None,
+    split_override: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -100,10 +111,25 @@ def slstm_backward(
     coef = torch.empty((T, B, 9, H), dtype=torch.float32, device=dev)
     d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
     d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
-    # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
     epc = 8 if bf16 else 4
-    r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
-           .reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).permute(0, 1, 3, 4, 2, 5).contiguous())
+    groups = NH * ((B + 15) // 16)
+    S = dh // 64
+    # a head over S compute units where the head dim allows it and all workgroups fit the device at once
+    split = (dh in (128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
+    if split_override is not None:
+        split = bool(split_override)
+    if split:
+        # R transposed per slice of 64 hidden units (gate units k = g*64 + a%64), tiled as MFMA operands:
+        # [NH][S][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
+        r_t = (r32.view(NH, 4, S, 64, dh).permute(0, 2, 4, 1, 3).reshape(NH, S, dh, 256).to(wx.dtype)  # [NH,S,d,k]
+               .reshape(NH, S, dh // 16, 16, 256 // (4 * epc), 4, epc).permute(0, 1, 2, 4, 5, 3, 6).contiguous())
+        exchange = torch.empty(2 * groups * S * 16 * dh, dtype=torch.float32, device=dev)
+        counters = torch.zeros(2 * groups + 1, dtype=torch.int32, device=dev)
+    else:
+        # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
+        r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
+               .reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).permute(0, 1, 3, 4, 2, 5).contiguous())
+        exchange = counters = None
     d_h = d_h.to(wx.dtype).contiguous()
     if d_s_final is not None:
         d_s_final = d_s_final.to(torch.float32).contiguous()
@@ -126,6 +152,10 @@ def slstm_backward(
     a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
     a.d_s0 = d_s0.data_ptr()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
+    a.split = 1 if split else 0
+    a.exchange = exchange.data_ptr() if split else None
+    a.counters = counters.data_ptr() if split else None
+    a.spin_limit = 0
     marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
@@ -143,6 +173,9 @@ def slstm_backward(
     dl = d_wx.view(B, T, 4, NH, dh).permute(3, 2, 4, 1, 0).reshape(NH, 4 * dh, T * B)  # [NH, 4*dh, (t, b)]
     d_r = torch.bmm(dl, yp)                                                            # [NH, 4*dh, dh]
     d_bias = d_wx.view(B * T, 4, NH, dh).sum(0).transpose(0, 1).contiguous()
+    if split and timings is None and int(counters[-1].item()):  # (a synchronisation; training calls are not latency-bound)
+        raise EngineError("xlstm_amd: a wait between the compute units of a head ran out in the backward pass "
+                          "(other work held compute units); the gradients are invalid")
     return d_wx, d_r, d_bias, d_s0
 
 
