@@ -135,3 +135,24 @@ def test_cell_autograd_matches_the_oracle(dtype, tol):
                 d_s0=_rel(st.grad.float().cpu().numpy()[:3], o_s0[:3]))
     print(errs, flush=True)
     assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
+
+
+def test_a_wait_between_compute_units_that_runs_out_is_reported():
+    """Host-forced: with a spin limit of one poll the workgroups of a head give up on each other at once (every kernel
+    still exits normally).  The call must raise, or - when all peers happened to be there - return the usual result."""
+    from xlstm_amd import functional as F
+
+    B, T, NH, dh = 16, 12, 4, 256
+    wx, r, b, _ = make_problem(95, B, T, NH, dh, rscale=2.0, bf16=True)
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev).bfloat16()
+    r_t, b_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    d_h = torch.randn(T, B, NH * dh, generator=torch.Generator().manual_seed(7)).to(dev).bfloat16()
+    h, _ = F.slstm_forward(wx_t, r_t, b_t)
+    good = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True)
+    try:
+        got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=1)
+    except F.EngineError as e:
+        assert "ran out" in str(e)
+    else:
+        assert torch.equal(got[0], good[0])

@@ -168,7 +168,7 @@ class sLSTMCellConfig:
         self.num_states = rnn_function_registry[self.function]["states"]
 
 
-BACKWARD_HEAD_DIMS = (64, 128, 256)  # what xs_slstm_backward covers
+BACKWARD_HEAD_DIMS = (64, 128, 256, 512)  # what xs_slstm_backward covers (512: bfloat16 inputs only)
 
 
 class _ForwardOnly(torch.autograd.Function):

@@ -63,6 +63,7 @@ def slstm_backward(
     d_s_final: Optional[torch.Tensor] = None,
     timings: Optional[dict] = None,
     split_override: Optional[bool] = None,
+    spin_limit: int = 0,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -74,7 +75,9 @@ def slstm_backward(
     Two kernels of the engine (``xs_slstm_backward_prepare``, ``xs_slstm_backward``) around three plain library GEMMs and
     a reduction: ``R.h_{t-1}`` for all steps at once in front, and the gradients of R and the bias, which are sums over
     all steps of products of the gate deltas with the outputs, behind.  ``timings`` (a dict) receives three events around
-    the two kernels.
+    the two kernels.  Where the head dim allows it (128, 256; 512 in bfloat16) and the workgroups fit the device at once,
+    a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
+    kernel); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
     """
     lib = _lib.load()
     _require_cuda("wx", wx)
@@ -155,7 +158,7 @@ def slstm_backward(
     a.split = 1 if split else 0
     a.exchange = exchange.data_ptr() if split else None
     a.counters = counters.data_ptr() if split else None
-    a.spin_limit = 0
+    a.spin_limit = int(spin_limit)
     marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
