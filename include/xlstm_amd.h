@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 8
+#define XS_ABI_VERSION 9
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -254,7 +254,8 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  * xs_slstm_backward_prepare  walks forward in time over raw = wx + ry + bias, where ry[t,b,h,g,a] =
  *   sum_d y_{t-1}[b,h,d] * r[h][g*dh+a][d] is given for all steps at once (one batched GEMM over the outputs of the
  *   forward call, shifted by one step, rows that start a document zeroed), and writes nine float32 coefficients per
- *   step and element into coef [T,B,9,H].
+ *   step and element into coef [T,B,9,H] (with split != 0: T * ceil(B/16)*16 * 9 * H floats, in the order the split
+ *   kernel reads them).
  * xs_slstm_backward          one launch for all T steps, reverse in time: d_wx [B,T,4,NH,dh] (float32, the gradient
  *   with respect to the raw gates: the gradient of wx, and with the outputs what the gradients of R and the bias are
  *   sums of, slstm_backward.cu:381-386, 52-108) and d_s0 [4,B,H] (the m part is zero).
@@ -275,7 +276,7 @@ typedef struct xs_slstm_bwd_args {
   const float *s0;           /* [4,B,H] or NULL (prepare) */
   const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */
   int64_t reset_stride_b;
-  float *coef;               /* [T,B,9,H]: written by prepare, read by backward */
+  float *coef;               /* [T,B,9,H] ([T,ceil(B/16)*16,9,H] with split): written by prepare, read by backward */
   const void *d_h;           /* [T,B,H]: gradient with respect to h_out (backward) */
   const float *d_s_final;    /* [4,B,H] or NULL: gradient with respect to the final state; y, c, n are used (backward) */
   const void *r_t;           /* (backward) */
@@ -284,10 +285,12 @@ typedef struct xs_slstm_bwd_args {
   float *d_s0;               /* [4,B,H] (backward) */
   void *stream;
   /* backward, optional: a head spread over dh/64 compute units (head dims 128, 256; 512 in bf16).  With split != 0,
-   * r_t is tiled per workgroup slice, [NH][dh/64][dh/16][KS/KC][KC/EPC][16][EPC] over the KS = 256 gate units
-   * k = g*64 + (a % 64) of the 64 hidden units a of a slice; exchange is a float32 buffer of
-   * 2 * NH * ceil(B/16) * (dh/64) * 16 * dh elements, counters 2 * NH * ceil(B/16) + 1 words that are ZERO when the call
-   * starts (the last one is set when a bounded wait between the compute units of a head ran out: d_s0 is NaN then).
+   * r_t holds R transposed with K ordered k = 256*(a/64) + 64*g + a%64 (a the hidden unit, g the gate), tiled as MFMA
+   * operands per owner of the output columns and per wave: [NH][dh/64][8][K/8/KC][4][KC/EPC][16][EPC], EPC the elements
+   * of 16 bytes and KC = 4*EPC; exchange is a 16-byte aligned buffer of 4 * NH * ceil(B/16) * 16 * 4*dh elements of
+   * dtype and counters 1 + NH * ceil(B/16) 32-bit words; the library initialises both in front of the kernel, and the
+   * FIRST word is nonzero after the call when a bounded wait between the compute units of a head ran out (d_s0 is NaN
+   * then).
    * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once. */
   int32_t split;
   void *exchange;

@@ -38,7 +38,10 @@ struct BwdPrepParams {
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
-  float *coef;               // [T,B,9,H]
+  float *coef;               // [T,B,9,H], or with tiled != 0 [T][ceil(B/16)][NH][dh/64][16 rows][9][64 units]: what a workgroup
+                             // of the split kernel reads per step is one piece of 36 KiB (planes 4 KiB apart, as in the
+                             // plain layout, all fall on the same memory channel)
+  int tiled;
 };
 
 template <bool BF16>
@@ -82,15 +85,21 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     const float rn = __builtin_amdgcn_rcpf(nnew);
     const float ynew = og * cnew * rn;
     float *dst = p.coef + ((long long)t * p.B + b) * 9 * H + col;
+    long long js = H;
+    if (p.tiled) {
+      const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (p.dh >> 6) + (a >> 6);
+      dst = p.coef + (piece * 16 + (b & 15)) * (9 * 64) + (a & 63);
+      js = 64;
+    }
     dst[0] = og * rn;
-    dst[(long long)H] = ynew * rn;
-    dst[2ll * H] = ig * tz;
-    dst[3ll * H] = ig;
-    dst[4ll * H] = fg * one_minus_fsig * c;
-    dst[5ll * H] = fg * one_minus_fsig * n;
-    dst[6ll * H] = ig * (1.0f - tz * tz);
-    dst[7ll * H] = (1.0f - og) * ynew;
-    dst[8ll * H] = fg;
+    dst[1 * js] = ynew * rn;
+    dst[2 * js] = ig * tz;
+    dst[3 * js] = ig;
+    dst[4 * js] = fg * one_minus_fsig * c;
+    dst[5 * js] = fg * one_minus_fsig * n;
+    dst[6 * js] = ig * (1.0f - tz * tz);
+    dst[7 * js] = (1.0f - og) * ynew;
+    dst[8 * js] = fg;
     c = cnew; n = nnew; m = mnew;
   }
 }
@@ -260,69 +269,218 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// The reverse pass with a head SPREAD OVER S = dh / 64 workgroups (compute units), the forward's idea turned round:
-// workgroup s of a (head, 16-row tile) group owns 64 hidden units.  Its slice of R transposed - the 256 gate units of
-// its own 64 units by all dh input units, 128 KiB in bf16 at head dim 256 - stays in the registers of its eight waves
-// for the whole call, its MFMAs need only the gate deltas of its OWN units, and what travels per step is a
-// reduce-scatter of partial sums: every workgroup writes its 16 x dh partial result, waits for the S - 1 others of its
-// group (one arrival counter per step parity, two buffers: a workgroup that is a step ahead writes the other one), and
-// adds up, in the order of the workgroups, the S partial sums of its own 64 columns.  Nothing is read from memory per
-// step but the coefficients of the workgroup's own 16 x 64 elements.
+// The reverse pass with a head SPREAD OVER S = dh / 64 workgroups (compute units), built like the forward's sequence
+// kernel: workgroup s of a (head, 16-row tile) group owns 64 hidden units.  It computes the step's gate deltas of its
+// own 16 x 64 elements, publishes them to its peers, and computes what reaches ITS 64 units of y_{t-1}:
+// delta [16 x 4 dh] . R^T [4 dh x 64].  That slice of R transposed (128 KiB in bf16 at head dim 256) stays in the
+// registers of the eight waves for the whole call, each wave holding one eighth of K for all 64 columns; the eight
+// partial results are added up through LDS.  Per step a workgroup writes its 16 x 256 deltas (8 KiB in bf16) and reads
+// the group's 16 x 4 dh, straight into MFMA operand registers; nothing else is read from memory per step but the
+// coefficients of its own elements, which are fetched two steps ahead.
 //
-// All workgroups of a group run on one XCD (workgroup i is dispatched to XCD i % 8) and must be resident at once; the
-// host launches at most as many as there are compute units.  Waits are bounded: when one runs out the call's abort
-// word is set, every workgroup stops waiting, and the gradient of the initial state is overwritten with NaN.
+// The exchange is a ring of kBwdRing slots per group, slot n % kBwdRing for the n-th step of the call, laid out as
+// MFMA A operands: [K / KC][16 rows][4][16 bytes] with KC = 32 (bf16) or 16 (float32) and K index
+// k = 256 s + 64 gate + unit % 64.  A word is data or the "not written yet" pattern (all ones, which no value takes:
+// NaNs are made canonical).  A reader polls its 16-byte chunks until none holds the pattern.  A workgroup that
+// publishes step n also re-arms its words of step n - 2: it has read all deltas of step n - 1, which every peer
+// computed from a complete set of step n - 2.  The re-arm is acknowledged before the workgroup's poll of step n
+// returns (accesses of a wave complete in order), so before it publishes step n + 1; a peer that polls the slot again
+// for step n - 2 + kBwdRing has seen that publication and finds the pattern or the new data, never the old.  The
+// library fills the ring with the pattern in front of the kernel.
+//
+// All workgroups of a group run on one XCD (workgroup i is dispatched to XCD i % 8): plain stores reach the XCD's L2,
+// and the polls read past the first-level cache.  All workgroups must be resident at once; the host launches at most
+// as many as there are compute units.  Waits are bounded: when one runs out the call's abort word is set, every wave
+// stops waiting, and the gradient of the initial state is overwritten with NaN.
+constexpr int kBwdRing = 4;
+
 struct BwdSplitParams {
   int B, T, NH, dh;
-  const float *coef;
+  const float *coef;         // [T][ceil(B/16)][NH][S][16 rows][9][64 units]
   const void *d_h;
   const float *d_s_final;
-  const void *r_ts;          // R transposed per workgroup slice, tiled as MFMA fragments:
-                             // [NH][S][dh / 16][KSTEPS][64 lanes][16 bytes], k = g 64 + (unit % 64) inside a slice
+  const void *r_ts;          // R transposed per workgroup and wave, tiled as MFMA B operands:
+                             // [NH][S][8 waves][KSTEPS][4 column blocks][64 lanes][16 bytes]
   const uint8_t *reset;
   long long reset_sb;
   float *d_wx;
   long long d_wx_sb, d_wx_st;
   float *d_s0;
-  float *xch;                // [2][groups][S][16][dh] partial sums
-  unsigned int *cnt;         // [groups][2] arrival counters, then one abort word; zero at the start of a call
+  void *xch;                 // [kBwdRing][groups][K / KC][16][4][16 bytes], all ones at the start
+  unsigned int *abort_word;  // zero at the start of a call
+  unsigned int *progress;    // [groups]: the step of the call that the group has reached (for the prefetching workgroups)
+  int main_locals;           // workgroups per XCD that compute; those behind them (one per XCD, if any) prefetch
   long long spin_limit;
 };
 
-template <bool BF16, int NB>  // eight waves, NB 16-column blocks each: dh = 128 NB, S = 2 NB workgroups per group
-__global__ __launch_bounds__(512) void slstm_bwd_split_kernel(BwdSplitParams p) {
+// fills the exchange ring with the "not written yet" pattern and clears the abort word in front of the split kernel
+// (a kernel, not a memset: a caller may capture the call in a graph)
+__global__ __launch_bounds__(256) void slstm_bwd_arm_kernel(uint4 *xch, long long n16, unsigned int *words, int nwords) {
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride)
+    xch[i] = uint4{0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu, 0xFFFFFFFFu};
+  if (blockIdx.x == 0)
+    for (int i = threadIdx.x; i < nwords; i += blockDim.x) words[i] = 0u;
+}
+
+// One workgroup per XCD that brings what the XCD's groups will read from memory - coefficients and d_h - into the XCD's
+// L2, a few steps ahead of them.  A compute unit returns its loads in the order they were issued, whichever wave issued
+// them: a miss that goes to HBM holds up every poll of the exchange ring behind it, and a step took 2.7 us at config 2
+// with the inputs fetched by the workgroup itself (by its polling waves or by others, one step ahead or two) against
+// 2.0 us with inputs that were already in the L2.  So another compute unit takes the misses.  Nothing depends on
+// these workgroups: they follow the groups' progress words at a distance, and stop when those stop.
+constexpr int kBwdAhead = 12;  // steps the prefetch may run ahead (1.2 MiB of a 4 MiB L2 at config 2)
+template <bool BF16>
+__device__ __forceinline__ void bwd_prefetch(const BwdSplitParams &p, int xcd) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  constexpr int EPC = 16 / ESZ;
+  const int S = p.dh >> 6, H = p.NH * p.dh, NT = (p.B + 15) >> 4, ngroups = p.NH * NT;
+  const int tid = threadIdx.x, nthreads = blockDim.x;
+  if (xcd >= ngroups) return;
+  // A touch is a load that writes LDS, not a register: nothing waits for these loads before the end, and a register
+  // that a load in flight is going to write would be handed out again by the compiler in the meantime.  Every touch of
+  // every wave lands in the same kilobyte, which nobody reads.
+  __shared__ uint4 dump[64];
+  const uint32_t dump_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dump);
+  auto touch_lines = [&](const char *base, int bytes, int first_line, int lines, int line_stride_lines, int per_run) {
+    // lines first_line + tid, + nthreads, ... of `lines`; line l is at base + ((l / per_run) * line_stride_lines + l % per_run) * 128
+    const unsigned long long b = reinterpret_cast<unsigned long long>(base);
+    const u32x4_t rs = {uniform((uint32_t)b), uniform((uint32_t)(b >> 32) & 0xFFFFu), (uint32_t)bytes, 0x00020000u};
+    for (int l0 = first_line; l0 < lines; l0 += nthreads) {  // (uniform trip count: lanes past the end ask past the buffer's end)
+      const int l = l0 + tid;
+      const int off = l < lines ? ((l / per_run) * line_stride_lines + l % per_run) * 128 : 0x7FFFFF00;
+      lds_direct_fetch_b128(rs, uniform(dump_lds), off);
+    }
+  };
+  __shared__ int stop;
+  if (tid == 0) stop = 0;
+  __syncthreads();
+  for (int m0 = 0; m0 < p.T; m0 += 4) {
+    if (m0 >= kBwdAhead) {
+      if (tid == 0) {
+        for (int g = xcd; g < ngroups && !stop; g += 8) {
+          int spins = 0;
+          while ((int)__hip_atomic_load(p.progress + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kBwdAhead < m0) {
+            if (++spins > (1 << 16) || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { stop = 1; break; }
+            __builtin_amdgcn_s_sleep(8);
+          }
+        }
+      }
+      __syncthreads();
+      if (stop) break;
+    }
+    for (int m = m0; m < m0 + 4 && m < p.T; ++m) {
+      const int t = p.T - 1 - m;
+      for (int g = xcd; g < ngroups; g += 8) {
+        const int head = g % p.NH, tile = g / p.NH, row0 = tile * 16;
+        const int piece_lines = 16 * 9 * 64 * 4 / 128;
+        const char *cbase = reinterpret_cast<const char *>(p.coef) + ((((long long)t * NT + tile) * p.NH + head) * S) * (piece_lines * 128ll);
+        touch_lines(cbase, S * piece_lines * 128, 0, S * piece_lines, 1, 1);
+        const int rows = p.B - row0 < 16 ? p.B - row0 : 16, per_row = p.dh * ESZ / 128;
+        const char *dbase = reinterpret_cast<const char *>(p.d_h) + (((long long)t * p.B + row0) * H + (long long)head * p.dh) * ESZ;
+        touch_lines(dbase, ((rows - 1) * H + p.dh) * ESZ, 0, rows * per_row, H * ESZ / 128, per_row);
+      }
+    }
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
+constexpr int kBwdPartStride = 68;  // floats between the rows of a wave's partial tile in LDS (no bank conflicts)
+constexpr int kBwdCoefBytes = 16 * 9 * 64 * 4;  // a step's coefficients of a workgroup: 16 rows, 9 of them, 64 units
+constexpr int bwd_feed_slot_bytes(bool bf16) { return kBwdCoefBytes + 16 * 64 * (bf16 ? 2 : 4); }  // ... and its d_h
+constexpr int bwd_split_lds_bytes(bool feed, bool bf16) {
+  return feed ? 8 * 16 * kBwdPartStride * 4 + 2 * bwd_feed_slot_bytes(bf16) : 2 * 8 * 16 * kBwdPartStride * 4;
+}
+
+// FEED: four more waves that do nothing but bring the steps' inputs from memory to LDS, two steps ahead, with loads
+// that write LDS directly (no registers, and every wait of these waves is written by hand: a wave's loads return in
+// the order they were issued, and the compiler waits for all of them wherever it waits for one).  The same order is
+// why the polling waves must not fetch the inputs themselves: a poll issued behind a step's 40 KiB of coefficients
+// comes back no sooner than they do, from HBM, and the step took 2.9 us at config 2 that way instead of 1.5 us
+// without the fetch.  Twelve waves leave 168 registers a lane, which the variants with 128 registers of R transposed
+// (float32 at head dim 256, bf16 at 512) do not fit: they run without feeders.
+//
+// With feeders a step has two barriers: B', behind which the slot that the step's inputs were read from is free for
+// the inputs of the step after the next, and A, in front of which the wave's partial tile is written and the next
+// step's inputs have landed.  (Without: one barrier, two sets of partial tiles.)
+template <bool BF16, int NB, bool FEED>  // eight compute waves; dh = 128 NB, S = 2 NB workgroups per group
+__global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSplitParams p) {
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int EPC = 16 / ESZ;               // elements of a 16-byte chunk
+  constexpr int KC = 4 * EPC;                 // K of one chunk row: what one MFMA (bf16) or four (float32) take
   constexpr int dh = NB * 128;
   constexpr int UW = 64;                      // hidden units of a workgroup
   constexpr int S = dh / UW;
-  constexpr int KS = 4 * UW;                  // gate units of a workgroup: its share of K
-  constexpr int KSTEPS = KS / (4 * EPC);
-  constexpr int LDK = KS + EPC;
-  __shared__ __attribute__((aligned(16))) char tile[16 * LDK * ESZ];
-  __shared__ int gave_up;
+  constexpr int K = 4 * dh;
+  constexpr int KSTEPS = K / 8 / KC;          // chunks of a wave: its eighth of K
+  constexpr int SLOT = 16 * K * ESZ;          // bytes of a group's slot
+  constexpr int PART = 16 * kBwdPartStride;   // floats of a wave's partial tile
+  extern __shared__ __attribute__((aligned(16))) float part[];  // [2][8 waves][16 rows][kBwdPartStride]
   const int H = p.NH * dh;
   const long long BH = (long long)p.B * H;
   const int ngroups = p.NH * ((p.B + 15) / 16);
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  if (local >= p.main_locals) {
+    bwd_prefetch<BF16>(p, xcd);
+    return;
+  }
   const int group = (local / S) * 8 + xcd, s = local % S;
   if (group >= ngroups) return;
   const int head = group % p.NH;
   const int row0 = (group / p.NH) * 16;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
-  unsigned int *const abort_word = p.cnt + 2 * ngroups;
-  if (tid == 0) gave_up = 0;
-  // ---- this workgroup's slice of R transposed -> registers, once
-  uint4 bq[KSTEPS][NB];
+  constexpr int FSLOT = bwd_feed_slot_bytes(BF16);
+  char *const feed = reinterpret_cast<char *>(part + 8 * PART);  // [2 slots][16 rows][9][64 units] float32, then d_h [16][64]
+  const long long coef_piece0 = ((((long long)(row0 >> 4)) * p.NH + head) * S + s) * kBwdCoefBytes;  // + t * coef_step
+  const long long coef_step = (long long)((p.B + 15) >> 4) * p.NH * S * kBwdCoefBytes;
+  if (FEED && wave >= 8) {
+    const int f = (int)uniform((uint32_t)wave) - 8;
+    const uint32_t feed_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)feed);
+    const int rows_there = p.B - row0 < 16 ? p.B - row0 : 16;
+    const uint32_t dh_records = (uint32_t)(((long long)(rows_there - 1) * H + 64) * ESZ);
+    // d_h: a load covers 8 rows of 128 bytes (bf16; the waves' two halves twice over) or 4 rows of 256 bytes
+    const int dh_part = BF16 ? (f & 1) : f;
+    const int dh_voff = BF16 ? ((dh_part * 8 + (lane >> 3)) * H * 2 + (lane & 7) * 16) : ((dh_part * 4 + (lane >> 4)) * H * 4 + (lane & 15) * 16);
+    auto request = [&](int n) {  // the inputs of step n of the call -> slot n % 2: ten loads a wave
+      const int t = p.T - 1 - n;
+      const unsigned long long cb = reinterpret_cast<unsigned long long>(p.coef) + (unsigned long long)(coef_piece0 + t * coef_step);
+      const u32x4_t crs = {uniform((uint32_t)cb), uniform((uint32_t)(cb >> 32) & 0xFFFFu), (uint32_t)kBwdCoefBytes, 0x00020000u};
+      const uint32_t slot = feed_lds + (n & 1) * FSLOT;
+#pragma unroll
+      for (int k = 0; k < 9; ++k) lds_direct_fetch_b128(crs, uniform(slot + (f * 9 + k) * 1024), (f * 9 + k) * 1024 + lane * 16);
+      const unsigned long long db = reinterpret_cast<unsigned long long>(p.d_h) + (unsigned long long)((((long long)t * p.B + row0) * H + (long long)head * dh + s * UW) * ESZ);
+      const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), dh_records, 0x00020000u};
+      lds_direct_fetch_b128(drs, uniform(slot + kBwdCoefBytes + dh_part * 1024), dh_voff);
+    };
+    request(0);
+    if (p.T > 1) {
+      request(1);
+      asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __syncthreads();  // (slot 0 is in place)
+    for (int n = 0; n < p.T; ++n) {
+      __syncthreads();  // B'(n): slot n % 2 has been read
+      if (n + 2 < p.T) {
+        request(n + 2);
+        asm volatile("s_waitcnt vmcnt(10)" ::: "memory");  // (all but the ten just issued: step n + 1 has landed)
+      } else {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
+      __syncthreads();  // A(n)
+    }
+    return;
+  }
+  // ---- this wave's share of the workgroup's slice of R transposed -> registers, once
+  uint4 bq[KSTEPS][4];
   {
-    const char *base = reinterpret_cast<const char *>(p.r_ts) + ((long long)(head * S + s) * (dh / 16) * KSTEPS * 64 << 4);
+    const char *base = reinterpret_cast<const char *>(p.r_ts) + ((((long long)(head * S + s) * 8 + wave) * KSTEPS * 4 * 64) << 4);
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks)
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb)
-        bq[ks][nb] = *reinterpret_cast<const uint4 *>(base + ((((long long)(wave * NB + nb) * KSTEPS + ks) * 64 + lane) << 4));
+      for (int cb = 0; cb < 4; ++cb) bq[ks][cb] = *reinterpret_cast<const uint4 *>(base + (((ks * 4 + cb) * 64 + lane) << 4));
   }
-  // ---- the thread's two elements: row prow, units s 64 + 2 pu, + 1 of the head
+  // ---- the thread's two elements: row prow, units s 64 + pu, + 1 of the head
   const int prow = tid >> 5, pu = (tid & 31) * 2;
   const int row = row0 + prow;
   const bool there = row < p.B;
@@ -333,122 +491,174 @@ __global__ __launch_bounds__(512) void slstm_bwd_split_kernel(BwdSplitParams p) 
 #pragma unroll
     for (int e = 0; e < 2; ++e) { dy[e] = p.d_s_final[o + e]; dc[e] = p.d_s_final[BH + o + e]; dn[e] = p.d_s_final[2 * BH + o + e]; }
   }
-  __syncthreads();
-  // the step's inputs of the thread's elements, fetched one step ahead (while the workgroup waits for its peers)
-  f32x2 c9[9], dh2;
-  bool restart = false;
-  auto fetch_step = [&](int t) {
-    if (!there) return;
-    restart = p.reset && p.reset[(long long)row * p.reset_sb + t];
-    const long long e = (long long)t * p.B + row;
-    const float *cf = p.coef + e * 9 * H + ecol;
+  // where the thread's deltas of gate g go in a slot, and where the wave's chunks come from
+  int pub_off[4];
 #pragma unroll
-    for (int j = 0; j < 9; ++j) c9[j] = *reinterpret_cast<const f32x2 *>(cf + (long long)j * H);
+  for (int g = 0; g < 4; ++g) {
+    const int k = s * 4 * UW + g * UW + pu;
+    pub_off[g] = (((k / KC) * 16 + prow) * 4 + (k % KC) / EPC) * 16 + (k % EPC) * ESZ;
+  }
+  const int poll_off = (r16 * 4 + q) * 16;
+  char *const ring = reinterpret_cast<char *>(p.xch) + (long long)group * SLOT;
+  const long long ring_stride = (long long)ngroups * SLOT;
+  // the step's inputs of the thread's elements, two sets used in turn: each is requested two steps ahead, right after
+  // a poll has come back, so that the next poll (loads return in order) does not queue up behind it
+  struct StepIn { f32x2 c9[9], dh2; bool restart; };
+  StepIn in0, in1;
+  auto fetch_step = [&](StepIn &in, int t) {
+    in.restart = false;
+    if (!there || t < 0) return;
+    in.restart = p.reset && p.reset[(long long)row * p.reset_sb + t];
+    const long long e = (long long)t * p.B + row;
+    const float *cf = p.coef + ((((long long)t * ((p.B + 15) >> 4) + (row0 >> 4)) * p.NH + head) * S + s) * (16 * 9 * 64) + prow * (9 * 64) + pu;
+#pragma unroll
+    for (int j = 0; j < 9; ++j) in.c9[j] = *reinterpret_cast<const f32x2 *>(cf + j * 64);
     if (BF16) {
       const uint32_t w = *reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint16_t *>(p.d_h) + e * H + ecol);
-      dh2 = f32x2{__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u)};
+      in.dh2 = f32x2{__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u)};
     } else {
-      dh2 = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(p.d_h) + e * H + ecol);
+      in.dh2 = *reinterpret_cast<const f32x2 *>(reinterpret_cast<const float *>(p.d_h) + e * H + ecol);
     }
   };
-  fetch_step(p.T - 1);
-  for (int t = p.T - 1; t >= 0; --t) {
-    const int n = p.T - 1 - t, par = n & 1;
-    // ---- the gradient of the step for the thread's elements; gate deltas to d_wx and, as the A operand, to LDS
+  bool gave_up = false;
+  uint32_t restart_raw = 0u;  // (FEED) the reset flag of the thread's row at the next step, as loaded
+  auto step = [&](StepIn &in, int t) {
+    const int n = p.T - 1 - t;
+    if (FEED) {
+      const char *slot = feed + (n & 1) * FSLOT;
+      const float *src = reinterpret_cast<const float *>(slot) + prow * (9 * 64) + pu;
+#pragma unroll
+      for (int j = 0; j < 9; ++j) in.c9[j] = *reinterpret_cast<const f32x2 *>(src + j * 64);
+      if (BF16) {
+        const uint32_t w = *reinterpret_cast<const uint32_t *>(slot + kBwdCoefBytes + prow * 128 + pu * 2);
+        in.dh2 = f32x2{__uint_as_float(w << 16), __uint_as_float(w & 0xFFFF0000u)};
+      } else {
+        in.dh2 = *reinterpret_cast<const f32x2 *>(slot + kBwdCoefBytes + prow * 256 + pu * 4);
+      }
+      in.restart = restart_raw != 0u;
+      __syncthreads();  // B'(n)
+    }
+    // ---- the gradient of the step for the thread's elements
     float delta[4][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}, {0.0f, 0.0f}, {0.0f, 0.0f}};
-    const bool restart_now = restart;
+    const bool restart_now = in.restart;
     if (there) {
-      const float dh_in[2] = {dh2[0], dh2[1]};
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
-        const float dyt = dh_in[k] + dy[k];
-        const float dct = dc[k] + dyt * c9[0][k];
-        const float dnt = dn[k] - dyt * c9[1][k];
-        delta[0][k] = c9[2][k] * dct + c9[3][k] * dnt;
-        delta[1][k] = c9[4][k] * dct + c9[5][k] * dnt;
-        delta[2][k] = c9[6][k] * dct;
-        delta[3][k] = c9[7][k] * dyt;
-        dc[k] = restart_now ? 0.0f : c9[8][k] * dct;  // (a row that starts a document at t took nothing from the step before)
-        dn[k] = restart_now ? 0.0f : c9[8][k] * dnt;
+        const float dyt = in.dh2[k] + dy[k];
+        const float dct = dc[k] + dyt * in.c9[0][k];
+        const float dnt = dn[k] - dyt * in.c9[1][k];
+        delta[0][k] = in.c9[2][k] * dct + in.c9[3][k] * dnt;
+        delta[1][k] = in.c9[4][k] * dct + in.c9[5][k] * dnt;
+        delta[2][k] = in.c9[6][k] * dct;
+        delta[3][k] = in.c9[7][k] * dyt;
+        dc[k] = restart_now ? 0.0f : in.c9[8][k] * dct;  // (a row that starts a document at t took nothing from the step before)
+        dn[k] = restart_now ? 0.0f : in.c9[8][k] * dnt;
       }
+    }
+    // ---- publish the deltas (rows outside the batch: zeros), re-arm the words of two steps ago
+    {
+      char *const cur = ring + (n % kBwdRing) * ring_stride;
+      char *const old = ring + ((n + kBwdRing - 2) % kBwdRing) * ring_stride;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        if (BF16) {
+          uint32_t w = pack_bf16x2(delta[g][0], delta[g][1]);
+          if ((w & 0xFFFFu) == 0xFFFFu) w = (w & 0xFFFF0000u) | 0x7FC0u;   // (keep the pattern unique)
+          if (w >= 0xFFFF0000u) w = (w & 0xFFFFu) | 0x7FC00000u;
+          *reinterpret_cast<uint32_t *>(cur + pub_off[g]) = w;
+          *reinterpret_cast<uint32_t *>(old + pub_off[g]) = 0xFFFFFFFFu;
+        } else {
+          float d0 = delta[g][0], d1 = delta[g][1];
+          if (d0 != d0) d0 = kPoison;
+          if (d1 != d1) d1 = kPoison;
+          *reinterpret_cast<f32x2 *>(cur + pub_off[g]) = f32x2{d0, d1};
+          *reinterpret_cast<f32x2 *>(old + pub_off[g]) = f32x2{__uint_as_float(kSentinel32), __uint_as_float(kSentinel32)};
+        }
+      }
+    }
+    // ---- the group's deltas of the wave's eighth of K: polled straight into the A operand registers
+    uint4 areg[KSTEPS];
+    {
+      const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(ring + (n % kBwdRing) * ring_stride, 0, SLOT, 0x00020000);
+      constexpr int kPastL1 = 16;  // (the load's scope bits: served by the L2)
+      long long spins = 0;
+      for (;;) {
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks)
+          areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, poll_off, (wave * KSTEPS + ks) * 1024, kPastL1));
+        uint32_t mark = 0u;
+#pragma unroll
+        for (int ks = 0; ks < KSTEPS; ++ks) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[ks]));
+        if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mark)) == 0ull || gave_up) break;
+        if (++spins > p.spin_limit || ((spins & 255) == 0 && __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
+          __hip_atomic_store(p.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          gave_up = true;
+          break;
+        }
+      }
+    }
+    if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
+    // ---- behind the poll: the inputs of the step after the next, then the step's gate deltas to d_wx
+    if (!FEED) fetch_step(in, t - 2);
+    if (FEED && there && p.reset && t > 0) restart_raw = p.reset[(long long)row * p.reset_sb + t - 1];  // (used by the next step)
+    if (there) {
       float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
 #pragma unroll
       for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
     }
+    // ---- delta [16 x K/8] . R^T [K/8 x 64]: the wave's partial result, to LDS
+    f32x4 acc[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int k = g * UW + pu;
-      if (BF16) *reinterpret_cast<uint32_t *>(tile + ((long long)prow * LDK + k) * 2) = pack_bf16x2(delta[g][0], delta[g][1]);
-      else *reinterpret_cast<f32x2 *>(tile + ((long long)prow * LDK + k) * 4) = f32x2{delta[g][0], delta[g][1]};
-    }
-    __syncthreads();
-    // ---- this workgroup's share of what reaches y_{t-1}: delta [16 x KS] . R^T slice [KS x dh], 16 NB columns per wave
-    f32x4 acc[NB];
-#pragma unroll
-    for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int cb = 0; cb < 4; ++cb) acc[cb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int ks = 0; ks < KSTEPS; ++ks) {
-      const uint4 av = *reinterpret_cast<const uint4 *>(tile + ((long long)r16 * LDK + ks * 4 * EPC + q * EPC) * ESZ);
+      const uint4 av = areg[ks];
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        const uint4 bv = bq[ks][nb];
+      for (int cb = 0; cb < 4; ++cb) {
+        const uint4 bv = bq[ks][cb];
         if (BF16) {
-          acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc[nb], 0, 0, 0);
+          acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, bv), acc[cb], 0, 0, 0);
         } else {
           const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {bv.x, bv.y, bv.z, bv.w};
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            acc[nb] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[nb], 0, 0, 0);
+            acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[cb], 0, 0, 0);
         }
       }
     }
-    // ---- partial sums out (past the first-level cache: the peers read them), then the group's arrival counter
-    float *const mine = p.xch + ((((long long)par * ngroups + group) * S + s) * 16) * dh;
+    // (two sets of tiles, used in turn: a wave writes the tiles of step n + 2 only after every peer has published
+    // step n + 2, for which it needed all of this workgroup's deltas of step n + 1, computed from the sums below)
+    float *const tiles = part + (FEED ? 0 : (n & 1) * 8 * PART);
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int cb = 0; cb < 4; ++cb)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        __hip_atomic_store(mine + (long long)(4 * q + i) * dh + (wave * NB + nb) * 16 + r16, acc[nb][i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    // The stores above are device-scope stores: acknowledged means visible to every compute unit.  Waiting for the
-    // acknowledgements and then for the workgroup's other waves orders them in front of the counter without a fence
-    // (a device-scope fence writes back and invalidates caches: two of them cost more than the rest of the step).
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    if (t > 0) fetch_step(t - 1);  // (behind the wait for the acknowledgements, which would be a wait for these loads too)
-    __syncthreads();  // (every wave's partial sums are out; the tile may be written again)
-    if (tid == 0) {
-      unsigned int *const counter = p.cnt + 2 * group + par;
-      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned int want = (unsigned int)S * (unsigned int)((n >> 1) + 1);
-      if (!gave_up) {
-        long long spins = 0;
-        while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
-          if (++spins > p.spin_limit || ((spins & 255) == 0 && __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
-            __hip_atomic_store(abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            gave_up = 1;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(1);
-        }
-      }
-    }
+      for (int i = 0; i < 4; ++i) tiles[wave * PART + (4 * q + i) * kBwdPartStride + cb * 16 + r16] = acc[cb][i];
     __syncthreads();
-    // ---- the S partial sums of the thread's two columns, in the order of the workgroups (device-scope loads: not from
-    //      the first-level cache, which may still hold what the buffer held two steps ago)
-    {
-      const float *src = p.xch + ((((long long)par * ngroups + group) * S) * 16 + prow) * dh + s * UW + pu;
-      float sum0 = 0.0f, sum1 = 0.0f;
+    // ---- the eight partial results of the thread's two columns, in the order of the waves
+    float sum0 = 0.0f, sum1 = 0.0f;
 #pragma unroll
-      for (int peer = 0; peer < S; ++peer) {
-        sum0 += __hip_atomic_load(src + (long long)peer * 16 * dh, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        sum1 += __hip_atomic_load(src + (long long)peer * 16 * dh + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-      dy[0] = restart_now ? 0.0f : sum0;
-      dy[1] = restart_now ? 0.0f : sum1;
+    for (int w = 0; w < 8; ++w) {
+      const f32x2 v = *reinterpret_cast<const f32x2 *>(tiles + w * PART + prow * kBwdPartStride + pu);
+      sum0 += v[0];
+      sum1 += v[1];
     }
+    dy[0] = restart_now ? 0.0f : sum0;
+    dy[1] = restart_now ? 0.0f : sum1;
+  };
+  if (!FEED) {
+    fetch_step(in0, p.T - 1);
+    fetch_step(in1, p.T - 2);
+  } else {
+    if (there && p.reset) restart_raw = p.reset[(long long)row * p.reset_sb + p.T - 1];
+    __syncthreads();  // (the feeders' first slot is in place)
+  }
+  for (int t = p.T - 1; t >= 0; t -= 2) {
+    step(in0, t);
+    if (t > 0) step(in1, t - 1);
   }
   // ---- gradient w.r.t. the initial state (the stabiliser's part is zero by the rule; NaN all over when a wait ran out)
   if (there) {
-    const bool poisoned = gave_up || __hip_atomic_load(abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool poisoned = gave_up || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const long long o = (long long)row * H + ecol;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {

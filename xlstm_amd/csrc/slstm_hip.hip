@@ -395,6 +395,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.ry = a->ry; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
+    p.tiled = a->split ? 1 : 0;
     const long long blocks = ((long long)a->B * H + 255) / 256;
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
     hipLaunchKernelGGL(bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
@@ -415,13 +416,24 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
       q.reset = a->reset; q.reset_sb = a->reset_stride_b;
       q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
-      q.xch = (float *)a->exchange; q.cnt = a->counters;
+      if (((uintptr_t)a->exchange % 16)) return fail(XS_ERR_ALIGN, "exchange must be 16-byte aligned");
+      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1;
+      q.main_locals = (int)(grid / 8);
+      const bool prefetchers = grid + 8 <= device_cus();  // (one more workgroup per XCD, where there is room)
       q.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+      const long long n16 = (long long)kBwdRing * ngroups * 16 * 4 * a->dh * (bf16 ? 2 : 4) / 16;
+      hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
+                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
       void (*ks)(BwdSplitParams) = nullptr;
-      if (a->dh == 128) ks = bf16 ? slstm_bwd_split_kernel<true, 1> : slstm_bwd_split_kernel<false, 1>;
-      else if (a->dh == 256) ks = bf16 ? slstm_bwd_split_kernel<true, 2> : slstm_bwd_split_kernel<false, 2>;
-      else ks = slstm_bwd_split_kernel<true, 4>;
-      hipLaunchKernelGGL(ks, dim3((unsigned)grid), dim3(512), 0, stream, q);
+      bool feed = true;  // (feeder waves where the registers allow twelve waves)
+      if (a->dh == 128) ks = bf16 ? slstm_bwd_split_kernel<true, 1, true> : slstm_bwd_split_kernel<false, 1, true>;
+      else if (a->dh == 256 && bf16) ks = slstm_bwd_split_kernel<true, 2, true>;
+      else if (a->dh == 256) { ks = slstm_bwd_split_kernel<false, 2, false>; feed = false; }
+      else { ks = slstm_bwd_split_kernel<true, 4, false>; feed = false; }
+      const int lds = bwd_split_lds_bytes(feed, bf16);
+      if (hipFuncSetAttribute((const void *)ks, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+        return fail(XS_ERR_LAUNCH, "the split backward kernel cannot have %d bytes of LDS", lds);
+      hipLaunchKernelGGL(ks, dim3((unsigned)(grid + (prefetchers ? 8 : 0))), dim3(feed ? 768 : 512), lds, stream, q);
       const hipError_t es = hipGetLastError();
       if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
       return XS_OK;

@@ -111,7 +111,6 @@ def slstm_backward(
         r32 = r32.bfloat16().float()
     yp = y_prev.view(T * B, NH, dh).transpose(0, 1)                      # [NH, T*B, dh]
     ry = torch.bmm(yp, r32.transpose(1, 2)).transpose(0, 1).contiguous()  # [T*B, NH, 4*dh] = [T,B,NH,4,dh]
-    coef = torch.empty((T, B, 9, H), dtype=torch.float32, device=dev)
     d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
     d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
     epc = 8 if bf16 else 4
@@ -121,13 +120,17 @@ def slstm_backward(
     split = (dh in (128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
     if split_override is not None:
         split = bool(split_override)
+    # (the split kernel reads the coefficients in pieces of 16 rows: its buffer covers whole row tiles)
+    coef = torch.empty((T, (B + 15) // 16 * 16 if split else B, 9, H), dtype=torch.float32, device=dev)
     if split:
-        # R transposed per slice of 64 hidden units (gate units k = g*64 + a%64), tiled as MFMA operands:
-        # [NH][S][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
-        r_t = (r32.view(NH, 4, S, 64, dh).permute(0, 2, 4, 1, 3).reshape(NH, S, dh, 256).to(wx.dtype)  # [NH,S,d,k]
-               .reshape(NH, S, dh // 16, 16, 256 // (4 * epc), 4, epc).permute(0, 1, 2, 4, 5, 3, 6).contiguous())
-        exchange = torch.empty(2 * groups * S * 16 * dh, dtype=torch.float32, device=dev)
-        counters = torch.zeros(2 * groups + 1, dtype=torch.int32, device=dev)
+        # R transposed with K ordered (owner slice, gate, unit % 64), tiled as the MFMA B operands of the workgroup
+        # that owns the output columns and of the wave that owns the eighth of K:
+        # [NH][S][8 waves][chunks of a wave][4 column blocks][k chunk of 4][column % 16][k % EPC]
+        ksteps = 4 * dh // 8 // (4 * epc)
+        r_t = (r32.view(NH, 4, S, 64, dh).permute(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh).to(wx.dtype)   # [NH, k, d]
+               .view(NH, 8, ksteps, 4, epc, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
+        exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=wx.dtype, device=dev)
+        counters = torch.empty(1 + groups, dtype=torch.int32, device=dev)
     else:
         # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
         r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
@@ -176,7 +179,7 @@ def slstm_backward(
     dl = d_wx.view(B, T, 4, NH, dh).permute(3, 2, 4, 1, 0).reshape(NH, 4 * dh, T * B)  # [NH, 4*dh, (t, b)]
     d_r = torch.bmm(dl, yp)                                                            # [NH, 4*dh, dh]
     d_bias = d_wx.view(B * T, 4, NH, dh).sum(0).transpose(0, 1).contiguous()
-    if split and timings is None and int(counters[-1].item()):  # (a synchronisation; training calls are not latency-bound)
+    if split and timings is None and int(counters[0].item()):  # (a synchronisation; training calls are not latency-bound)
         raise EngineError("xlstm_amd: a wait between the compute units of a head ran out in the backward pass "
                           "(other work held compute units); the gradients are invalid")
     return d_wx, d_r, d_bias, d_s0
