@@ -33,7 +33,7 @@ struct BwdPrepParams {
   int B, T, NH, dh;
   const void *wx;            // [B,T,4,NH,dh], strides in elements
   long long wx_sb, wx_st;
-  const float *ry;           // [T,B,NH,4,dh] float32: R.h_{t-1}
+  const float *ry;           // [NH,B,T,4,dh] float32: R.h_{t-1}
   const float *bias;         // [NH,4,dh]
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
@@ -57,20 +57,39 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
   for (int g = 0; g < 4; ++g) bias_g[g] = p.bias[((long long)head * 4 + g) * p.dh + a];
   float c = 0.0f, n = 0.0f, m = 0.0f;
   if (p.s0) { c = p.s0[BH + idx]; n = p.s0[2 * BH + idx]; m = p.s0[3 * BH + idx]; }
-  auto load_raw = [&](int t, float (&raw)[4]) {
+  // One wave per compute unit or so: nothing hides a load's way to memory and back but the thread's own requests.
+  // W.x and R.h of a step are requested kPrepAhead steps ahead into a ring of register sets (the loop is unrolled
+  // over it) and stay as they came until their step: anything computed from a load right behind its request would
+  // make the wave wait for it there.
+  constexpr int kPrepAhead = 6;
+  typename std::conditional<BF16, uint16_t, float>::type ring_wx[kPrepAhead][4];
+  float ring_ry[kPrepAhead][4];
+  uint8_t rst[kPrepAhead];
+  auto request = [&](int t, int slot) {
+    if (t >= p.T) return;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const long long wo = (long long)b * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + col;
-      const float w = BF16 ? bf16_bits_to_float(reinterpret_cast<const uint16_t *>(p.wx)[wo]) : reinterpret_cast<const float *>(p.wx)[wo];
-      raw[g] = (w + p.ry[((((long long)t * p.B + b) * p.NH + head) * 4 + g) * p.dh + a]) + bias_g[g];
+      if constexpr (BF16) ring_wx[slot][g] = reinterpret_cast<const uint16_t *>(p.wx)[wo];
+      else ring_wx[slot][g] = reinterpret_cast<const float *>(p.wx)[wo];
+      ring_ry[slot][g] = p.ry[((((long long)head * p.B + b) * p.T + t) * 4 + g) * p.dh + a];
     }
+    if (p.reset) rst[slot] = p.reset[(long long)b * p.reset_sb + t];
   };
-  float nxt[4];
-  load_raw(0, nxt);
-  for (int t = 0; t < p.T; ++t) {
-    float raw[4] = {nxt[0], nxt[1], nxt[2], nxt[3]};
-    if (t + 1 < p.T) load_raw(t + 1, nxt);  // (one step ahead: the loads of a thread's next step do not depend on this one)
-    if (p.reset && p.reset[(long long)b * p.reset_sb + t]) { c = 0.0f; n = 0.0f; m = 0.0f; }
+#pragma unroll
+  for (int i = 0; i < kPrepAhead; ++i) { rst[i] = 0; request(i, i); }
+  auto one_step = [&](int t, int slot) {
+    float raw[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float w;
+      if constexpr (BF16) w = bf16_bits_to_float(ring_wx[slot][g]);
+      else w = ring_wx[slot][g];
+      raw[g] = (w + ring_ry[slot][g]) + bias_g[g];
+    }
+    const bool restart = rst[slot] != 0;
+    request(t + kPrepAhead, slot);
+    if (restart) { c = 0.0f; n = 0.0f; m = 0.0f; }
     // the forward's update (slstm_pointwise), with the gate values kept
     const float sigf_neg = __expf(-fabsf(raw[1]));
     const float lfm = m + (fminf(raw[1], 0.0f) - 0.69314718055994531f * __builtin_amdgcn_logf(1.0f + sigf_neg));
@@ -101,6 +120,11 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     dst[7 * js] = (1.0f - og) * ynew;
     dst[8 * js] = fg;
     c = cnew; n = nnew; m = mnew;
+  };
+  for (int t0 = 0; t0 < p.T; t0 += kPrepAhead) {
+#pragma unroll
+    for (int i = 0; i < kPrepAhead; ++i)
+      if (t0 + i < p.T) one_step(t0 + i, i);
   }
 }
 
