@@ -475,23 +475,19 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
       const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), dh_records, 0x00020000u};
       lds_direct_fetch_b128(drs, uniform(slot + kBwdCoefBytes + dh_part * 1024), dh_voff);
     };
+    // Slot n % 2 is free behind barrier B'(n), but the inputs of step n + 2 are asked for only behind barrier A(n),
+    // when the compute waves add up, read LDS and do arithmetic: right behind B' they publish and poll, and 38 KiB
+    // of requests in front of those in the compute unit's queue cost the group a poll round (4.6 -> 4.2 ms at
+    // config 2).
     request(0);
-    if (p.T > 1) {
-      request(1);
-      asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (p.T > 1) request(1);
     __syncthreads();  // (slot 0 is in place)
     for (int n = 0; n < p.T; ++n) {
       __syncthreads();  // B'(n): slot n % 2 has been read
-      if (n + 2 < p.T) {
-        request(n + 2);
-        asm volatile("s_waitcnt vmcnt(10)" ::: "memory");  // (all but the ten just issued: step n + 1 has landed)
-      } else {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the inputs of step n + 1, requested a step ago, have landed)
       __syncthreads();  // A(n)
+      if (n + 2 < p.T) request(n + 2);
     }
     return;
   }
@@ -523,6 +519,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
     pub_off[g] = (((k / KC) * 16 + prow) * 4 + (k % KC) / EPC) * 16 + (k % EPC) * ESZ;
   }
   const int poll_off = (r16 * 4 + q) * 16;
+  const int wave_u = (int)uniform((uint32_t)wave);  // (on the scalar unit: the polls' slot offsets are scalar operands)
   char *const ring = reinterpret_cast<char *>(p.xch) + (long long)group * SLOT;
   const long long ring_stride = (long long)ngroups * SLOT;
   // the step's inputs of the thread's elements, two sets used in turn: each is requested two steps ahead, right after
@@ -586,18 +583,20 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         if (BF16) {
-          uint32_t w = pack_bf16x2(delta[g][0], delta[g][1]);
-          if ((w & 0xFFFFu) == 0xFFFFu) w = (w & 0xFFFF0000u) | 0x7FC0u;   // (keep the pattern unique)
-          if (w >= 0xFFFF0000u) w = (w & 0xFFFFu) | 0x7FC00000u;
-          *reinterpret_cast<uint32_t *>(cur + pub_off[g]) = w;
-          *reinterpret_cast<uint32_t *>(old + pub_off[g]) = 0xFFFFFFFFu;
+          // (the pattern stays unique: a half of all ones, which only a NaN can give, becomes 0xFFFE, a NaN as well)
+          const u16x2_t w = __builtin_elementwise_min(__builtin_bit_cast(u16x2_t, pack_bf16x2(delta[g][0], delta[g][1])), u16x2_t{0xFFFE, 0xFFFE});
+          *reinterpret_cast<uint32_t *>(cur + pub_off[g]) = __builtin_bit_cast(uint32_t, w);
         } else {
           float d0 = delta[g][0], d1 = delta[g][1];
           if (d0 != d0) d0 = kPoison;
           if (d1 != d1) d1 = kPoison;
           *reinterpret_cast<f32x2 *>(cur + pub_off[g]) = f32x2{d0, d1};
-          *reinterpret_cast<f32x2 *>(old + pub_off[g]) = f32x2{__uint_as_float(kSentinel32), __uint_as_float(kSentinel32)};
         }
+      }
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {  // (behind all of the step's deltas: those are waited for)
+        if (BF16) *reinterpret_cast<uint32_t *>(old + pub_off[g]) = 0xFFFFFFFFu;
+        else *reinterpret_cast<f32x2 *>(old + pub_off[g]) = f32x2{__uint_as_float(kSentinel32), __uint_as_float(kSentinel32)};
       }
     }
     // ---- the group's deltas of the wave's eighth of K: polled straight into the A operand registers
@@ -609,7 +608,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
       for (;;) {
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks)
-          areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, poll_off, (wave * KSTEPS + ks) * 1024, kPastL1));
+          areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(rs, poll_off, (wave_u * KSTEPS + ks) * 1024, kPastL1));
         uint32_t mark = 0u;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[ks]));
