@@ -21,10 +21,11 @@
 //                              operand of MFMAs against R transposed (K = 4 dh gate units, N = dh input units), whose
 //                              result - the gradient that reaches y_{t-1} through the recurrence - stays in the
 //                              registers of the lanes that need it for the next step (the accumulator layout is the
-//                              layout of the pointwise part).  R transposed is read from the L2 every step.
-//
-// This is a first version: a head is not spread over compute units (no exchange between workgroups), so a step is bound
-// by one compute unit's path to the L2 (4 dh x dh operands per step), and head dims are 64, 128 or 256.
+//                              layout of the pointwise part).  R transposed is read from the L2 every step: a step is
+//                              bound by one compute unit's path to the L2 (4 dh x dh operands per step).  Head dims 64,
+//                              128, 256; used for 64 and for launches that the split kernel cannot hold.
+//   slstm_bwd_split_kernel     the same pass with a head spread over dh / 64 compute units that exchange their gate
+//                              deltas every step (head dims 128, 256, 512 in bf16); described in front of it.
 #pragma once
 
 namespace {
