@@ -219,12 +219,17 @@ def bench_backward(device, iters=3):
     # what the reverse kernel has to move per step and element: nine coefficients and the four gate deltas in float32,
     # the output gradient in bf16; R transposed once (the gate deltas that the compute units of a head exchange stay in the L2)
     nbytes = (9 * 4 + 4 * 4 + 2) * B * T * H + NH * 4 * dh * dh * 2
+    traffic = None
+    traffic_file = os.path.join(ROOT, "profiles", "traffic_bwd_cfg2.json")
+    if os.path.exists(traffic_file):
+        traffic = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
     return {"workload": "backward pass at config 2: B=16 T=2048 D=1024 NH=4 bf16, documents mean 512",
             "ms": float(np.median(total)), "prepare_kernel_ms": float(np.median(prep)), "reverse_kernel_ms": rev_ms,
             "tokens_per_s": B * T / (float(np.median(total)) * 1e-3), "finite": bool(torch.isfinite(out[0]).all()),
             "roofline": {"bound": "hbm", "achieved": nbytes / (rev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                         "frac": nbytes / (rev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
-                         "kernel": "slstm_bwd_split_kernel<bf16,NB=2,FEED>", "algorithmic_bytes_per_launch": nbytes}}
+                         "frac": nbytes / (rev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
+                         "kernel": "slstm_bwd_split_kernel<bf16,NB=2,FEED>", "algorithmic_bytes_per_launch": nbytes,
+                         "traffic_source": "profiles/traffic_bwd_cfg2.json (rocprofv3 counters of a separate run, not of this one)"}}
 
 
 def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
