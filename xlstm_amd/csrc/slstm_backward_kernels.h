@@ -600,6 +600,17 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
         else *reinterpret_cast<f32x2 *>(old + pub_off[g]) = f32x2{__uint_as_float(kSentinel32), __uint_as_float(kSentinel32)};
       }
     }
+    // ---- between the publication and the first look at the peers' deltas, which need a while to land: the step's
+    //      gate deltas to d_wx and a short sleep (reverse kernel at config 2: 4.25 ms with these stores behind the poll,
+    //      4.14 with them here, 4.11 / 4.06 with 256 / 512 cycles of sleep on top, 4.16 / 4.50 with 1024 / 1536)
+    if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
+    if (FEED && there && p.reset && t > 0) restart_raw = p.reset[(long long)row * p.reset_sb + t - 1];  // (used by the next step)
+    if (there) {
+      float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
+#pragma unroll
+      for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
+    }
+    __builtin_amdgcn_s_sleep(8);
     // ---- the group's deltas of the wave's eighth of K: polled straight into the A operand registers
     uint4 areg[KSTEPS];
     {
@@ -621,15 +632,8 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
         }
       }
     }
-    if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
-    // ---- behind the poll: the inputs of the step after the next, then the step's gate deltas to d_wx
+    // ---- behind the poll: the inputs of the step after the next
     if (!FEED) fetch_step(in, t - 2);
-    if (FEED && there && p.reset && t > 0) restart_raw = p.reset[(long long)row * p.reset_sb + t - 1];  // (used by the next step)
-    if (there) {
-      float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
-#pragma unroll
-      for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
-    }
     // ---- delta [16 x K/8] . R^T [K/8 x 64]: the wave's partial result, to LDS
     f32x4 acc[4];
 #pragma unroll
