@@ -33,6 +33,8 @@ CASES = [
 
 # what the kernel that spreads a head over dh / 64 compute units adds: head dim 512 (bf16), many row tiles
 SPLIT_CASES = [
+    (False, 3, 1, 2, 128, False),     # one step: the feeders' first slot only
+    (True, 17, 2, 2, 256, True),      # two steps, two row tiles
     (True, 9, 7, 2, 512, True),
     (True, 100, 5, 2, 256, True),
     (False, 50, 6, 4, 128, True),
