@@ -284,7 +284,7 @@ typedef struct xs_slstm_bwd_args {
   int64_t d_wx_stride_b, d_wx_stride_t;
   float *d_s0;               /* [4,B,H] (backward) */
   void *stream;
-  /* backward, optional: a head spread over dh/64 compute units (head dims 128, 256; 512 in bf16).  With split != 0,
+  /* backward, optional: a head spread over dh/64 compute units (head dims 64, 128, 256; 512 in bf16).  With split != 0,
    * r_t holds R transposed with K ordered k = 256*(a/64) + 64*g + a%64 (a the hidden unit, g the gate), tiled as MFMA
    * operands per owner of the output columns and per wave: [NH][dh/64][8][K/8/KC][4][KC/EPC][16][EPC], EPC the elements
    * of 16 bytes and KC = 4*EPC; exchange is a 16-byte aligned buffer of 4 * NH * ceil(B/16) * 16 * 4*dh elements of

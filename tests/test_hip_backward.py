@@ -46,8 +46,6 @@ SPLIT_CASES = [
 def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, split):
     from xlstm_amd import functional as F
 
-    if split and dh == 64:
-        pytest.skip("head dim 64 is one workgroup's worth: no split")
     if not split and dh == 512:
         pytest.skip("head dim 512 has the split kernel only")
     print("case backward", bf16, B, T, NH, dh, masked, split, flush=True)

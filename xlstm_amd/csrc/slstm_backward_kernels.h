@@ -23,9 +23,9 @@
 //                              registers of the lanes that need it for the next step (the accumulator layout is the
 //                              layout of the pointwise part).  R transposed is read from the L2 every step: a step is
 //                              bound by one compute unit's path to the L2 (4 dh x dh operands per step).  Head dims 64,
-//                              128, 256; used for 64 and for launches that the split kernel cannot hold.
+//                              128, 256; used for launches that the split kernel cannot hold.
 //   slstm_bwd_split_kernel     the same pass with a head spread over dh / 64 compute units that exchange their gate
-//                              deltas every step (head dims 128, 256, 512 in bf16); described in front of it.
+//                              deltas every step (head dims 64 - one unit, the same step - 128, 256, 512 in bf16); described in front of it.
 #pragma once
 
 namespace {
@@ -427,14 +427,14 @@ constexpr int bwd_split_lds_bytes(bool feed, bool bf16) {
 // With feeders a step has two barriers: B', behind which the slot that the step's inputs were read from is free for
 // the inputs of the step after the next, and A, in front of which the wave's partial tile is written and the next
 // step's inputs have landed.  (Without: one barrier, two sets of partial tiles.)
-template <bool BF16, int NB, bool FEED>  // eight compute waves; dh = 128 NB, S = 2 NB workgroups per group
+template <bool BF16, int S, bool FEED>  // eight compute waves; S workgroups per group, dh = 64 S (S = 1: one workgroup
+                                        // per head and row tile, the same step with nobody else to wait for)
 __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSplitParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int EPC = 16 / ESZ;               // elements of a 16-byte chunk
   constexpr int KC = 4 * EPC;                 // K of one chunk row: what one MFMA (bf16) or four (float32) take
-  constexpr int dh = NB * 128;
   constexpr int UW = 64;                      // hidden units of a workgroup
-  constexpr int S = dh / UW;
+  constexpr int dh = S * UW;
   constexpr int K = 4 * dh;
   constexpr int KSTEPS = K / 8 / KC;          // chunks of a wave: its eighth of K
   constexpr int SLOT = 16 * K * ESZ;          // bytes of a group's slot

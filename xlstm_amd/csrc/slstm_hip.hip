@@ -404,7 +404,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");
     if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
     if (a->split) {
-      if (a->dh != 128 && a->dh != 256 && !(a->dh == 512 && bf16))
+      if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && bf16))
         return fail(XS_ERR_UNSUPPORTED, "backward pass over several compute units per head: head dim %d not supported", a->dh);
       if (!a->exchange || !a->counters) return fail(XS_ERR_NULL, "exchange and counters are required with split");
       const int S = a->dh / 64;
@@ -426,10 +426,11 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
                          (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
       void (*ks)(BwdSplitParams) = nullptr;
       bool feed = true;  // (feeder waves where the registers allow twelve waves)
-      if (a->dh == 128) ks = bf16 ? slstm_bwd_split_kernel<true, 1, true> : slstm_bwd_split_kernel<false, 1, true>;
-      else if (a->dh == 256 && bf16) ks = slstm_bwd_split_kernel<true, 2, true>;
-      else if (a->dh == 256) { ks = slstm_bwd_split_kernel<false, 2, false>; feed = false; }
-      else { ks = slstm_bwd_split_kernel<true, 4, false>; feed = false; }
+      if (a->dh == 64) ks = bf16 ? slstm_bwd_split_kernel<true, 1, true> : slstm_bwd_split_kernel<false, 1, true>;
+      else if (a->dh == 128) ks = bf16 ? slstm_bwd_split_kernel<true, 2, true> : slstm_bwd_split_kernel<false, 2, true>;
+      else if (a->dh == 256 && bf16) ks = slstm_bwd_split_kernel<true, 4, true>;
+      else if (a->dh == 256) { ks = slstm_bwd_split_kernel<false, 4, false>; feed = false; }
+      else { ks = slstm_bwd_split_kernel<true, 8, false>; feed = false; }
       const int lds = bwd_split_lds_bytes(feed, bf16);
       if (hipFuncSetAttribute((const void *)ks, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
         return fail(XS_ERR_LAUNCH, "the split backward kernel cannot have %d bytes of LDS", lds);

@@ -75,7 +75,7 @@ def slstm_backward(
     Two kernels of the engine (``xs_slstm_backward_prepare``, ``xs_slstm_backward``) around three plain library GEMMs and
     a reduction: ``R.h_{t-1}`` for all steps at once in front, and the gradients of R and the bias, which are sums over
     all steps of products of the gate deltas with the outputs, behind.  ``timings`` (a dict) receives three events around
-    the two kernels.  Where the head dim allows it (128, 256; 512 in bfloat16) and the workgroups fit the device at once,
+    the two kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
     """
@@ -120,7 +120,7 @@ def slstm_backward(
     groups = NH * ((B + 15) // 16)
     S = dh // 64
     # a head over S compute units where the head dim allows it and all workgroups fit the device at once
-    split = (dh in (128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
+    split = (dh in (64, 128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
     if split_override is not None:
         split = bool(split_override)
     # (the split kernel reads the coefficients in pieces of 16 rows: its buffer covers whole row tiles)
