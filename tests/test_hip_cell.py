@@ -193,12 +193,22 @@ def test_float16_input_is_computed_in_float32_and_rounded_back():
 
 
 def test_backward_raises_for_head_dims_without_backward_kernels():
-    wx, r, b, _ = make_problem(24, 1, 2, 1, 16)
+    wx, r, b, _ = make_problem(24, 1, 2, 1, 384)  # (float32: the backward kernels end at head dim 256)
     cell = _cell_from(r, b, dtype="float32").train()
     x = torch.from_numpy(wx).cuda().requires_grad_(True)
     out, _ = cell(x)
     with pytest.raises(RuntimeError, match="backward pass for head dims"):
         out.sum().backward()
+
+
+def test_backward_of_a_small_head_dim_runs_padded():
+    wx, r, b, _ = make_problem(24, 2, 5, 2, 16)
+    cell = _cell_from(r, b, dtype="float32").train()
+    x = torch.from_numpy(wx).cuda().requires_grad_(True)
+    out, _ = cell(x)
+    out.sum().backward()
+    assert x.grad is not None and torch.isfinite(x.grad).all() and x.grad.abs().max() > 0
+    assert cell._recurrent_kernel_.grad is not None and torch.isfinite(cell._recurrent_kernel_.grad).all()
 
 
 def test_unsupported_head_dim_is_an_error_not_a_wrong_answer():

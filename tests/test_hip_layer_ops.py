@@ -227,7 +227,7 @@ def test_layer_with_engine_pre_ops_equals_layer_with_torch_pre_ops():
 
 def test_layer_under_autograd_keeps_the_pytorch_ops_and_trains_through_the_cell():
     """The engine's layer kernels record no graph: with grad enabled the layer keeps its PyTorch ops around the cell,
-    and the cell's own backward kernels carry the gradient (head dims 64, 128, 256); other head dims raise."""
+    and the cell's own backward kernels carry the gradient (head dims in between their sizes run padded)."""
     from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
 
     torch.manual_seed(12)
@@ -242,9 +242,9 @@ def test_layer_under_autograd_keeps_the_pytorch_ops_and_trains_through_the_cell(
     grads = [p.grad for p in layer.parameters()]
     assert all(g is not None and torch.isfinite(g.float()).all() for g in grads)
     assert x.grad is not None and torch.isfinite(x.grad.float()).all() and x.grad.float().abs().max() > 0
-    small = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=8, backend="hip")).to(DEV).bfloat16()  # head dim 32
-    with pytest.raises(RuntimeError, match="backward pass for head dims"):
-        small(x.detach()).float().sum().backward()
+    small = sLSTMLayer(sLSTMLayerConfig(embedding_dim=256, num_heads=8, backend="hip")).to(DEV).bfloat16()  # head dim 32: padded
+    small(x.detach()).float().sum().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad.float()).all() for p in small.parameters())
 
 
 def test_layer_ops_accept_empty_inputs():

@@ -168,7 +168,7 @@ class sLSTMCellConfig:
         self.num_states = rnn_function_registry[self.function]["states"]
 
 
-BACKWARD_HEAD_DIMS = (64, 128, 256, 512)  # what xs_slstm_backward covers (512: bfloat16 inputs only)
+BACKWARD_MAX_HEAD_DIM = {torch.float32: 256, torch.bfloat16: 512}  # what xs_slstm_backward covers (smaller head dims padded up)
 
 
 class _ForwardOnly(torch.autograd.Function):
@@ -182,7 +182,7 @@ class _ForwardOnly(torch.autograd.Function):
     @staticmethod
     def backward(ctx, *grads):
         raise RuntimeError(
-            f"sLSTMCell backend 'hip' has a backward pass for head dims {BACKWARD_HEAD_DIMS} only; "
+            "sLSTMCell backend 'hip' has a backward pass for head dims up to 256 (float32) and 512 (bfloat16) only; "
             "use the reference's 'cuda' or 'vanilla' backend to train this shape"
         )
 
@@ -492,7 +492,7 @@ class sLSTMCell_hip(nn.Module):
             input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
             or (state is not None and state.requires_grad)
         ):
-            if self.head_dim in BACKWARD_HEAD_DIMS and x.is_cuda:
+            if x.is_cuda and self.head_dim <= BACKWARD_MAX_HEAD_DIM.get(x.dtype, 0):
                 h, s = _CellFunction.apply(x, self._recurrent_kernel_, self._bias_, state, h, s, reset_mask,
                                            self.config.num_heads)
             else:

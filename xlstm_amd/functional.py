@@ -52,6 +52,15 @@ def _compute_units(dev) -> int:
     return _CU_COUNT[idx]
 
 
+def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
+    """The head dim that the backward kernels run a head dim ``dh`` as (64, 128, 256, and 512 with bfloat16 inputs; sizes in
+    between are padded up by ``slstm_backward``), or None when there is none."""
+    for size in (64, 128, 256, 512):
+        if dh <= size and (size < 512 or dtype == torch.bfloat16):
+            return size
+    return None
+
+
 def slstm_backward(
     wx: torch.Tensor,
     r: torch.Tensor,
@@ -87,9 +96,36 @@ def slstm_backward(
     if wx.dtype not in _DTYPE_CODE:
         raise TypeError(f"wx dtype {wx.dtype} not supported by the hip backend (float32 or bfloat16)")
     bf16 = wx.dtype == torch.bfloat16
-    dev = wx.device
     if tuple(h_out.shape) != (T, B, H) or tuple(d_h.shape) != (T, B, H):
         raise ValueError(f"h_out and d_h must be [S, B, H] = {(T, B, H)}")
+    dh_k = backward_kernel_head_dim(dh, wx.dtype)
+    if dh_k is None:
+        raise EngineError(f"xlstm_amd: no backward kernel for head dim {dh} with {wx.dtype} inputs "
+                          f"(up to 512 with bfloat16, up to 256 with float32)")
+    if dh_k != dh:
+        # A head dim between the kernels' sizes runs as the next size up with units that are not there: their W.x, bias
+        # and rows and columns of R are zero, so they neither see nor touch the real units, and their results are cut off.
+        pad = dh_k - dh
+        B_, T_ = int(wx.shape[0]), int(wx.shape[1])
+        Fn = torch.nn.functional
+
+        def widen(x, lead):  # [*lead, NH*dh] -> [*lead, NH, dh_k], zeros behind the real units
+            return Fn.pad(x.reshape(*lead, NH, dh), (0, pad))
+
+        wx_p = widen(wx, (B_, T_, 4)).reshape(B_, T_, 4 * NH * dh_k)
+        r_p = Fn.pad(r.reshape(NH, 4, dh, dh), (0, pad, 0, pad)).reshape(NH, 4 * dh_k, dh_k)
+        bias_p = Fn.pad(bias, (0, pad))
+        s0_p = widen(s0, (4, B_)).reshape(4, B_, NH * dh_k) if s0 is not None else None
+        h_p = widen(h_out, (T_, B_)).reshape(T_, B_, NH * dh_k)
+        dh_p = widen(d_h, (T_, B_)).reshape(T_, B_, NH * dh_k)
+        dsf_p = widen(d_s_final, (4, B_)).reshape(4, B_, NH * dh_k) if d_s_final is not None else None
+        d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
+                                                 split_override=split_override, spin_limit=spin_limit)
+        return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
+                d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
+                d_bias[..., :dh].contiguous(),
+                d_s0.view(4, B_, NH, dh_k)[..., :dh].reshape(4, B_, H))
+    dev = wx.device
     if wx.stride(2) != 1 or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H):
         wx = wx.contiguous()
     bias = bias.to(torch.float32).contiguous()
