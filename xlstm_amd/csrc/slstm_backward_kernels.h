@@ -301,12 +301,12 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
 // registers of the eight waves for the whole call, each wave holding one eighth of K for all 64 columns; the eight
 // partial results are added up through LDS.  Per step a workgroup writes its 16 x 256 deltas (8 KiB in bf16) and reads
 // the group's 16 x 4 dh, straight into MFMA operand registers; nothing else is read from memory per step but the
-// coefficients of its own elements, which are fetched two steps ahead.
+// coefficients and d_h of its own elements (by feeder waves, or two steps ahead: see FEED below).
 //
 // The exchange is a ring of kBwdRing slots per group, slot n % kBwdRing for the n-th step of the call, laid out as
 // MFMA A operands: [K / KC][16 rows][4][16 bytes] with KC = 32 (bf16) or 16 (float32) and K index
 // k = 256 s + 64 gate + unit % 64.  A word is data or the "not written yet" pattern (all ones, which no value takes:
-// NaNs are made canonical).  A reader polls its 16-byte chunks until none holds the pattern.  A workgroup that
+// a NaN that would is changed into another NaN).  A reader polls its 16-byte chunks until none holds the pattern.  A workgroup that
 // publishes step n also re-arms its words of step n - 2: it has read all deltas of step n - 1, which every peer
 // computed from a complete set of step n - 2.  The re-arm is acknowledged before the workgroup's poll of step n
 // returns (accesses of a wave complete in order), so before it publishes step n + 1; a peer that polls the slot again
