@@ -72,7 +72,42 @@ def test_a_copy_of_a_register_with_a_hand_issued_load_in_flight_is_found():
     assert isa_check.inflight_register_uses(TO_LDS) == []
 
 
+_LISTING = {}
+
+
+def _compiled_listing(tmp_path):
+    if "text" not in _LISTING:  # (one compilation for the tests of this file)
+        _LISTING["text"] = isa_check.emit_assembly(os.path.join(tmp_path, "device.s"))
+    return _LISTING["text"]
+
+
 def test_the_kernels_as_compiled_have_neither(tmp_path):
-    listing = isa_check.emit_assembly(os.path.join(tmp_path, "device.s"))
+    listing = _compiled_listing(tmp_path)
     assert listing.count("ASMSTART") > 50  # (the listing really is the kernels')
     assert isa_check.check(listing) == []
+
+
+def test_the_backward_kernel_with_feeder_waves_keeps_its_registers_and_polls_with_scalar_offsets(tmp_path):
+    """Two properties of slstm_bwd_split_kernel that its speed rests on and that only the assembly shows: the variants
+    with feeder waves (twelve waves: 168 registers a lane) do not spill, and the polls of the exchange ring take their
+    slot offset from a scalar register (with the offset in a vector register the compiler wraps every poll in a loop
+    over the distinct values of the lanes)."""
+    import re
+
+    listing = _compiled_listing(tmp_path)
+    meta = listing[listing.index("amdhsa.kernels:"):]
+    seen = 0
+    for entry in re.split(r"\n  - ", meta)[1:]:
+        name = re.search(r"\.name:\s+(\S+)", entry)
+        if not name or "slstm_bwd_split_kernel" not in name.group(1) or not name.group(1).endswith("ELb1EEEvNS_14BwdSplitParamsE"):
+            continue
+        seen += 1
+        assert int(re.search(r"\.vgpr_count:\s*(\d+)", entry).group(1)) <= 168, name.group(1)
+        assert int(re.search(r"\.private_segment_fixed_size:\s*(\d+)", entry).group(1)) == 0, name.group(1)
+        body = listing[listing.index(name.group(1) + ":"):]
+        body = body[: body.index(".end_amdhsa_kernel")].split("\n")
+        polls = [i for i, line in enumerate(body) if "buffer_load_dwordx4" in line and "sc1" in line]
+        assert polls, name.group(1)
+        for i in polls:
+            assert not any("v_readfirstlane" in line for line in body[max(0, i - 6): i]), (name.group(1), body[i - 6: i + 1])
+    assert seen == 5  # bf16 at head dims 64, 128, 256; float32 at 64, 128
