@@ -32,6 +32,30 @@ CASES = [
 
 
 # what the kernel that spreads a head over dh / 64 compute units adds: head dim 512 (bf16), many row tiles
+def test_a_batch_with_more_row_tiles_than_the_device_holds_runs_in_slices_of_rows():
+    """B = 500 at head dim 256 with two heads is 32 row tiles x 2 heads x 4 compute units = 256 workgroups, more than
+    the device holds beside the prefetching ones: two launches of the split kernel over slices of rows, against the
+    oracle."""
+    from xlstm_amd import functional as F
+
+    B, T, NH, dh = 500, 3, 2, 256
+    H = NH * dh
+    wx, r, b, s0 = make_problem(93, B, T, NH, dh, rscale=2.0, bf16=True, with_state=True)
+    reset = geometric_reset_mask(8, B, T, 2)
+    d_h = torch.from_numpy(np.random.default_rng(94).standard_normal((T, B, H)).astype(np.float32)).bfloat16().float().numpy()
+    r = torch.from_numpy(r).bfloat16().float().numpy()
+    dev = torch.device("cuda:0")
+    wx_t, r_t, b_t = torch.from_numpy(wx).to(dev).bfloat16(), r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    s0_t, m_t = torch.from_numpy(s0).to(dev), torch.from_numpy(reset).to(dev)
+    h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
+    d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev))
+    torch.cuda.synchronize()
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h)
+    errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
+                d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
+    assert all(np.isfinite(v) and v <= 2e-2 for v in errs.values()), errs
+
+
 PADDED_CASES = [
     # head dims between the kernels' sizes: run as the next size up with zero units
     (False, 3, 6, 2, 16, True),

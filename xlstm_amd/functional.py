@@ -126,6 +126,23 @@ def slstm_backward(
                 d_bias[..., :dh].contiguous(),
                 d_s0.view(4, B_, NH, dh_k)[..., :dh].reshape(4, B_, H))
     dev = wx.device
+    # The kernel that spreads a head over dh/64 compute units needs all its workgroups on the device at once.  A batch
+    # with more row tiles than that runs in slices of rows (rows do not meet in the backward pass but in the sums for
+    # R and the bias), rather than with one workgroup per head, which takes 7 times as long per step.
+    if split_override is not False:
+        room = (_compute_units(dev) - 8) // (8 * (dh // 64)) * 8      # groups per launch, the prefetching workgroups kept
+        tiles_per_launch = room // NH
+        if tiles_per_launch >= 1 and (B + 15) // 16 > tiles_per_launch:
+            rows = tiles_per_launch * 16
+            parts = []
+            for b0 in range(0, B, rows):
+                b1 = min(B, b0 + rows)
+                parts.append(slstm_backward(
+                    wx[b0:b1], r, bias, None if s0 is None else s0[:, b0:b1], None if reset_mask is None else reset_mask[b0:b1],
+                    h_out[:, b0:b1], d_h[:, b0:b1], None if d_s_final is None else d_s_final[:, b0:b1],
+                    timings=None, split_override=split_override, spin_limit=spin_limit))
+            return (torch.cat([q[0] for q in parts], 0), sum(q[1] for q in parts), sum(q[2] for q in parts),
+                    torch.cat([q[3] for q in parts], 1))
     if wx.stride(2) != 1 or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H):
         wx = wx.contiguous()
     bias = bias.to(torch.float32).contiguous()
