@@ -251,7 +251,7 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  * reference's per-timestep launches (slstm_backward.cu:291-319) and the state history and gate cache its forward
  * writes for them (slstm.cc:79-108); the forward entry points above store nothing for training.
  *
- * xs_slstm_backward_prepare  walks forward in time over raw = wx + ry + bias, where ry[h,b,t,g,a] =
+ * xs_slstm_backward_prepare  walks forward in time over raw = wx + ry + bias, where ry[h,b,t,a,g] =
  *   sum_d y_{t-1}[b,h,d] * r[h][g*dh+a][d] is given for all steps at once (one batched GEMM over the outputs of the
  *   forward call, shifted by one step, rows that start a document zeroed), and writes nine float32 coefficients per
  *   step and element into coef [T,B,9,H] (with split != 0: T * ceil(B/16)*16 * 9 * H floats, in the order the split
@@ -271,7 +271,7 @@ typedef struct xs_slstm_bwd_args {
   int32_t dtype;
   const void *wx;            /* [B,T,4,NH,dh], strides in elements, innermost 4*H contiguous (prepare) */
   int64_t wx_stride_b, wx_stride_t;
-  const float *ry;           /* [NH,B,T,4,dh] (prepare) */
+  const float *ry;           /* [NH,B,T,dh,4] (prepare) */
   const float *bias;         /* [NH,4,dh] (prepare) */
   const float *s0;           /* [4,B,H] or NULL (prepare) */
   const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */

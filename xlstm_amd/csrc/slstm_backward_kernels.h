@@ -34,7 +34,7 @@ struct BwdPrepParams {
   int B, T, NH, dh;
   const void *wx;            // [B,T,4,NH,dh], strides in elements
   long long wx_sb, wx_st;
-  const float *ry;           // [NH,B,T,4,dh] float32: R.h_{t-1}
+  const float *ry;           // [NH,B,T,dh,4] float32: R.h_{t-1}, the four gates of a unit side by side
   const float *bias;         // [NH,4,dh]
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
@@ -62,9 +62,10 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
   // W.x and R.h of a step are requested kPrepAhead steps ahead into a ring of register sets (the loop is unrolled
   // over it) and stay as they came until their step: anything computed from a load right behind its request would
   // make the wave wait for it there.
-  constexpr int kPrepAhead = 6;
+  constexpr int kPrepAhead = 6;  // (10 and 16: the same time; with the nine stores of a step at most 63 memory operations are
+                                 // in flight, four steps' worth, whatever the ring holds)
   typename std::conditional<BF16, uint16_t, float>::type ring_wx[kPrepAhead][4];
-  float ring_ry[kPrepAhead][4];
+  f32x4 ring_ry[kPrepAhead];  // (the four gates of the element in one load)
   uint8_t rst[kPrepAhead];
   auto request = [&](int t, int slot) {
     if (t >= p.T) return;
@@ -73,8 +74,8 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
       const long long wo = (long long)b * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + col;
       if constexpr (BF16) ring_wx[slot][g] = reinterpret_cast<const uint16_t *>(p.wx)[wo];
       else ring_wx[slot][g] = reinterpret_cast<const float *>(p.wx)[wo];
-      ring_ry[slot][g] = p.ry[((((long long)head * p.B + b) * p.T + t) * 4 + g) * p.dh + a];
     }
+    ring_ry[slot] = *reinterpret_cast<const f32x4 *>(p.ry + ((((long long)head * p.B + b) * p.T + t) * p.dh + a) * 4);
     if (p.reset) rst[slot] = p.reset[(long long)b * p.reset_sb + t];
   };
 #pragma unroll
