@@ -611,7 +611,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
 #pragma unroll
       for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
     }
-    __builtin_amdgcn_s_sleep(8);
+    if (S > 1) __builtin_amdgcn_s_sleep(8);  // (a workgroup that is its own group has its deltas in the L2 by the time it asks)
     // ---- the group's deltas of the wave's eighth of K: polled straight into the A operand registers
     uint4 areg[KSTEPS];
     {
