@@ -45,52 +45,104 @@ struct BwdPrepParams {
   int tiled;
 };
 
+// 16 bytes (or one byte) per lane from a buffer straight into LDS, lane i's bytes at lds_addr + 16 i (+ 4 i).  The wait
+// states in front: the descriptor may sit in scalar registers that a vector instruction has just written, and the
+// compiler does not look for that hazard inside a statement like this.
+__device__ __forceinline__ void bwd_fetch_to_lds_b128(u32x4_t rsrc, uint32_t lds_addr, uint32_t voffset) {
+  asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+__device__ __forceinline__ void bwd_fetch_to_lds_u8(u32x4_t rsrc, uint32_t lds_addr, uint32_t voffset) {
+  asm volatile("s_nop 4\n\ts_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_ubyte %1, %2, 0 offen lds"
+               :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+
+// One workgroup per (batch row, 64 hidden units): wave 0 walks through time, waves 1 to 3 bring its inputs to LDS -
+// W.x, R.h and the reset flag, one wave each, one load a step - in blocks of kPrepBlock steps, two or three blocks ahead, with
+// loads that write LDS directly and waits written by hand.  With the inputs fetched by the walking wave itself, into
+// registers six steps ahead, the kernel took 0.95 ms at config 2 and 0.36 ms without its loads: a wave has at most
+// 63 memory operations in flight, the nine stores of a step among them, which is four steps' worth of loads against a
+// way to HBM and back of several microseconds, and there is about one such wave per compute unit.
+constexpr int kPrepBlock = 8;
 template <bool BF16>
 __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p) {
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int WXB = 4 * 64 * ESZ;           // W.x of a step: [4 gates][64 units]
+  constexpr int RYB = 64 * 16;                // R.h of a step: [64 units][4 gates] float32
+  constexpr int SLOT = WXB + RYB + 16;        // ... and the row's reset flag
+  constexpr int NR = BF16 ? 4 : 3;            // blocks in the ring (48 KiB either way): NR - 1 of them ahead
+  __shared__ __attribute__((aligned(16))) char ring[NR * kPrepBlock * SLOT];
   const int H = p.NH * p.dh;
-  const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
-  if (idx >= (long long)p.B * H) return;
-  const int b = (int)(idx / H), col = (int)(idx - (long long)b * H);
-  const int head = col / p.dh, a = col - head * p.dh;
-  const long long BH = (long long)p.B * H;
+  const int slices = H >> 6;
+  const int b = blockIdx.x / slices, col0 = (blockIdx.x - b * slices) << 6;
+  const int head = col0 / p.dh, a0 = col0 - head * p.dh;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = (int)uniform((uint32_t)(tid >> 6));
+  const int nblocks = (p.T + kPrepBlock - 1) / kPrepBlock;
+  const uint32_t ring_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)ring);
+  if (wave > 0) {
+    // ---- a loader wave.  Block k sits in ring part k % NR; it is asked for behind barrier k - NR + 1 (when the walking
+    //      wave is through with block k - NR, which sat there) and has landed in front of barrier k.
+    auto descriptor = [&](const void *base, uint32_t bytes) {
+      const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+      return u32x4_t{uniform((uint32_t)a), uniform((uint32_t)(a >> 32) & 0xFFFFu), bytes, 0x00020000u};
+    };
+    auto request_block = [&](int k) {  // eight loads, whatever T is (steps past the end ask for the last step again)
+#pragma unroll
+      for (int i = 0; i < kPrepBlock; ++i) {
+        int t = k * kPrepBlock + i;
+        t = t < p.T ? t : p.T - 1;
+        const uint32_t slot = ring_lds + ((k % NR) * kPrepBlock + i) * SLOT;
+        if (wave == 1) {        // W.x: a gate's 64 units are 128 bytes (bf16: 8 lanes) or 256 (float32: 16 lanes)
+          constexpr int LPG = 64 * ESZ / 16;
+          const char *base = reinterpret_cast<const char *>(p.wx) + ((long long)b * p.wx_sb + (long long)t * p.wx_st + col0) * ESZ;
+          const uint32_t voff = (uint32_t)(((long long)(lane / LPG) * H) * ESZ + (lane % LPG) * 16);
+          const u32x4_t rs = descriptor(base, (uint32_t)((3ll * H + 64) * ESZ));
+          const uint32_t dst = uniform(slot);
+          if (lane < 4 * LPG) bwd_fetch_to_lds_b128(rs, dst, voff);  // (only these lanes write LDS)
+        } else if (wave == 2) {  // R.h: the slice's 64 units x 4 gates are 1 KiB in a row
+          const float *base = p.ry + ((((long long)head * p.B + b) * p.T + t) * p.dh + a0) * 4;
+          bwd_fetch_to_lds_b128(descriptor(base, 1024u), uniform(slot + WXB), (uint32_t)lane * 16u);
+        } else {                 // the row's reset flag (lane 0; without a mask: nothing is read, the word is not used)
+          const unsigned char *base = p.reset ? p.reset + (long long)b * p.reset_sb + t : reinterpret_cast<const unsigned char *>(p.wx);
+          const u32x4_t rs = descriptor(base, 1u);
+          const uint32_t dst = uniform(slot + WXB + RYB);
+          if (lane == 0) bwd_fetch_to_lds_u8(rs, dst, 0u);
+        }
+      }
+    };
+    // (blocks past the end are asked for like the others - their steps are the last step again, their ring part is
+    // free - so that every wait below is for the same count)
+#pragma unroll
+    for (int j = 0; j < NR - 1; ++j) request_block(j);
+    for (int k = 0; k < nblocks; ++k) {
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kPrepBlock * (NR - 2)) : "memory");  // (block k has landed)
+      __syncthreads();  // barrier k: the walking wave is through with block k - 1
+      request_block(k + NR - 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+  // ---- the walking wave: lane = unit of the slice
+  const int col = col0 + lane, a = a0 + lane;
+  const long long BH = (long long)p.B * H, idx = (long long)b * H + col;
   float bias_g[4];
 #pragma unroll
   for (int g = 0; g < 4; ++g) bias_g[g] = p.bias[((long long)head * 4 + g) * p.dh + a];
   float c = 0.0f, n = 0.0f, m = 0.0f;
   if (p.s0) { c = p.s0[BH + idx]; n = p.s0[2 * BH + idx]; m = p.s0[3 * BH + idx]; }
-  // One wave per compute unit or so: nothing hides a load's way to memory and back but the thread's own requests.
-  // W.x and R.h of a step are requested kPrepAhead steps ahead into a ring of register sets (the loop is unrolled
-  // over it) and stay as they came until their step: anything computed from a load right behind its request would
-  // make the wave wait for it there.
-  constexpr int kPrepAhead = 6;  // (10 and 16: the same time; with the nine stores of a step at most 63 memory operations are
-                                 // in flight, four steps' worth, whatever the ring holds)
-  typename std::conditional<BF16, uint16_t, float>::type ring_wx[kPrepAhead][4];
-  f32x4 ring_ry[kPrepAhead];  // (the four gates of the element in one load)
-  uint8_t rst[kPrepAhead];
-  auto request = [&](int t, int slot) {
-    if (t >= p.T) return;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const long long wo = (long long)b * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + col;
-      if constexpr (BF16) ring_wx[slot][g] = reinterpret_cast<const uint16_t *>(p.wx)[wo];
-      else ring_wx[slot][g] = reinterpret_cast<const float *>(p.wx)[wo];
-    }
-    ring_ry[slot] = *reinterpret_cast<const f32x4 *>(p.ry + ((((long long)head * p.B + b) * p.T + t) * p.dh + a) * 4);
-    if (p.reset) rst[slot] = p.reset[(long long)b * p.reset_sb + t];
-  };
-#pragma unroll
-  for (int i = 0; i < kPrepAhead; ++i) { rst[i] = 0; request(i, i); }
-  auto one_step = [&](int t, int slot) {
+  const bool has_mask = p.reset != nullptr;
+  auto one_step = [&](int t, const char *slot) {
     float raw[4];
+    const f32x4 ry = *reinterpret_cast<const f32x4 *>(slot + WXB + lane * 16);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       float w;
-      if constexpr (BF16) w = bf16_bits_to_float(ring_wx[slot][g]);
-      else w = ring_wx[slot][g];
-      raw[g] = (w + ring_ry[slot][g]) + bias_g[g];
+      if constexpr (BF16) w = bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(slot + (g * 64 + lane) * 2));
+      else w = *reinterpret_cast<const float *>(slot + (g * 64 + lane) * 4);
+      raw[g] = (w + ry[g]) + bias_g[g];
     }
-    const bool restart = rst[slot] != 0;
-    request(t + kPrepAhead, slot);
+    const bool restart = has_mask && (*reinterpret_cast<const uint32_t *>(slot + WXB + RYB) & 0xFFu) != 0u;
     if (restart) { c = 0.0f; n = 0.0f; m = 0.0f; }
     // the forward's update (slstm_pointwise), with the gate values kept
     const float sigf_neg = __expf(-fabsf(raw[1]));
@@ -123,10 +175,13 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     dst[8 * js] = fg;
     c = cnew; n = nnew; m = mnew;
   };
-  for (int t0 = 0; t0 < p.T; t0 += kPrepAhead) {
+  for (int k = 0; k < nblocks; ++k) {
+    __syncthreads();  // barrier k
 #pragma unroll
-    for (int i = 0; i < kPrepAhead; ++i)
-      if (t0 + i < p.T) one_step(t0 + i, i);
+    for (int i = 0; i < kPrepBlock; ++i) {
+      const int t = k * kPrepBlock + i;
+      if (t < p.T) one_step(t, ring + ((k % NR) * kPrepBlock + i) * SLOT);
+    }
   }
 }
 

@@ -396,7 +396,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.ry = a->ry; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
     p.tiled = a->split ? 1 : 0;
-    const long long blocks = ((long long)a->B * H + 255) / 256;
+    const long long blocks = (long long)a->B * (H / 64);  // (head dims are multiples of 64 here)
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
     hipLaunchKernelGGL(bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
   } else {
