@@ -57,21 +57,27 @@ __device__ __forceinline__ void bwd_fetch_to_lds_u8(u32x4_t rsrc, uint32_t lds_a
                :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
 }
 
-// One workgroup per (batch row, 64 hidden units): wave 0 walks through time, waves 1 to 3 bring its inputs to LDS -
+// One workgroup per (batch row, 64 hidden units): wave 0 walks through time, waves 4 to 6 store what it leaves in LDS
+// (three coefficients each), waves 1 to 3 bring its inputs to LDS -
 // W.x, R.h and the reset flag, one wave each, one load a step - in blocks of kPrepBlock steps, two or three blocks ahead, with
 // loads that write LDS directly and waits written by hand.  With the inputs fetched by the walking wave itself, into
 // registers six steps ahead, the kernel took 0.95 ms at config 2 and 0.36 ms without its loads: a wave has at most
 // 63 memory operations in flight, the nine stores of a step among them, which is four steps' worth of loads against a
 // way to HBM and back of several microseconds, and there is about one such wave per compute unit.
 constexpr int kPrepBlock = 8;
+constexpr int bwd_prepare_lds_bytes(bool bf16) {  // the ring of inputs and two blocks of results
+  return (bf16 ? 4 : 3) * kPrepBlock * (4 * 64 * (bf16 ? 2 : 4) + 64 * 16 + 16) + 2 * kPrepBlock * 9 * 64 * 4;
+}
 template <bool BF16>
-__global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p) {
+__global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int WXB = 4 * 64 * ESZ;           // W.x of a step: [4 gates][64 units]
   constexpr int RYB = 64 * 16;                // R.h of a step: [64 units][4 gates] float32
   constexpr int SLOT = WXB + RYB + 16;        // ... and the row's reset flag
   constexpr int NR = BF16 ? 4 : 3;            // blocks in the ring (48 KiB either way): NR - 1 of them ahead
-  __shared__ __attribute__((aligned(16))) char ring[NR * kPrepBlock * SLOT];
+  extern __shared__ __attribute__((aligned(16))) char prep_lds[];
+  char *const ring = prep_lds;                                                    // [NR][kPrepBlock] slots of inputs
+  float *const outs = reinterpret_cast<float *>(prep_lds + NR * kPrepBlock * SLOT);  // [2][kPrepBlock][9][64]: results
   const int H = p.NH * p.dh;
   const int slices = H >> 6;
   const int b = blockIdx.x / slices, col0 = (blockIdx.x - b * slices) << 6;
@@ -80,6 +86,36 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
   const int wave = (int)uniform((uint32_t)(tid >> 6));
   const int nblocks = (p.T + kPrepBlock - 1) / kPrepBlock;
   const uint32_t ring_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)ring);
+  if (wave >= 4) {
+    // ---- a storer wave: three of the nine coefficients of every step, a block behind the walking wave (which leaves
+    //      them in LDS: with its own nine stores a step in its 63 operations in flight, the acknowledgements of those
+    //      stores set its pace, 0.66 ms at config 2)
+    const int col = col0 + lane, a = a0 + lane, j0 = 3 * (wave - 4);
+    auto store_block = [&](int k) {
+#pragma unroll
+      for (int i = 0; i < kPrepBlock; ++i) {
+        const int t = k * kPrepBlock + i;
+        if (t >= p.T) break;
+        float *dst = p.coef + ((long long)t * p.B + b) * 9 * H + col;
+        long long js = H;
+        if (p.tiled) {
+          const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (p.dh >> 6) + (a >> 6);
+          dst = p.coef + (piece * 16 + (b & 15)) * (9 * 64) + (a & 63);
+          js = 64;
+        }
+        const float *src = outs + (((k & 1) * kPrepBlock + i) * 9 + j0) * 64 + lane;
+#pragma unroll
+        for (int j = 0; j < 3; ++j) dst[(j0 + j) * js] = src[j * 64];
+      }
+    };
+    for (int k = 0; k < nblocks; ++k) {
+      __syncthreads();  // barrier k
+      if (k > 0) store_block(k - 1);
+    }
+    __syncthreads();    // the last block's results are in LDS
+    store_block(nblocks - 1);
+    return;
+  }
   if (wave > 0) {
     // ---- a loader wave.  Block k sits in ring part k % NR; it is asked for behind barrier k - NR + 1 (when the walking
     //      wave is through with block k - NR, which sat there) and has landed in front of barrier k.
@@ -121,6 +157,7 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
       request_block(k + NR - 1);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();    // (the storers' last barrier)
     return;
   }
   // ---- the walking wave: lane = unit of the slice
@@ -132,17 +169,28 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
   float c = 0.0f, n = 0.0f, m = 0.0f;
   if (p.s0) { c = p.s0[BH + idx]; n = p.s0[2 * BH + idx]; m = p.s0[3 * BH + idx]; }
   const bool has_mask = p.reset != nullptr;
-  auto one_step = [&](int t, const char *slot) {
+  // (a block's inputs are read from LDS in one go, in front of its eight steps: read per step, each read would be
+  // waited for with nothing else to do, and the compiler does not move them up past the writes of the results)
+  struct StepInputs { f32x4 ry; typename std::conditional<BF16, uint16_t, float>::type wx[4]; uint32_t flag; };
+  auto read_inputs = [&](const char *slot, StepInputs &in) {
+    in.ry = *reinterpret_cast<const f32x4 *>(slot + WXB + lane * 16);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      if constexpr (BF16) in.wx[g] = *reinterpret_cast<const uint16_t *>(slot + (g * 64 + lane) * 2);
+      else in.wx[g] = *reinterpret_cast<const float *>(slot + (g * 64 + lane) * 4);
+    }
+    in.flag = has_mask ? *reinterpret_cast<const uint32_t *>(slot + WXB + RYB) : 0u;
+  };
+  auto one_step = [&](const StepInputs &in, float *out) {
     float raw[4];
-    const f32x4 ry = *reinterpret_cast<const f32x4 *>(slot + WXB + lane * 16);
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       float w;
-      if constexpr (BF16) w = bf16_bits_to_float(*reinterpret_cast<const uint16_t *>(slot + (g * 64 + lane) * 2));
-      else w = *reinterpret_cast<const float *>(slot + (g * 64 + lane) * 4);
-      raw[g] = (w + ry[g]) + bias_g[g];
+      if constexpr (BF16) w = bf16_bits_to_float(in.wx[g]);
+      else w = in.wx[g];
+      raw[g] = (w + in.ry[g]) + bias_g[g];
     }
-    const bool restart = has_mask && (*reinterpret_cast<const uint32_t *>(slot + WXB + RYB) & 0xFFu) != 0u;
+    const bool restart = (in.flag & 0xFFu) != 0u;
     if (restart) { c = 0.0f; n = 0.0f; m = 0.0f; }
     // the forward's update (slstm_pointwise), with the gate values kept
     const float sigf_neg = __expf(-fabsf(raw[1]));
@@ -157,32 +205,29 @@ __global__ __launch_bounds__(256) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     const float nnew = fg * n + ig;
     const float rn = __builtin_amdgcn_rcpf(nnew);
     const float ynew = og * cnew * rn;
-    float *dst = p.coef + ((long long)t * p.B + b) * 9 * H + col;
-    long long js = H;
-    if (p.tiled) {
-      const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (p.dh >> 6) + (a >> 6);
-      dst = p.coef + (piece * 16 + (b & 15)) * (9 * 64) + (a & 63);
-      js = 64;
-    }
-    dst[0] = og * rn;
-    dst[1 * js] = ynew * rn;
-    dst[2 * js] = ig * tz;
-    dst[3 * js] = ig;
-    dst[4 * js] = fg * one_minus_fsig * c;
-    dst[5 * js] = fg * one_minus_fsig * n;
-    dst[6 * js] = ig * (1.0f - tz * tz);
-    dst[7 * js] = (1.0f - og) * ynew;
-    dst[8 * js] = fg;
+    out[0 * 64] = og * rn;
+    out[1 * 64] = ynew * rn;
+    out[2 * 64] = ig * tz;
+    out[3 * 64] = ig;
+    out[4 * 64] = fg * one_minus_fsig * c;
+    out[5 * 64] = fg * one_minus_fsig * n;
+    out[6 * 64] = ig * (1.0f - tz * tz);
+    out[7 * 64] = (1.0f - og) * ynew;
+    out[8 * 64] = fg;
     c = cnew; n = nnew; m = mnew;
   };
   for (int k = 0; k < nblocks; ++k) {
     __syncthreads();  // barrier k
+    StepInputs in[kPrepBlock];
+#pragma unroll
+    for (int i = 0; i < kPrepBlock; ++i) read_inputs(ring + ((k % NR) * kPrepBlock + i) * SLOT, in[i]);
 #pragma unroll
     for (int i = 0; i < kPrepBlock; ++i) {
       const int t = k * kPrepBlock + i;
-      if (t < p.T) one_step(t, ring + ((k % NR) * kPrepBlock + i) * SLOT);
+      if (t < p.T) one_step(in[i], outs + ((k & 1) * kPrepBlock + i) * 9 * 64 + lane);
     }
   }
+  __syncthreads();  // (the storers' last barrier)
 }
 
 struct BwdParams {

@@ -398,7 +398,11 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.tiled = a->split ? 1 : 0;
     const long long blocks = (long long)a->B * (H / 64);  // (head dims are multiples of 64 here)
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
-    hipLaunchKernelGGL(bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, p);
+    void (*kp)(BwdPrepParams) = bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>;
+    const int plds = bwd_prepare_lds_bytes(bf16);
+    if (hipFuncSetAttribute((const void *)kp, hipFuncAttributeMaxDynamicSharedMemorySize, plds) != hipSuccess)
+      return fail(XS_ERR_LAUNCH, "the prepare kernel cannot have %d bytes of LDS", plds);
+    hipLaunchKernelGGL(kp, dim3((unsigned)blocks), dim3(448), plds, stream, p);
   } else {
     if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
     if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");
