@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 9
+#define XS_ABI_VERSION 10
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -75,10 +75,10 @@ enum {
  *                             its workgroups running at once), so one of them
  *                             waits, within spin_limit, until the other is done.
  *   stream                    hipStream_t (NULL = the null stream).
- *   spin_limit                bound on every wait between compute units, in poll
- *                             iterations; 0 selects the default.  When a wait
- *                             runs out the kernel records it in the status block
- *                             and finishes without waiting any further.
+ *   spin_limit                bound on every wait between compute units (a step: between
+ *                             the waves of a workgroup), in poll iterations; 0 selects
+ *                             the default.  When a wait runs out the kernel records it
+ *                             in the status block and finishes without waiting any further.
  *   h_prev [B, NH*dh]         optional, xs_slstm_step with bf16 wx only (ignored
  *                             otherwise): the y plane of s0 rounded to bf16, i.e.
  *                             the h_out of the previous step.  The kernel rounds
@@ -110,7 +110,8 @@ typedef struct xs_slstm_args {
 /* Status block at the start of the workspace, written by the kernels. */
 typedef struct xs_slstm_status {
   uint32_t aborted;     /* 1 if a bounded wait ran out: the results are invalid, and every workgroup that finished after
-                           the give-up has overwritten its part of h_out and s_out with NaN */
+                           the give-up has overwritten its part of h_out and s_out with NaN (a step: the workgroup
+                           whose waves gave up on each other writes NaN for its tile) */
   uint32_t abort_wg;    /* workgroup that gave up first */
   uint32_t abort_step;  /* timestep it was waiting for */
   uint32_t max_spins;   /* largest number of poll iterations any wait needed */
@@ -119,7 +120,9 @@ typedef struct xs_slstm_status {
   uint32_t step_kernel; /* 1 if the call ran the single-token step kernel (xs_slstm_step, or xs_slstm_forward with T == 1) */
   uint32_t rows_per_workgroup; /* sequence kernels: batch rows a workgroup handles (4, 8, 16, 32 = two row tiles, 64 = four
                                   row tiles: the kernel with MFMA waves and gating waves), of the last launch; 0 after a step */
-  uint32_t reserved[8];
+  uint32_t pipelined_step; /* 1 if the step ran the pipelined step kernel (bf16, head dim 256, whole tiles, a state, no mask,
+                              h_prev given), 0 if the tile kernel; 0 after a sequence call */
+  uint32_t reserved[7];
 } xs_slstm_status;
 
 /* Library / ABI identification.  Replaces nothing (the reference keys its JIT
@@ -295,7 +298,19 @@ typedef struct xs_slstm_bwd_args {
   int32_t split;
   void *exchange;
   uint32_t *counters;
-  int64_t spin_limit;        /* 0 = default */
+  int64_t spin_limit;        /* bound of the waits between the compute units of a head, in looks; 0 = default; negative:
+                                every such wait gives up at its first look (forces the error path from the host: the
+                                kernel still runs to its end, counters[0] is set and d_s0 is NaN) */
+  /* backward, the two options of the reference's native backward pass (cell.py:84-87):
+   * recurrent_cut != 0       no gradient passes from a step to the y it started from: the product with R transposed is
+   *                          left out (sLSTMFunc.backward_cut, slstm.cc:223-304, slstm_backward_cut.cu:265-312); c and n
+   *                          still pass theirs on, and d_s0's y plane is zero.
+   * recurrent_clipval > 0    the gradient that reaches y_t from step t+1 is clipped to +-recurrent_clipval before d_h is
+   *                          added (slstm_pointwise.cu:136-143); the y plane of d_s_final counts as coming from outside
+   *                          (the reference receives it through the same argument as d_h) and is not clipped.
+   *                          0, negative or not finite: no clipping. */
+  int32_t recurrent_cut;
+  float recurrent_clipval;
 } xs_slstm_bwd_args;
 
 int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);

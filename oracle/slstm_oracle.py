@@ -44,7 +44,7 @@ def _lib():
             fn.argtypes = [ctypes.c_void_p] * 7 + [ctypes.c_int] * 5
         if hasattr(lib, "slstm_oracle_backward_f64"):  # (a library built before the backward oracle existed has none)
             lib.slstm_oracle_backward_f64.restype = ctypes.c_int
-            lib.slstm_oracle_backward_f64.argtypes = [ctypes.c_void_p] * 11 + [ctypes.c_int] * 5
+            lib.slstm_oracle_backward_f64.argtypes = [ctypes.c_void_p] * 11 + [ctypes.c_int] * 6 + [ctypes.c_double]
         _LIB = lib
     return _LIB
 
@@ -112,10 +112,13 @@ def slstm_forward_per_document(wx, r_ext, b_ext, reset, dtype=np.float64):
     return h, s
 
 
-def slstm_backward(wx, r_ext, b_ext, s0, reset, d_h, d_s_final=None, n0_rule=N0_PER_ELEMENT):
+def slstm_backward(wx, r_ext, b_ext, s0, reset, d_h, d_s_final=None, n0_rule=N0_PER_ELEMENT, recurrent_cut=False,
+                   recurrent_clipval=None):
     """Gradients of a loss with d loss / d h_out = ``d_h`` [T,B,H] (and d loss / d final state = ``d_s_final`` [4,B,H])
     with respect to W.x [B,T,4H], R_ext [NH,dh,4,dh], b_ext [NH,4,dh] and the initial state [4,B,H], in float64, by
-    the rule of the reference's native kernel: the stabiliser m is a constant (slstm_pointwise.cu:118-196)."""
+    the rule of the reference's native kernel: the stabiliser m is a constant (slstm_pointwise.cu:118-196).
+    ``recurrent_cut`` leaves out the gradient from a step to the y it started from (slstm_backward_cut.cu:265-312),
+    ``recurrent_clipval`` clips that gradient to +-clipval before d_h is added (slstm_pointwise.cu:136-143)."""
     lib = _lib()
     B, T = wx.shape[0], wx.shape[1]
     NH, dh = r_ext.shape[0], r_ext.shape[1]
@@ -127,7 +130,8 @@ def slstm_backward(wx, r_ext, b_ext, s0, reset, d_h, d_s_final=None, n0_rule=N0_
     d_wx = np.zeros((B, T, 4 * H)); d_r = np.zeros((NH, dh, 4, dh)); d_b = np.zeros((NH, 4, dh)); d_s0 = np.zeros((4, B, H))
     ptr = lambda a: None if a is None else a.ctypes.data_as(ctypes.c_void_p)
     rc = lib.slstm_oracle_backward_f64(ptr(wx_), ptr(r_), ptr(b_), ptr(s0_), ptr(rs_), ptr(dh_), ptr(dsf_), ptr(d_wx),
-                                       ptr(d_r), ptr(d_b), ptr(d_s0), B, T, NH, dh, n0_rule)
+                                       ptr(d_r), ptr(d_b), ptr(d_s0), B, T, NH, dh, n0_rule, int(bool(recurrent_cut)),
+                                       float(recurrent_clipval) if recurrent_clipval is not None else 0.0)
     if rc != 0:
         raise MemoryError("slstm_oracle_backward_f64 failed")
     return d_wx, d_r, d_b, d_s0

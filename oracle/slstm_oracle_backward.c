@@ -16,11 +16,24 @@
  * or m it is not the derivative of the forward as written; the vanilla path's autograd differs there, and so does
  * this restatement (tests/golden/bwd_state_loss.npz documents the difference).
  *
+ * Two options of the reference's native backward are restated as well:
+ *   recurrent_cut      no gradient passes from a step to the y it started from: the contraction with R transposed is
+ *                      left out (xlstm/blocks/slstm/src/cuda/slstm_backward_cut.cu:265-312 against
+ *                      slstm_backward.cu:314-319; chosen by cell.py:580-583).  c and n still pass their gradients on.
+ *   recurrent_clipval  the gradient that reaches y_t through the recurrence is clipped to +-clipval before the
+ *                      gradient from outside is added (slstm_pointwise.cu:136-143).  What comes from outside (d_h, and
+ *                      at the last step the y part of d_s_final, which the reference receives through the same
+ *                      argument, slstm_backward.cu:367-370; ds starts as zeros, slstm.cc:178-179) is not clipped.  <= 0 or not finite: no clipping.
+ *
  * Pinning status:
  *   slstm_oracle_backward_f64: pinned by (a) central finite differences of slstm_oracle_forward_f64 for losses that
  *     are linear forms of the outputs, in every input (W.x, R, bias, initial y/c/n), (b) the gradients that the
  *     reference's vanilla cell returns through autograd for such losses (tests/golden/bwd_*.npz), (c) rows that a
- *     reset mask cuts: the gradient of a packed row equals the gradients of its documents run alone.
+ *     reset mask cuts: the gradient of a packed row equals the gradients of its documents run alone, (d) the
+ *     d_s_final argument (y, c, n) by the chain rule: the gradients of a sequence equal those of its two halves when
+ *     the second half's d_s0 is the first half's d_s_final, (e) recurrent_cut by the gradient of the same outputs
+ *     computed with R = 0 from inputs that already contain R y_{t-1} (the pinned path), (f) recurrent_clipval by a
+ *     step-by-step restatement in numpy around one-step calls (tests/test_oracle_backward.py).
  *
  * Layouts as in slstm_oracle.c; d_h [T, B, NH*dh] is the gradient of the loss with respect to h_out, d_s_final
  * [4, B, NH*dh] (may be NULL) with respect to the final state; outputs d_wx [B, T, 4, NH, dh], d_r_ext [NH, dh, 4, dh],
@@ -40,7 +53,8 @@ static double bw_sigmoid(double x) {
 
 int slstm_oracle_backward_f64(const double *wx, const double *r_ext, const double *b_ext, const double *s0,
                               const uint8_t *reset, const double *d_h, const double *d_s_final, double *d_wx,
-                              double *d_r_ext, double *d_b_ext, double *d_s0, int B, int T, int NH, int dh, int n0_rule) {
+                              double *d_r_ext, double *d_b_ext, double *d_s0, int B, int T, int NH, int dh, int n0_rule,
+                              int recurrent_cut, double recurrent_clipval) {
   const size_t H = (size_t)NH * dh, BH = (size_t)B * H;
   /* ---- forward, keeping what the backward needs: the state BEFORE every step (after the reset) and after it, and
    *      the gate values the native kernel caches (exp(i - m'), raw f, tanh z, sigmoid o) */
@@ -64,6 +78,7 @@ int slstm_oracle_backward_f64(const double *wx, const double *r_ext, const doubl
       for (size_t k = 0; k < BH; ++k)
         if (n[k] != 0) { all_n_zero = 0; break; }
     double *after = sa + (size_t)t * 4 * BH, *g = gc + (size_t)t * 4 * BH;
+#pragma omp parallel for collapse(2) schedule(static)
     for (int b = 0; b < B; ++b)
       for (int h = 0; h < NH; ++h)
         for (int a = 0; a < dh; ++a) {
@@ -93,11 +108,17 @@ int slstm_oracle_backward_f64(const double *wx, const double *r_ext, const doubl
   memset(d_r_ext, 0, (size_t)NH * dh * 4 * dh * sizeof(double));
   memset(d_b_ext, 0, (size_t)NH * 4 * dh * sizeof(double));
   if (d_s_final) memcpy(dcur, d_s_final, 4 * BH * sizeof(double));
+  const int clip = isfinite(recurrent_clipval) && recurrent_clipval > 0;
   for (int t = T - 1; t >= 0; --t) {
     const double *before = sb + (size_t)t * 4 * BH, *after = sa + (size_t)t * 4 * BH, *g = gc + (size_t)t * 4 * BH;
     for (size_t idx = 0; idx < BH; ++idx) {
       /* slstm_pointwise.cu:139-190 */
-      const double dy_total = d_h[(size_t)t * BH + idx] + dcur[idx];
+      double dy_recurrent = dcur[idx];
+      if (clip && t < T - 1) { /* (at the last step dcur holds what came from outside: the y part of d_s_final) */
+        if (dy_recurrent > recurrent_clipval) dy_recurrent = recurrent_clipval;
+        if (dy_recurrent < -recurrent_clipval) dy_recurrent = -recurrent_clipval;
+      }
+      const double dy_total = d_h[(size_t)t * BH + idx] + dy_recurrent;
       double dc_total = dcur[BH + idx], dn_total = dcur[2 * BH + idx];
       const double ig = g[idx], fraw = g[BH + idx], zv = g[2 * BH + idx], og = g[3 * BH + idx];
       const double c_old = before[BH + idx], n_old = before[2 * BH + idx], m_old = before[3 * BH + idx];
@@ -115,8 +136,10 @@ int slstm_oracle_backward_f64(const double *wx, const double *r_ext, const doubl
       dcur[idx] = 0; dcur[BH + idx] = fg * dc_total; dcur[2 * BH + idx] = fg * dn_total; dcur[3 * BH + idx] = 0;
     }
     /* gradient of W.x and the bias; of R and of the y the step started from (slstm_backward.cu:314-319, 381-386) */
-    for (int b = 0; b < B; ++b)
-      for (int h = 0; h < NH; ++h)
+    /* (heads do not meet: one thread per head keeps every sum in the order of the plain loops) */
+#pragma omp parallel for schedule(static)
+    for (int h = 0; h < NH; ++h)
+      for (int b = 0; b < B; ++b)
         for (int q = 0; q < 4; ++q)
           for (int a = 0; a < dh; ++a) {
             const size_t k = (size_t)h * dh + a;
@@ -126,7 +149,7 @@ int slstm_oracle_backward_f64(const double *wx, const double *r_ext, const doubl
             for (int d = 0; d < dh; ++d) {
               const size_t yi = (size_t)b * H + (size_t)h * dh + d;
               d_r_ext[(((size_t)h * dh + d) * 4 + q) * dh + a] += before[yi] * dv;
-              dcur[yi] += dv * r_ext[(((size_t)h * dh + d) * 4 + q) * dh + a];
+              if (!recurrent_cut) dcur[yi] += dv * r_ext[(((size_t)h * dh + d) * 4 + q) * dh + a];
             }
           }
     /* a row that starts a document at t took nothing from the step before */

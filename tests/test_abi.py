@@ -32,7 +32,8 @@ def test_abi_version_and_struct_mirror():
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
-    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8  # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more
+    # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more, int32 + float
+    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8 + 8
 
 
 def test_backward_argument_errors_without_touching_the_gpu():
@@ -45,6 +46,31 @@ def test_backward_argument_errors_without_touching_the_gpu():
     assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -1  # coef missing
     a.dtype = 5
     assert lib.xs_slstm_backward(ctypes.byref(a)) == -3
+
+
+def test_backward_alignment_errors_without_touching_the_gpu():
+    """What the backward kernels fetch in pieces of 16 bytes (W.x, R.h, the coefficients, d_h) or write in pairs of
+    floats (d_wx) must be aligned for it: XS_ERR_ALIGN before anything is launched (fake addresses, never used)."""
+    lib = _lib.load()
+    a = _lib.SlstmBwdArgs()
+    a.B, a.T, a.NH, a.dh, a.dtype = 2, 3, 2, 64, _lib.XS_BF16
+    H = 128
+    a.coef, a.wx, a.ry, a.bias = 0x100000, 0x200000, 0x300000, 0x400000
+    a.wx_stride_b, a.wx_stride_t = 3 * 4 * H, 4 * H
+    for field, bad in (("wx", 0x200002), ("wx_stride_t", 4 * H + 1), ("wx_stride_b", 3 * 4 * H + 4), ("ry", 0x300008),
+                       ("coef", 0x100004)):
+        keep = getattr(a, field)
+        setattr(a, field, bad)
+        assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -4, field
+        assert b"aligned" in lib.xs_last_error()
+        setattr(a, field, keep)
+    a.d_h, a.r_t, a.d_wx, a.d_s0 = 0x500000, 0x600000, 0x700000, 0x800000
+    a.d_wx_stride_b, a.d_wx_stride_t = 3 * 4 * H, 4 * H
+    for field, bad in (("d_h", 0x500002), ("r_t", 0x600008), ("d_wx", 0x700004), ("d_wx_stride_t", 4 * H + 1), ("coef", 0x100008)):
+        keep = getattr(a, field)
+        setattr(a, field, bad)
+        assert lib.xs_slstm_backward(ctypes.byref(a)) == -4, field
+        setattr(a, field, keep)
 
 
 def test_argument_errors_without_touching_the_gpu():

@@ -170,8 +170,13 @@ def test_cell_autograd_matches_the_oracle(dtype, tol):
 
 
 def test_a_wait_between_compute_units_that_runs_out_is_reported():
-    """Host-forced: with a spin limit of one poll the workgroups of a head give up on each other at once (every kernel
-    still exits normally).  The call must raise, or - when all peers happened to be there - return the usual result."""
+    """Host-forced: a negative spin limit makes every wait between the workgroups of a head give up at its first look
+    (every kernel still exits normally).  The call must raise, the gradient of the initial state must be NaN, and the
+    next call must be the usual one.  (A bound of one look does not do it: the peers' deltas are always there by the
+    second look, as five calls in a row showed.)"""
+    import ctypes
+
+    from xlstm_amd import _lib
     from xlstm_amd import functional as F
 
     B, T, NH, dh = 16, 12, 4, 256
@@ -182,9 +187,165 @@ def test_a_wait_between_compute_units_that_runs_out_is_reported():
     d_h = torch.randn(T, B, NH * dh, generator=torch.Generator().manual_seed(7)).to(dev).bfloat16()
     h, _ = F.slstm_forward(wx_t, r_t, b_t)
     good = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True)
-    try:
-        got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=1)
-    except F.EngineError as e:
-        assert "ran out" in str(e)
-    else:
-        assert torch.equal(got[0], good[0])
+    with pytest.raises(F.EngineError, match="ran out"):
+        F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=-1)
+    # the same call with the synchronisation left to the caller (timings asked for): nothing raises, d_s0 is NaN
+    t = {}
+    got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=-1, timings=t)
+    torch.cuda.synchronize()
+    assert bool(torch.isnan(got[3][:3]).all())
+    again = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True)  # the next call is unaffected
+    assert torch.equal(again[0], good[0]) and torch.equal(again[3], good[3])
+
+
+def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=None, **opts):
+    """The engine's backward and the oracle's on one seeded problem; returns the four relative errors."""
+    from xlstm_amd import functional as F
+
+    H = NH * dh
+    wx, r, b, s0 = make_problem(seed, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=with_state)
+    reset = geometric_reset_mask(seed + 1, B, T, mean_len or max(2, T // 2)) if masked else None
+    if reset is not None and with_state:
+        reset[0, 0] = 0
+    d_h = np.random.default_rng(seed + 2).standard_normal((T, B, H)).astype(np.float32)
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev)
+    if bf16:
+        wx_t = wx_t.bfloat16()
+        d_h = torch.from_numpy(d_h).bfloat16().float().numpy()
+        r = torch.from_numpy(r).bfloat16().float().numpy()
+    r_t, b_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    s0_t = torch.from_numpy(s0).to(dev) if s0 is not None else None
+    m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
+    dsf_t = torch.from_numpy(d_sf).to(dev) if d_sf is not None else None
+    h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
+    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override")}
+    d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), dsf_t, **kw)
+    torch.cuda.synchronize()
+    okw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval")}
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf, **okw)
+    errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
+                d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
+    return errs, (d_wx, d_r, d_b, d_s0), (o_wx, o_r, o_b, o_s0)
+
+
+def test_backward_over_2048_steps_bf16_packed_documents():
+    """The length of BASELINE config 2 (T = 2048, 4 heads of 256, bf16, packed geometric documents) on a few batch
+    rows (rows are independent; the oracle affords three of them): what 2048 reverse steps on bf16 operands do to the
+    error, against the float64 oracle.  Tolerance 2e-2."""
+    print("case backward T=2048 bf16 B=3", flush=True)
+    errs, _, _ = _run_both(True, 3, 2048, 4, 256, 301, masked=True, with_state=False, mean_len=512)
+    print("backward, T = 2048, bf16:", errs, flush=True)
+    assert all(np.isfinite(v) and v <= 2e-2 for v in errs.values()), errs
+
+
+def test_backward_config1_shape_fp32_full_size():
+    """BASELINE config 1 at full size (B 4, T 256, 4 heads of 128, float32, zero state): 1e-5 against the oracle."""
+    print("case backward config 1 fp32", flush=True)
+    errs, _, _ = _run_both(False, 4, 256, 4, 128, 302, masked=False, with_state=False)
+    print("backward, config 1:", errs, flush=True)
+    assert all(np.isfinite(v) and v <= 1e-5 for v in errs.values()), errs
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 11, 2, 64, True), (False, 20, 9, 2, 128, True), (True, 16, 12, 4, 256, True),
+                                                  (False, 4, 10, 2, 128, False), (True, 9, 8, 2, 512, True)])
+def test_the_gradient_of_the_final_state_by_the_chain_rule(bf16, B, T, NH, dh, split):
+    """``d_s_final`` on the GPU, pinned the way the oracle's is: the gradients of a sequence are those of its second
+    part, started from the state after step k - 1, and of its first part with the second part's ``d_s0`` as the
+    gradient of its final state.  d_wx and d_s0 of the two calls reproduce the whole call's (float32: to rounding;
+    bf16: the hand-over itself is exact, the deltas then differ by the rounding of the operands), and the y, c and n
+    planes all carry something."""
+    from xlstm_amd import functional as F
+
+    k = T // 2
+    H = NH * dh
+    wx, r, b, s0 = make_problem(310, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=True)
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev)
+    if bf16:
+        wx_t = wx_t.bfloat16()
+    r_t, b_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    s0_t = torch.from_numpy(s0).to(dev)
+    d_h = torch.randn(T, B, H, generator=torch.Generator().manual_seed(311)).to(dev).to(wx_t.dtype)
+    h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t)
+    whole = F.slstm_backward(wx_t, r_t, b_t, s0_t, None, h, d_h, split_override=split)
+    h_a, s_k = F.slstm_forward(wx_t[:, :k], r_t, b_t, s0_t)
+    h_b, _ = F.slstm_forward(wx_t[:, k:], r_t, b_t, s_k)
+    assert torch.equal(torch.cat([h_a, h_b]), h)
+    tail = F.slstm_backward(wx_t[:, k:], r_t, b_t, s_k, None, h_b, d_h[k:].contiguous(), split_override=split)
+    assert all(float(tail[3][i].abs().max()) > 0 for i in range(3)) and not bool(tail[3][3].any())
+    head = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), tail[3], split_override=split)
+    torch.cuda.synchronize()
+    tol = 2e-2 if bf16 else 1e-5
+
+    def rel(a, g):
+        return float((a - g).abs().max() / max(1.0, float(g.abs().max())))
+
+    errs = dict(d_wx=rel(torch.cat([head[0], tail[0]], 1), whole[0]), d_r=rel(head[1] + tail[1], whole[1]),
+                d_b=rel(head[2] + tail[2], whole[2]), d_s0=rel(head[3], whole[3]))
+    print("chain rule", bf16, B, T, NH, dh, split, errs, flush=True)
+    assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
+    # not vacuous: without the hand-over the first part's gradients are not the whole call's
+    plain = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), split_override=split)
+    assert rel(plain[0], whole[0][:, :k]) > 10 * tol
+    # and against the oracle, d_s_final given
+    d_sf = tail[3].cpu().numpy()
+    o = so.slstm_backward(wx[:, :k], torch.from_numpy(r).to(wx_t.dtype).float().numpy(), b, s0, None,
+                          d_h[:k].float().cpu().numpy(), d_sf)
+    assert _rel(head[0].cpu().numpy(), o[0]) <= tol and _rel(head[3].cpu().numpy(), o[3]) <= tol
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (False, 20, 7, 2, 128, True), (True, 16, 10, 4, 256, True),
+                                                  (False, 4, 12, 4, 256, False), (True, 9, 7, 2, 512, True), (True, 6, 9, 2, 128, False),
+                                                  (False, 7, 6, 2, 256, True)])
+@pytest.mark.parametrize("opts", [dict(recurrent_cut=True), dict(recurrent_clipval=0.05), dict(recurrent_clipval=1.0),
+                                  dict(recurrent_cut=True, recurrent_clipval=0.05)],
+                         ids=["cut", "clip0.05", "clip1", "cut+clip"])
+def test_recurrent_cut_and_clipval_against_the_oracle(bf16, B, T, NH, dh, split, opts):
+    """``gradient_recurrent_cut`` / ``gradient_recurrent_clipval`` of the reference's native backward pass
+    (slstm_backward_cut.cu:265-312, slstm_pointwise.cu:136-143) in both reverse kernels, with a mask, a state and a
+    gradient of the final state, against the oracle's flags (pinned in tests/test_oracle_backward.py)."""
+    H = NH * dh
+    d_sf = np.random.default_rng(320).standard_normal((4, B, H)).astype(np.float32)
+    d_sf[3] = 0.0
+    print("case cut/clip", bf16, B, T, NH, dh, split, opts, flush=True)
+    errs, got, want = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, split_override=split, **opts)
+    print(errs, flush=True)
+    tol = 2e-2 if bf16 else 1e-5
+    assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
+    if opts.get("recurrent_cut"):
+        assert not bool(got[3][0].any())  # nothing reaches the y of the initial state
+    # the option bites: the plain gradient of the same problem is something else
+    if opts.get("recurrent_cut") or opts.get("recurrent_clipval", 1.0) < 1.0:
+        _, got_plain, _ = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, split_override=split)
+        assert float((got_plain[0] - got[0]).abs().max()) > 1e-3
+
+
+def test_cell_config_gradient_recurrent_cut_and_clipval():
+    """The cell hands ``gradient_recurrent_cut`` / ``gradient_recurrent_clipval`` of its config to the backward pass
+    (cell.py:84-87, 580-583 of the reference); a clip value below 1 would also clip the reference's forward
+    (cell.py:200-210) and is refused at construction."""
+    from tests.test_hip_cell import _cell_from
+    from xlstm_amd.cell import sLSTMCell, sLSTMCellConfig
+
+    B, T, NH, dh = 3, 8, 2, 64
+    H = NH * dh
+    wx, r, b, s0 = make_problem(330, B, T, NH, dh, rscale=2.0, with_state=True)
+    w = np.random.default_rng(331).standard_normal((T, B, H)).astype(np.float32) * 4.0
+    for kw in (dict(gradient_recurrent_cut=True), dict(gradient_recurrent_clipval=1.0)):
+        cell = _cell_from(r, b, dtype="float32", **kw).train()
+        x = torch.from_numpy(wx).cuda().requires_grad_(True)
+        st = torch.from_numpy(s0).cuda().requires_grad_(True)
+        out, _ = cell(x, st)                               # [B, NH, T, dh]
+        (out * torch.from_numpy(w).cuda().view(T, B, NH, dh).permute(1, 2, 0, 3)).sum().backward()
+        o = so.slstm_backward(wx, r, b, s0, None, w, None, recurrent_cut=kw.get("gradient_recurrent_cut", False),
+                              recurrent_clipval=kw.get("gradient_recurrent_clipval"))
+        plain = so.slstm_backward(wx, r, b, s0, None, w, None)
+        assert np.abs(plain[0] - o[0]).max() > 1e-3, "the option does not bite in this problem"
+        d_r_ext = cell._recurrent_kernel_int2ext(cell._recurrent_kernel_.grad).cpu().numpy()
+        errs = dict(d_wx=_rel(x.grad.cpu().numpy(), o[0]), d_r=_rel(d_r_ext, o[1]),
+                    d_s0=_rel(st.grad.cpu().numpy()[:3], o[3][:3]))
+        print(kw, errs, flush=True)
+        assert all(v <= 1e-5 for v in errs.values()), errs
+    with pytest.raises(NotImplementedError, match="gradient_recurrent_clipval"):
+        sLSTMCell(sLSTMCellConfig(hidden_size=H, num_heads=NH, backend="hip", gradient_recurrent_clipval=0.5))

@@ -71,7 +71,9 @@ def test_config2_and_config4_cell_packed_documents_full_size(B, mean_len, name):
 
 def test_config3_decode_full_width():
     """B=256, D=2048 (8 x 256), bf16: 128-token prefill, then 1024 consecutive T=1 steps carrying the state,
-    as BASELINE states it."""
+    as BASELINE states it, driven the way the benchmark's decode leg drives them: a ``StepPlan`` whose every step
+    gets the h of the step before as its bf16 operand.  That is the pipelined step kernel, and the status block must
+    say so; the first 64 steps are run a second time without the operand hint (the tile kernel)."""
     B, NH, dh, PRE, STEPS = 256, 8, 256, 128, 1024
     H = NH * dh
     print("config 3: building inputs on the device", flush=True)
@@ -87,24 +89,75 @@ def test_config3_decode_full_width():
     from xlstm_amd import functional as F
 
     ws = F.workspace_for(B, 1, NH, dh, wx_t.device)
+    plan = F.StepPlan(B, r_t, b_t, wx_dtype=torch.bfloat16, workspace=ws)
     h_dec = torch.empty(STEPS, B, H, dtype=torch.bfloat16, device=DEV)
     s_a, s_b = s.clone(), torch.empty_like(s)
+    wx_steps = wx_t[:, PRE:].transpose(0, 1).contiguous()  # [STEPS, B, 4H]: a step's W.x as the layer hands it over
     for t in range(STEPS):
-        F.slstm_forward(wx_t[:, PRE + t:PRE + t + 1], r_step, b_t, s_a, None, step=True, workspace=ws,
-                        h_out=h_dec[t:t + 1], s_out=s_b)
+        plan(wx_steps[t], s_a, s_b, h_dec[t], h_prev=h_dec[t - 1] if t else h_pre[PRE - 1])
         s_a, s_b = s_b, s_a
     torch.cuda.synchronize()
-    assert F.read_status(ws)["step_kernel"] == 1
+    st = F.read_status(ws)
+    print("config 3: status after the last step", st, flush=True)
+    assert st["step_kernel"] == 1 and st["pipelined_step"] == 1 and st["aborted"] == 0
     # property at full size: decoding step by step == one sequence call, bit for bit
     print("config 3: one sequence call over all 1152 tokens", flush=True)
     h_all, s_all = _hip(wx_t, r_t, b_t)
     assert torch.equal(h_all[:PRE], h_pre) and torch.equal(h_all[PRE:], h_dec) and torch.equal(s_all, s_a)
+    # the same steps without the operand hint: the tile kernel, the same bits
+    s_a, s_b = s.clone(), torch.empty_like(s)
+    h_tile = torch.empty(64, B, H, dtype=torch.bfloat16, device=DEV)
+    for t in range(64):
+        F.slstm_forward(wx_t[:, PRE + t:PRE + t + 1], r_step, b_t, s_a, None, step=True, workspace=ws,
+                        h_out=h_tile[t:t + 1], s_out=s_b)
+        s_a, s_b = s_b, s_a
+    torch.cuda.synchronize()
+    st = F.read_status(ws)
+    assert st["step_kernel"] == 1 and st["pipelined_step"] == 0
+    assert torch.equal(h_tile, h_dec[:64])
     # oracle on a few rows (rows are independent)
     rows = [0, 17, 255]
     h_ref, s_ref = so.slstm_forward(wx_t[rows].float().cpu().numpy(), r, b)
     assert max_err(h_all[:, rows].float().cpu().numpy(), h_ref) <= 2e-2
     assert max_err(s_all[:, rows].cpu().numpy(), s_ref) <= 2e-2
     assert tuple(h_all.shape) == (PRE + STEPS, B, H)
+
+
+def test_pipelined_step_whose_waves_give_up_on_each_other_says_so():
+    """Host-forced: with a spin limit of one look the waves of a workgroup of the pipelined step kernel give up on
+    each other at once (every wave still runs to its end).  Either some workgroup gave up - then the status block says
+    so and that workgroup's tile of the outputs is NaN - or every wait happened to be satisfied at the first look and
+    the step is the usual one.  The test prints which of the two it saw."""
+    from xlstm_amd import _lib
+    from xlstm_amd import functional as F
+    import ctypes
+
+    B, NH, dh = 256, 8, 256
+    H = NH * dh
+    g = torch.Generator(device=DEV).manual_seed(104)
+    wx = torch.randn(B, 1, 4 * H, generator=g, device=DEV).bfloat16()
+    _, r, b, _ = make_problem(104, 1, 1, NH, dh)
+    r_t, b_t = _params(r, b)
+    s0 = torch.randn(4, B, H, generator=g, device=DEV)
+    s0[2] = s0[2].abs() + 1.0
+    s0[0] = s0[0].bfloat16().float()
+    h_prev = s0[0].bfloat16()
+    ws = F.workspace_for(B, 1, NH, dh, wx.device)
+    good_h, good_s = F.slstm_forward(wx, r_t.bfloat16(), b_t, s0, None, step=True, workspace=ws, h_prev=h_prev)
+    torch.cuda.synchronize()
+    assert F.read_status(ws)["pipelined_step"] == 1
+    h, s = F.slstm_forward(wx, r_t.bfloat16(), b_t, s0, None, step=True, workspace=ws, h_prev=h_prev, spin_limit=1)
+    torch.cuda.synchronize()
+    st = F.read_status(ws)
+    if st["aborted"]:
+        print("pipelined step, spin limit 1: gave up (workgroup %d); NaN tiles" % st["abort_wg"], flush=True)
+        assert not bool(torch.isfinite(h.float()).all()) and not bool(torch.isfinite(s).all())
+        # a tile is all NaN or untouched by the give-up: what is finite is the usual result
+        ok = torch.isfinite(h.float())
+        assert torch.equal(h[ok], good_h[ok])
+    else:
+        print("pipelined step, spin limit 1: every wait was satisfied at the first look", flush=True)
+        assert torch.equal(h, good_h) and torch.equal(s, good_s)
 
 
 def test_config5_large_heads_full_size():

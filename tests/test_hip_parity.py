@@ -188,17 +188,33 @@ def test_spin_limit_runs_out_is_reported_not_hung():
     between compute units.  The kernel must finish, flag the call and poison its outputs."""
     wx, r, b, _ = make_problem(16, 16, 64, 4, 256, bf16=True)
     h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
-    h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
-    assert status["aborted"] in (0, 1)
-    if status["aborted"]:
-        assert status["abort_step"] >= 1
-    _assert_flagged_or_right(h, s, status, h_ref, s_ref)
+    # (256 workgroups that look for their 15 peers exactly once: some peer is always a moment late.  Should every look
+    # ever succeed the call is simply right, so the call is made up to five times until the give-up path has run.)
+    seen = []
+    for _ in range(5):
+        h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
+        assert status["aborted"] in (0, 1)
+        seen.append(status["aborted"])
+        if status["aborted"]:
+            assert status["abort_step"] >= 1
+        _assert_flagged_or_right(h, s, status, h_ref, s_ref)
+        if status["aborted"]:
+            break
+    print("one row tile, spin limit 1: aborted flags of the calls made:", seen, flush=True)
+    assert seen[-1] == 1, "the give-up path never ran"
     # four row tiles per workgroup: the drainer wave's wait for the compute waves is bounded the same way
     wx, r, b, _ = make_problem(17, 64, 6, 4, 1024, bf16=True)
     h_ref, s_ref = so.slstm_forward(wx, r, b, None, None)
-    h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
-    assert status["aborted"] in (0, 1)
-    _assert_flagged_or_right(h, s, status, h_ref, s_ref)
+    seen = []
+    for _ in range(5):
+        h, s, status = _run_hip(wx, r, b, bf16=True, spin_limit=1)
+        assert status["aborted"] in (0, 1)
+        seen.append(status["aborted"])
+        _assert_flagged_or_right(h, s, status, h_ref, s_ref)
+        if status["aborted"]:
+            break
+    print("four row tiles, spin limit 1: aborted flags of the calls made:", seen, flush=True)
+    assert seen[-1] == 1, "the give-up path never ran"
     # and the next call on the same device is unaffected
     h2, s2, status2 = _run_hip(wx, r, b, bf16=True)
     assert status2["aborted"] == 0
@@ -227,11 +243,11 @@ def test_cell_raises_for_an_aborted_call_at_the_next_host_contact():
                                workspace=ws, spin_limit=1)
         cell._watch(ws)
         torch.cuda.synchronize()
-        if F.read_status(ws)["aborted"]:
-            assert not bool(torch.isfinite(s).all())
-            with pytest.raises(F.EngineError, match="gave up waiting"):
-                cell.check_status()
-        else:
+        gave_up = bool(F.read_status(ws)["aborted"])
+        print("cell watch, spin limit 1: the call gave up:", gave_up, flush=True)
+        assert gave_up, "256 workgroups looking for their peers exactly once all found them"
+        assert not bool(torch.isfinite(s).all())
+        with pytest.raises(F.EngineError, match="gave up waiting"):
             cell.check_status()
         out2, st2 = cell(x)  # the cell keeps working
         cell.check_status()

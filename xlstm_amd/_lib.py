@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 
 XS_F32, XS_BF16 = 0, 1
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 EXPORTS = (
     "xs_abi_version",
@@ -79,6 +79,8 @@ class SlstmBwdArgs(ctypes.Structure):
         ("exchange", ctypes.c_void_p),
         ("counters", ctypes.c_void_p),
         ("spin_limit", ctypes.c_int64),
+        ("recurrent_cut", ctypes.c_int32),
+        ("recurrent_clipval", ctypes.c_float),
     ]
 
 
@@ -141,7 +143,8 @@ class SlstmStatus(ctypes.Structure):
         ("aborted", ctypes.c_uint32), ("abort_wg", ctypes.c_uint32), ("abort_step", ctypes.c_uint32),
         ("max_spins", ctypes.c_uint32), ("xcd_mixed", ctypes.c_uint32), ("launches", ctypes.c_uint32),
         ("step_kernel", ctypes.c_uint32), ("rows_per_workgroup", ctypes.c_uint32),
-        ("reserved", ctypes.c_uint32 * 8),
+        ("pipelined_step", ctypes.c_uint32),
+        ("reserved", ctypes.c_uint32 * 7),
     ]
 
 

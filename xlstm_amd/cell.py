@@ -17,7 +17,9 @@ What differs, on purpose:
   * the stabiliser uses the native kernel's per-element ``n == 0`` rule
     (slstm_pointwise.cu:79), which equals the vanilla rule for every state the
     cell itself can produce;
-  * forward only: the hip backend is an inference engine, ``backward`` raises;
+  * training: the forward stores nothing for it; ``loss.backward()`` recomputes what it needs and runs the engine's
+    backward kernels (``functional.slstm_backward``), with the reference's ``gradient_recurrent_cut`` and
+    ``gradient_recurrent_clipval``.  Head dims beyond the backward kernels' range raise in ``backward``;
   * a call with S == 1 -- what the reference's ``sLSTMLayer.step`` makes for every decoded
     token (layer.py:113-115) -- runs the single-token step kernel, bit-identical to the same
     step inside a longer call.
@@ -90,8 +92,8 @@ class ParameterProxy:
 @dataclass
 class sLSTMCellConfig:
     """Field-for-field the reference's config (cell.py:61-163); the fields that
-    only parameterise its CUDA build (batch_size, constants, gradient clipping)
-    are accepted and ignored by the hip backend."""
+    only parameterise its CUDA build (batch_size, constants, the dtype_* of its
+    intermediate buffers) are accepted and ignored by the hip backend."""
 
     hidden_size: int = -1
     num_heads: int = 4
@@ -194,9 +196,9 @@ class _CellFunction(torch.autograd.Function):
     what the forward call returned for ``x, r, bias, state, mask``; nothing else is stored for the backward."""
 
     @staticmethod
-    def forward(ctx, x, r, bias, state, h, s, mask, num_heads):
+    def forward(ctx, x, r, bias, state, h, s, mask, num_heads, cut, clipval):
         ctx.save_for_backward(x, r, bias, h, *(() if state is None else (state,)))
-        ctx.mask, ctx.num_heads = mask, num_heads
+        ctx.mask, ctx.num_heads, ctx.cut, ctx.clipval = mask, num_heads, cut, clipval
         return h.view_as(h), s.view_as(s)
 
     @staticmethod
@@ -206,9 +208,9 @@ class _CellFunction(torch.autograd.Function):
         NH, dh = ctx.num_heads, r.shape[2]
         d_wx, d_r, d_bias, d_s0 = F_hip.slstm_backward(
             x.detach(), r.detach(), bias.detach().view(NH, 4, dh), None if state is None else state.detach(), ctx.mask,
-            h, d_h, d_s)
+            h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval)
         return (d_wx.to(x.dtype), d_r.to(r.dtype), d_bias.reshape(bias.shape).to(bias.dtype),
-                None if state is None else d_s0.to(state.dtype), None, None, None, None)
+                None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None)
 
 
 class _Runtime:
@@ -263,6 +265,16 @@ class sLSTMCell_hip(nn.Module):
             # the reference's native kernel clips y to +-clipval when built with it (slstm_pointwise.cu:107-110);
             # the hip kernels have no such path, and ignoring the setting would change results silently
             raise NotImplementedError("sLSTMCell backend 'hip' does not implement forward_clipval; leave it None")
+        clipval = self.config.gradient_recurrent_clipval
+        if clipval is not None and not clipval >= 1.0:
+            # The reference's cuda build clips y to +-gradient_recurrent_clipval in the FORWARD as well (cell.py:200-210
+            # hands that value, not forward_clipval, to SLSTM_FORWARD_CLIPVAL; slstm_pointwise.cu:107-110).  |y| <= 1 for
+            # every state the cell reaches from a zero state (y = sigmoid(o) c / n, c / n a weighted mean of tanh values),
+            # so a bound of 1 or more leaves the forward as it is and is implemented (the backward kernels clip);
+            # a smaller one would change the forward, which the hip kernels do not do.
+            raise NotImplementedError(
+                "sLSTMCell backend 'hip' implements gradient_recurrent_clipval >= 1 only: the reference clips the "
+                "forward's y to the same bound, which the hip forward kernels do not do")
         # optional: keep the carried state in float32 instead of the input dtype
         self.keep_state_fp32 = False
         # workspaces of the sequence kernel, one per (device, stream), the status words of calls in flight, caches
@@ -494,7 +506,8 @@ class sLSTMCell_hip(nn.Module):
         ):
             if x.is_cuda and self.head_dim <= BACKWARD_MAX_HEAD_DIM.get(x.dtype, 0):
                 h, s = _CellFunction.apply(x, self._recurrent_kernel_, self._bias_, state, h, s, reset_mask,
-                                           self.config.num_heads)
+                                           self.config.num_heads, bool(self.config.gradient_recurrent_cut),
+                                           self.config.gradient_recurrent_clipval)
             else:
                 h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
         output = self._permute_output(h)
@@ -542,7 +555,8 @@ class sLSTMCell_hip(nn.Module):
                 or torch.is_autocast_enabled()):
             return None
         if torch.is_grad_enabled() and (
-                input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad):
+                input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
+                or state.requires_grad):
             return None
         self._check_input(input)
         B = input.shape[0]

@@ -243,7 +243,15 @@ struct BwdParams {
   float *d_wx;               // [B,T,4,NH,dh] float32, strides in elements
   long long d_wx_sb, d_wx_st;
   float *d_s0;               // [4,B,H]
+  int cut;                   // no gradient from a step to the y it started from (slstm_backward_cut.cu:265-312)
+  float clip;                // > 0: that gradient is clipped to +-clip before d_h is added (slstm_pointwise.cu:136-143); 0: not
 };
+
+// The gradient that reached y_t through the recurrence, as the step's gradient takes it in: clipped when the call asks
+// for it, except at the last step, where it is the y part of d_s_final and comes from outside.
+__device__ __forceinline__ float bwd_recurrent_dy(float dy, float clip, bool last_step) {
+  return (clip > 0.0f && !last_step) ? __builtin_amdgcn_fmed3f(dy, -clip, clip) : dy;
+}
 
 // NW waves, each with NB 16-column blocks of the result (dh = 16 NB NW: wave w owns input units 16 NB w .. + 16 NB - 1).
 // More waves with fewer blocks each keep more loads in flight: a step is made of memory latency.
@@ -323,7 +331,7 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
           const int unit = (wave * NB + nb) * 16 + r16;
           float delta[4] = {0.0f, 0.0f, 0.0f, 0.0f};
           if (there[ii]) {
-            const float dyt = dh_in[ii][nb] + dy[nb][i];
+            const float dyt = dh_in[ii][nb] + bwd_recurrent_dy(dy[nb][i], p.clip, t == p.T - 1);
             const float dct = dc[nb][i] + dyt * cf[ii][nb][0];
             const float dnt = dn[nb][i] - dyt * cf[ii][nb][1];
             delta[0] = cf[ii][nb][2] * dct + cf[ii][nb][3] * dnt;
@@ -348,9 +356,11 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
     }
     __syncthreads();
     // ---- what reaches y_{t-1} through the recurrence: delta [16 rows x K] . R^T [K x dh], this wave's dh / 4 columns
+    //      (nothing when the call cuts that path)
     f32x4 acc[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) acc[nb] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    if (!p.cut) {
 #pragma unroll
     for (int j = 0; j < NG; ++j) {
       fetch_group(j + 1 < NG ? j + 1 : 0, bq[(j + 1) & 1]);
@@ -371,6 +381,7 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
           }
         }
       }
+    }
     }
     __syncthreads();  // (the tile is written again in the next step)
 #pragma unroll
@@ -437,6 +448,8 @@ struct BwdSplitParams {
   unsigned int *progress;    // [groups]: the step of the call that the group has reached (for the prefetching workgroups)
   int main_locals;           // workgroups per XCD that compute; those behind them (one per XCD, if any) prefetch
   long long spin_limit;
+  int cut;                   // as in BwdParams
+  float clip;
 };
 
 // fills the exchange ring with the "not written yet" pattern and clears the abort word in front of the split kernel
@@ -667,7 +680,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
     if (there) {
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
-        const float dyt = in.dh2[k] + dy[k];
+        const float dyt = in.dh2[k] + bwd_recurrent_dy(dy[k], p.clip, n == 0);
         const float dct = dc[k] + dyt * in.c9[0][k];
         const float dnt = dn[k] - dyt * in.c9[1][k];
         delta[0][k] = in.c9[2][k] * dct + in.c9[3][k] * dnt;
@@ -678,8 +691,10 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
         dn[k] = restart_now ? 0.0f : in.c9[8][k] * dnt;
       }
     }
-    // ---- publish the deltas (rows outside the batch: zeros), re-arm the words of two steps ago
-    {
+    // ---- publish the deltas (rows outside the batch: zeros), re-arm the words of two steps ago.  A call that cuts
+    //      the gradient through y needs none of the exchange: every workgroup is on its own.
+    const bool cut = p.cut != 0;
+    if (!cut) {
       char *const cur = ring + (n % kBwdRing) * ring_stride;
       char *const old = ring + ((n + kBwdRing - 2) % kBwdRing) * ring_stride;
 #pragma unroll
@@ -713,6 +728,13 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
 #pragma unroll
       for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
     }
+    if (cut) {
+      if (!FEED) fetch_step(in, t - 2);
+      __syncthreads();  // (the step's one barrier behind the publication: the feeders count on it)
+      dy[0] = 0.0f;
+      dy[1] = 0.0f;
+      return;
+    }
     if (S > 1) __builtin_amdgcn_s_sleep(8);  // (a workgroup that is its own group has its deltas in the L2 by the time it asks)
     // ---- the group's deltas of the wave's eighth of K: polled straight into the A operand registers
     uint4 areg[KSTEPS];
@@ -727,7 +749,8 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
         uint32_t mark = 0u;
 #pragma unroll
         for (int ks = 0; ks < KSTEPS; ++ks) mark = mark_join<BF16>(mark, chunk_mark<BF16>(areg[ks]));
-        if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mark)) == 0ull || gave_up) break;
+        // (a negative spin limit is the host's way to make every wait run out at its first look: the error path, forced)
+        if ((__builtin_amdgcn_ballot_w64(mark_has_sentinel<BF16>(mark)) == 0ull && p.spin_limit >= 0) || gave_up) break;
         if (++spins > p.spin_limit || ((spins & 255) == 0 && __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT))) {
           __hip_atomic_store(p.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           gave_up = true;

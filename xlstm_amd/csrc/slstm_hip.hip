@@ -187,6 +187,7 @@ int run_step(const xs_slstm_args *a) {
   p.B = B; p.NH = NH; p.dh = dh;
   p.n_unit_tiles = (dh + 31) / 32;
   p.n_row_tiles = (B + 63) / 64;
+  p.spin_limit = a->spin_limit > 0 ? (a->spin_limit < (1ll << 30) ? (int)a->spin_limit : (1 << 30)) : (1 << 22);
   const long long nwg = (long long)NH * p.n_unit_tiles * p.n_row_tiles;
   if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
   const dim3 grid((unsigned)nwg);
@@ -391,6 +392,12 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (prepare) {
     if (!a->wx || !a->ry || !a->bias) return fail(XS_ERR_NULL, "wx, ry and bias are required");
     if (a->wx_stride_t < 4 * H || (a->B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");
+    {  // (W.x and R.h go straight into LDS in pieces of 16 bytes)
+      const long long esz = bf16 ? 2 : 4;
+      if (((uintptr_t)a->wx % 16) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16))
+        return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
+      if (((uintptr_t)a->ry % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "ry and coef must be 16-byte aligned");
+    }
     BwdPrepParams p;
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
@@ -406,7 +413,13 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   } else {
     if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
     if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");
+    // (d_h and the coefficients are fetched in pieces of 16 bytes, d_wx is written in pairs of floats)
+    if (((uintptr_t)a->d_h % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "d_h and coef must be 16-byte aligned");
+    if (((uintptr_t)a->d_wx % 8) || (a->d_wx_stride_b % 2) || (a->d_wx_stride_t % 2))
+      return fail(XS_ERR_ALIGN, "d_wx must be 8-byte aligned and its strides even");
     if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
+    // (0, negative, NaN or infinite: no clipping)
+    const float clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
     if (a->split) {
       if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && bf16))
         return fail(XS_ERR_UNSUPPORTED, "backward pass over several compute units per head: head dim %d not supported", a->dh);
@@ -424,7 +437,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1;
       q.main_locals = (int)(grid / 8);
       const bool prefetchers = grid + 8 <= device_cus();  // (one more workgroup per XCD, where there is room)
-      q.spin_limit = a->spin_limit > 0 ? a->spin_limit : kDefaultSpinLimit;
+      q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;  // (negative: every wait gives up at once)
+      q.cut = a->recurrent_cut != 0; q.clip = clip;
       const long long n16 = (long long)kBwdRing * ngroups * 16 * 4 * a->dh * (bf16 ? 2 : 4) / 16;
       hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
                          (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
@@ -448,6 +462,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.coef = a->coef; p.d_h = a->d_h; p.d_s_final = a->d_s_final; p.r_t = a->r_t;
     p.reset = a->reset; p.reset_sb = a->reset_stride_b;
     p.d_wx = a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t; p.d_s0 = a->d_s0;
+    p.cut = a->recurrent_cut != 0; p.clip = clip;
     void (*kern)(BwdParams) = nullptr;
     int waves = 0;
 #ifndef XS_BWD_NB256

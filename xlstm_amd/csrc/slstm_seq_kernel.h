@@ -508,6 +508,15 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   const int xlane = ((wave * KW + q * EPC) >> 4) * XTILE + (r16 * 16 + ((q * EPC) & 15)) * ESZ;
   const int xtile_stride = p.G * XTILE;
   auto xconst = [&](int c, int mt_) { return ((c * 4 * EPC) >> 4) * XTILE + mt_ * xtile_stride; };
+  // Where the time loop of the compute waves starts relative to a 32-byte boundary of the code moves the time per step
+  // by 3 % (config 2, all eight phases measured twice: 1.690 / 1.707 / 1.717 / 1.718 / 1.720 / 1.738 / 1.751 / 1.752 ms,
+  // the same 32 bytes further on): the instruction fetch of a wave that comes out of a poll or a barrier.  Without the
+  // alignment the phase is whatever the code in front of the loop leaves (one more store there cost 1 %); with it the
+  // phase is chosen, per variant where one has been measured.
+#ifndef XS_LOOP_PAD
+#define XS_LOOP_PAD ((BF16 && NCH == 2 && MT == 1 && FULL && !BURST && !FMAC) ? 3 : 0)
+#endif
+  asm volatile(".p2align 5\n\t.rept %0\n\ts_nop 0\n\t.endr" :: "n"(XS_LOOP_PAD));
   for (int t = 0; t < p.T; ++t) {
     // all 16-byte polls of this step go through one buffer descriptor based at slot (t-1)
     // (the descriptor ends with the slot: a chunk past the last member reads zeros)

@@ -38,6 +38,7 @@ struct StepParams {
   int B, NH, dh;
   int n_unit_tiles, n_row_tiles;
   const void *h_prev;  // optional bf16 copy of the y plane of s0 (see the HB variant)
+  int spin_limit;      // bound of the waits between the waves of a workgroup (the pipelined kernel)
 };
 
 // Workgroup i runs on XCD i % 8.  The workgroups of one head share its h rows and its R, so they

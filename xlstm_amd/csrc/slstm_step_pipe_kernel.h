@@ -43,12 +43,14 @@ namespace {
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
-// (bounded like every other wait of the engine; the other waves of the workgroup always get there)
-__device__ __forceinline__ void wait_lds_counter(uint32_t *counter, uint32_t want) {
-  for (int spins = 0; spins < (1 << 22); ++spins) {
-    if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= want) break;
+// Bounded like every other wait of the engine (the other waves of the workgroup always get there); false when the
+// bound ran out.  The caller then marks the workgroup as given up, and what it stores is NaN.
+__device__ __forceinline__ bool wait_lds_counter(uint32_t *counter, uint32_t want, int spin_limit) {
+  for (int spins = 0; spins < spin_limit; ++spins) {
+    if (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= want) return true;
     __builtin_amdgcn_s_sleep(1);
   }
+  return __hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) >= want;
 }
 
 constexpr int kStepPipeThreads = 768;  // 4 MFMA waves + 8 gating waves
@@ -70,7 +72,7 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
   unsigned char *const cnm = hbuf + NHB * 64 * 256;                   // [3][64 rows][128 B]
   unsigned char *const wxl = cnm + 3 * 64 * 128;                      // [4 gates][64 rows][64 B]
   unsigned char *const rbuf = wxl + 4 * 64 * 64;                      // [2 K halves][128 columns][256 B], pieces swizzled
-  uint32_t *const counters = reinterpret_cast<uint32_t *>(rbuf + 2 * kHalfR);  // h_landed, -, -, -, summed[4], s_landed[4]
+  uint32_t *const counters = reinterpret_cast<uint32_t *>(rbuf + 2 * kHalfR);  // h_landed, -, -, -, summed[4], s_landed[4], gave_up
   // sums of (row tile rt, gate g), [16 rows][SROW] floats: inside the 8 KiB of K half rt / 2 that held gate g's columns
   auto sums_of = [&](int rt, int g) { return reinterpret_cast<float *>(rbuf + (rt >> 1) * kHalfR + g * 8192 + (rt & 1) * (16 * SROW * 4)); };
 
@@ -83,10 +85,22 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
   const int H = p.NH * DH;
   const long long BH = (long long)p.B * H;
 
+  // the status block: one launch, the step kernel, the pipelined one.  (Device-scope stores, like the stores of a
+  // workgroup that gives up: both reach the same place in the same order they were made.  Workgroup 0 is the first
+  // to be dispatched, and nobody gives up before its operands are a memory round trip overdue.)
   if (blockIdx.x == 0 && threadIdx.x < 16)
-    reinterpret_cast<uint32_t *>(p.status)[threadIdx.x] = (threadIdx.x == 5 || threadIdx.x == 6) ? 1u : 0u;  // one launch, the step kernel
-  if (threadIdx.x < 12) counters[threadIdx.x] = 0u;
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p.status) + threadIdx.x,
+                       (threadIdx.x == 5 || threadIdx.x == 6 || threadIdx.x == 8) ? 1u : 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x < 13) counters[threadIdx.x] = 0u;
   lds_barrier();  // the only workgroup barrier: the counters start at zero
+  // a wait inside the workgroup ran out: the workgroup's outputs become NaN and the status block says so
+  auto give_up = [&]() {
+    if (lane == 0) {
+      __hip_atomic_store(&counters[12], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      __hip_atomic_store(&p.status->abort_wg, (uint32_t)blockIdx.x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&p.status->aborted, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  };
 
   // ---- the old c, n, m and W.x (what is furthest away): a gating wave requests its share of the two row tiles its
   //      group gates, the earlier row tile first (10 loads per row tile, 3 + 2 or 2 + 3 per wave)
@@ -173,7 +187,7 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
       for (int ch = 0; ch < NK; ++ch)
         rf[ut][ch] = *reinterpret_cast<const uint4 *>(rbuf + (ch >> 2) * kHalfR + (wave * 32 + ut * 16 + r16) * 256 + swz[ch & 3]);
     if (wave == 0) XS_PSTAMP(1);
-    wait_lds_counter(&counters[0], 4u);  // h of all row tiles, from all four MFMA waves
+    if (!wait_lds_counter(&counters[0], 4u, p.spin_limit)) give_up();  // h of all row tiles, from all four MFMA waves
     asm volatile("" ::: "memory");
     // B operand: h of row 16 rt + r16, k-step ch.  The fragments of the next row tile are read while the MFMAs of this
     // one run (everything has landed: nothing else stands between the row tiles but the LDS round trip).
@@ -252,8 +266,7 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
       if (lane == 0) __hip_atomic_fetch_add(&counters[8 + rt], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
       if (wave == 4) XS_PSTAMP(16);
     }
-    wait_lds_counter(&counters[8 + rt], 4u);
-    wait_lds_counter(&counters[4 + rt], 4u);
+    if (!wait_lds_counter(&counters[8 + rt], 4u, p.spin_limit) || !wait_lds_counter(&counters[4 + rt], 4u, p.spin_limit)) give_up();
     asm volatile("" ::: "memory");
     if (wave == 4 || wave == 8) XS_PSTAMP(17 + 2 * rt);
     float2 s2[4];
@@ -266,6 +279,8 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
     const float2 c2 = *reinterpret_cast<const float2 *>(cnm + (0 * 64 + row) * 128 + pair * 8);
     const float2 n2 = *reinterpret_cast<const float2 *>(cnm + (1 * 64 + row) * 128 + pair * 8);
     const float2 m2 = *reinterpret_cast<const float2 *>(cnm + (2 * 64 + row) * 128 + pair * 8);
+    // (an MFMA wave that gave up said so before it reported its sums; this wave's own give_up is in LDS order before this read)
+    const bool poisoned = __hip_atomic_load(&counters[12], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0u;
     float yv[2], cv[2], nv[2], mv[2];
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
@@ -277,7 +292,8 @@ __global__ __launch_bounds__(kStepPipeThreads) void slstm_step_pipe_kernel(StepP
       }
       CellState st{0.0f, i ? c2.y : c2.x, i ? n2.y : n2.x, i ? m2.y : m2.x};
       slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
-      yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
+      yv[i] = poisoned ? kPoison : st.y; cv[i] = poisoned ? kPoison : st.c;
+      nv[i] = poisoned ? kPoison : st.n; mv[i] = poisoned ? kPoison : st.m;
     }
     if (rti == 0) {
       // The second row tile's share, before this row tile's stores go out: loads and stores share the counter and a

@@ -73,6 +73,8 @@ def slstm_backward(
     timings: Optional[dict] = None,
     split_override: Optional[bool] = None,
     spin_limit: int = 0,
+    recurrent_cut: bool = False,
+    recurrent_clipval: Optional[float] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -87,6 +89,9 @@ def slstm_backward(
     the two kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
+    ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
+    to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
+    clipped to +-value before ``d_h`` is added, ``slstm_pointwise.cu:136-143``).
     """
     lib = _lib.load()
     _require_cuda("wx", wx)
@@ -120,7 +125,8 @@ def slstm_backward(
         dh_p = widen(d_h, (T_, B_)).reshape(T_, B_, NH * dh_k)
         dsf_p = widen(d_s_final, (4, B_)).reshape(4, B_, NH * dh_k) if d_s_final is not None else None
         d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
-                                                 split_override=split_override, spin_limit=spin_limit)
+                                                 split_override=split_override, spin_limit=spin_limit,
+                                                 recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval)
         return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
                 d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
                 d_bias[..., :dh].contiguous(),
@@ -140,11 +146,14 @@ def slstm_backward(
                 parts.append(slstm_backward(
                     wx[b0:b1], r, bias, None if s0 is None else s0[:, b0:b1], None if reset_mask is None else reset_mask[b0:b1],
                     h_out[:, b0:b1], d_h[:, b0:b1], None if d_s_final is None else d_s_final[:, b0:b1],
-                    timings=None, split_override=split_override, spin_limit=spin_limit))
+                    timings=None, split_override=split_override, spin_limit=spin_limit,
+                    recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval))
             return (torch.cat([q[0] for q in parts], 0), sum(q[1] for q in parts), sum(q[2] for q in parts),
                     torch.cat([q[3] for q in parts], 1))
-    if wx.stride(2) != 1 or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H):
-        wx = wx.contiguous()
+    esz = wx.element_size()
+    if (wx.stride(2) != 1 or wx.data_ptr() % 16 or (wx.stride(0) * esz) % 16 or (wx.stride(1) * esz) % 16
+            or wx.stride(1) < 4 * H or (B > 1 and wx.stride(0) < 4 * H)):
+        wx = wx.contiguous()  # (the same condition as in the forward: the kernels fetch W.x in pieces of 16 bytes)
     bias = bias.to(torch.float32).contiguous()
     if s0 is not None:
         s0 = s0.to(torch.float32).contiguous()
@@ -222,6 +231,8 @@ def slstm_backward(
     a.exchange = exchange.data_ptr() if split else None
     a.counters = counters.data_ptr() if split else None
     a.spin_limit = int(spin_limit)
+    a.recurrent_cut = 1 if recurrent_cut else 0
+    a.recurrent_clipval = float(recurrent_clipval) if recurrent_clipval is not None else 0.0
     marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
