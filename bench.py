@@ -184,6 +184,65 @@ def bench_decode(device, steps=1024, prefill=128):
     }
 
 
+def measure_stage(device, stage, steps, members=16, two_xcds=0, rows=4, reps=5):
+    """Median time (us) of one call of ``xs_measure_stage`` with ``steps`` iterations, by HIP events on the stream the
+    kernel is launched on; ``None`` if one of its bounded waits ran out."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from xlstm_amd import _lib
+
+    lib = _lib.load()
+    ws = torch.zeros(256 + 32 * 8 * 16 * 512, dtype=torch.uint8, device=device)
+    a = _lib.MeasureArgs()
+    a.stage, a.members, a.two_xcds, a.rows, a.steps = stage, members, two_xcds, rows, steps
+    a.workspace, a.workspace_bytes = ws.data_ptr(), ws.numel()
+    a.stream = torch.cuda.current_stream(device).cuda_stream
+    times = []
+    for i in range(reps + 1):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        rc = lib.xs_measure_stage(ctypes.byref(a))
+        e1.record()
+        torch.cuda.synchronize()
+        if rc != 0:
+            raise RuntimeError(f"xs_measure_stage failed ({rc}): {_lib.last_error()}")
+        if stage in (_lib.STAGE_EXCHANGE, _lib.STAGE_CHAIN) and int(ws[:4].view(torch.int32)[0]):
+            return None
+        if i:
+            times.append(e0.elapsed_time(e1) * 1e3)
+    return float(np.median(times))
+
+
+def serial_bound(device):
+    """The dependency chain of one timestep, measured by ``xs_measure_stage`` (the product kernel's instructions, layouts
+    and exchange protocol; every iteration needs the result of the one before).  ``config2_chain``: the whole chain as
+    one loop - poll, MFMAs, sums through LDS and the barrier, gating, publication - on 16 head groups of 16 compute
+    units, with none of the product kernel's other work: the serial bound of a step of this structure.  The stages alone
+    (each its own loop, so their sum is more than the chain: every loop pays its own entry and waits) say where it
+    goes.  Per-iteration times are differences between two step counts, so launches and set-up cancel.  Also the floor
+    of a dependent launch (the decode step's)."""
+    from xlstm_amd import _lib
+
+    def per_step(stage, n=20000, **kw):
+        lo, hi = measure_stage(device, stage, n, **kw), measure_stage(device, stage, 3 * n, **kw)
+        return None if lo is None or hi is None else (hi - lo) / (2 * n)
+
+    chain = per_step(_lib.STAGE_CHAIN, rows=4)
+    ex16 = per_step(_lib.STAGE_EXCHANGE, members=16, rows=4)
+    mm = per_step(_lib.STAGE_CONTRACTION)
+    ga = per_step(_lib.STAGE_GATING)
+    ex64 = per_step(_lib.STAGE_EXCHANGE, n=5000, members=64, two_xcds=1, rows=16)
+    ex32 = per_step(_lib.STAGE_EXCHANGE, n=5000, members=32, rows=16)
+    launch = per_step(_lib.STAGE_LAUNCH, n=2000)
+    return {"config2_chain_us_per_step": chain,
+            "stages_alone_us": {"exchange_16_units_one_xcd_4_rows": ex16, "mfma_and_lds_reduction": mm, "gating": ga},
+            "exchange_32_units_one_xcd_16_rows_us": ex32, "exchange_64_units_two_xcds_16_rows_us": ex64,
+            "dependent_launch_us": launch}
+
+
 def bench_backward(device, iters=3):
     """The backward pass at BASELINE config 2 (B=16, T=2048, D=1024, NH=4, bf16, packed documents): the whole call
     (three library GEMMs and a reduction around the engine's two kernels) and the two kernels by HIP events."""
@@ -497,6 +556,10 @@ def main():
     ap.add_argument("--phase-profile", action="store_true",
                     help="per-phase cycle tables of the sequence kernels from the measurement build of the library "
                          "(python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so)")
+    ap.add_argument("--serial-bound", action="store_true",
+                    help="only measure the stages of a timestep's dependency chain and the launch floor (their own JSON line)")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="leave out the other BASELINE configs, the backward pass and the serial bound (profiling runs)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 1 GiB device copy 5 times (scales the rocprofv3 FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -527,6 +590,9 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         print(json.dumps({"copy_bytes_each_way": src.numel() * 4, "copies": 5}))
+        return
+    if args.serial_bound:
+        print(json.dumps({"serial_bound": serial_bound(device)}))
         return
     if args.decode_only:
         print(json.dumps({"decode": bench_decode(device)}))
@@ -606,6 +672,31 @@ def main():
     if os.path.exists(traffic_file):
         out["roofline"]["traffic"] = json.load(open(traffic_file)).get("hbm_bytes_per_launch")
         out["roofline"]["traffic_source"] = "profiles/traffic_seq_cfg2.json (rocprofv3 counters of a separate run, not of this one)"
+    lean = args.headline_only or args.no_decode  # (profiling runs want the one kernel)
+    if not lean:
+        # the stages of the chain measured in this run, and what the measured step is against their sum
+        sb = serial_bound(device)
+        out["roofline"]["serial_bound_stages_us"] = sb
+        if sb.get("config2_chain_us_per_step"):
+            out["roofline"]["serial_bound_us_per_step"] = sb["config2_chain_us_per_step"]
+            out["roofline"]["frac_of_serial_bound"] = sb["config2_chain_us_per_step"] / (kern_ms * 1e3 / T)
+            out["roofline"]["serial_bound_source"] = ("measured in this run: xs_measure_stage(XS_STAGE_CHAIN), the step's "
+                                                      "dependency chain alone on 16 head groups of 16 compute units")
+        # the other BASELINE configurations and the backward pass, compact (full rows: --all-configs)
+        c1 = bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0)
+        c4 = bench_config(device, "config 4 (one sLSTM cell): B=8 T=2048 D=1024 NH=4 bf16, documents mean 768", 8, 2048, 4, 256, True, 768)
+        c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=3)
+        bw = bench_backward(device)
+        out["other_configs"] = [
+            {"workload": c["workload"], "ms": c["ms"], "us_per_timestep": c["us_per_timestep"], "aborted": c["aborted"],
+             "roofline": ({"bound": "mfma", "frac": c["tflops"] / MFMA_BF16_PEAK_TFLOPS, "achieved": c["tflops"], "unit": "TFLOP/s",
+                           "peak": MFMA_BF16_PEAK_TFLOPS, "kernel": "slstm_seq_roles_kernel<bf16,NCH=8,FULL>"} if c is c5 else
+                          {"bound": "hbm", "frac": c["hbm_GBs"] / HBM_PEAK_GBS, "achieved": c["hbm_GBs"], "unit": "GB/s",
+                           "peak": HBM_PEAK_GBS})}
+            for c in (c1, c4, c5)]
+        out["backward"] = {k: bw[k] for k in ("workload", "ms", "finite") if k in bw}
+        out["backward"]["kernels_ms"] = {k: v for k, v in bw.items() if k.endswith("_ms")}
+        out["backward"]["roofline"] = bw["roofline"]
     if args.all_configs:
         out["all_configs"] = [
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),
@@ -620,6 +711,16 @@ def main():
         out["layer"] = bench_layer(device, args.layer_iters, args.layer_decode_steps)
     if not args.no_decode:
         out["decode"] = bench_decode(device)
+        if not lean:
+            # a decode step is one dependent launch: its floor is the launch itself plus the step's bytes at the HBM peak
+            launch = out["roofline"]["serial_bound_stages_us"].get("dependent_launch_us")
+            if launch:
+                dr = out["decode"]["roofline"]
+                dr["dependent_launch_floor_us"] = launch
+                dr["serial_bound_us_per_step"] = launch + dr["algorithmic_bytes_per_launch"] / (HBM_PEAK_GBS * 1e3)
+                dr["frac_of_serial_bound"] = dr["serial_bound_us_per_step"] / min(
+                    out["decode"]["gpu_us_per_step"], out["decode"]["graph_us_per_step"] or 1e9)
+                dr["serial_bound_source"] = "measured in this run: back-to-back launches of an empty kernel + bytes / HBM peak"
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(wx_c, r_ext_c, bias_c, mask_c)
     print(json.dumps(out), flush=True)

@@ -316,6 +316,34 @@ typedef struct xs_slstm_bwd_args {
 int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);
 int xs_slstm_backward(const xs_slstm_bwd_args *args);
 
+/*
+ * Measurement (no counterpart in the reference): one stage of the dependency chain of a timestep of the sequence
+ * kernel, run alone for `steps` iterations in which every iteration needs the result of the one before, with the
+ * product kernel's instructions, layouts and exchange protocol.  The caller times the call (events on `stream`) at two
+ * step counts and divides the difference; the sum of the three stages is the serial bound of a step.
+ *   XS_STAGE_EXCHANGE     `members` compute units (8, 16, 32 or 64; one XCD, or with two_xcds != 0 half each on XCDs 0
+ *                         and 4 with device-scope stores) publish a 16 x 16 bf16 tile each and poll the group's tile of
+ *                         `rows` batch rows until it is complete.  Workspace: 256 + 8 * members * 512 bytes; word 0 is
+ *                         nonzero afterwards if a wait ran out (other work held compute units), word 1 the longest wait.
+ *   XS_STAGE_CONTRACTION  one workgroup: 4 waves x 4 gates x 2 MFMAs (head dim 256), partial sums through LDS, barrier.
+ *   XS_STAGE_GATING       one workgroup: the exponential gating of one element per lane, y rounded to bf16.
+ *   XS_STAGE_LAUNCH       `steps` launches of an empty kernel, back to back: the floor of a dependent launch.
+ *   XS_STAGE_CHAIN        the three stages as ONE loop in the product kernel's order (poll, MFMAs, sums through LDS and
+ *                         the barrier, gating, publication) on head groups of 16 compute units placed as the product places
+ *                         them, as many as the device holds, tiles of `rows` batch rows; constant W.x, no mask, no output
+ *                         tensor, none of the product kernel's other waves: what a step costs when only the chain is
+ *                         left.  Workspace: 256 + (compute units / 16) * 8 * 16 * 512 bytes; words 0 and 1 as above.
+ */
+enum { XS_STAGE_EXCHANGE = 0, XS_STAGE_CONTRACTION = 1, XS_STAGE_GATING = 2, XS_STAGE_LAUNCH = 3, XS_STAGE_CHAIN = 4 };
+typedef struct xs_measure_args {
+  int32_t stage, members, two_xcds, rows, steps;
+  void *workspace;
+  size_t workspace_bytes;
+  void *stream;
+} xs_measure_args;
+
+int xs_measure_stage(const xs_measure_args *args);
+
 #ifdef __cplusplus
 }
 #endif

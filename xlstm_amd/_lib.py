@@ -28,6 +28,7 @@ EXPORTS = (
     "xs_causal_conv_silu",
     "xs_headwise_gates",
     "xs_headwise_group_norm",
+    "xs_measure_stage",
 )
 
 
@@ -136,6 +137,21 @@ class NormArgs(ctypes.Structure):
     ]
 
 
+STAGE_EXCHANGE, STAGE_CONTRACTION, STAGE_GATING, STAGE_LAUNCH, STAGE_CHAIN = 0, 1, 2, 3, 4
+
+
+class MeasureArgs(ctypes.Structure):
+    """Mirror of ``xs_measure_args``."""
+
+    _fields_ = [
+        ("stage", ctypes.c_int32), ("members", ctypes.c_int32), ("two_xcds", ctypes.c_int32), ("rows", ctypes.c_int32),
+        ("steps", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_size_t),
+        ("stream", ctypes.c_void_p),
+    ]
+
+
 class SlstmStatus(ctypes.Structure):
     """Mirror of ``xs_slstm_status`` (first bytes of the workspace)."""
 
@@ -181,6 +197,8 @@ def load() -> ctypes.CDLL:
     lib.xs_headwise_gates.argtypes = [ctypes.POINTER(GatesArgs)]
     lib.xs_headwise_group_norm.restype = ctypes.c_int
     lib.xs_headwise_group_norm.argtypes = [ctypes.POINTER(NormArgs)]
+    lib.xs_measure_stage.restype = ctypes.c_int
+    lib.xs_measure_stage.argtypes = [ctypes.POINTER(MeasureArgs)]
     if lib.xs_abi_version() != ABI_VERSION:
         raise RuntimeError(f"xlstm_amd: ABI version {lib.xs_abi_version()} != expected {ABI_VERSION}; rebuild")
     _LIB = lib

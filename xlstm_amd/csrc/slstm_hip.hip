@@ -34,6 +34,7 @@
 #include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
 #include "slstm_backward_kernels.h"
+#include "slstm_serial_bound.h"
 
 // ---------------------------------------------------------------------------
 // Scratch of the entry point that allocates nothing (xs_slstm_forward_static): status block, placement words and
@@ -617,6 +618,64 @@ int run_group_norm(const xs_norm_args *a) {
   return XS_OK;
 }
 
+// ---- measurement: one stage of the dependency chain of a timestep, alone (slstm_serial_bound.h)
+int run_stage(const xs_measure_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->steps <= 0) return fail(XS_ERR_SHAPE, "steps must be positive");
+  hipStream_t stream = (hipStream_t)a->stream;
+  StageParams p{};
+  p.steps = a->steps;
+  p.words = nullptr;
+  if (a->stage == XS_STAGE_LAUNCH) {
+    for (int i = 0; i < a->steps; ++i) hipLaunchKernelGGL(stage_empty_kernel, dim3(1), dim3(64), 0, stream);
+  } else {
+    if (!a->workspace || ((uintptr_t)a->workspace % 256)) return fail(XS_ERR_WORKSPACE, "a 256-byte aligned workspace is required");
+    p.words = (unsigned int *)a->workspace;
+    if (a->stage == XS_STAGE_EXCHANGE) {
+      const int G = a->members;
+      if (G != 8 && G != 16 && G != 32 && G != 64) return fail(XS_ERR_SHAPE, "members must be 8, 16, 32 or 64");
+      if (a->rows < 1 || a->rows > 16) return fail(XS_ERR_SHAPE, "rows must be 1..16");
+      const int cus = device_cus();
+      const int per_xcd = a->two_xcds ? G / 2 : G;
+      if (cus <= 0 || per_xcd > cus / 8) return fail(XS_ERR_DEVICE, "%d workgroups do not fit one XCD of this device at once", per_xcd);
+      const size_t ring = (size_t)kRing * G * 512;
+      if (a->workspace_bytes < 256 + ring) return fail(XS_ERR_WORKSPACE, "the exchange stage needs %zu bytes of workspace", 256 + ring);
+      p.members = G; p.two_xcds = a->two_xcds ? 1 : 0; p.rows = a->rows;
+      p.ring = (char *)a->workspace + 256;
+      p.spin_limit = kDefaultSpinLimit;
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, (uint32_t *)a->workspace, (size_t)64, 0u);
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(64), dim3(256), 0, stream, (uint32_t *)p.ring, ring / 4, kSentinel32);
+      void (*k)(StageParams) = G == 8 ? stage_exchange_kernel<1> : (G == 16 ? stage_exchange_kernel<2> : (G == 32 ? stage_exchange_kernel<4> : stage_exchange_kernel<8>));
+      hipLaunchKernelGGL(k, dim3(8 * per_xcd), dim3(256), 0, stream, p);
+    } else if (a->stage == XS_STAGE_CHAIN) {
+      const int G = 16;  // (head dim 256)
+      const int cus = device_cus();
+      const int per_xcd = cus > 0 ? (cus / 8) / G : 0;  // head groups per XCD, as many as fit: the product's launch at config 2
+      if (per_xcd < 1) return fail(XS_ERR_DEVICE, "a head group of %d workgroups does not fit one XCD of this device", G);
+      if (a->rows < 1 || a->rows > 16) return fail(XS_ERR_SHAPE, "rows must be 1..16");
+      const size_t ring = (size_t)8 * per_xcd * kRing * G * 512;
+      if (a->workspace_bytes < 256 + ring) return fail(XS_ERR_WORKSPACE, "the chain stage needs %zu bytes of workspace", 256 + ring);
+      p.members = G; p.two_xcds = 0; p.rows = a->rows;
+      p.ring = (char *)a->workspace + 256;
+      p.spin_limit = kDefaultSpinLimit;
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, (uint32_t *)a->workspace, (size_t)64, 0u);
+      hipLaunchKernelGGL(fill_u32_kernel, dim3(64), dim3(256), 0, stream, (uint32_t *)p.ring, ring / 4, kSentinel32);
+      hipLaunchKernelGGL(stage_chain_kernel, dim3(8 * per_xcd * G), dim3(256), 0, stream, p);
+    } else if (a->stage == XS_STAGE_CONTRACTION) {
+      if (a->workspace_bytes < 256) return fail(XS_ERR_WORKSPACE, "256 bytes of workspace are required");
+      hipLaunchKernelGGL(stage_contraction_kernel<2>, dim3(1), dim3(256), 0, stream, p);
+    } else if (a->stage == XS_STAGE_GATING) {
+      if (a->workspace_bytes < 256) return fail(XS_ERR_WORKSPACE, "256 bytes of workspace are required");
+      hipLaunchKernelGGL(stage_gating_kernel, dim3(1), dim3(256), 0, stream, p);
+    } else {
+      return fail(XS_ERR_SHAPE, "unknown stage %d", a->stage);
+    }
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "measurement kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 // host side of the static scratch array: its device address, per device
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
@@ -692,6 +751,11 @@ int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args) {
 int xs_slstm_backward(const xs_slstm_bwd_args *args) {
   g_err[0] = 0;
   return run_backward(args, false);
+}
+
+int xs_measure_stage(const xs_measure_args *args) {
+  g_err[0] = 0;
+  return run_stage(args);
 }
 
 int xs_causal_conv_silu(const xs_conv_args *args) {
