@@ -311,10 +311,27 @@ typedef struct xs_slstm_bwd_args {
    *                          0, negative or not finite: no clipping. */
   int32_t recurrent_cut;
   float recurrent_clipval;
+  /* the forward call's outputs and recurrent matrix, and the gradients of the parameters */
+  const void *h_out;         /* [T,B,H] in dtype: what the forward call returned (params; prepare when ry is NULL) */
+  const void *r;             /* [NH,4*dh,dh] in dtype, as the forward takes it (prepare when ry is NULL) */
+  float *d_r;                /* [NH,4*dh,dh] float32: gradient of r in that layout (params) */
+  float *d_bias;             /* [NH,4,dh] float32 (params) */
 } xs_slstm_bwd_args;
 
 int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);
 int xs_slstm_backward(const xs_slstm_bwd_args *args);
+
+/*
+ * xs_slstm_backward_params   the gradients of the recurrent matrix and the bias from the gate deltas that
+ *   xs_slstm_backward left in d_wx and the forward's outputs: d_r[h][g*dh+a][d] = sum over rows and steps of
+ *   d_wx[b,t,g,h,a] * y_{t-1}[b,h,d] (y_{-1} the y plane of s0; zero where reset[b,t] is set), d_bias[h][g][a] = sum of
+ *   d_wx[b,t,g,h,a].  Replaces the strided-batched GEMM and the bias aggregation behind the reference's time loop
+ *   (slstm_backward.cu:381-386, 52-108).  Uses B, T, NH, dh (a multiple of 64), dtype, d_wx and its strides, h_out, s0,
+ *   reset, d_r, d_bias, stream.  With bf16 the deltas are rounded to bf16 for the product (float32 sums), as the
+ *   reference's gate cache is.  The sums over slices of B*T are added with float atomics: their last bits depend on
+ *   the order the compute units finish in.
+ */
+int xs_slstm_backward_params(const xs_slstm_bwd_args *args);
 
 /*
  * Measurement (no counterpart in the reference): one stage of the dependency chain of a timestep of the sequence

@@ -25,6 +25,7 @@ EXPORTS = (
     "xs_slstm_forward_static",
     "xs_slstm_backward_prepare",
     "xs_slstm_backward",
+    "xs_slstm_backward_params",
     "xs_causal_conv_silu",
     "xs_headwise_gates",
     "xs_headwise_group_norm",
@@ -82,6 +83,10 @@ class SlstmBwdArgs(ctypes.Structure):
         ("spin_limit", ctypes.c_int64),
         ("recurrent_cut", ctypes.c_int32),
         ("recurrent_clipval", ctypes.c_float),
+        ("h_out", ctypes.c_void_p),
+        ("r", ctypes.c_void_p),
+        ("d_r", ctypes.c_void_p),
+        ("d_bias", ctypes.c_void_p),
     ]
 
 
@@ -188,7 +193,7 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmArgs)]
-    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
+    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmBwdArgs)]
     lib.xs_causal_conv_silu.restype = ctypes.c_int

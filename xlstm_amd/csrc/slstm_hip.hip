@@ -34,6 +34,7 @@
 #include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
 #include "slstm_backward_kernels.h"
+#include "slstm_backward_params_kernel.h"
 #include "slstm_serial_bound.h"
 
 // ---------------------------------------------------------------------------
@@ -486,6 +487,64 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   return XS_OK;
 }
 
+// ---- backward pass: the gradients of R and the bias from the gate deltas and the forward's outputs
+int run_backward_params(const xs_slstm_bwd_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
+  if (a->dtype != XS_F32 && a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
+  if (a->dh % 64 != 0) return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d is not a multiple of 64", a->dh);
+  if (!a->d_r || !a->d_bias) return fail(XS_ERR_NULL, "d_r and d_bias are required");
+  const bool bf16 = a->dtype == XS_BF16;
+  const long long H = (long long)a->NH * a->dh;
+  hipStream_t stream = (hipStream_t)a->stream;
+  const size_t nr = (size_t)a->NH * 4 * a->dh * a->dh, nb = (size_t)4 * H;
+  if (((uintptr_t)a->d_r % 4) || ((uintptr_t)a->d_bias % 4)) return fail(XS_ERR_ALIGN, "d_r and d_bias must be 4-byte aligned");
+  const bool empty = a->B == 0 || a->T == 0;
+  if (!empty) {
+    if (!a->d_wx || !a->h_out) return fail(XS_ERR_NULL, "d_wx and h_out are required");
+    if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
+    if (((uintptr_t)a->d_wx % 16) || (a->d_wx_stride_b % 4) || (a->d_wx_stride_t % 4))
+      return fail(XS_ERR_ALIGN, "d_wx and its row/step strides must be 16-byte aligned");
+    if (((uintptr_t)a->h_out % 16) || ((uintptr_t)a->s0 % 16)) return fail(XS_ERR_ALIGN, "h_out and s0 must be 16-byte aligned");
+    if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
+  }
+  // (the slices of K are added into the results: they start at zero)
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(256), dim3(256), 0, stream, (uint32_t *)a->d_r, nr, 0u);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(4), dim3(256), 0, stream, (uint32_t *)a->d_bias, nb, 0u);
+  if (!empty) {
+    BwdParamParams p;
+    p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
+    p.d_wx = a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t;
+    p.h_out = a->h_out; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b;
+    p.d_r = a->d_r; p.d_bias = a->d_bias;
+    p.tchunks = (a->T + kParamKC - 1) / kParamKC;
+    const int nt = a->dh % 256 == 0 ? 256 : (a->dh % 128 == 0 ? 128 : 64);
+    const int tiles = (4 * a->dh / kParamMT) * (a->dh / nt);
+    const long long nchunks = (long long)a->B * p.tchunks;
+    // slices of K: enough workgroups for two per compute unit, no slice shorter than four chunks
+    const int cus = device_cus() > 0 ? device_cus() : 256;
+    long long ks = (2ll * cus + (long long)a->NH * tiles - 1) / ((long long)a->NH * tiles);
+    if (ks > nchunks / 4) ks = nchunks / 4;
+    if (ks < 1) ks = 1;
+    p.ksplit = (int)ks;
+    const long long groups = (long long)a->NH * ks;
+    const long long grid = (groups + 7) / 8 * 8 * tiles;
+    if (grid > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one launch");
+    void (*kern)(BwdParamParams);
+    if (bf16) kern = nt == 256 ? slstm_bwd_param_kernel<true, 256> : (nt == 128 ? slstm_bwd_param_kernel<true, 128> : slstm_bwd_param_kernel<true, 64>);
+    else kern = nt == 256 ? slstm_bwd_param_kernel<false, 256> : (nt == 128 ? slstm_bwd_param_kernel<false, 128> : slstm_bwd_param_kernel<false, 64>);
+    const size_t lds = (size_t)bwd_param_lds_bytes(bf16, nt);
+    if (lds > 64 * 1024) {
+      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
+      if (rc != XS_OK) return rc;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(512), lds, stream, p);
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "parameter gradient kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 int run_conv(const xs_conv_args *a) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->D <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d D=%d", a->B, a->T, a->D);
@@ -756,6 +815,11 @@ int xs_slstm_backward(const xs_slstm_bwd_args *args) {
 int xs_measure_stage(const xs_measure_args *args) {
   g_err[0] = 0;
   return run_stage(args);
+}
+
+int xs_slstm_backward_params(const xs_slstm_bwd_args *args) {
+  g_err[0] = 0;
+  return run_backward_params(args);
 }
 
 int xs_causal_conv_silu(const xs_conv_args *args) {

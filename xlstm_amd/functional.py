@@ -246,13 +246,18 @@ def slstm_backward(
             marks.append(torch.cuda.Event(enable_timing=True))
             marks[-1].record()
             timings["events"] = marks  # prepare = [0] -> [1], reverse kernel = [1] -> [2]
-    # d R[h][g dh + a][d] = sum over steps and rows of delta[b,t,g,h,a] * y_{t-1}[b,h,d]; d bias = sum of delta
-    # (the deltas of a gate and head are a transposed matrix inside d_wx as it lies, 4 NH of them a regular batch, and the
-    # outputs are broadcast over the gates: measured at config 2 0.79 ms, against 0.89 with the outputs repeated by
-    # hand, 0.79 + a copy with d_wx brought into another order, and 1.7 as four products of NH matrices)
-    dl = d_wx.view(B * T, 4, NH, dh).permute(1, 2, 3, 0)                                 # [4, NH, dh, B*T]
-    d_r = torch.matmul(dl, yp.unsqueeze(0)).permute(1, 0, 2, 3).reshape(NH, 4 * dh, dh)  # [NH, 4*dh, dh]
-    d_bias = d_wx.view(B * T, 4, NH, dh).sum(0).transpose(0, 1).contiguous()
+        # d R[h][g dh + a][d] = sum over steps and rows of delta[b,t,g,h,a] * y_{t-1}[b,h,d]; d bias = sum of delta: the
+        # engine's third backward kernel, from d_wx as it lies and the forward's outputs
+        d_r = torch.empty((NH, 4 * dh, dh), dtype=torch.float32, device=dev)
+        d_bias = torch.empty((NH, 4, dh), dtype=torch.float32, device=dev)
+        h_c = h_out if h_out.is_contiguous() and h_out.dtype == wx.dtype else h_out.to(wx.dtype).contiguous()
+        a.h_out, a.d_r, a.d_bias = h_c.data_ptr(), d_r.data_ptr(), d_bias.data_ptr()
+        rc = lib.xs_slstm_backward_params(ctypes.byref(a))
+        if rc != 0:
+            raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+        if timings is not None:
+            marks.append(torch.cuda.Event(enable_timing=True))
+            marks[-1].record()  # parameter gradients = [2] -> [3]
     if split and timings is None and int(counters[0].item()):  # (a synchronisation; training calls are not latency-bound)
         raise EngineError("xlstm_amd: a wait between the compute units of a head ran out in the backward pass "
                           "(other work held compute units); the gradients are invalid")
