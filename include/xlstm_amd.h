@@ -254,11 +254,10 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  * reference's per-timestep launches (slstm_backward.cu:291-319) and the state history and gate cache its forward
  * writes for them (slstm.cc:79-108); the forward entry points above store nothing for training.
  *
- * xs_slstm_backward_prepare  walks forward in time over raw = wx + ry + bias, where ry[h,b,t,a,g] =
- *   sum_d y_{t-1}[b,h,d] * r[h][g*dh+a][d] is given for all steps at once (one batched GEMM over the outputs of the
- *   forward call, shifted by one step, rows that start a document zeroed), and writes nine float32 coefficients per
- *   step and element into coef [T,B,9,H] (with split != 0: T * ceil(B/16)*16 * 9 * H floats, in the order the split
- *   kernel reads them).
+ * xs_slstm_backward_prepare  walks forward in time over raw = wx + R.y_{t-1} + bias, recomputing R.y_{t-1} from the
+ *   outputs h_out of the forward call (y_{-1} the y plane of s0; zero where reset[b,t] is set) and r, and writes nine
+ *   float32 coefficients per step and element into coef [T,B,9,H] (with split != 0: T * ceil(B/16)*16 * 9 * H floats,
+ *   in the order the split kernel reads them).
  * xs_slstm_backward          one launch for all T steps, reverse in time: d_wx [B,T,4,NH,dh] (float32, the gradient
  *   with respect to the raw gates: the gradient of wx, and with the outputs what the gradients of R and the bias are
  *   sums of, slstm_backward.cu:381-386, 52-108) and d_s0 [4,B,H] (the m part is zero).
@@ -266,7 +265,8 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  * dtype is the type of wx, d_h and r_t (XS_F32 or XS_BF16).  r_t is R transposed - element (input unit d, gate
  * unit k = g*dh + a) of head h is the reference's external view recurrent_kernel[h][d][g][a] (cell.py:234-242) -
  * tiled as MFMA operands: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC] with EPC = 16 bytes of elements (8 bf16, 4 f32)
- * and KC = 4*EPC, so that what the 64 lanes of a wave load for one k-step is 1 KiB in a row.  Head dims: 64, 128, 256.
+ * and KC = 4*EPC, so that what the 64 lanes of a wave load for one k-step is 1 KiB in a row.  Head dims: 64, 128, 256
+ * (512 with bf16 and split).
  * The caller owns every buffer; both calls only enqueue kernels on `stream`.
  */
 typedef struct xs_slstm_bwd_args {
@@ -274,7 +274,7 @@ typedef struct xs_slstm_bwd_args {
   int32_t dtype;
   const void *wx;            /* [B,T,4,NH,dh], strides in elements, innermost 4*H contiguous (prepare) */
   int64_t wx_stride_b, wx_stride_t;
-  const float *ry;           /* [NH,B,T,dh,4] (prepare) */
+  const float *ry;           /* unused (an earlier version took R.y_{t-1} of all steps here); pass NULL */
   const float *bias;         /* [NH,4,dh] (prepare) */
   const float *s0;           /* [4,B,H] or NULL (prepare) */
   const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */
@@ -312,8 +312,8 @@ typedef struct xs_slstm_bwd_args {
   int32_t recurrent_cut;
   float recurrent_clipval;
   /* the forward call's outputs and recurrent matrix, and the gradients of the parameters */
-  const void *h_out;         /* [T,B,H] in dtype: what the forward call returned (params; prepare when ry is NULL) */
-  const void *r;             /* [NH,4*dh,dh] in dtype, as the forward takes it (prepare when ry is NULL) */
+  const void *h_out;         /* [T,B,H] in dtype: what the forward call returned (prepare, params) */
+  const void *r;             /* [NH,4*dh,dh] in dtype, the forward's layout (prepare) */
   float *d_r;                /* [NH,4*dh,dh] float32: gradient of r in that layout (params) */
   float *d_bias;             /* [NH,4,dh] float32 (params) */
 } xs_slstm_bwd_args;

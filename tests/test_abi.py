@@ -32,8 +32,8 @@ def test_abi_version_and_struct_mirror():
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
-    # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more, int32 + float
-    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8 + 8
+    # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more, int32 + float, 4 pointers
+    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8 + 8 + 4 * 8
 
 
 def test_backward_argument_errors_without_touching_the_gpu():
@@ -55,10 +55,10 @@ def test_backward_alignment_errors_without_touching_the_gpu():
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = 2, 3, 2, 64, _lib.XS_BF16
     H = 128
-    a.coef, a.wx, a.ry, a.bias = 0x100000, 0x200000, 0x300000, 0x400000
+    a.coef, a.wx, a.r, a.bias, a.h_out = 0x100000, 0x200000, 0x300000, 0x400000, 0x900000
     a.wx_stride_b, a.wx_stride_t = 3 * 4 * H, 4 * H
-    for field, bad in (("wx", 0x200002), ("wx_stride_t", 4 * H + 1), ("wx_stride_b", 3 * 4 * H + 4), ("ry", 0x300008),
-                       ("coef", 0x100004)):
+    for field, bad in (("wx", 0x200002), ("wx_stride_t", 4 * H + 1), ("wx_stride_b", 3 * 4 * H + 4), ("r", 0x300008),
+                       ("h_out", 0x900004), ("coef", 0x100004)):
         keep = getattr(a, field)
         setattr(a, field, bad)
         assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -4, field
@@ -70,6 +70,12 @@ def test_backward_alignment_errors_without_touching_the_gpu():
         keep = getattr(a, field)
         setattr(a, field, bad)
         assert lib.xs_slstm_backward(ctypes.byref(a)) == -4, field
+        setattr(a, field, keep)
+    a.d_r, a.d_bias = 0xA00000, 0xB00000
+    for field, bad in (("d_wx", 0x700004), ("d_wx_stride_t", 4 * H + 2), ("h_out", 0x900008)):
+        keep = getattr(a, field)
+        setattr(a, field, bad)
+        assert lib.xs_slstm_backward_params(ctypes.byref(a)) == -4, field
         setattr(a, field, keep)
 
 

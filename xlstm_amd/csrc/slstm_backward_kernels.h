@@ -7,8 +7,8 @@
 // differentiation (its gradient is written as zero, slstm_pointwise.cu:187-190).
 //
 //   slstm_bwd_prepare_kernel   one thread per (batch row, hidden unit) walks FORWARD through time over
-//                              raw = W.x + R.h_{t-1} + bias (R.h_{t-1} for all steps at once is one batched GEMM over the
-//                              stored outputs, done by the caller) and leaves, per step and element, the nine
+//                              raw = W.x + R.h_{t-1} + bias (R.h_{t-1} from the stored outputs, by MFMA waves of the same
+//                              workgroup a block of steps ahead) and leaves, per step and element, the nine
 //                              coefficients that make the gradient of a step a handful of multiply-adds:
 //                                dc' = dc + dy a0          dn' = dn - dy a1
 //                                d_i = a2 dc' + a3 dn'     d_f = a4 dc' + a5 dn'     d_z = a6 dc'     d_o = a7 dy
@@ -34,7 +34,8 @@ struct BwdPrepParams {
   int B, T, NH, dh;
   const void *wx;            // [B,T,4,NH,dh], strides in elements
   long long wx_sb, wx_st;
-  const float *ry;           // [NH,B,T,dh,4] float32: R.h_{t-1}, the four gates of a unit side by side
+  const void *r;             // [NH, 4 dh, dh] in the type of the operands: R as the forward takes it (K contiguous)
+  const void *h_out;         // [T,B,H] in the type of the operands: the forward's outputs
   const float *bias;         // [NH,4,dh]
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
@@ -57,40 +58,125 @@ __device__ __forceinline__ void bwd_fetch_to_lds_u8(u32x4_t rsrc, uint32_t lds_a
                :: "s"(lds_addr), "v"(voffset), "s"(rsrc) : "memory", "m0");
 }
 
-// One workgroup per (batch row, 64 hidden units): wave 0 walks through time, waves 4 to 6 store what it leaves in LDS
-// (three coefficients each), waves 1 to 3 bring its inputs to LDS -
-// W.x, R.h and the reset flag, one wave each, one load a step - in blocks of kPrepBlock steps, two or three blocks ahead, with
-// loads that write LDS directly and waits written by hand.  With the inputs fetched by the walking wave itself, into
-// registers six steps ahead, the kernel took 0.95 ms at config 2 and 0.36 ms without its loads: a wave has at most
-// 63 memory operations in flight, the nine stores of a step among them, which is four steps' worth of loads against a
-// way to HBM and back of several microseconds, and there is about one such wave per compute unit.
+// One workgroup per (batch row, 64 hidden units), twelve waves:
+//   wave 0        walks through time: lane = unit, the forward's own update with the gate values kept, nine
+//                 coefficients per step into LDS.
+//   wave 1        brings the steps' inputs to an LDS ring - W.x of the slice, the row's output of the step before (the
+//                 operand of R), the reset flag: three loads a step - in blocks of kPrepBlock steps, up to three blocks
+//                 ahead, with loads that write LDS directly and waits written by hand.  (With the inputs fetched by the
+//                 walking wave itself, into registers six steps ahead, the kernel took 0.95 ms at config 2 and 0.36 ms
+//                 without its loads: a wave has at most 63 memory operations in flight, the nine stores of a step among
+//                 them, against a way to HBM and back of several microseconds.)
+//   waves 2, 3    store what the walking wave leaves in LDS (five and four coefficients each), a block behind it: with
+//                 its own nine stores a step in its 63 operations in flight, the acknowledgements of those stores set
+//                 the walking wave's pace.
+//   waves 4 - 11  R.y_{t-1} of the slice's 64 units x 4 gates for the steps of the NEXT block: MFMAs over the outputs in
+//                 the ring (rows that start a document zero; in front of step 0 the y of the initial state) against
+//                 their 32 columns of R, which stay in registers for the whole call; results into the ring, where the
+//                 walking wave finds them next to W.x.  The reference caches the gate values of the forward instead
+//                 (slstm.cc:79-108); an earlier version of this kernel read R.h from a tensor that a library GEMM over
+//                 all steps had written (1 KiB per step and workgroup more to fetch, 0.5 GB at config 2).
 constexpr int kPrepBlock = 8;
-constexpr int bwd_prepare_lds_bytes(bool bf16) {  // the ring of inputs and two blocks of results
-  return (bf16 ? 4 : 3) * kPrepBlock * (4 * 64 * (bf16 ? 2 : 4) + 64 * 16 + 16) + 2 * kPrepBlock * 9 * 64 * 4;
+constexpr int kPrepRing = 4;  // blocks in the ring
+constexpr int kPrepThreads = 768;
+constexpr int bwd_prepare_slot_bytes(bool bf16, int dh) { return 4 * 64 * (bf16 ? 2 : 4) + 64 * 16 + 16 + dh * (bf16 ? 2 : 4); }
+constexpr int bwd_prepare_lds_bytes(bool bf16, int dh) {  // the ring of inputs and two blocks of results
+  return kPrepRing * kPrepBlock * bwd_prepare_slot_bytes(bf16, dh) + 2 * kPrepBlock * 9 * 64 * 4;
 }
-template <bool BF16>
-__global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p) {
+template <bool BF16, int DH>
+__global__ __launch_bounds__(kPrepThreads) void slstm_bwd_prepare_kernel(BwdPrepParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int EPC = 16 / ESZ;               // elements of a 16-byte chunk
   constexpr int WXB = 4 * 64 * ESZ;           // W.x of a step: [4 gates][64 units]
-  constexpr int RYB = 64 * 16;                // R.h of a step: [64 units][4 gates] float32
-  constexpr int SLOT = WXB + RYB + 16;        // ... and the row's reset flag
-  constexpr int NR = BF16 ? 4 : 3;            // blocks in the ring (48 KiB either way): NR - 1 of them ahead
+  constexpr int RYB = 64 * 16;                // R.y of a step: [64 units][4 gates] float32
+  constexpr int HOFF = WXB + RYB + 16;        // ... the row's reset flag, then the operand row: y_{t-1} of the head, DH elements
+  constexpr int SLOT = bwd_prepare_slot_bytes(BF16, DH);
+  constexpr int NR = kPrepRing;
+  constexpr int KSTEPS = DH / (4 * EPC);      // 16-byte chunks of an operand row per lane group
   extern __shared__ __attribute__((aligned(16))) char prep_lds[];
   char *const ring = prep_lds;                                                    // [NR][kPrepBlock] slots of inputs
   float *const outs = reinterpret_cast<float *>(prep_lds + NR * kPrepBlock * SLOT);  // [2][kPrepBlock][9][64]: results
-  const int H = p.NH * p.dh;
+  const int H = p.NH * DH;
   const int slices = H >> 6;
   const int b = blockIdx.x / slices, col0 = (blockIdx.x - b * slices) << 6;
-  const int head = col0 / p.dh, a0 = col0 - head * p.dh;
+  const int head = col0 / DH, a0 = col0 - head * DH;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = (int)uniform((uint32_t)(tid >> 6));
   const int nblocks = (p.T + kPrepBlock - 1) / kPrepBlock;
   const uint32_t ring_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)ring);
+  const long long BH = (long long)p.B * H;
+  // Barriers, the same for every wave: P (block 0's inputs have landed), then barrier k in front of the walking wave's
+  // block k (the MFMA waves have left R.y of block k in the ring, the inputs of block k + 1 have landed), then one
+  // behind the last block.
   if (wave >= 4) {
-    // ---- a storer wave: three of the nine coefficients of every step, a block behind the walking wave (which leaves
-    //      them in LDS: with its own nine stores a step in its 63 operations in flight, the acknowledgements of those
-    //      stores set its pace, 0.66 ms at config 2)
-    const int col = col0 + lane, a = a0 + lane, j0 = 3 * (wave - 4);
+    // ---- an MFMA wave: columns 32 mw .. + 31 of the slice's 256, column c = 4 * unit + gate (the order the walking
+    //      wave reads them in)
+    const int mw = wave - 4, q = lane >> 4, r16 = lane & 15;
+    uint4 rreg[KSTEPS][2];
+#pragma unroll
+    for (int cb = 0; cb < 2; ++cb) {
+      const int c = 32 * mw + 16 * cb + r16;
+      const long long row = (long long)head * 4 * DH + (long long)(c & 3) * DH + a0 + (c >> 2);
+      const char *src = reinterpret_cast<const char *>(p.r) + row * DH * ESZ;
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) rreg[ks][cb] = *reinterpret_cast<const uint4 *>(src + (ks * 4 + q) * 16);
+    }
+    auto block_product = [&](int k) {  // R.y of the steps of block k: rows 0 .. 7 of the MFMA tile, the rest is padding
+      const int t = k * kPrepBlock + (r16 & 7);
+      const char *slot = ring + ((k % NR) * kPrepBlock + (r16 & 7)) * SLOT;
+      bool zero = r16 >= kPrepBlock || t >= p.T;
+      if (p.reset && !zero) zero = (*reinterpret_cast<const uint32_t *>(slot + WXB + RYB) & 0xFFu) != 0u;
+      f32x4 acc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+      for (int ks = 0; ks < KSTEPS; ++ks) {
+        uint4 av = *reinterpret_cast<const uint4 *>(slot + HOFF + (ks * 4 + q) * 16);
+        if (t == 0) {  // in front of the first step: the y of the initial state, rounded as the forward rounds it
+          av = uint4{0u, 0u, 0u, 0u};
+          if (p.s0) {
+            const float *src = p.s0 + (long long)b * H + (long long)head * DH + (ks * 4 + q) * EPC;
+            const float4 lo = *reinterpret_cast<const float4 *>(src);
+            if (BF16) {
+              const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
+              av = uint4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y), pack_bf16x2(hi.z, hi.w)};
+            } else {
+              av = __builtin_bit_cast(uint4, lo);
+            }
+          }
+        }
+        if (zero) av = uint4{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb) {
+          if (BF16) {
+            acc[cb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, rreg[ks][cb]), acc[cb], 0, 0, 0);
+          } else {
+            const uint32_t aw[4] = {av.x, av.y, av.z, av.w}, bw[4] = {rreg[ks][cb].x, rreg[ks][cb].y, rreg[ks][cb].z, rreg[ks][cb].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[cb] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(aw[e]), __uint_as_float(bw[e]), acc[cb], 0, 0, 0);
+          }
+        }
+      }
+      if (q < 2) {  // lane (q, r16) holds steps 4 q .. 4 q + 3 of column r16 of each block of 16 columns
+#pragma unroll
+        for (int cb = 0; cb < 2; ++cb)
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            *reinterpret_cast<float *>(ring + ((k % NR) * kPrepBlock + 4 * q + e) * SLOT + WXB + (32 * mw + 16 * cb + r16) * 4) = acc[cb][e];
+      }
+    };
+    __syncthreads();  // P
+    block_product(0);
+    for (int k = 0; k < nblocks; ++k) {
+      __syncthreads();  // barrier k
+      if (k + 1 < nblocks) block_product(k + 1);
+    }
+    __syncthreads();    // (behind the last block)
+    return;
+  }
+  if (wave >= 2) {
+    // ---- a storer wave: five (wave 2) or four (wave 3) of the nine coefficients of every step, a block behind the
+    //      walking wave
+    const int col = col0 + lane, a = a0 + lane, j0 = wave == 2 ? 0 : 5, nj = wave == 2 ? 5 : 4;
     auto store_block = [&](int k) {
 #pragma unroll
       for (int i = 0; i < kPrepBlock; ++i) {
@@ -99,15 +185,17 @@ __global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p)
         float *dst = p.coef + ((long long)t * p.B + b) * 9 * H + col;
         long long js = H;
         if (p.tiled) {
-          const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (p.dh >> 6) + (a >> 6);
+          const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (DH >> 6) + (a >> 6);
           dst = p.coef + (piece * 16 + (b & 15)) * (9 * 64) + (a & 63);
           js = 64;
         }
         const float *src = outs + (((k & 1) * kPrepBlock + i) * 9 + j0) * 64 + lane;
 #pragma unroll
-        for (int j = 0; j < 3; ++j) dst[(j0 + j) * js] = src[j * 64];
+        for (int j = 0; j < 5; ++j)
+          if (j < nj) dst[(j0 + j) * js] = src[j * 64];
       }
     };
+    __syncthreads();  // P
     for (int k = 0; k < nblocks; ++k) {
       __syncthreads();  // barrier k
       if (k > 0) store_block(k - 1);
@@ -116,30 +204,37 @@ __global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     store_block(nblocks - 1);
     return;
   }
-  if (wave > 0) {
-    // ---- a loader wave.  Block k sits in ring part k % NR; it is asked for behind barrier k - NR + 1 (when the walking
-    //      wave is through with block k - NR, which sat there) and has landed in front of barrier k.
+  if (wave == 1) {
+    // ---- the loader wave.  Block k sits in ring part k % NR; it is asked for behind barrier k - NR + 1 (when the
+    //      walking wave is through with block k - NR, which sat there) and has landed in front of barrier k - 1, when
+    //      the MFMA waves take its operand rows.
     auto descriptor = [&](const void *base, uint32_t bytes) {
       const unsigned long long a = reinterpret_cast<unsigned long long>(base);
       return u32x4_t{uniform((uint32_t)a), uniform((uint32_t)(a >> 32) & 0xFFFFu), bytes, 0x00020000u};
     };
-    auto request_block = [&](int k) {  // eight loads, whatever T is (steps past the end ask for the last step again)
+    constexpr int LPG = 64 * ESZ / 16;        // lanes that cover a gate's 64 units of W.x
+    constexpr int HL = DH * ESZ / 16;         // lanes that cover an operand row (16 .. 64)
+    auto request_block = [&](int k) {  // 3 x 8 loads, whatever T is (steps past the end ask for the last step again)
 #pragma unroll
       for (int i = 0; i < kPrepBlock; ++i) {
         int t = k * kPrepBlock + i;
         t = t < p.T ? t : p.T - 1;
         const uint32_t slot = ring_lds + ((k % NR) * kPrepBlock + i) * SLOT;
-        if (wave == 1) {        // W.x: a gate's 64 units are 128 bytes (bf16: 8 lanes) or 256 (float32: 16 lanes)
-          constexpr int LPG = 64 * ESZ / 16;
+        {  // W.x: a gate's 64 units are 128 bytes (bf16: 8 lanes) or 256 (float32: 16 lanes)
           const char *base = reinterpret_cast<const char *>(p.wx) + ((long long)b * p.wx_sb + (long long)t * p.wx_st + col0) * ESZ;
           const uint32_t voff = (uint32_t)(((long long)(lane / LPG) * H) * ESZ + (lane % LPG) * 16);
           const u32x4_t rs = descriptor(base, (uint32_t)((3ll * H + 64) * ESZ));
           const uint32_t dst = uniform(slot);
           if (lane < 4 * LPG) bwd_fetch_to_lds_b128(rs, dst, voff);  // (only these lanes write LDS)
-        } else if (wave == 2) {  // R.h: the slice's 64 units x 4 gates are 1 KiB in a row
-          const float *base = p.ry + ((((long long)head * p.B + b) * p.T + t) * p.dh + a0) * 4;
-          bwd_fetch_to_lds_b128(descriptor(base, 1024u), uniform(slot + WXB), (uint32_t)lane * 16u);
-        } else {                 // the row's reset flag (lane 0; without a mask: nothing is read, the word is not used)
+        }
+        {  // the operand row: the head's outputs of step t - 1 (step 0: any row, the MFMA waves take the initial state)
+          const int tp = t > 0 ? t - 1 : 0;
+          const char *base = reinterpret_cast<const char *>(p.h_out) + ((long long)tp * BH + (long long)b * H + (long long)head * DH) * ESZ;
+          const u32x4_t rs = descriptor(base, (uint32_t)(DH * ESZ));
+          const uint32_t dst = uniform(slot + HOFF);
+          if (lane < HL) bwd_fetch_to_lds_b128(rs, dst, (uint32_t)lane * 16u);
+        }
+        {  // the row's reset flag (lane 0; without a mask: nothing is read, the word is not used)
           const unsigned char *base = p.reset ? p.reset + (long long)b * p.reset_sb + t : reinterpret_cast<const unsigned char *>(p.wx);
           const u32x4_t rs = descriptor(base, 1u);
           const uint32_t dst = uniform(slot + WXB + RYB);
@@ -149,23 +244,26 @@ __global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     };
     // (blocks past the end are asked for like the others - their steps are the last step again, their ring part is
     // free - so that every wait below is for the same count)
-#pragma unroll
-    for (int j = 0; j < NR - 1; ++j) request_block(j);
+    request_block(0);
+    request_block(1);
+    request_block(2);
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(3 * kPrepBlock * 2) : "memory");  // (block 0 has landed)
+    __syncthreads();  // P
     for (int k = 0; k < nblocks; ++k) {
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(kPrepBlock * (NR - 2)) : "memory");  // (block k has landed)
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(3 * kPrepBlock) : "memory");    // (block k + 1 has landed)
       __syncthreads();  // barrier k: the walking wave is through with block k - 1
       request_block(k + NR - 1);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();    // (the storers' last barrier)
+    __syncthreads();    // (behind the last block)
     return;
   }
   // ---- the walking wave: lane = unit of the slice
-  const int col = col0 + lane, a = a0 + lane;
-  const long long BH = (long long)p.B * H, idx = (long long)b * H + col;
+  const int a = a0 + lane;
+  const long long idx = (long long)b * H + col0 + lane;
   float bias_g[4];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) bias_g[g] = p.bias[((long long)head * 4 + g) * p.dh + a];
+  for (int g = 0; g < 4; ++g) bias_g[g] = p.bias[((long long)head * 4 + g) * DH + a];
   float c = 0.0f, n = 0.0f, m = 0.0f;
   if (p.s0) { c = p.s0[BH + idx]; n = p.s0[2 * BH + idx]; m = p.s0[3 * BH + idx]; }
   const bool has_mask = p.reset != nullptr;
@@ -216,6 +314,7 @@ __global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p)
     out[8 * 64] = fg;
     c = cnew; n = nnew; m = mnew;
   };
+  __syncthreads();  // P
   for (int k = 0; k < nblocks; ++k) {
     __syncthreads();  // barrier k
     StepInputs in[kPrepBlock];
@@ -227,7 +326,7 @@ __global__ __launch_bounds__(448) void slstm_bwd_prepare_kernel(BwdPrepParams p)
       if (t < p.T) one_step(in[i], outs + ((k & 1) * kPrepBlock + i) * 9 * 64 + lane);
     }
   }
-  __syncthreads();  // (the storers' last barrier)
+  __syncthreads();  // (behind the last block)
 }
 
 struct BwdParams {

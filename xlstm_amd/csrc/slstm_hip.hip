@@ -392,26 +392,33 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
   hipStream_t stream = (hipStream_t)a->stream;
   if (prepare) {
-    if (!a->wx || !a->ry || !a->bias) return fail(XS_ERR_NULL, "wx, ry and bias are required");
+    if (!a->wx || !a->r || !a->h_out || !a->bias) return fail(XS_ERR_NULL, "wx, r, h_out and bias are required");
     if (a->wx_stride_t < 4 * H || (a->B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");
-    {  // (W.x and R.h go straight into LDS in pieces of 16 bytes)
+    {  // (W.x and the outputs go straight into LDS in pieces of 16 bytes, R is read in such pieces)
       const long long esz = bf16 ? 2 : 4;
       if (((uintptr_t)a->wx % 16) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16))
         return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
-      if (((uintptr_t)a->ry % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "ry and coef must be 16-byte aligned");
+      if (((uintptr_t)a->r % 16) || ((uintptr_t)a->h_out % 16) || ((uintptr_t)a->s0 % 16) || ((uintptr_t)a->coef % 16))
+        return fail(XS_ERR_ALIGN, "r, h_out, s0 and coef must be 16-byte aligned");
     }
     BwdPrepParams p;
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
-    p.ry = a->ry; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
+    p.r = a->r; p.h_out = a->h_out; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
     p.tiled = a->split ? 1 : 0;
     const long long blocks = (long long)a->B * (H / 64);  // (head dims are multiples of 64 here)
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
-    void (*kp)(BwdPrepParams) = bf16 ? slstm_bwd_prepare_kernel<true> : slstm_bwd_prepare_kernel<false>;
-    const int plds = bwd_prepare_lds_bytes(bf16);
-    if (hipFuncSetAttribute((const void *)kp, hipFuncAttributeMaxDynamicSharedMemorySize, plds) != hipSuccess)
-      return fail(XS_ERR_LAUNCH, "the prepare kernel cannot have %d bytes of LDS", plds);
-    hipLaunchKernelGGL(kp, dim3((unsigned)blocks), dim3(448), plds, stream, p);
+    void (*kp)(BwdPrepParams) = nullptr;
+    switch (a->dh) {
+      case 64: kp = bf16 ? slstm_bwd_prepare_kernel<true, 64> : slstm_bwd_prepare_kernel<false, 64>; break;
+      case 128: kp = bf16 ? slstm_bwd_prepare_kernel<true, 128> : slstm_bwd_prepare_kernel<false, 128>; break;
+      case 256: kp = bf16 ? slstm_bwd_prepare_kernel<true, 256> : slstm_bwd_prepare_kernel<false, 256>; break;
+      default: kp = slstm_bwd_prepare_kernel<true, 512>; break;  // (512 with bf16: checked above)
+    }
+    const int plds = bwd_prepare_lds_bytes(bf16, a->dh);
+    const int rc = ensure_dynamic_lds((const void *)kp, (size_t)plds);
+    if (rc != XS_OK) return rc;
+    hipLaunchKernelGGL(kp, dim3((unsigned)blocks), dim3(kPrepThreads), plds, stream, p);
   } else {
     if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
     if (((uintptr_t)a->r_t % 16)) return fail(XS_ERR_ALIGN, "r_t must be 16-byte aligned");

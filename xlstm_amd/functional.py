@@ -1,5 +1,5 @@
-"""Tensor-level entry points of the HIP engine (torch is used for device memory
-and streams only; all arithmetic happens in the HIP kernels).
+"""Tensor-level entry points of the HIP engine (torch is used for device memory,
+streams and layout changes of the parameters only; all arithmetic happens in the HIP kernels).
 
 Layouts are the external ones of the reference cell:
   wx    [B, S, 4*H]   gate pre-activations, last dim ordered (gate, head, unit)
@@ -83,10 +83,11 @@ def slstm_backward(
     gradient with respect to ``h_out`` and ``d_s_final[4,B,H]`` (optional) with respect to the final state.  Returns
     ``(d_wx[B,S,4H] float32, d_r[NH,4*dh,dh], d_bias[NH,4,dh], d_s0[4,B,H])``.
 
-    Two kernels of the engine (``xs_slstm_backward_prepare``, ``xs_slstm_backward``) around three plain library GEMMs and
-    a reduction: ``R.h_{t-1}`` for all steps at once in front, and the gradients of R and the bias, which are sums over
-    all steps of products of the gate deltas with the outputs, behind.  ``timings`` (a dict) receives three events around
-    the two kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
+    Three kernels of the engine: ``xs_slstm_backward_prepare`` (a forward walk over the stored outputs that leaves nine
+    coefficients per step and element), ``xs_slstm_backward`` (the reverse pass) and ``xs_slstm_backward_params`` (the
+    gradients of R and the bias, sums over all steps of products of the gate deltas with the outputs); what torch does
+    here is allocating the buffers and bringing R into the kernels' operand order.  ``timings`` (a dict) receives four
+    events around the three kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
@@ -159,27 +160,11 @@ def slstm_backward(
         s0 = s0.to(torch.float32).contiguous()
     if reset_mask is not None:
         reset_mask = (reset_mask != 0).to(torch.uint8).contiguous()
-    # the operand of every step as the forward saw it: y_{t-1} (the initial y in front), rows that start a document zero,
-    # in the type of the forward's operands (h_out is), batch-major like d_wx: the two meet in the product for d_r
-    y_prev = torch.empty((B, T, H), dtype=wx.dtype, device=dev)
-    y_prev[:, 0] = s0[0] if s0 is not None else 0.0
-    if T > 1:
-        y_prev[:, 1:] = h_out[:-1].transpose(0, 1)
-    if reset_mask is not None:
-        y_prev.masked_fill_(reset_mask.bool().unsqueeze(-1), 0.0)
     r32 = r.to(torch.float32)
-    yp = y_prev.float().view(B * T, NH, dh).transpose(0, 1)               # [NH, B*T, dh]
-
-    def by_unit(rr):  # rows of R ordered (unit, gate): the four gate values of a unit end up side by side in R.h
-        return rr.view(NH, 4, dh, dh).transpose(1, 2).reshape(NH, 4 * dh, dh)
-
     if bf16:
-        # the forward's own product: bf16 operands, float32 sums (0.18 against 0.66 ms at config 2 for the float32 one)
-        r16 = r32.bfloat16()
-        r32 = r16.float()
-        ry = torch.bmm(y_prev.view(B * T, NH, dh).transpose(0, 1), by_unit(r16).transpose(1, 2), out_dtype=torch.float32)
-    else:
-        ry = torch.bmm(yp, by_unit(r32).transpose(1, 2))                  # [NH, B*T, 4*dh] = [NH,B,T,dh,4]
+        r32 = r32.bfloat16().float()  # (the forward rounds R to bf16)
+    r_fwd = r32.to(wx.dtype).contiguous()  # R as the forward multiplies by it: the prepare kernel recomputes R.y_{t-1} from it
+    h_c = h_out if h_out.is_contiguous() and h_out.dtype == wx.dtype else h_out.to(wx.dtype).contiguous()
     d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
     d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
     epc = 8 if bf16 else 4
@@ -214,7 +199,8 @@ def slstm_backward(
     a.dtype = _DTYPE_CODE[wx.dtype]
     a.wx = wx.data_ptr()
     a.wx_stride_b, a.wx_stride_t = wx.stride(0), wx.stride(1)
-    a.ry = ry.data_ptr()
+    a.ry = None
+    a.r, a.h_out = r_fwd.data_ptr(), h_c.data_ptr()
     a.bias = bias.data_ptr()
     a.s0 = s0.data_ptr() if s0 is not None else None
     a.reset = reset_mask.data_ptr() if reset_mask is not None else None
@@ -250,8 +236,7 @@ def slstm_backward(
         # engine's third backward kernel, from d_wx as it lies and the forward's outputs
         d_r = torch.empty((NH, 4 * dh, dh), dtype=torch.float32, device=dev)
         d_bias = torch.empty((NH, 4, dh), dtype=torch.float32, device=dev)
-        h_c = h_out if h_out.is_contiguous() and h_out.dtype == wx.dtype else h_out.to(wx.dtype).contiguous()
-        a.h_out, a.d_r, a.d_bias = h_c.data_ptr(), d_r.data_ptr(), d_bias.data_ptr()
+        a.d_r, a.d_bias = d_r.data_ptr(), d_bias.data_ptr()
         rc = lib.xs_slstm_backward_params(ctypes.byref(a))
         if rc != 0:
             raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
