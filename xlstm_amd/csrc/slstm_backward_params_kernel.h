@@ -85,7 +85,7 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
   const bool y_thread = tid < kParamKC * NROWTHREADS;  // (NT 64: 256 threads cover the chunk)
   float bsum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
 
-  struct Staged { float4 d[2]; uint4 y[YPASS < 1 ? 1 : YPASS][BF16 ? 1 : 2]; };
+  struct Staged { float4 d[2]; uint4 y[YPASS < 1 ? 1 : YPASS][BF16 ? 1 : 2]; uint32_t flag[YPASS < 1 ? 1 : YPASS]; };
   auto fetch = [&](long long c, Staged &s) {
     const int b = (int)(c / p.tchunks), t0 = (int)(c % p.tchunks) * kParamKC;
     {  // delta
@@ -102,8 +102,10 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
       const int t = t0 + yk + ps * (512 / NROWTHREADS);
 #pragma unroll
       for (int e = 0; e < (BF16 ? 1 : 2); ++e) s.y[ps][e] = uint4{0u, 0u, 0u, 0u};
+      s.flag[ps] = 0u;
       if (!y_thread || t >= p.T) continue;
-      if (p.reset && p.reset[(long long)b * p.reset_sb + t]) continue;  // a row that starts a document: the operand was zero
+      // (the flag is looked at when the chunk is staged: a test here would wait for every load issued so far)
+      if (p.reset) s.flag[ps] = p.reset[(long long)b * p.reset_sb + t];
       const long long col = (long long)head * dh + n0 + yn;
       if (t == 0) {
         if (!p.s0) continue;
@@ -140,12 +142,14 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
 #pragma unroll
       for (int ps = 0; ps < (YPASS < 1 ? 1 : YPASS); ++ps) {
         elem_t *bdst = Bs + ((long long)buf * kParamKC + yk + ps * (512 / NROWTHREADS)) * LDB + yn;
+        const bool keep = s.flag[ps] == 0u;  // (a row that starts a document at this step: the forward's operand was zero)
+        const uint4 y0 = keep ? s.y[ps][0] : uint4{0u, 0u, 0u, 0u};
         if (BF16) {
-          *reinterpret_cast<uint2 *>(bdst) = uint2{s.y[ps][0].x, s.y[ps][0].y};
-          *reinterpret_cast<uint2 *>(bdst + 4) = uint2{s.y[ps][0].z, s.y[ps][0].w};
+          *reinterpret_cast<uint2 *>(bdst) = uint2{y0.x, y0.y};
+          *reinterpret_cast<uint2 *>(bdst + 4) = uint2{y0.z, y0.w};
         } else {
-          *reinterpret_cast<uint4 *>(bdst) = s.y[ps][0];
-          *reinterpret_cast<uint4 *>(bdst + 4) = s.y[ps][BF16 ? 0 : 1];
+          *reinterpret_cast<uint4 *>(bdst) = y0;
+          *reinterpret_cast<uint4 *>(bdst + 4) = keep ? s.y[ps][BF16 ? 0 : 1] : uint4{0u, 0u, 0u, 0u};
         }
       }
     }
@@ -159,16 +163,10 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
   const int am = wm * (MTILES * 16) + r16;   // this lane's row of an A fragment inside the workgroup's 128 (+ 16 per tile)
   const int bn = wn * 64 + r16;              // ... column of a B fragment (+ 16 per tile)
 
-  Staged st;
-  if (c_lo < c_hi) {
-    fetch(c_lo, st);
-    stage(st, 0);
-  }
-  __syncthreads();
-  for (long long c = c_lo; c < c_hi; ++c) {
-    const int buf = (int)((c - c_lo) & 1);
-    const bool more = c + 1 < c_hi;
-    if (more) fetch(c + 1, st);  // (in flight under the MFMAs below)
+  // Two chunks are in flight beyond the one in LDS (two sets of staging registers, used in turn): with one, every
+  // chunk cost a whole memory latency (0.36 ms at B 16 x T 2048 x D 1024; 64 KiB a compute unit in flight are what
+  // keeps the memory system busy)
+  auto compute = [&](int buf) {
     const elem_t *A = As + (long long)buf * kParamKC * LDA, *Bm = Bs + (long long)buf * kParamKC * LDB;
     if constexpr (BF16) {
       // one MFMA k-step = the whole chunk: lane group q takes k = 8 q .. 8 q + 7
@@ -203,8 +201,24 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
           for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[i], bf[j], acc[i][j], 0, 0, 0);
       }
     }
-    if (more) stage(st, buf ^ 1);  // (the other buffer: everybody left it before the barrier that opened this chunk)
+  };
+  Staged sa, sb;
+  if (c_lo < c_hi) {
+    fetch(c_lo, sa);
+    if (c_lo + 1 < c_hi) fetch(c_lo + 1, sb);
+    stage(sa, 0);
+    if (c_lo + 2 < c_hi) fetch(c_lo + 2, sa);
+  }
+  __syncthreads();
+  auto iteration = [&](long long c, Staged &next, int buf) {  // `next` holds chunk c + 1 and is refilled with chunk c + 3
+    compute(buf);
+    if (c + 1 < c_hi) stage(next, buf ^ 1);  // (the other buffer: everybody left it before the barrier that opened this chunk)
+    if (c + 3 < c_hi) fetch(c + 3, next);
     __syncthreads();
+  };
+  for (long long c = c_lo; c < c_hi; c += 2) {
+    iteration(c, sb, 0);
+    if (c + 1 < c_hi) iteration(c + 1, sa, 1);
   }
 
   // ---- the slice's share of d_r: lane (q, r16) holds rows 4 q .. 4 q + 3, column r16 of every 16 x 16 tile

@@ -459,8 +459,10 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       else if (a->dh == 256) { ks = slstm_bwd_split_kernel<false, 4, false>; feed = false; }
       else { ks = slstm_bwd_split_kernel<true, 8, false>; feed = false; }
       const int lds = bwd_split_lds_bytes(feed, bf16);
-      if (hipFuncSetAttribute((const void *)ks, hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
-        return fail(XS_ERR_LAUNCH, "the split backward kernel cannot have %d bytes of LDS", lds);
+      {
+        const int rc = ensure_dynamic_lds((const void *)ks, (size_t)lds);
+        if (rc != XS_OK) return rc;
+      }
       hipLaunchKernelGGL(ks, dim3((unsigned)(grid + (prefetchers ? 8 : 0))), dim3(feed ? 768 : 512), lds, stream, q);
       const hipError_t es = hipGetLastError();
       if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
@@ -483,8 +485,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     const int esz = bf16 ? 2 : 4;
     const size_t lds = (size_t)16 * (4 * a->dh + 16 / esz) * esz;  // the delta tile
     if (lds > 64 * 1024) {
-      const hipError_t ea = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      if (ea != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel: %zu bytes of LDS refused: %s", lds, hipGetErrorString(ea));
+      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), lds);
+      if (rc != XS_OK) return rc;
     }
     const long long blocks = (long long)a->NH * ((a->B + 15) / 16);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(waves * 64), lds, stream, p);
