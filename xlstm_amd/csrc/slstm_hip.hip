@@ -321,6 +321,11 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
     else
       kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
                   : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
+    // row tiles of at most 4 rows, bf16, whole K ranges up to 512: the compute waves split the columns by unit, not K
+    if (bf16 && MT == 1 && rows_per_wg == 4 && full && nch <= 4 && G <= 32) {
+      kern = nch == 1 ? slstm_seq_kernel<true, 1, 1, true, false, false, true>
+                      : (nch == 2 ? slstm_seq_kernel<true, 2, 1, true, false, false, true> : slstm_seq_kernel<true, 4, 1, true, false, false, true>);
+    }
 #ifdef XS_SMALL_BATCH_FMA
     // the measured alternative for small batches (see the kernel): only in a library built for that measurement
     if (MT == 1 && rows_per_wg == 4 && nch <= 2 && full) {

@@ -153,9 +153,12 @@ __device__ __forceinline__ uint32_t seq_handshake(const SeqParams &p, int wg, in
 // 4 (fp32) inputs of every real row - fetched from the lane that holds them - into its own column's weights, and
 // the four lane groups' partial sums over K are added with two cross-lane steps.  The sums are formed in a different
 // order than the MFMA forms them, so the bits differ from the MFMA path (and from the decode kernel).
-template <bool BF16, int NCH, int MT, bool FULL, bool BURST, bool FMAC = false>
+// QUAD: row tiles of at most 4 rows (bf16, FULL, one row tile): the four compute waves split the workgroup's 64
+// columns by UNIT instead of splitting K, see "waves 0-3, QUAD" below.
+template <bool BF16, int NCH, int MT, bool FULL, bool BURST, bool FMAC = false, bool QUAD = false>
 __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
   static_assert(!FMAC || MT == 1, "the FMA contraction is for one row tile of at most 4 rows");
+  static_assert(!QUAD || (BF16 && MT == 1 && FULL && !BURST && !FMAC), "the unit-split compute waves exist for bf16, one full row tile");
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
   constexpr int KW = NCH * 4 * EPC;      // input units per wave
   constexpr int ESZ = BF16 ? 2 : 4;
@@ -409,6 +412,188 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     }
     __builtin_amdgcn_s_barrier();  // final barrier
     asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(sink));
+    return;
+  }
+
+  // =========================================================================
+  // waves 0-3, QUAD: row tiles of at most 4 rows.  With K split over the four waves (below), a step's chain runs
+  // through LDS: partial tiles out, a barrier, sixteen partial values back in and added up, and only one of the four
+  // waves gates real rows.  Here wave w owns units 4 w .. 4 w + 3 of the workgroup's 16 with all four gates (16
+  // columns) and the WHOLE of K: it polls the whole h tile of the group (4 rows x dh, 16 bytes per lane from the 16
+  // lanes whose MFMA row is a real one), multiplies, and gates its own 16 elements; nothing crosses between the waves.
+  // The batch rows sit at MFMA rows 0, 4, 8, 12, so the sum of (row b, column n) arrives in lane group b, lane n, and
+  // the four gates of a unit meet in the unit's lane through three row shifts (no LDS).  K is accumulated in the same
+  // four quarters and folded in the same order as everywhere else: the same bits.  The barrier of the step (the
+  // feeder's W.x, the drainer's h) is passed in front of the poll.  The exchange ring is [slot][member][4 rows]
+  // [16 units]: the group's h of a step is 8 dh bytes in a row.
+  // =========================================================================
+  if constexpr (QUAD) {
+    __builtin_amdgcn_s_setprio(3);
+    constexpr int NK = 4 * NCH;                // MFMA k-steps over the head dim (dh = 32 NK)
+    const int q = lane >> 4, r16 = lane & 15;
+    uint4 rreg[NK];
+    {
+      const int a = a0 + 4 * wave + (r16 & 3);
+      const long long rowoff = ((long long)head * 4 * dh + (long long)(r16 >> 2) * dh + a) * dh;
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks) {
+        const long long off = rowoff + ks * 32 + q * 8;
+        if (p.r_bf16) {
+          rreg[ks] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const uint16_t *>(p.r) + off);
+        } else {
+          const float4 lo = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.r) + off);
+          const float4 hi = *reinterpret_cast<const float4 *>(reinterpret_cast<const float *>(p.r) + off + 4);
+          rreg[ks] = uint4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y), pack_bf16x2(hi.z, hi.w)};
+        }
+      }
+    }
+    // gating role: lane group = batch row of the tile, lanes 0-3 of the group = the wave's four units
+    const int gb = q, gu = 4 * wave + (r16 & 3);
+    const bool gate_lane = r16 < 4;
+    const int ua = a0 + gu, col = head * dh + ua;
+    const int brow = rowbase + gb;
+    float bias_g[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) bias_g[g] = p.bias[((long long)head * 4 + g) * dh + ua];
+    CellState st{0.0f, 0.0f, 0.0f, 0.0f};
+    if (p.s0 && brow < rend) {
+      const long long o = (long long)brow * H + col;
+      st.y = p.s0[o]; st.c = p.s0[BH + o]; st.n = p.s0[2 * BH + o]; st.m = p.s0[3 * BH + o];
+    }
+    bool aborted = false;
+    uint32_t max_spins = 0;
+    lds_barrier();  // prologue barrier
+    const bool cross = cross_s != 0u;
+    constexpr int QTILE = 4 * 16 * 2;          // bytes a member publishes per step
+    const int xslot = p.G * QTILE;
+    char *const xbase = reinterpret_cast<char *>(p.xbuf) + (long long)gi * kRing * xslot;
+    // operand: MFMA row r16 is batch row r16 / 4 when r16 % 4 == 0, nothing otherwise; k-step ks, lane group q: units
+    // 32 ks + 8 q .. + 7 = member 2 ks + q / 2, its units 8 (q % 2) .. + 7
+    const int arow = rowbase + (r16 >> 2);
+    const bool a_lane = (r16 & 3) == 0 && arow < rend;
+    const int xl = a_lane ? (q >> 1) * QTILE + (r16 >> 2) * 32 + (q & 1) * 16 : 0x7FFFFF00;
+    const long long xo = (long long)member * (QTILE / 2) + gb * 16 + gu;
+#ifndef XS_QUAD_PAD
+#define XS_QUAD_PAD 2
+#endif
+    asm volatile(".p2align 5\n\t.rept %0\n\ts_nop 0\n\t.endr" :: "n"(XS_QUAD_PAD));
+    for (int t = 0; t < p.T; ++t) {
+      const __amdgpu_buffer_rsrc_t hrs = __builtin_amdgcn_make_buffer_rsrc(xbase + ((t + kRing - 1) % kRing) * xslot, 0, xslot, 0x00020000);
+      uint16_t *const hcur = reinterpret_cast<uint16_t *>(xbase + (t % kRing) * xslot);
+      uint16_t *const hold = reinterpret_cast<uint16_t *>(xbase + ((t + kRing - 2) % kRing) * xslot);
+      uint4 areg[NK];
+      // The step's barrier and what the gating needs from LDS come FIRST, then a pause of 64 cycles, then the poll:
+      // whatever stands between the poll's return and the MFMAs is on the chain, and a poll that leaves the moment
+      // the workgroup has published finds the peers' words unwritten and has to go round again.  Measured at B 16 x
+      // T 2048 x 4 heads of 256 (ms per call): barrier and LDS reads under the poll 1.81, in front of it 1.63, with
+      // the pause 1.51 (twice as long: 1.53, four times: 1.66); then the loop's start moved over the eight phases of a
+      // 32-byte line of code: 1.485 .. 1.557, the best one taken.  (K split over the waves, below: 1.70.)
+      const int buf = t & 1;
+      float wxv[4];
+      lds_barrier();  // barrier #t: W.x of this step is in LDS, the h of two steps ago has been drained
+#pragma unroll
+      for (int g = 0; g < 4; ++g) wxv[g] = wxs[buf][g][gb * kTileStride + gu];
+      const bool row_reset = rfl[t & 3][r16 >> 2] != 0u;   // (the operand's row: it contributes R.0 = 0 exactly)
+      const bool gate_reset = rfl[t & 3][gb] != 0u;
+#ifndef XS_QUAD_SLEEP
+#define XS_QUAD_SLEEP 1
+#endif
+      if (XS_QUAD_SLEEP > 0) __builtin_amdgcn_s_sleep(XS_QUAD_SLEEP);
+      if (t > 0) {
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks)
+          areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, ks * 2 * QTILE, 16));
+      } else {
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks) {
+          areg[ks] = make_uint4(0, 0, 0, 0);
+          if (a_lane && p.s0) {
+            const float *src = p.s0 + (long long)arow * H + head * dh + ks * 32 + q * 8;
+            const float4 lo = *reinterpret_cast<const float4 *>(src);
+            const float4 hi = *reinterpret_cast<const float4 *>(src + 4);
+            areg[ks] = uint4{pack_bf16x2(lo.x, lo.y), pack_bf16x2(lo.z, lo.w), pack_bf16x2(hi.x, hi.y), pack_bf16x2(hi.z, hi.w)};
+          }
+        }
+      }
+      if (t > 0 && !aborted) {
+        uint32_t spins = 0;
+        for (;;) {
+          uint32_t ma = 0u;
+#pragma unroll
+          for (int ks = 0; ks < NK; ++ks) ma = mark_join<true>(ma, chunk_mark<true>(areg[ks]));
+          if (__builtin_amdgcn_ballot_w64(mark_has_sentinel<true>(ma)) == 0ull) break;
+#pragma unroll
+          for (int ks = 0; ks < NK; ++ks)
+            areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, ks * 2 * QTILE, 16));
+          spins += 1;
+          if ((spins & 1023u) == 0u && __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) {
+            aborted = true;
+            break;
+          }
+          if ((long long)spins >= spin_limit) {
+            aborted = true;
+            if (atomicExch(&p.status->aborted, 1u) == 0u) {
+              p.status->abort_wg = (uint32_t)wg;
+              p.status->abort_step = (uint32_t)t;
+            }
+            break;
+          }
+        }
+        max_spins = spins > max_spins ? spins : max_spins;
+      }
+      if (__builtin_amdgcn_ballot_w64(row_reset) != 0ull) {
+#pragma unroll
+        for (int ks = 0; ks < NK; ++ks)
+          if (row_reset) areg[ks] = make_uint4(0, 0, 0, 0);
+      }
+      // the four quarters of K, each its own chain from zero, folded in the order of the other kernels' waves
+      f32x4 acc[4];
+#pragma unroll
+      for (int w4 = 0; w4 < 4; ++w4) acc[w4] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int c = 0; c < NCH; ++c)
+#pragma unroll
+        for (int w4 = 0; w4 < 4; ++w4)
+          acc[w4] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, areg[w4 * NCH + c]),
+                                                            __builtin_bit_cast(bf16x8, rreg[w4 * NCH + c]), acc[w4], 0, 0, 0);
+      float mine = acc[0][0];
+      mine += acc[1][0];
+      mine += acc[2][0];
+      mine += acc[3][0];
+      // lane (row, gate g, unit u) -> the unit's lane (row, 0, u): lanes 4, 8, 12 further on in the row of 16
+      const int mi = __float_as_int(mine);
+      const float ry1 = __int_as_float(__builtin_amdgcn_update_dpp(0, mi, 0x104, 0xF, 0xF, true));  // row_shl:4
+      const float ry2 = __int_as_float(__builtin_amdgcn_update_dpp(0, mi, 0x108, 0xF, 0xF, true));  // row_shl:8
+      const float ry3 = __int_as_float(__builtin_amdgcn_update_dpp(0, mi, 0x10C, 0xF, 0xF, true));  // row_shl:12
+      const float raw0 = (wxv[0] + mine) + bias_g[0], raw1 = (wxv[1] + ry1) + bias_g[1];
+      const float raw2 = (wxv[2] + ry2) + bias_g[2], raw3 = (wxv[3] + ry3) + bias_g[3];
+      if (gate_reset) st = CellState{0.0f, 0.0f, 0.0f, 0.0f};
+      slstm_pointwise(raw0, raw1, raw2, raw3, st);
+      const float y = st.y;
+      if (gate_lane) {
+        const uint16_t v = (uint16_t)float_to_bf16_bits(y);
+        if (cross) {
+          __hip_atomic_store(hcur + xo, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(hold + xo, (uint16_t)kSentinel16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        } else {
+          hcur[xo] = v;
+          hold[xo] = (uint16_t)kSentinel16;
+        }
+        hst[t & 3][gb * 16 + gu] = y;
+      }
+#pragma unroll
+      for (int ks = 0; ks < NK; ++ks)  // (the operand registers stay reserved to the end of the iteration)
+        asm volatile("" :: "v"(areg[ks].x), "v"(areg[ks].y), "v"(areg[ks].z), "v"(areg[ks].w));
+    }
+    for (int j = NIT; j < NITpad; ++j) lds_barrier();  // padding iterations of the feeder
+    lds_barrier();                                     // final barrier
+    const bool poisoned = __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
+    if (gate_lane && brow < rend) {
+      const long long o = (long long)brow * H + col;
+      if (poisoned) st = CellState{kPoison, kPoison, kPoison, kPoison};
+      p.s_out[o] = st.y; p.s_out[BH + o] = st.c; p.s_out[2 * BH + o] = st.n; p.s_out[3 * BH + o] = st.m;
+    }
+    if (lane == 0 && max_spins) atomicMax(&p.status->max_spins, max_spins);
     return;
   }
 
