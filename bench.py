@@ -219,7 +219,7 @@ def measure_stage(device, stage, steps, members=16, two_xcds=0, rows=4, reps=5):
 def serial_bound(device):
     """The dependency chain of one timestep, measured by ``xs_measure_stage`` (the product kernel's instructions, layouts
     and exchange protocol; every iteration needs the result of the one before).  ``config2_chain``: the whole chain as
-    one loop - poll, MFMAs, sums through LDS and the barrier, gating, publication - on 16 head groups of 16 compute
+    one loop - barrier, poll, MFMAs, fold and row shifts, gating, publication - on 16 head groups of 16 compute
     units, with none of the product kernel's other work: the serial bound of a step of this structure.  The stages alone
     (each its own loop, so their sum is more than the chain: every loop pays its own entry and waits) say where it
     goes.  Per-iteration times are differences between two step counts, so launches and set-up cancel.  Also the floor
@@ -238,7 +238,7 @@ def serial_bound(device):
     ex32 = per_step(_lib.STAGE_EXCHANGE, n=5000, members=32, rows=16)
     launch = per_step(_lib.STAGE_LAUNCH, n=2000)
     return {"config2_chain_us_per_step": chain,
-            "stages_alone_us": {"exchange_16_units_one_xcd_4_rows": ex16, "mfma_and_lds_reduction": mm, "gating": ga},
+            "stages_alone_us": {"exchange_16_units_one_xcd_4_rows": ex16, "mfma_fold_and_row_shifts": mm, "gating": ga},
             "exchange_32_units_one_xcd_16_rows_us": ex32, "exchange_64_units_two_xcds_16_rows_us": ex64,
             "dependent_launch_us": launch}
 
@@ -665,7 +665,7 @@ def main():
                    "tokens_per_step": B * T},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,BURST=0>", "kernel_ms": kern_ms,
+                     "kernel": "slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,BURST=0,FMAC=0,QUAD=1>", "kernel_ms": kern_ms,
                      "algorithmic_bytes_per_launch": nbytes, "us_per_timestep": kern_ms * 1e3 / T,
                      "max_poll_rounds": status["max_spins"],
                      "tflops": 8.0 * B * T * NH * dh * dh / (kern_ms * 1e-3) / 1e12},

@@ -342,11 +342,14 @@ int xs_slstm_backward_params(const xs_slstm_bwd_args *args);
  *                         and 4 with device-scope stores) publish a 16 x 16 bf16 tile each and poll the group's tile of
  *                         `rows` batch rows until it is complete.  Workspace: 256 + 8 * members * 512 bytes; word 0 is
  *                         nonzero afterwards if a wait ran out (other work held compute units), word 1 the longest wait.
- *   XS_STAGE_CONTRACTION  one workgroup: 4 waves x 4 gates x 2 MFMAs (head dim 256), partial sums through LDS, barrier.
+ *                         With rows <= 4 inside one XCD: the layout of the kernel for such tiles, every wave polls the
+ *                         whole tile.
+ *   XS_STAGE_CONTRACTION  one workgroup: a wave's 8 MFMAs over K = 256 in four chains, their fold, the three row shifts
+ *                         that bring a unit's four gates together.
  *   XS_STAGE_GATING       one workgroup: the exponential gating of one element per lane, y rounded to bf16.
  *   XS_STAGE_LAUNCH       `steps` launches of an empty kernel, back to back: the floor of a dependent launch.
- *   XS_STAGE_CHAIN        the three stages as ONE loop in the product kernel's order (poll, MFMAs, sums through LDS and
- *                         the barrier, gating, publication) on head groups of 16 compute units placed as the product places
+ *   XS_STAGE_CHAIN        the three stages as ONE loop in the order of the kernel for tiles of 4 rows (barrier, pause,
+ *                         poll, MFMAs, fold, row shifts, gating, publication) on head groups of 16 compute units placed as the product places
  *                         them, as many as the device holds, tiles of `rows` batch rows; constant W.x, no mask, no output
  *                         tensor, none of the product kernel's other waves: what a step costs when only the chain is
  *                         left.  Workspace: 256 + (compute units / 16) * 8 * 16 * 512 bytes; words 0 and 1 as above.

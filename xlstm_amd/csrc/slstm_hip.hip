@@ -719,6 +719,9 @@ int run_stage(const xs_measure_args *a) {
       hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, stream, (uint32_t *)a->workspace, (size_t)64, 0u);
       hipLaunchKernelGGL(fill_u32_kernel, dim3(64), dim3(256), 0, stream, (uint32_t *)p.ring, ring / 4, kSentinel32);
       void (*k)(StageParams) = G == 8 ? stage_exchange_kernel<1> : (G == 16 ? stage_exchange_kernel<2> : (G == 32 ? stage_exchange_kernel<4> : stage_exchange_kernel<8>));
+      // tiles of at most 4 rows inside one XCD: the layout and the polls of the kernel for such tiles
+      if (a->rows <= 4 && !a->two_xcds && G <= 32)
+        k = G == 8 ? stage_exchange_quad_kernel<4> : (G == 16 ? stage_exchange_quad_kernel<8> : stage_exchange_quad_kernel<16>);
       hipLaunchKernelGGL(k, dim3(8 * per_xcd), dim3(256), 0, stream, p);
     } else if (a->stage == XS_STAGE_CHAIN) {
       const int G = 16;  // (head dim 256)

@@ -474,7 +474,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     const int xl = a_lane ? (q >> 1) * QTILE + (r16 >> 2) * 32 + (q & 1) * 16 : 0x7FFFFF00;
     const long long xo = (long long)member * (QTILE / 2) + gb * 16 + gu;
 #ifndef XS_QUAD_PAD
-#define XS_QUAD_PAD 2
+#define XS_QUAD_PAD 4
 #endif
     asm volatile(".p2align 5\n\t.rept %0\n\ts_nop 0\n\t.endr" :: "n"(XS_QUAD_PAD));
     for (int t = 0; t < p.T; ++t) {
@@ -482,12 +482,15 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       uint16_t *const hcur = reinterpret_cast<uint16_t *>(xbase + (t % kRing) * xslot);
       uint16_t *const hold = reinterpret_cast<uint16_t *>(xbase + ((t + kRing - 2) % kRing) * xslot);
       uint4 areg[NK];
-      // The step's barrier and what the gating needs from LDS come FIRST, then a pause of 64 cycles, then the poll:
-      // whatever stands between the poll's return and the MFMAs is on the chain, and a poll that leaves the moment
-      // the workgroup has published finds the peers' words unwritten and has to go round again.  Measured at B 16 x
-      // T 2048 x 4 heads of 256 (ms per call): barrier and LDS reads under the poll 1.81, in front of it 1.63, with
-      // the pause 1.51 (twice as long: 1.53, four times: 1.66); then the loop's start moved over the eight phases of a
-      // 32-byte line of code: 1.485 .. 1.557, the best one taken.  (K split over the waves, below: 1.70.)
+      // The step's barrier and what the gating needs from LDS come FIRST, then one s_sleep, then the poll: whatever
+      // stands between the poll's return and the MFMAs is on the chain.  Measured at B 16 x T 2048 x 4 heads of 256 (ms
+      // per call): barrier and LDS reads under the poll 1.81, in front of it 1.63, with the s_sleep 1.52 (two of
+      // them 1.53 - 1.57, four 1.66).  What the s_sleep gives is not the delay - the same cycles spent in s_nop cost
+      // instead (32 cycles 1.61, 64 1.69, 128 1.91), and it does as well behind the poll's issue or in front of the
+      // barrier (1.52 - 1.53) - but the issue slots: a wave asleep leaves its SIMD to the feeder, drainer and prefetch
+      // waves, which these waves' raised priority otherwise keeps waiting (no s_sleep but priority 0 from the barrier
+      // to the poll: 1.53).  Then the loop's start moved over the eight phases of a 32-byte line of code:
+      // 1.517 .. 1.573, the best one taken.  (K split over the waves, below: 1.70.)
       const int buf = t & 1;
       float wxv[4];
       lds_barrier();  // barrier #t: W.x of this step is in LDS, the h of two steps ago has been drained
@@ -499,6 +502,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #define XS_QUAD_SLEEP 1
 #endif
       if (XS_QUAD_SLEEP > 0) __builtin_amdgcn_s_sleep(XS_QUAD_SLEEP);
+      asm volatile("");  // (the compiler keeps what stands in front of this statement in front of the poll)
       if (t > 0) {
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks)
