@@ -387,12 +387,12 @@ def phase_profile(device):
     # config 2: slstm_seq_kernel, one row tile of 4 rows; per timestep
     T = 2048
     st, ms = run(16, T, 4, 256, 512)
-    names = ["poll (request to complete operand)", "mfma + partial sums to LDS", "barrier", "LDS sum + gating",
-             "publish + stage h", "loop top"]
-    out["config 2 (slstm_seq_kernel<bf16,NCH=2,MT=1,FULL>), cycles per timestep, workgroup 0"] = {
+    names = {5: "loop top", 2: "barrier", 1: "W.x and flags out of LDS + s_sleep", 0: "poll (request to complete operand)",
+             7: "8 MFMAs + fold + row shifts", 3: "exponential gating", 4: "publish + re-arm + stage h"}
+    out["config 2 (slstm_seq_kernel<bf16,NCH=2,MT=1,FULL,QUAD>), cycles per timestep, workgroup 0"] = {
         "ms_per_call_with_stamps": ms,
-        "compute waves 0-3": {n: [round(float(st[w][i] / T)) for w in range(4)] for i, n in enumerate(names)},
-        "compute waves: sum": [round(float(st[w][:6].sum() / T)) for w in range(4)],
+        "compute waves 0-3": {n: [round(float(st[w][i] / T)) for w in range(4)] for i, n in names.items()},
+        "compute waves: sum": [round(float((st[w][:6].sum() + st[w][7]) / T)) for w in range(4)],
         "compute waves: polls repeated per step": [round(float(st[w][6] / T), 2) for w in range(4)],
         "feeder wave": {"W.x into LDS": round(float(st[4][0] / T)), "issue": round(float(st[4][1] / T)),
                         "barrier": round(float(st[4][2] / T))},

@@ -349,3 +349,76 @@ def test_cell_config_gradient_recurrent_cut_and_clipval():
         assert all(v <= 1e-5 for v in errs.values()), errs
     with pytest.raises(NotImplementedError, match="gradient_recurrent_clipval"):
         sLSTMCell(sLSTMCellConfig(hidden_size=H, num_heads=NH, backend="hip", gradient_recurrent_clipval=0.5))
+
+
+@pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (True, 16, 12, 4, 256, True), (False, 4, 10, 2, 128, False)])
+def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
+    """A caller without torch arithmetic - the binding a maintainer would put in place of the reference's
+    ``sLSTMFunc.backward`` (slstm.cc:137-221, which returns {dx, ds0, dR, db} from one native call): forward, then the
+    three backward entry points, through ctypes with buffers the caller owns; the recurrent matrix is brought into the
+    reverse kernel's operand order with numpy on the host.  All four gradients against the oracle."""
+    import ctypes
+
+    from xlstm_amd import _lib
+    from xlstm_amd import functional as F
+
+    lib = _lib.load()
+    H = NH * dh
+    wx, r, b, s0 = make_problem(340, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=True)
+    reset = geometric_reset_mask(341, B, T, max(2, T // 2))
+    reset[0, 0] = 0
+    rng = np.random.default_rng(342)
+    d_h = rng.standard_normal((T, B, H)).astype(np.float32)
+    d_sf = rng.standard_normal((4, B, H)).astype(np.float32)
+    d_sf[3] = 0.0
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    dev = torch.device("cuda:0")
+    if bf16:
+        d_h = torch.from_numpy(d_h).bfloat16().float().numpy()
+        r = torch.from_numpy(r).bfloat16().float().numpy()
+    r_k = r_ext_to_kernel(torch.from_numpy(r)).numpy()                       # [NH, 4 dh, dh], the forward's layout
+    # R transposed in the reverse kernel's operand order (include/xlstm_amd.h), by numpy
+    epc = 8 if bf16 else 4
+    if split:
+        S, ksteps = dh // 64, 4 * dh // 8 // (4 * epc)
+        r_t = (r_k.reshape(NH, 4, S, 64, dh).transpose(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh)
+               .reshape(NH, 8, ksteps, 4, epc, S, 4, 16).transpose(0, 5, 1, 2, 6, 3, 7, 4))
+    else:
+        r_t = r_k.transpose(0, 2, 1).reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).transpose(0, 1, 3, 4, 2, 5)
+    dev_t = lambda a, dt=torch.float32: torch.from_numpy(np.ascontiguousarray(a)).to(dev).to(dt)
+    wx_t, r_fwd, rt_t, b_t, s0_t = dev_t(wx, tdt), dev_t(r_k, tdt), dev_t(r_t, tdt), dev_t(b), dev_t(s0)
+    m_t = torch.from_numpy(reset).to(dev)
+    dh_t, dsf_t = dev_t(d_h, tdt), dev_t(d_sf)
+    h, _ = F.slstm_forward(wx_t, r_fwd if bf16 else dev_t(r_k), b_t, s0_t, m_t)
+    groups = NH * ((B + 15) // 16)
+    rows = (B + 15) // 16 * 16 if split else B
+    coef = torch.empty(T * rows * 9 * H, dtype=torch.float32, device=dev)
+    d_wx = torch.empty(B, T, 4 * H, dtype=torch.float32, device=dev)
+    d_s0 = torch.empty(4, B, H, dtype=torch.float32, device=dev)
+    d_r = torch.empty(NH, 4 * dh, dh, dtype=torch.float32, device=dev)
+    d_b = torch.empty(NH, 4, dh, dtype=torch.float32, device=dev)
+    exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=tdt, device=dev)
+    counters = torch.empty(1 + groups, dtype=torch.int32, device=dev)
+    a = _lib.SlstmBwdArgs()
+    a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
+    a.wx, a.wx_stride_b, a.wx_stride_t = wx_t.data_ptr(), wx_t.stride(0), wx_t.stride(1)
+    a.r, a.h_out, a.bias, a.s0 = r_fwd.data_ptr(), h.data_ptr(), b_t.data_ptr(), s0_t.data_ptr()
+    a.reset, a.reset_stride_b = m_t.data_ptr(), m_t.stride(0)
+    a.coef, a.d_h, a.d_s_final, a.r_t = coef.data_ptr(), dh_t.data_ptr(), dsf_t.data_ptr(), rt_t.data_ptr()
+    a.d_wx, a.d_wx_stride_b, a.d_wx_stride_t, a.d_s0 = d_wx.data_ptr(), d_wx.stride(0), d_wx.stride(1), d_s0.data_ptr()
+    a.d_r, a.d_bias = d_r.data_ptr(), d_b.data_ptr()
+    a.stream = torch.cuda.current_stream().cuda_stream
+    a.split = 1 if split else 0
+    a.exchange, a.counters = (exchange.data_ptr(), counters.data_ptr()) if split else (None, None)
+    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
+        rc = fn(ctypes.byref(a))
+        assert rc == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    if split:
+        assert int(counters[0]) == 0
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
+    tol = 2e-2 if bf16 else 1e-5
+    errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
+                d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
+    print("C ABI backward", bf16, B, T, NH, dh, split, errs, flush=True)
+    assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs

@@ -97,9 +97,16 @@ __global__ __launch_bounds__(kPrepThreads) void slstm_bwd_prepare_kernel(BwdPrep
   char *const ring = prep_lds;                                                    // [NR][kPrepBlock] slots of inputs
   float *const outs = reinterpret_cast<float *>(prep_lds + NR * kPrepBlock * SLOT);  // [2][kPrepBlock][9][64]: results
   const int H = p.NH * DH;
-  const int slices = H >> 6;
-  const int b = blockIdx.x / slices, col0 = (blockIdx.x - b * slices) << 6;
-  const int head = col0 / DH, a0 = col0 - head * DH;
+  // The DH / 64 workgroups of a (batch row, head) read the same operand rows (the head's outputs): they take
+  // consecutive slots of ONE XCD (workgroup i runs on XCD i % 8), so those rows come from HBM into one L2 once.
+  // (Dealt out in launch order they sat on different XCDs and each fetched its own copy: 539 MB read at
+  // B 16 x T 2048 x 4 heads of 256 for 340 of W.x, outputs and R.)
+  constexpr int SPH = DH >> 6;                       // slices per head
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int pair = (slot / SPH) * 8 + xcd;           // (batch row, head) pair
+  if (pair >= p.B * p.NH) return;
+  const int b = pair / p.NH, head = pair - b * p.NH, a0 = (slot % SPH) << 6;
+  const int col0 = head * DH + a0;
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = (int)uniform((uint32_t)(tid >> 6));
   const int nblocks = (p.T + kPrepBlock - 1) / kPrepBlock;

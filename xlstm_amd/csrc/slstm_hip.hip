@@ -411,7 +411,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.r = a->r; p.h_out = a->h_out; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
     p.tiled = a->split ? 1 : 0;
-    const long long blocks = (long long)a->B * (H / 64);  // (head dims are multiples of 64 here)
+    // (batch row, head) pairs dealt out over the XCDs, the dh / 64 slices of a pair on one of them
+    const long long blocks = ((long long)a->B * a->NH + 7) / 8 * 8 * (a->dh / 64);
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
     void (*kp)(BwdPrepParams) = nullptr;
     switch (a->dh) {

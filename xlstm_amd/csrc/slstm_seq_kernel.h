@@ -462,6 +462,13 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     }
     bool aborted = false;
     uint32_t max_spins = 0;
+#ifdef XS_PROFILE
+    long long qprof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long qtick = clock64();
+#define XS_QTICK(i) do { const long long now_ = clock64(); qprof[i] += now_ - qtick; qtick = now_; } while (0)
+#else
+#define XS_QTICK(i) do { } while (0)
+#endif
     lds_barrier();  // prologue barrier
     const bool cross = cross_s != 0u;
     constexpr int QTILE = 4 * 16 * 2;          // bytes a member publishes per step
@@ -493,7 +500,9 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       // 1.517 .. 1.573, the best one taken.  (K split over the waves, below: 1.70.)
       const int buf = t & 1;
       float wxv[4];
+      XS_QTICK(5);
       lds_barrier();  // barrier #t: W.x of this step is in LDS, the h of two steps ago has been drained
+      XS_QTICK(2);
 #pragma unroll
       for (int g = 0; g < 4; ++g) wxv[g] = wxs[buf][g][gb * kTileStride + gu];
       const bool row_reset = rfl[t & 3][r16 >> 2] != 0u;   // (the operand's row: it contributes R.0 = 0 exactly)
@@ -503,6 +512,10 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #endif
       if (XS_QUAD_SLEEP > 0) __builtin_amdgcn_s_sleep(XS_QUAD_SLEEP);
       asm volatile("");  // (the compiler keeps what stands in front of this statement in front of the poll)
+#ifdef XS_PROFILE
+      asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#endif
+      XS_QTICK(1);
       if (t > 0) {
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks)
@@ -544,7 +557,11 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
           }
         }
         max_spins = spins > max_spins ? spins : max_spins;
+#ifdef XS_PROFILE
+        qprof[6] += spins;
+#endif
       }
+      XS_QTICK(0);
       if (__builtin_amdgcn_ballot_w64(row_reset) != 0ull) {
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks)
@@ -571,9 +588,17 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
       const float ry3 = __int_as_float(__builtin_amdgcn_update_dpp(0, mi, 0x10C, 0xF, 0xF, true));  // row_shl:12
       const float raw0 = (wxv[0] + mine) + bias_g[0], raw1 = (wxv[1] + ry1) + bias_g[1];
       const float raw2 = (wxv[2] + ry2) + bias_g[2], raw3 = (wxv[3] + ry3) + bias_g[3];
+#ifdef XS_PROFILE
+      asm volatile("" :: "v"(raw0), "v"(raw1), "v"(raw2), "v"(raw3));
+#endif
+      XS_QTICK(7);
       if (gate_reset) st = CellState{0.0f, 0.0f, 0.0f, 0.0f};
       slstm_pointwise(raw0, raw1, raw2, raw3, st);
       const float y = st.y;
+#ifdef XS_PROFILE
+      asm volatile("" :: "v"(y));
+#endif
+      XS_QTICK(3);
       if (gate_lane) {
         const uint16_t v = (uint16_t)float_to_bf16_bits(y);
         if (cross) {
@@ -588,9 +613,18 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #pragma unroll
       for (int ks = 0; ks < NK; ++ks)  // (the operand registers stay reserved to the end of the iteration)
         asm volatile("" :: "v"(areg[ks].x), "v"(areg[ks].y), "v"(areg[ks].z), "v"(areg[ks].w));
+      XS_QTICK(4);
     }
     for (int j = NIT; j < NITpad; ++j) lds_barrier();  // padding iterations of the feeder
     lds_barrier();                                     // final barrier
+#ifdef XS_PROFILE
+    // slots: 0 poll (issue to complete operand), 1 LDS reads + s_sleep, 2 barrier, 3 gating, 4 publication + staging,
+    // 5 loop top, 6 polls repeated, 7 MFMAs + fold + row shifts
+    if (lane == 0 && member == 0 && gi == 0) {
+      long long *dst = reinterpret_cast<long long *>(p.wg_xcc + kStampWord) + wave * 8;
+      for (int i = 0; i < 8; ++i) dst[i] = qprof[i];
+    }
+#endif
     const bool poisoned = __hip_atomic_load(&p.status->aborted, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u;
     if (gate_lane && brow < rend) {
       const long long o = (long long)brow * H + col;
