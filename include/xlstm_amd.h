@@ -279,7 +279,7 @@ typedef struct xs_slstm_bwd_args {
   const float *s0;           /* [4,B,H] or NULL (prepare) */
   const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */
   int64_t reset_stride_b;
-  float *coef;               /* [T,B,9,H] ([T,ceil(B/16)*16,9,H] with split): written by prepare, read by backward */
+  float *coef;               /* [T,B,9,H] ([T,ceil(B/16)*16,9,H] with split, [T,ceil(B/4)*4,9,H] with split == 2): written by prepare, read by backward */
   const void *d_h;           /* [T,B,H]: gradient with respect to h_out (backward) */
   const float *d_s_final;    /* [4,B,H] or NULL: gradient with respect to the final state; y, c, n are used (backward) */
   const void *r_t;           /* (backward) */
@@ -294,6 +294,10 @@ typedef struct xs_slstm_bwd_args {
    * dtype and counters 1 + NH * ceil(B/16) 32-bit words; the library initialises both in front of the kernel, and the
    * FIRST word is nonzero after the call when a bounded wait between the compute units of a head ran out (d_s0 is NaN
    * then).
+   * split == 2 (XS_BF16, head dims 64, 128, 256): row tiles of 4 rows instead of 16, four times the workgroups, a
+   * shorter step; for batches whose NH * ceil(B/4) * dh/64 workgroups fit the device.  Then K is ordered k = 4*a + g,
+   * r_t is tiled the same way, coef is [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units], exchange has
+   * 4 * NH * ceil(B/4) * 4 * 4*dh elements and counters 1 + NH * ceil(B/4) words.
    * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once. */
   int32_t split;
   void *exchange;

@@ -73,14 +73,31 @@ SPLIT_CASES = [
 ]
 
 
-@pytest.mark.parametrize("split", [False, True], ids=["one-unit", "split"])
-@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES + SPLIT_CASES + PADDED_CASES)
-def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, split):
+def _row_tile_of(kernel, bf16, dh):
+    """``kernel``: "one-unit" (one workgroup per head), "split" (a head over dh/64 compute units, row tiles of 16 rows),
+    "quad" (the same in row tiles of 4 rows: bf16, head dims up to 256).  Returns (split_override, row_tile_override)."""
+    if kernel == "quad" and (not bf16 or dh > 256):
+        pytest.skip("row tiles of 4 rows: bf16 and head dims up to 256")
+    return kernel != "one-unit", {"one-unit": None, "split": 16, "quad": 4}[kernel]
+
+
+QUAD_CASES = [
+    (True, 1, 1, 1, 64, False),       # one row, one step
+    (True, 2, 3, 1, 128, True),       # fewer steps than the feeder wave runs ahead
+    (True, 7, 4, 3, 256, True),       # a ragged second row tile, as many steps as feeder slots
+    (True, 6, 5, 2, 64, True),
+]
+
+
+@pytest.mark.parametrize("kernel", ["one-unit", "split", "quad"])
+@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES + SPLIT_CASES + PADDED_CASES + QUAD_CASES)
+def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, kernel):
     from xlstm_amd import functional as F
 
+    split, row_tile = _row_tile_of(kernel, bf16, (dh + 63) // 64 * 64)
     if not split and dh > 256:
         pytest.skip("head dim 512 (and what is padded up to it) has the split kernel only")
-    print("case backward", bf16, B, T, NH, dh, masked, split, flush=True)
+    print("case backward", bf16, B, T, NH, dh, masked, kernel, flush=True)
     H = NH * dh
     wx, r, b, s0 = make_problem(91, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=masked)
     reset = geometric_reset_mask(7, B, T, max(2, T // 2)) if masked else None
@@ -102,7 +119,7 @@ def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, split):
     m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
     d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), torch.from_numpy(d_sf).to(dev),
-                                            split_override=split)
+                                            split_override=split, row_tile_override=row_tile)
     torch.cuda.synchronize()
     o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
     o_r_k = r_ext_to_kernel(torch.from_numpy(o_r)).numpy()
@@ -169,7 +186,8 @@ def test_cell_autograd_matches_the_oracle(dtype, tol):
     assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
 
 
-def test_a_wait_between_compute_units_that_runs_out_is_reported():
+@pytest.mark.parametrize("row_tile", [16, 4])
+def test_a_wait_between_compute_units_that_runs_out_is_reported(row_tile):
     """Host-forced: a negative spin limit makes every wait between the workgroups of a head give up at its first look
     (every kernel still exits normally).  The call must raise, the gradient of the initial state must be NaN, and the
     next call must be the usual one.  (A bound of one look does not do it: the peers' deltas are always there by the
@@ -186,16 +204,26 @@ def test_a_wait_between_compute_units_that_runs_out_is_reported():
     r_t, b_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
     d_h = torch.randn(T, B, NH * dh, generator=torch.Generator().manual_seed(7)).to(dev).bfloat16()
     h, _ = F.slstm_forward(wx_t, r_t, b_t)
-    good = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True)
+    print("case backward give-up, row tile", row_tile, flush=True)
+    kw = dict(split_override=True, row_tile_override=row_tile)
+    good = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, **kw)
     with pytest.raises(F.EngineError, match="ran out"):
-        F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=-1)
+        F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, spin_limit=-1, **kw)
     # the same call with the synchronisation left to the caller (timings asked for): nothing raises, d_s0 is NaN
     t = {}
-    got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True, spin_limit=-1, timings=t)
+    got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, spin_limit=-1, timings=t, **kw)
     torch.cuda.synchronize()
     assert bool(torch.isnan(got[3][:3]).all())
-    again = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, split_override=True)  # the next call is unaffected
+    again = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, **kw)  # the next call is unaffected
     assert torch.equal(again[0], good[0]) and torch.equal(again[3], good[3])
+
+
+_ORACLE_RESULTS = {}
+
+
+def _kernel_kw(split):
+    """False: one workgroup per head; True: a head over dh/64 compute units in row tiles of 16 rows; 4: in row tiles of 4."""
+    return dict(split_override=bool(split), row_tile_override=None if split is False else (4 if split == 4 and split is not True else 16))
 
 
 def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=None, **opts):
@@ -219,22 +247,27 @@ def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=
     m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
     dsf_t = torch.from_numpy(d_sf).to(dev) if d_sf is not None else None
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
-    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override")}
+    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override", "row_tile_override")}
     d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), dsf_t, **kw)
     torch.cuda.synchronize()
     okw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval")}
-    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf, **okw)
+    key = (bf16, B, T, NH, dh, seed, masked, with_state, mean_len, None if d_sf is None else d_sf.tobytes(), tuple(sorted(okw.items())))
+    if key not in _ORACLE_RESULTS:  # (the same problem through several kernels: the oracle runs once)
+        _ORACLE_RESULTS[key] = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf, **okw)
+    o_wx, o_r, o_b, o_s0 = _ORACLE_RESULTS[key]
     errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
                 d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
     return errs, (d_wx, d_r, d_b, d_s0), (o_wx, o_r, o_b, o_s0)
 
 
-def test_backward_over_2048_steps_bf16_packed_documents():
+@pytest.mark.parametrize("row_tile", [4, 16])
+def test_backward_over_2048_steps_bf16_packed_documents(row_tile):
     """The length of BASELINE config 2 (T = 2048, 4 heads of 256, bf16, packed geometric documents) on a few batch
     rows (rows are independent; the oracle affords three of them): what 2048 reverse steps on bf16 operands do to the
-    error, against the float64 oracle.  Tolerance 2e-2."""
-    print("case backward T=2048 bf16 B=3", flush=True)
-    errs, _, _ = _run_both(True, 3, 2048, 4, 256, 301, masked=True, with_state=False, mean_len=512)
+    error, against the float64 oracle, in both row tilings of the kernel that spreads a head over four compute units
+    (4 rows: what config 2 itself runs).  Tolerance 2e-2."""
+    print("case backward T=2048 bf16 B=3 row tile", row_tile, flush=True)
+    errs, _, _ = _run_both(True, 3, 2048, 4, 256, 301, masked=True, with_state=False, mean_len=512, row_tile_override=row_tile)
     print("backward, T = 2048, bf16:", errs, flush=True)
     assert all(np.isfinite(v) and v <= 2e-2 for v in errs.values()), errs
 
@@ -248,7 +281,8 @@ def test_backward_config1_shape_fp32_full_size():
 
 
 @pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 11, 2, 64, True), (False, 20, 9, 2, 128, True), (True, 16, 12, 4, 256, True),
-                                                  (False, 4, 10, 2, 128, False), (True, 9, 8, 2, 512, True)])
+                                                  (False, 4, 10, 2, 128, False), (True, 9, 8, 2, 512, True),
+                                                  (True, 16, 12, 4, 256, 4), (True, 7, 10, 2, 128, 4)])
 def test_the_gradient_of_the_final_state_by_the_chain_rule(bf16, B, T, NH, dh, split):
     """``d_s_final`` on the GPU, pinned the way the oracle's is: the gradients of a sequence are those of its second
     part, started from the state after step k - 1, and of its first part with the second part's ``d_s0`` as the
@@ -268,13 +302,13 @@ def test_the_gradient_of_the_final_state_by_the_chain_rule(bf16, B, T, NH, dh, s
     s0_t = torch.from_numpy(s0).to(dev)
     d_h = torch.randn(T, B, H, generator=torch.Generator().manual_seed(311)).to(dev).to(wx_t.dtype)
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t)
-    whole = F.slstm_backward(wx_t, r_t, b_t, s0_t, None, h, d_h, split_override=split)
+    whole = F.slstm_backward(wx_t, r_t, b_t, s0_t, None, h, d_h, **_kernel_kw(split))
     h_a, s_k = F.slstm_forward(wx_t[:, :k], r_t, b_t, s0_t)
     h_b, _ = F.slstm_forward(wx_t[:, k:], r_t, b_t, s_k)
     assert torch.equal(torch.cat([h_a, h_b]), h)
-    tail = F.slstm_backward(wx_t[:, k:], r_t, b_t, s_k, None, h_b, d_h[k:].contiguous(), split_override=split)
+    tail = F.slstm_backward(wx_t[:, k:], r_t, b_t, s_k, None, h_b, d_h[k:].contiguous(), **_kernel_kw(split))
     assert all(float(tail[3][i].abs().max()) > 0 for i in range(3)) and not bool(tail[3][3].any())
-    head = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), tail[3], split_override=split)
+    head = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), tail[3], **_kernel_kw(split))
     torch.cuda.synchronize()
     tol = 2e-2 if bf16 else 1e-5
 
@@ -286,7 +320,7 @@ def test_the_gradient_of_the_final_state_by_the_chain_rule(bf16, B, T, NH, dh, s
     print("chain rule", bf16, B, T, NH, dh, split, errs, flush=True)
     assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
     # not vacuous: without the hand-over the first part's gradients are not the whole call's
-    plain = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), split_override=split)
+    plain = F.slstm_backward(wx_t[:, :k], r_t, b_t, s0_t, None, h_a, d_h[:k].contiguous(), **_kernel_kw(split))
     assert rel(plain[0], whole[0][:, :k]) > 10 * tol
     # and against the oracle, d_s_final given
     d_sf = tail[3].cpu().numpy()
@@ -297,7 +331,7 @@ def test_the_gradient_of_the_final_state_by_the_chain_rule(bf16, B, T, NH, dh, s
 
 @pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (False, 20, 7, 2, 128, True), (True, 16, 10, 4, 256, True),
                                                   (False, 4, 12, 4, 256, False), (True, 9, 7, 2, 512, True), (True, 6, 9, 2, 128, False),
-                                                  (False, 7, 6, 2, 256, True)])
+                                                  (False, 7, 6, 2, 256, True), (True, 16, 10, 4, 256, 4), (True, 5, 9, 2, 64, 4)])
 @pytest.mark.parametrize("opts", [dict(recurrent_cut=True), dict(recurrent_clipval=0.05), dict(recurrent_clipval=1.0),
                                   dict(recurrent_cut=True, recurrent_clipval=0.05)],
                          ids=["cut", "clip0.05", "clip1", "cut+clip"])
@@ -309,7 +343,7 @@ def test_recurrent_cut_and_clipval_against_the_oracle(bf16, B, T, NH, dh, split,
     d_sf = np.random.default_rng(320).standard_normal((4, B, H)).astype(np.float32)
     d_sf[3] = 0.0
     print("case cut/clip", bf16, B, T, NH, dh, split, opts, flush=True)
-    errs, got, want = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, split_override=split, **opts)
+    errs, got, want = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, **_kernel_kw(split), **opts)
     print(errs, flush=True)
     tol = 2e-2 if bf16 else 1e-5
     assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
@@ -317,7 +351,7 @@ def test_recurrent_cut_and_clipval_against_the_oracle(bf16, B, T, NH, dh, split,
         assert not bool(got[3][0].any())  # nothing reaches the y of the initial state
     # the option bites: the plain gradient of the same problem is something else
     if opts.get("recurrent_cut") or opts.get("recurrent_clipval", 1.0) < 1.0:
-        _, got_plain, _ = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, split_override=split)
+        _, got_plain, _ = _run_both(bf16, B, T, NH, dh, 321, masked=True, with_state=True, d_sf=d_sf, **_kernel_kw(split))
         assert float((got_plain[0] - got[0]).abs().max()) > 1e-3
 
 
@@ -351,7 +385,8 @@ def test_cell_config_gradient_recurrent_cut_and_clipval():
         sLSTMCell(sLSTMCellConfig(hidden_size=H, num_heads=NH, backend="hip", gradient_recurrent_clipval=0.5))
 
 
-@pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (True, 16, 12, 4, 256, True), (False, 4, 10, 2, 128, False)])
+@pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (True, 16, 12, 4, 256, True), (False, 4, 10, 2, 128, False),
+                                                  (True, 14, 12, 4, 256, 4)])
 def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     """A caller without torch arithmetic - the binding a maintainer would put in place of the reference's
     ``sLSTMFunc.backward`` (slstm.cc:137-221, which returns {dx, ds0, dR, db} from one native call): forward, then the
@@ -379,7 +414,12 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     r_k = r_ext_to_kernel(torch.from_numpy(r)).numpy()                       # [NH, 4 dh, dh], the forward's layout
     # R transposed in the reverse kernel's operand order (include/xlstm_amd.h), by numpy
     epc = 8 if bf16 else 4
-    if split:
+    tile_rows = 4 if split == 4 and split is not True else 16  # (split: False, True = row tiles of 16 rows, 4 = of 4 rows)
+    if tile_rows == 4:
+        S, ksteps = dh // 64, 4 * dh // 8 // 32                               # K ordered (unit, gate)
+        r_t = (r_k.reshape(NH, 4, dh, dh).transpose(0, 2, 1, 3).reshape(NH, 4 * dh, dh)
+               .reshape(NH, 8, ksteps, 4, 8, S, 4, 16).transpose(0, 5, 1, 2, 6, 3, 7, 4))
+    elif split:
         S, ksteps = dh // 64, 4 * dh // 8 // (4 * epc)
         r_t = (r_k.reshape(NH, 4, S, 64, dh).transpose(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh)
                .reshape(NH, 8, ksteps, 4, epc, S, 4, 16).transpose(0, 5, 1, 2, 6, 3, 7, 4))
@@ -390,14 +430,14 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     m_t = torch.from_numpy(reset).to(dev)
     dh_t, dsf_t = dev_t(d_h, tdt), dev_t(d_sf)
     h, _ = F.slstm_forward(wx_t, r_fwd if bf16 else dev_t(r_k), b_t, s0_t, m_t)
-    groups = NH * ((B + 15) // 16)
-    rows = (B + 15) // 16 * 16 if split else B
+    groups = NH * ((B + tile_rows - 1) // tile_rows)
+    rows = (B + tile_rows - 1) // tile_rows * tile_rows if split else B
     coef = torch.empty(T * rows * 9 * H, dtype=torch.float32, device=dev)
     d_wx = torch.empty(B, T, 4 * H, dtype=torch.float32, device=dev)
     d_s0 = torch.empty(4, B, H, dtype=torch.float32, device=dev)
     d_r = torch.empty(NH, 4 * dh, dh, dtype=torch.float32, device=dev)
     d_b = torch.empty(NH, 4, dh, dtype=torch.float32, device=dev)
-    exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=tdt, device=dev)
+    exchange = torch.empty(4 * groups * tile_rows * 4 * dh, dtype=tdt, device=dev)
     counters = torch.empty(1 + groups, dtype=torch.int32, device=dev)
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
@@ -408,7 +448,7 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     a.d_wx, a.d_wx_stride_b, a.d_wx_stride_t, a.d_s0 = d_wx.data_ptr(), d_wx.stride(0), d_wx.stride(1), d_s0.data_ptr()
     a.d_r, a.d_bias = d_r.data_ptr(), d_b.data_ptr()
     a.stream = torch.cuda.current_stream().cuda_stream
-    a.split = 1 if split else 0
+    a.split = (2 if tile_rows == 4 else 1) if split else 0
     a.exchange, a.counters = (exchange.data_ptr(), counters.data_ptr()) if split else (None, None)
     for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
         rc = fn(ctypes.byref(a))

@@ -40,9 +40,9 @@ struct BwdPrepParams {
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
-  float *coef;               // [T,B,9,H], or with tiled != 0 [T][ceil(B/16)][NH][dh/64][16 rows][9][64 units]: what a workgroup
-                             // of the split kernel reads per step is one piece of 36 KiB (planes 4 KiB apart, as in the
-                             // plain layout, all fall on the same memory channel)
+  float *coef;               // [T,B,9,H], or with tiled = R (16 or 4) [T][ceil(B/R)][NH][dh/64][R rows][9][64 units]: what a
+                             // workgroup of the split kernels reads per step is one piece of 36 (9) KiB (planes 4 KiB apart,
+                             // as in the plain layout, all fall on the same memory channel)
   int tiled;
 };
 
@@ -192,8 +192,9 @@ __global__ __launch_bounds__(kPrepThreads) void slstm_bwd_prepare_kernel(BwdPrep
         float *dst = p.coef + ((long long)t * p.B + b) * 9 * H + col;
         long long js = H;
         if (p.tiled) {
-          const long long piece = (((long long)t * ((p.B + 15) >> 4) + (b >> 4)) * p.NH + head) * (DH >> 6) + (a >> 6);
-          dst = p.coef + (piece * 16 + (b & 15)) * (9 * 64) + (a & 63);
+          const int tr = p.tiled;
+          const long long piece = (((long long)t * ((p.B + tr - 1) / tr) + b / tr) * p.NH + head) * (DH >> 6) + (a >> 6);
+          dst = p.coef + (piece * tr + b % tr) * (9 * 64) + (a & 63);
           js = 64;
         }
         const float *src = outs + (((k & 1) * kPrepBlock + i) * 9 + j0) * 64 + lane;
@@ -575,10 +576,10 @@ __global__ __launch_bounds__(256) void slstm_bwd_arm_kernel(uint4 *xch, long lon
 // 2.0 us with inputs that were already in the L2.  So another compute unit takes the misses.  Nothing depends on
 // these workgroups: they follow the groups' progress words at a distance, and stop when those stop.
 constexpr int kBwdAhead = 12;  // steps the prefetch may run ahead (1.2 MiB of a 4 MiB L2 at config 2)
-template <bool BF16>
+template <bool BF16, int ROWS = 16>  // ROWS: batch rows of a row tile
 __device__ __forceinline__ void bwd_prefetch(const BwdSplitParams &p, int xcd) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  const int S = p.dh >> 6, H = p.NH * p.dh, NT = (p.B + 15) >> 4, ngroups = p.NH * NT;
+  const int S = p.dh >> 6, H = p.NH * p.dh, NT = (p.B + ROWS - 1) / ROWS, ngroups = p.NH * NT;
   const int tid = threadIdx.x, nthreads = blockDim.x;
   if (xcd >= ngroups) return;
   // A touch is a load that writes LDS, not a register: nothing waits for these loads before the end, and a register
@@ -616,11 +617,11 @@ __device__ __forceinline__ void bwd_prefetch(const BwdSplitParams &p, int xcd) {
     for (int m = m0; m < m0 + 4 && m < p.T; ++m) {
       const int t = p.T - 1 - m;
       for (int g = xcd; g < ngroups; g += 8) {
-        const int head = g % p.NH, tile = g / p.NH, row0 = tile * 16;
-        const int piece_lines = 16 * 9 * 64 * 4 / 128;
+        const int head = g % p.NH, tile = g / p.NH, row0 = tile * ROWS;
+        const int piece_lines = ROWS * 9 * 64 * 4 / 128;
         const char *cbase = reinterpret_cast<const char *>(p.coef) + ((((long long)t * NT + tile) * p.NH + head) * S) * (piece_lines * 128ll);
         touch_lines(cbase, S * piece_lines * 128, 0, S * piece_lines, 1, 1);
-        const int rows = p.B - row0 < 16 ? p.B - row0 : 16, per_row = p.dh * ESZ / 128;
+        const int rows = p.B - row0 < ROWS ? p.B - row0 : ROWS, per_row = p.dh * ESZ / 128;
         const char *dbase = reinterpret_cast<const char *>(p.d_h) + (((long long)t * p.B + row0) * H + (long long)head * p.dh) * ESZ;
         touch_lines(dbase, ((rows - 1) * H + p.dh) * ESZ, 0, rows * per_row, H * ESZ / 128, per_row);
       }

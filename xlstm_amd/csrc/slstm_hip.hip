@@ -34,6 +34,7 @@
 #include "slstm_step_pipe_kernel.h"
 #include "slstm_layer_kernels.h"
 #include "slstm_backward_kernels.h"
+#include "slstm_backward_quad_kernel.h"
 #include "slstm_backward_params_kernel.h"
 #include "slstm_serial_bound.h"
 
@@ -410,7 +411,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.r = a->r; p.h_out = a->h_out; p.bias = a->bias; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
-    p.tiled = a->split ? 1 : 0;
+    p.tiled = a->split == 2 ? 4 : (a->split ? 16 : 0);
     // (batch row, head) pairs dealt out over the XCDs, the dh / 64 slices of a pair on one of them
     const long long blocks = ((long long)a->B * a->NH + 7) / 8 * 8 * (a->dh / 64);
     if (blocks > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many elements for one launch");
@@ -435,6 +436,42 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     if (a->d_wx_stride_t < 4 * H || (a->B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
     // (0, negative, NaN or infinite: no clipping)
     const float clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
+    if (a->split == 2) {
+      // row tiles of 4 rows (bf16, head dims up to 256): four times the workgroups of the 16-row kernel, a shorter step
+      if (!bf16 || (a->dh != 64 && a->dh != 128 && a->dh != 256))
+        return fail(XS_ERR_UNSUPPORTED, "backward pass with row tiles of 4 rows: bf16 and head dim 64, 128 or 256 (got %d)", a->dh);
+      if (!a->exchange || !a->counters) return fail(XS_ERR_NULL, "exchange and counters are required with split");
+      if (((uintptr_t)a->exchange % 16)) return fail(XS_ERR_ALIGN, "exchange must be 16-byte aligned");
+      if (a->reset && 3 * a->reset_stride_b + a->T >= 0x7FFFFF00ll) return fail(XS_ERR_UNSUPPORTED, "reset rows too far apart for row tiles of 4 rows");
+      if (3 * H * 2 + 1024 >= 0x7FFFFF00ll) return fail(XS_ERR_UNSUPPORTED, "rows too long for row tiles of 4 rows");
+      const int S = a->dh / 64;
+      const long long ngroups = (long long)a->NH * ((a->B + 3) / 4);
+      const long long grid = (ngroups + 7) / 8 * 8 * S;
+      if (grid > device_cus()) return fail(XS_ERR_DEVICE, "%lld workgroups of the backward pass with row tiles of 4 rows do not fit %d compute units at once", grid, device_cus());
+      BwdSplitParams q;
+      q.B = a->B; q.T = a->T; q.NH = a->NH; q.dh = a->dh;
+      q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
+      q.reset = a->reset; q.reset_sb = a->reset_stride_b;
+      q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1;
+      q.main_locals = (int)(grid / 8);
+      const bool prefetchers = grid + 8 <= device_cus();
+      q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;
+      q.cut = a->recurrent_cut != 0; q.clip = clip;
+      const long long n16 = (long long)kBwdRing * ngroups * 4 * 4 * a->dh * 2 / 16;
+      hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
+                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
+      void (*kq)(BwdSplitParams) = a->dh == 64 ? slstm_bwd_quad_kernel<1> : (a->dh == 128 ? slstm_bwd_quad_kernel<2> : slstm_bwd_quad_kernel<4>);
+      const int lds = bwd_quad_lds_bytes();
+      {
+        const int rc = ensure_dynamic_lds((const void *)kq, (size_t)lds);
+        if (rc != XS_OK) return rc;
+      }
+      hipLaunchKernelGGL(kq, dim3((unsigned)(grid + (prefetchers ? 8 : 0))), dim3(576), lds, stream, q);
+      const hipError_t es = hipGetLastError();
+      if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
+      return XS_OK;
+    }
     if (a->split) {
       if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && bf16))
         return fail(XS_ERR_UNSUPPORTED, "backward pass over several compute units per head: head dim %d not supported", a->dh);

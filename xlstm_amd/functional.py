@@ -73,6 +73,7 @@ def slstm_backward(
     timings: Optional[dict] = None,
     split_override: Optional[bool] = None,
     spin_limit: int = 0,
+    row_tile_override: Optional[int] = None,
     recurrent_cut: bool = False,
     recurrent_clipval: Optional[float] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -89,7 +90,8 @@ def slstm_backward(
     here is allocating the buffers and bringing R into the kernels' operand order.  ``timings`` (a dict) receives four
     events around the three kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
-    kernel); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
+    kernel), in row tiles of 4 rows where four times the workgroups fit (bfloat16, head dims up to 256;
+    ``row_tile_override`` = 16 or 4 forces either); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
     to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
     clipped to +-value before ``d_h`` is added, ``slstm_pointwise.cu:136-143``).
@@ -126,7 +128,7 @@ def slstm_backward(
         dh_p = widen(d_h, (T_, B_)).reshape(T_, B_, NH * dh_k)
         dsf_p = widen(d_s_final, (4, B_)).reshape(4, B_, NH * dh_k) if d_s_final is not None else None
         d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
-                                                 split_override=split_override, spin_limit=spin_limit,
+                                                 split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
                                                  recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval)
         return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
                 d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
@@ -147,7 +149,7 @@ def slstm_backward(
                 parts.append(slstm_backward(
                     wx[b0:b1], r, bias, None if s0 is None else s0[:, b0:b1], None if reset_mask is None else reset_mask[b0:b1],
                     h_out[:, b0:b1], d_h[:, b0:b1], None if d_s_final is None else d_s_final[:, b0:b1],
-                    timings=None, split_override=split_override, spin_limit=spin_limit,
+                    timings=None, split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
                     recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval))
             return (torch.cat([q[0] for q in parts], 0), sum(q[1] for q in parts), sum(q[2] for q in parts),
                     torch.cat([q[3] for q in parts], 1))
@@ -174,9 +176,23 @@ def slstm_backward(
     split = (dh in (64, 128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
     if split_override is not None:
         split = bool(split_override)
-    # (the split kernel reads the coefficients in pieces of 16 rows: its buffer covers whole row tiles)
-    coef = torch.empty((T, (B + 15) // 16 * 16 if split else B, 9, H), dtype=torch.float32, device=dev)
-    if split:
+    # row tiles of 4 rows (bf16, head dims up to 256) where four times the workgroups still fit, with the prefetching ones
+    groups4 = NH * ((B + 3) // 4)
+    quad = (split and bf16 and dh <= 256 and (groups4 + 7) // 8 * 8 * S + 8 <= _compute_units(dev)
+            and (reset_mask is None or 3 * reset_mask.stride(0) + T < 2 ** 31 - 256))
+    if row_tile_override is not None:
+        quad = split and row_tile_override == 4
+    # (the split kernels read the coefficients in pieces of a row tile: the buffer covers whole row tiles)
+    coef = torch.empty((T, ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else B, 9, H), dtype=torch.float32, device=dev)
+    if quad:
+        # R transposed with K ordered (unit, gate), tiled as the MFMA B operands of the workgroup that owns the output
+        # columns and of the wave that owns the eighth of K: [NH][S][8 waves][k-steps of a wave][4 column blocks][k / 8 % 4][column % 16][k % 8]
+        ksteps = 4 * dh // 8 // 32
+        r_t = (r32.view(NH, 4, dh, dh).permute(0, 2, 1, 3).reshape(NH, 4 * dh, dh).to(wx.dtype)           # [NH, k, d]
+               .view(NH, 8, ksteps, 4, 8, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
+        exchange = torch.empty(4 * groups4 * 4 * 4 * dh, dtype=wx.dtype, device=dev)
+        counters = torch.empty(1 + groups4, dtype=torch.int32, device=dev)
+    elif split:
         # R transposed with K ordered (owner slice, gate, unit % 64), tiled as the MFMA B operands of the workgroup
         # that owns the output columns and of the wave that owns the eighth of K:
         # [NH][S][8 waves][chunks of a wave][4 column blocks][k chunk of 4][column % 16][k % EPC]
@@ -213,7 +229,7 @@ def slstm_backward(
     a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
     a.d_s0 = d_s0.data_ptr()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
-    a.split = 1 if split else 0
+    a.split = (2 if quad else 1) if split else 0
     a.exchange = exchange.data_ptr() if split else None
     a.counters = counters.data_ptr() if split else None
     a.spin_limit = int(spin_limit)
