@@ -289,7 +289,7 @@ def bench_backward(device, iters=3):
             "tokens_per_s": B * T / (float(np.median(total)) * 1e-3), "finite": bool(torch.isfinite(out[0]).all()),
             "roofline": {"bound": "hbm", "achieved": nbytes / (rev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": nbytes / (rev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
-                         "kernel": "slstm_bwd_split_kernel<bf16,NB=2,FEED>", "algorithmic_bytes_per_launch": nbytes,
+                         "kernel": "slstm_bwd_quad_kernel<S=4>", "algorithmic_bytes_per_launch": nbytes,
                          "traffic_source": "profiles/traffic_bwd_cfg2.json (rocprofv3 counters of a separate run, not of this one)"}}
 
 
@@ -415,7 +415,45 @@ def phase_profile(device):
                               "W.x through the LDS corner": round(float(st[5][3] / n)),
                               "sum": round(float(st[5][:6].sum() / n))},
         }
+    out["backward, config 2 (slstm_bwd_quad_kernel<S=4>), cycles since the step's barrier, first workgroup"] = backward_phase_profile(device)
     return out
+
+
+def backward_phase_profile(device):
+    """When three waves of the reverse kernel's first workgroup pass fixed points of a timestep, in cycles since they left
+    the step's barrier (the measurement build leaves the sums in the m plane of ``d_s0``, which is zero otherwise)."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    B, T, NH, dh = 16, 2048, 4, 256
+    H = NH * dh
+    wx_c, r_ext_c, bias_c, mask_c = make_inputs(B, T, NH, dh, 512, torch.device("cpu"))
+    wx = wx_c.to(device)
+    r = r_ext_c.permute(0, 2, 3, 1).reshape(NH, 4 * dh, dh).contiguous().to(device)
+    bias, mask = bias_c.to(device), mask_c.to(device)
+    h, _ = F.slstm_forward(wx, r, bias, None, mask)
+    d_h = torch.randn(T, B, H, device=device).bfloat16()
+    ms = []
+    for _ in range(3):
+        tm = {}
+        out = F.slstm_backward(wx, r, bias, None, mask, h, d_h, timings=tm)
+        torch.cuda.synchronize()
+        ms.append(tm["events"][1].elapsed_time(tm["events"][2]))
+    words = out[3][3].reshape(-1)[:60].view(torch.int64).cpu().double()
+    st, fd = words[:24].view(3, 8) / T, words[24:30]
+    points = ["partial results added up", "deltas published", "first look issued at the earliest", "deltas complete",
+              "partial tile written", "barrier left (= the step)"]
+    res = {"reverse_kernel_ms_with_stamps": sorted(ms)[1]}
+    for w, row in zip(("wave 0 (forms the gradient; polls its own workgroup)", "wave 4 (polls its own workgroup)",
+                       "wave 6 (polls another workgroup)"), st):
+        res[w] = {n: round(float(v)) for n, v in zip(points, row[:6])}
+        res[w]["looks repeated per step"] = round(float(row[6]), 2)
+        res[w]["the look that found them issued"] = round(float(row[7]))
+    res["feeder wave 0"] = {"a request, issue to landed (sampled)": round(float(fd[0] / max(1.0, float(fd[1])))),
+                            "its request goes out (every fourth step)": round(float(fd[2] / (T / 4))),
+                            "its wait is over, per step": round(float(fd[4] / T)), "step": round(float(fd[5] / T))}
+    return res
 
 
 def bench_config4(device, iters=3):

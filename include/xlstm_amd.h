@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 10
+#define XS_ABI_VERSION 11
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -291,13 +291,13 @@ typedef struct xs_slstm_bwd_args {
    * r_t holds R transposed with K ordered k = 256*(a/64) + 64*g + a%64 (a the hidden unit, g the gate), tiled as MFMA
    * operands per owner of the output columns and per wave: [NH][dh/64][8][K/8/KC][4][KC/EPC][16][EPC], EPC the elements
    * of 16 bytes and KC = 4*EPC; exchange is a 16-byte aligned buffer of 4 * NH * ceil(B/16) * 16 * 4*dh elements of
-   * dtype and counters 1 + NH * ceil(B/16) 32-bit words; the library initialises both in front of the kernel, and the
-   * FIRST word is nonzero after the call when a bounded wait between the compute units of a head ran out (d_s0 is NaN
-   * then).
+   * dtype and counters 1 + 2 * NH * ceil(B/16) 32-bit words; the library initialises both in front of the kernel, and the
+   * FIRST word is nonzero after the call when a bounded wait between the compute units of a head ran out, or when the
+   * workgroups of a head did not run on one XCD as the exchange assumes (d_s0 is NaN then).
    * split == 2 (XS_BF16, head dims 64, 128, 256): row tiles of 4 rows instead of 16, four times the workgroups, a
    * shorter step; for batches whose NH * ceil(B/4) * dh/64 workgroups fit the device.  Then K is ordered k = 4*a + g,
    * r_t is tiled the same way, coef is [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units], exchange has
-   * 4 * NH * ceil(B/4) * 4 * 4*dh elements and counters 1 + NH * ceil(B/4) words.
+   * 4 * NH * ceil(B/4) * 4 * 4*dh elements and counters 1 + 2 * NH * ceil(B/4) words.
    * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once. */
   int32_t split;
   void *exchange;

@@ -438,7 +438,7 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     d_r = torch.empty(NH, 4 * dh, dh, dtype=torch.float32, device=dev)
     d_b = torch.empty(NH, 4, dh, dtype=torch.float32, device=dev)
     exchange = torch.empty(4 * groups * tile_rows * 4 * dh, dtype=tdt, device=dev)
-    counters = torch.empty(1 + groups, dtype=torch.int32, device=dev)
+    counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
     a.wx, a.wx_stride_b, a.wx_stride_t = wx_t.data_ptr(), wx_t.stride(0), wx_t.stride(1)

@@ -14,7 +14,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 
 XS_F32, XS_BF16 = 0, 1
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 EXPORTS = (
     "xs_abi_version",

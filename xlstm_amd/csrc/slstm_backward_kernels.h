@@ -553,6 +553,7 @@ struct BwdSplitParams {
   void *xch;                 // [kBwdRing][groups][K / KC][16][4][16 bytes], all ones at the start
   unsigned int *abort_word;  // zero at the start of a call
   unsigned int *progress;    // [groups]: the step of the call that the group has reached (for the prefetching workgroups)
+  unsigned int *placement;   // [groups], zero at the start: the XCDs that the group's workgroups found themselves on, one bit each
   int main_locals;           // workgroups per XCD that compute; those behind them (one per XCD, if any) prefetch
   long long spin_limit;
   int cut;                   // as in BwdParams
@@ -630,6 +631,20 @@ __device__ __forceinline__ void bwd_prefetch(const BwdSplitParams &p, int xcd) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 }
 
+// The workgroups of a group exchange their deltas with plain stores through the L2 of the XCD that they are launched
+// on by position (workgroup i on XCD i mod 8).  Each leaves the XCD it really runs on in the group's placement word, and
+// at the end of the call looks at what the others left: with more than one XCD among them the exchange may have read
+// words that were never written back (or a slot's previous content), so the call is flagged like one whose waits ran out.
+__device__ __forceinline__ void bwd_note_placement(const BwdSplitParams &p, int group) {
+  if (threadIdx.x == 0) atomicOr(p.placement + group, 1u << (__builtin_amdgcn_s_getreg(20 | (3 << 11)) & 0xFu));  // XCC_ID, bits [3:0]
+}
+__device__ __forceinline__ bool bwd_placement_mixed(const BwdSplitParams &p, int group) {
+  const unsigned int seen = __hip_atomic_load(p.placement + group, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const bool mixed = (seen & (seen - 1u)) != 0u;
+  if (mixed && threadIdx.x == 0) __hip_atomic_store(p.abort_word, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return mixed;
+}
+
 constexpr int kBwdPartStride = 68;  // floats between the rows of a wave's partial tile in LDS (no bank conflicts)
 constexpr int kBwdCoefBytes = 16 * 9 * 64 * 4;  // a step's coefficients of a workgroup: 16 rows, 9 of them, 64 units
 constexpr int bwd_feed_slot_bytes(bool bf16) { return kBwdCoefBytes + 16 * 64 * (bf16 ? 2 : 4); }  // ... and its d_h
@@ -674,6 +689,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
   const int head = group % p.NH;
   const int row0 = (group / p.NH) * 16;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
+  bwd_note_placement(p, group);
   constexpr int FSLOT = bwd_feed_slot_bytes(BF16);
   char *const feed = reinterpret_cast<char *>(part + 8 * PART);  // [2 slots][16 rows][9][64 units] float32, then d_h [16][64]
   const long long coef_piece0 = ((((long long)(row0 >> 4)) * p.NH + head) * S + s) * kBwdCoefBytes;  // + t * coef_step
@@ -920,8 +936,9 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
     if (t > 0) step(in1, t - 1);
   }
   // ---- gradient w.r.t. the initial state (the stabiliser's part is zero by the rule; NaN all over when a wait ran out)
+  const bool mixed = S > 1 && p.cut == 0 && bwd_placement_mixed(p, group);
   if (there) {
-    const bool poisoned = gave_up || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool poisoned = gave_up || mixed || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     const long long o = (long long)row * H + ecol;
 #pragma unroll
     for (int e = 0; e < 2; ++e) {

@@ -453,21 +453,38 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
       q.reset = a->reset; q.reset_sb = a->reset_stride_b;
       q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
-      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1;
+      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1; q.placement = a->counters + 1 + ngroups;
       q.main_locals = (int)(grid / 8);
-      const bool prefetchers = grid + 8 <= device_cus();
+      // prefetching workgroups per XCD: one per 40 KB that the XCD's groups read per step (a compute unit draws some
+      // 65 GB/s from memory, a step takes about a microsecond), as far as there are compute units left
+      int prefetchers = 0;
+      {
+        const long long groups_per_xcd = (ngroups + 7) / 8;
+        const long long step_bytes = groups_per_xcd * S * (kBwdQuadCoefBytes + 4 * 64 * 2);
+        long long want = (step_bytes + 39999) / 40000;
+        const long long room = (device_cus() - grid) / 8;
+        if (want > room) want = room;
+        if (want > 8) want = 8;
+        prefetchers = (int)(want < 0 ? 0 : want);
+      }
+#ifdef XS_BQ_NOPF
+      prefetchers = 0;
+#endif
+#ifdef XS_BQ_PF
+      if (prefetchers > XS_BQ_PF) prefetchers = XS_BQ_PF;
+#endif
       q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;
       q.cut = a->recurrent_cut != 0; q.clip = clip;
       const long long n16 = (long long)kBwdRing * ngroups * 4 * 4 * a->dh * 2 / 16;
       hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
-                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
+                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + 2 * ngroups));
       void (*kq)(BwdSplitParams) = a->dh == 64 ? slstm_bwd_quad_kernel<1> : (a->dh == 128 ? slstm_bwd_quad_kernel<2> : slstm_bwd_quad_kernel<4>);
       const int lds = bwd_quad_lds_bytes();
       {
         const int rc = ensure_dynamic_lds((const void *)kq, (size_t)lds);
         if (rc != XS_OK) return rc;
       }
-      hipLaunchKernelGGL(kq, dim3((unsigned)(grid + (prefetchers ? 8 : 0))), dim3(576), lds, stream, q);
+      hipLaunchKernelGGL(kq, dim3((unsigned)(grid + 8 * prefetchers)), dim3(kBwdQuadThreads), lds, stream, q);
       const hipError_t es = hipGetLastError();
       if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
       return XS_OK;
@@ -486,14 +503,14 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.reset = a->reset; q.reset_sb = a->reset_stride_b;
       q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
       if (((uintptr_t)a->exchange % 16)) return fail(XS_ERR_ALIGN, "exchange must be 16-byte aligned");
-      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1;
+      q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1; q.placement = a->counters + 1 + ngroups;
       q.main_locals = (int)(grid / 8);
       const bool prefetchers = grid + 8 <= device_cus();  // (one more workgroup per XCD, where there is room)
       q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;  // (negative: every wait gives up at once)
       q.cut = a->recurrent_cut != 0; q.clip = clip;
       const long long n16 = (long long)kBwdRing * ngroups * 16 * 4 * a->dh * (bf16 ? 2 : 4) / 16;
       hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
-                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + ngroups));
+                         (uint4 *)a->exchange, n16, a->counters, (int)(1 + 2 * ngroups));
       void (*ks)(BwdSplitParams) = nullptr;
       bool feed = true;  // (feeder waves where the registers allow twelve waves)
       if (a->dh == 64) ks = bf16 ? slstm_bwd_split_kernel<true, 1, true> : slstm_bwd_split_kernel<false, 1, true>;

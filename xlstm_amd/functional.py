@@ -191,7 +191,7 @@ def slstm_backward(
         r_t = (r32.view(NH, 4, dh, dh).permute(0, 2, 1, 3).reshape(NH, 4 * dh, dh).to(wx.dtype)           # [NH, k, d]
                .view(NH, 8, ksteps, 4, 8, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
         exchange = torch.empty(4 * groups4 * 4 * 4 * dh, dtype=wx.dtype, device=dev)
-        counters = torch.empty(1 + groups4, dtype=torch.int32, device=dev)
+        counters = torch.empty(1 + 2 * groups4, dtype=torch.int32, device=dev)
     elif split:
         # R transposed with K ordered (owner slice, gate, unit % 64), tiled as the MFMA B operands of the workgroup
         # that owns the output columns and of the wave that owns the eighth of K:
@@ -200,7 +200,7 @@ def slstm_backward(
         r_t = (r32.view(NH, 4, S, 64, dh).permute(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh).to(wx.dtype)   # [NH, k, d]
                .view(NH, 8, ksteps, 4, epc, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
         exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=wx.dtype, device=dev)
-        counters = torch.empty(1 + groups, dtype=torch.int32, device=dev)
+        counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     else:
         # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
         r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
@@ -261,7 +261,8 @@ def slstm_backward(
             marks[-1].record()  # parameter gradients = [2] -> [3]
     if split and timings is None and int(counters[0].item()):  # (a synchronisation; training calls are not latency-bound)
         raise EngineError("xlstm_amd: a wait between the compute units of a head ran out in the backward pass "
-                          "(other work held compute units); the gradients are invalid")
+                          "(other work held compute units, or the workgroups of a head were not placed on one XCD); "
+                          "the gradients are invalid")
     return d_wx, d_r, d_bias, d_s0
 
 
