@@ -325,6 +325,8 @@ __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSpli
       }
       XS_BTICK(1);
       // ---- while the deltas are on their way: d_wx, the progress word, the next step's inputs
+      //      (with the first look issued in front of these instead of behind them, and a longer sleep in front of it, the
+      //      kernel took 2.33 ms at config 2 instead of 2.20: the look then waits for the stores behind it as well)
       if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
       if (there) {
         float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
