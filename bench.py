@@ -276,6 +276,30 @@ def bench_backward(device, iters=3):
             rev.append(ev[1].elapsed_time(ev[2]))
             par.append(ev[2].elapsed_time(ev[3]))
     rev_ms = float(np.median(rev))
+    # the same with a training forward that leaves the coefficients (no forward walk in the backward call)
+    keep = {}
+    coef = F.backward_coefficients_buffer(wx, NH)
+    if coef is not None:
+        fwd_plain, fwd_keep, tot_keep = [], [], []
+        for i in range(iters + 1):
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+            e[0].record()
+            F.slstm_forward(wx, r, bias, None, mask)
+            e[1].record()
+            F.slstm_forward(wx, r, bias, None, mask, coef_out=coef)
+            e[2].record()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            out2 = F.slstm_backward(wx, r, bias, None, mask, h, d_h, coef=coef)
+            torch.cuda.synchronize()
+            if i:
+                tot_keep.append((time.perf_counter() - t0) * 1e3)
+                fwd_plain.append(e[0].elapsed_time(e[1]))
+                fwd_keep.append(e[1].elapsed_time(e[2]))
+        keep = {"with_forward_coefficients": {
+            "backward_ms": float(np.median(tot_keep)), "forward_ms": float(np.median(fwd_keep)),
+            "plain_forward_ms": float(np.median(fwd_plain)),
+            "same_gradients": bool(torch.allclose(out2[0], out[0], rtol=0, atol=2e-3 * float(out[0].abs().max())))}}
     # what the reverse kernel has to move per step and element: nine coefficients and the four gate deltas in float32,
     # the output gradient in bf16; R transposed once (the gate deltas that the compute units of a head exchange stay in the L2)
     nbytes = (9 * 4 + 4 * 4 + 2) * B * T * H + NH * 4 * dh * dh * 2
@@ -286,7 +310,7 @@ def bench_backward(device, iters=3):
     return {"workload": "backward pass at config 2: B=16 T=2048 D=1024 NH=4 bf16, documents mean 512",
             "ms": float(np.median(total)), "prepare_kernel_ms": float(np.median(prep)), "reverse_kernel_ms": rev_ms,
             "parameter_gradient_kernel_ms": float(np.median(par)),
-            "tokens_per_s": B * T / (float(np.median(total)) * 1e-3), "finite": bool(torch.isfinite(out[0]).all()),
+            "tokens_per_s": B * T / (float(np.median(total)) * 1e-3), "finite": bool(torch.isfinite(out[0]).all()), **keep,
             "roofline": {"bound": "hbm", "achieved": nbytes / (rev_ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": nbytes / (rev_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": traffic,
                          "kernel": "slstm_bwd_quad_kernel<S=4>", "algorithmic_bytes_per_launch": nbytes,
@@ -737,6 +761,8 @@ def main():
         out["backward"] = {k: bw[k] for k in ("workload", "ms", "finite") if k in bw}
         out["backward"]["kernels_ms"] = {k: v for k, v in bw.items() if k.endswith("_ms")}
         out["backward"]["roofline"] = bw["roofline"]
+        if "with_forward_coefficients" in bw:
+            out["backward"]["with_forward_coefficients"] = bw["with_forward_coefficients"]
     if args.all_configs:
         out["all_configs"] = [
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),

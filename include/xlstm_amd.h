@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 11
+#define XS_ABI_VERSION 12
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -87,6 +87,20 @@ enum {
  *                             bit for bit the same.  The caller vouches for the
  *                             copy: it is not compared with s0.  Not in the
  *                             reference.
+ *   coef_out                  optional, xs_slstm_forward only: a training forward.  The
+ *                             nine float32 coefficients per step and element that
+ *                             xs_slstm_backward_prepare would otherwise recompute, in the
+ *                             order xs_slstm_backward reads them with split == 2:
+ *                             [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units]
+ *                             (T * ceil(B/4)*4 * 9 * H floats).  Takes the place of the
+ *                             state history and gate cache that the reference's forward
+ *                             keeps for its backward (slstm.cc:79-108).  Only where the
+ *                             call runs in row tiles of 4 rows of one kernel: bf16 wx, head
+ *                             dim 128 or 256, a batch whose row tiles of 4 rows fit the
+ *                             device; otherwise XS_ERR_UNSUPPORTED before anything is
+ *                             launched (call again without it and use
+ *                             xs_slstm_backward_prepare).  h_out and s_out are bit for bit
+ *                             those of a call without it.
  */
 typedef struct xs_slstm_args {
   int32_t B, T, NH, dh;
@@ -105,6 +119,7 @@ typedef struct xs_slstm_args {
   void *stream;
   int64_t spin_limit;
   const void *h_prev;
+  float *coef_out;
 } xs_slstm_args;
 
 /* Status block at the start of the workspace, written by the kernels. */

@@ -462,3 +462,94 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
                 d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
     print("C ABI backward", bf16, B, T, NH, dh, split, errs, flush=True)
     assert all(np.isfinite(v) and v <= tol for v in errs.values()), errs
+
+
+@pytest.mark.parametrize("B,T,NH,dh,masked", [(16, 12, 4, 256, True), (6, 9, 2, 128, True), (4, 2, 2, 128, False), (9, 33, 1, 256, True)])
+def test_a_training_forward_leaves_the_coefficients_of_the_backward_pass(B, T, NH, dh, masked):
+    """``slstm_forward(..., coef_out=)`` (the forward's kernel for row tiles of 4 rows with the gate values kept): h and
+    the state are bit for bit those of the plain call, and the backward pass that takes the coefficients instead of
+    walking forward itself returns the gradients of the one that does (the same formulas compiled into two kernels: last
+    bits of a coefficient differ, and a gate delta that the compute units exchange in bf16 then rounds the other way:
+    2e-3 of the largest entry) and the oracle's (2e-2)."""
+    from xlstm_amd import functional as F
+
+    H = NH * dh
+    print("case forward coefficients", B, T, NH, dh, masked, flush=True)
+    wx, r, b, s0 = make_problem(350, B, T, NH, dh, rscale=2.0, bf16=True, with_state=masked)
+    reset = geometric_reset_mask(351, B, T, max(2, T // 2)) if masked else None
+    if reset is not None:
+        reset[0, 0] = 0
+    rng = np.random.default_rng(352)
+    d_h = torch.from_numpy(rng.standard_normal((T, B, H)).astype(np.float32)).bfloat16().float().numpy()
+    d_sf = rng.standard_normal((4, B, H)).astype(np.float32)
+    d_sf[3] = 0.0
+    r = torch.from_numpy(r).bfloat16().float().numpy()
+    dev = torch.device("cuda:0")
+    wx_t = torch.from_numpy(wx).to(dev).bfloat16()
+    r_t, b_t = r_ext_to_kernel(torch.from_numpy(r)).to(dev), torch.from_numpy(b).to(dev)
+    s0_t = torch.from_numpy(s0).to(dev) if s0 is not None else None
+    m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
+    dh_t, dsf_t = torch.from_numpy(d_h).to(dev), torch.from_numpy(d_sf).to(dev)
+    coef = F.backward_coefficients_buffer(wx_t, NH)
+    assert coef is not None and tuple(coef.shape) == (T, (B + 3) // 4 * 4, 9, H)
+    coef.fill_(float("nan"))
+    h_plain, s_plain = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
+    h, s = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t, coef_out=coef)
+    torch.cuda.synchronize()
+    assert torch.equal(h, h_plain) and torch.equal(s, s_plain)
+    # every coefficient of a row that exists has been written
+    tiles = coef.view(T, (B + 3) // 4, NH, dh // 64, 4, 9, 64)
+    rows_there = torch.arange((B + 3) // 4 * 4, device=dev).view(-1, 4) < B
+    assert bool(torch.isfinite(tiles.permute(1, 4, 0, 2, 3, 5, 6)[rows_there]).all())
+    got = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, dh_t, dsf_t, coef=coef)
+    ref = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, dh_t, dsf_t, row_tile_override=4)
+    torch.cuda.synchronize()
+    for name, a, g in zip(("d_wx", "d_r", "d_b", "d_s0"), got, ref):
+        assert _rel(a.cpu().numpy(), g.cpu().numpy()) <= 2e-3, name
+    o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
+    errs = dict(d_wx=_rel(got[0].cpu().numpy(), o_wx), d_r=_rel(got[1].cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
+                d_b=_rel(got[2].cpu().numpy(), o_b), d_s0=_rel(got[3].cpu().numpy(), o_s0))
+    print(errs, flush=True)
+    assert all(np.isfinite(v) and v <= 2e-2 for v in errs.values()), errs
+
+
+def test_calls_that_cannot_leave_coefficients_say_so_before_anything_runs():
+    """float32 inputs, head dims other than 128 and 256, batches whose row tiles of 4 rows do not fit the device: no
+    buffer is offered, and a call that is handed one all the same raises ``CoefficientsUnsupported``."""
+    from xlstm_amd import functional as F
+
+    dev = torch.device("cuda:0")
+    assert F.backward_coefficients_buffer(torch.zeros(4, 8, 4 * 256, device=dev), 2) is None                             # float32
+    assert F.backward_coefficients_buffer(torch.zeros(4, 8, 4 * 128, device=dev, dtype=torch.bfloat16), 2) is None        # head dim 64
+    assert F.backward_coefficients_buffer(torch.zeros(300, 8, 4 * 1024, device=dev, dtype=torch.bfloat16), 4) is None     # too many rows
+    B, T, NH, dh = 300, 3, 4, 256
+    H = NH * dh
+    wx = torch.randn(B, T, 4 * H, device=dev).bfloat16()
+    r = torch.randn(NH, 4 * dh, dh, device=dev) * 0.05
+    b = torch.zeros(NH, 4, dh, device=dev)
+    coef = torch.empty(T, (B + 3) // 4 * 4, 9, H, device=dev)
+    with pytest.raises(F.CoefficientsUnsupported):
+        F.slstm_forward(wx, r, b, coef_out=coef)
+    h, _ = F.slstm_forward(wx, r, b)  # the plain call is the usual one
+    assert bool(torch.isfinite(h.float()).all())
+
+
+def test_cell_that_keeps_the_backward_coefficients_has_the_same_gradients():
+    from tests.test_hip_cell import _cell_from
+
+    B, T, NH, dh = 8, 16, 2, 128
+    wx, r, b, s0 = make_problem(360, B, T, NH, dh, rscale=2.0, bf16=True, with_state=True)
+    r = torch.from_numpy(r).bfloat16().float().numpy()
+    mask = torch.from_numpy(geometric_reset_mask(361, B, T, 6)).cuda()
+    w = torch.randn(B, NH, T, dh, generator=torch.Generator().manual_seed(9)).cuda()
+    grads = []
+    for keep in (False, True):
+        cell = _cell_from(r, b, dtype="bfloat16").train()
+        cell.keep_backward_coefficients = keep
+        x = torch.from_numpy(wx).cuda().bfloat16().requires_grad_(True)
+        st = torch.from_numpy(s0).cuda().bfloat16().requires_grad_(True)
+        out, _ = cell(x, st, reset_mask=mask)
+        (out.float() * w).sum().backward()
+        grads.append((x.grad.float(), cell._recurrent_kernel_.grad.float(), cell._bias_.grad.float(), st.grad.float()))
+    for a, g in zip(grads[1], grads[0]):
+        assert float((a - g).abs().max()) <= 2e-3 * max(1.0, float(g.abs().max()))

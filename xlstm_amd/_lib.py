@@ -13,8 +13,9 @@ PKG = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_amd.so"))
 
 XS_F32, XS_BF16 = 0, 1
+XS_ERR_UNSUPPORTED = -5
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 EXPORTS = (
     "xs_abi_version",
@@ -53,6 +54,7 @@ class SlstmArgs(ctypes.Structure):
         ("stream", ctypes.c_void_p),
         ("spin_limit", ctypes.c_int64),
         ("h_prev", ctypes.c_void_p),
+        ("coef_out", ctypes.c_void_p),
     ]
 
 

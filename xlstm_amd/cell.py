@@ -196,9 +196,10 @@ class _CellFunction(torch.autograd.Function):
     what the forward call returned for ``x, r, bias, state, mask``; nothing else is stored for the backward."""
 
     @staticmethod
-    def forward(ctx, x, r, bias, state, h, s, mask, num_heads, cut, clipval):
+    def forward(ctx, x, r, bias, state, h, s, mask, num_heads, cut, clipval, coef):
         ctx.save_for_backward(x, r, bias, h, *(() if state is None else (state,)))
         ctx.mask, ctx.num_heads, ctx.cut, ctx.clipval = mask, num_heads, cut, clipval
+        ctx.coef = coef  # (what a training forward left for the backward pass, or None: see keep_backward_coefficients)
         return h.view_as(h), s.view_as(s)
 
     @staticmethod
@@ -208,9 +209,10 @@ class _CellFunction(torch.autograd.Function):
         NH, dh = ctx.num_heads, r.shape[2]
         d_wx, d_r, d_bias, d_s0 = F_hip.slstm_backward(
             x.detach(), r.detach(), bias.detach().view(NH, 4, dh), None if state is None else state.detach(), ctx.mask,
-            h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval)
+            h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval, coef=ctx.coef)
+        ctx.coef = None
         return (d_wx.to(x.dtype), d_r.to(r.dtype), d_bias.reshape(bias.shape).to(bias.dtype),
-                None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None)
+                None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None, None)
 
 
 class _Runtime:
@@ -244,6 +246,13 @@ class sLSTMCell_hip(nn.Module):
     """
 
     config_class = sLSTMCellConfig
+
+    #: Training: let the forward call leave the backward pass its coefficients (36 bytes per step and element, held
+    #: until the backward has run) where it can - bfloat16 inputs, head dim 128 or 256, a batch whose row tiles of 4
+    #: rows fit the device - instead of having the backward pass recompute them in a forward walk of its own.  The
+    #: reference's native forward always keeps its states and gate values (slstm.cc:79-108); here the default keeps
+    #: nothing.  The gradients are the same either way.
+    keep_backward_coefficients: bool = False
 
     def __init__(self, config: sLSTMCellConfig, skip_backend_init: bool = False):
         super().__init__()
@@ -487,27 +496,30 @@ class sLSTMCell_hip(nn.Module):
         if step and x.dtype == torch.bfloat16:
             r = self._bf16_recurrent_kernel()  # the step kernel reads R every token: keep it in the operand type
         ws = self._workspace(B, x.device) if x.is_cuda else None
-        h, s = F_hip.slstm_forward(
-            x,
-            r,
-            self._bias_.detach().view(self.config.num_heads, 4, self.head_dim),
-            state,
-            reset_mask,
-            step=step,
-            s_out=state_out,
-            workspace=ws,
+        wants_grad = torch.is_grad_enabled() and (
+            input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
+            or (state is not None and state.requires_grad)
         )
+        args = (x, r, self._bias_.detach().view(self.config.num_heads, 4, self.head_dim), state, reset_mask)
+        coef = None
+        if wants_grad and self.keep_backward_coefficients and x.is_cuda and not step:
+            coef = F_hip.backward_coefficients_buffer(x, self.config.num_heads)
+        h = s = None
+        if coef is not None:
+            try:
+                h, s = F_hip.slstm_forward(*args, s_out=state_out, workspace=ws, coef_out=coef)
+            except F_hip.CoefficientsUnsupported:  # (nothing has run: the plain forward, and the backward recomputes)
+                coef = None
+        if h is None:
+            h, s = F_hip.slstm_forward(*args, step=step, s_out=state_out, workspace=ws)
         self._rt.last_workspace = ws
         if not step and x.shape[1] > 1:
             self._watch(ws)
-        if torch.is_grad_enabled() and (
-            input.requires_grad or self._recurrent_kernel_.requires_grad or self._bias_.requires_grad
-            or (state is not None and state.requires_grad)
-        ):
+        if wants_grad:
             if x.is_cuda and self.head_dim <= BACKWARD_MAX_HEAD_DIM.get(x.dtype, 0):
                 h, s = _CellFunction.apply(x, self._recurrent_kernel_, self._bias_, state, h, s, reset_mask,
                                            self.config.num_heads, bool(self.config.gradient_recurrent_cut),
-                                           self.config.gradient_recurrent_clipval)
+                                           self.config.gradient_recurrent_clipval, coef)
             else:
                 h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
         output = self._permute_output(h)

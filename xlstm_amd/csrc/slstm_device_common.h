@@ -81,6 +81,23 @@ __device__ __forceinline__ void slstm_pointwise(float iraw, float fraw, float zr
   s.c = cnew; s.n = nnew; s.m = mnew;
 }
 
+// The same update with the gate values kept (a training forward leaves the backward pass its coefficients): the same
+// expressions in the same order, so the state and y have the bits of slstm_pointwise.
+struct GateValues { float og, ig, fg, tz, rn; };
+__device__ __forceinline__ void slstm_pointwise_keep(float iraw, float fraw, float zraw, float oraw, CellState &s, GateValues &k) {
+  const float lfm = s.m + (fminf(fraw, 0.0f) - 0.69314718055994531f * __builtin_amdgcn_logf(1.0f + __expf(-fabsf(fraw))));
+  const float mnew = (s.n == 0.0f) ? iraw : fmaxf(iraw, lfm);
+  k.og = __builtin_amdgcn_rcpf(1.0f + __expf(-oraw));
+  k.ig = fminf(__expf(iraw - mnew), 1.0f);
+  k.fg = fminf(__expf(lfm - mnew), 1.0f);
+  k.tz = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __expf(2.0f * zraw));
+  const float cnew = k.fg * s.c + k.ig * k.tz;
+  const float nnew = k.fg * s.n + k.ig;
+  k.rn = __builtin_amdgcn_rcpf(nnew);
+  s.y = k.og * cnew * k.rn;
+  s.c = cnew; s.n = nnew; s.m = mnew;
+}
+
 // ---------------------------------------------------------------------------
 // fill kernels (plain vector stores; also used instead of memset so that a
 // caller may capture the call in a graph)

@@ -323,9 +323,17 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
       kern = bf16 ? (full ? pick_kernel<true, true>(nch, MT, burst) : pick_kernel<true, false>(nch, MT, burst))
                   : (full ? pick_kernel<false, true>(nch, MT, burst) : pick_kernel<false, false>(nch, MT, burst));
     // row tiles of at most 4 rows, bf16, whole K ranges up to 512: the compute waves split the columns by unit, not K
-    if (bf16 && MT == 1 && rows_per_wg == 4 && full && nch <= 4 && G <= 32) {
+    const bool quad = bf16 && MT == 1 && rows_per_wg == 4 && full && nch <= 4 && G <= 32;
+    if (quad) {
       kern = nch == 1 ? slstm_seq_kernel<true, 1, 1, true, false, false, true>
                       : (nch == 2 ? slstm_seq_kernel<true, 2, 1, true, false, false, true> : slstm_seq_kernel<true, 4, 1, true, false, false, true>);
+    }
+    if (a->coef_out) {  // a training forward: the same kernel, leaving the backward pass its coefficients
+      if (!quad || (dh != 128 && dh != 256) || rows_per_launch < B)
+        return fail(XS_ERR_UNSUPPORTED, "coef_out: the call does not run in row tiles of 4 rows of one kernel (bf16, head dim 128 or 256, "
+                                        "ceil(B/4) * NH * dh/16 workgroups on the device at once)");
+      if (((uintptr_t)a->coef_out % 4)) return fail(XS_ERR_ALIGN, "coef_out must be 4-byte aligned");
+      kern = nch == 1 ? slstm_seq_kernel<true, 1, 1, true, false, false, true, true> : slstm_seq_kernel<true, 2, 1, true, false, false, true, true>;
     }
 #ifdef XS_SMALL_BATCH_FMA
     // the measured alternative for small batches (see the kernel): only in a library built for that measurement
@@ -368,6 +376,7 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
     p.b0 = b0; p.bend = bend; p.G = G; p.NBT = NBT; p.rows_per_wg = rows_per_wg;
     p.head0 = head0; p.NHL = NHL;
     p.spin_limit = a->spin_limit;
+    p.coef_out = a->coef_out;
     // a prefetch wave issues 2 (bf16) or 4 (fp32) scalar loads per batch row of a tile; 8 per wave and iteration
     // and 16 in all are what the scalar cache sustains, a tile that needs more goes without (prefetch waves that
     // fall behind hold up the barriers: measured 2x slower)
@@ -844,6 +853,13 @@ int xs_slstm_forward(const xs_slstm_args *args) {
   g_err[0] = 0;
   const int rc = validate(args, false);
   if (rc != XS_OK) return rc;
+  if (args->coef_out) {  // a training forward: is this one of the calls that can leave the coefficients? (launches nothing)
+    if (args->T < 1 || args->B < 1) return fail(XS_ERR_UNSUPPORTED, "coef_out: nothing to do for an empty call");
+    size_t need = 0;
+    const int rd = run_forward(args, &need);
+    if (rd != XS_OK) return rd;
+    return run_forward(args);  // (also for one token: the step kernels keep no gate values)
+  }
   // one token: the tiled step kernel (no waits between compute units, bit-identical to the sequence kernel)
   if (args->T == 1 && args->B > 0 && args->r_dtype == args->wx_dtype) return run_step(args);
   return run_forward(args);
@@ -853,6 +869,7 @@ int xs_slstm_forward_static(const xs_slstm_args *args) {
   g_err[0] = 0;
   int rc = validate(args, false, true);
   if (rc != XS_OK) return rc;
+  if (args->coef_out) return fail(XS_ERR_UNSUPPORTED, "coef_out goes with xs_slstm_forward");
   xs_slstm_args a = *args;
   rc = static_scratch(&a.workspace);
   if (rc != XS_OK) return rc;
@@ -871,6 +888,7 @@ int xs_slstm_step(const xs_slstm_args *args) {
   g_err[0] = 0;
   const int rc = validate(args, true);
   if (rc != XS_OK) return rc;
+  if (args->coef_out) return fail(XS_ERR_UNSUPPORTED, "coef_out goes with xs_slstm_forward");
   return run_step(args);
 }
 

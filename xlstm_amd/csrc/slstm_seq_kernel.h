@@ -27,6 +27,8 @@ struct SeqParams {
   int rows_per_wg;
   long long spin_limit;
   int prefetch;  // number of prefetch waves launched behind the six others (0 .. kMaxPrefetchWaves)
+  float *coef_out;  // COEF variant: the backward pass's nine coefficients per step and element,
+                    // [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units] (what slstm_bwd_quad_kernel reads); else unused
 };
 
 // ---------------------------------------------------------------------------
@@ -155,8 +157,11 @@ __device__ __forceinline__ uint32_t seq_handshake(const SeqParams &p, int wg, in
 // order than the MFMA forms them, so the bits differ from the MFMA path (and from the decode kernel).
 // QUAD: row tiles of at most 4 rows (bf16, FULL, one row tile): the four compute waves split the workgroup's 64
 // columns by UNIT instead of splitting K, see "waves 0-3, QUAD" below.
-template <bool BF16, int NCH, int MT, bool FULL, bool BURST, bool FMAC = false, bool QUAD = false>
+// COEF (with QUAD): a training forward: the compute waves also leave the nine coefficients per step and element that the
+// backward pass would otherwise recompute in a forward walk of its own (slstm_bwd_prepare_kernel), see "COEF" below.
+template <bool BF16, int NCH, int MT, bool FULL, bool BURST, bool FMAC = false, bool QUAD = false, bool COEF = false>
 __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm_seq_kernel(SeqParams p) {
+  static_assert(!COEF || QUAD, "coefficients for the backward pass come from the unit-split compute waves only");
   static_assert(!FMAC || MT == 1, "the FMA contraction is for one row tile of at most 4 rows");
   static_assert(!QUAD || (BF16 && MT == 1 && FULL && !BURST && !FMAC), "the unit-split compute waves exist for bf16, one full row tile");
   constexpr int EPC = BF16 ? 8 : 4;      // elements per 16-byte chunk
@@ -169,6 +174,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
   __shared__ float part[2][4][4][kTileFloats];  // [buffer][wave][gate][unit*stride + row]
   __shared__ float wxs[2][4][kTileFloats];      // [slot][gate][row*stride + unit]   W.x of one iteration
   __shared__ float hst[4][256];                 // [slot][row*16 + unit]             h on its way to HBM
+  __shared__ float cst[COEF ? 4 : 1][COEF ? 9 * 64 : 1];  // [slot][coefficient][row*16 + unit]  (COEF) on their way to HBM
   __shared__ uint32_t rfl[4][16];               // [slot][row]                       reset flags
   __shared__ uint32_t cross_s;
 
@@ -342,6 +348,24 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         }
       }
     };
+    // COEF: the coefficients of step t are staged one iteration later than its h (in the shadow of the next step's
+    // poll), between barriers #t+1 and #t+2, and leave three iterations behind: 4 rows x 9 coefficients x 16 units into
+    // the piece of the (row tile, head, slice of 64 units) that the backward's reverse kernel reads per step
+    float *coef_dst = nullptr;
+    long long coef_step = 0;
+    if constexpr (COEF) {
+      const int ntiles = (p.B + 3) >> 2, S = dh >> 6;
+      coef_step = (long long)ntiles * p.NH * S * (4 * 9 * 64);
+      coef_dst = p.coef_out + ((((long long)(rowbase >> 2)) * p.NH + head) * S + (a0 >> 6)) * (4 * 9 * 64)
+                 + (lane >> 4) * (9 * 64) + (a0 & 63) + (lane & 15);
+    }
+    auto drain_coef = [&](int t) {
+      if constexpr (COEF) {
+        float *dst = coef_dst + t * coef_step;
+#pragma unroll
+        for (int j = 0; j < 9; ++j) dst[j * 64] = cst[t & 3][j * 64 + lane];
+      }
+    };
     lds_barrier();  // prologue barrier
 #ifdef XS_PROFILE
     long long dprof[2] = {0, 0};
@@ -349,6 +373,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #endif
     for (int j = 0; j < NITpad; ++j) {
       if (j >= 2 && j - 2 < NIT) drain(j - 2);
+      if (COEF && j >= 3 && j - 3 < NIT) drain_coef(j - 3);
 #ifdef XS_PROFILE
       { const long long now_ = clock64(); dprof[0] += now_ - dt; dt = now_; }
 #endif
@@ -359,6 +384,8 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     }
     lds_barrier();  // final barrier
     for (int it = (NITpad >= 2 ? NITpad - 2 : 0); it < NIT; ++it) drain(it);
+    if (COEF)
+      for (int it = (NITpad >= 3 ? NITpad - 3 : 0); it < NIT; ++it) drain_coef(it);
     // A bounded wait ran out somewhere: whatever this workgroup computed from then on is built on operands that
     // never arrived.  A caller that does not read the status block must not mistake it for a result, so the
     // workgroup's part of h_out becomes NaN (the compute waves do the same to s_out).  Any workgroup that consumed
@@ -462,6 +489,26 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
     }
     bool aborted = false;
     uint32_t max_spins = 0;
+    // COEF: what the coefficients of the step before are made of, kept until the next step's poll is out
+    GateValues kept{0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+    float kept_y = 0.0f, kept_c = 0.0f, kept_n = 0.0f, kept_f = 0.0f;
+    auto stage_coefficients = [&](int t) {  // the nine coefficients of step t (see slstm_bwd_prepare_kernel) -> LDS
+      if constexpr (COEF) {
+        const float omf = __builtin_amdgcn_rcpf(1.0f + __expf(kept_f));  // 1 - sigmoid(f)
+        if (gate_lane) {
+          float *dst = &cst[t & 3][gb * 16 + gu];
+          dst[0 * 64] = kept.og * kept.rn;
+          dst[1 * 64] = kept_y * kept.rn;
+          dst[2 * 64] = kept.ig * kept.tz;
+          dst[3 * 64] = kept.ig;
+          dst[4 * 64] = kept.fg * omf * kept_c;
+          dst[5 * 64] = kept.fg * omf * kept_n;
+          dst[6 * 64] = kept.ig * (1.0f - kept.tz * kept.tz);
+          dst[7 * 64] = (1.0f - kept.og) * kept_y;
+          dst[8 * 64] = kept.fg;
+        }
+      }
+    };
 #ifdef XS_PROFILE
     long long qprof[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     long long qtick = clock64();
@@ -520,6 +567,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks)
           areg[ks] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(hrs, xl, ks * 2 * QTILE, 16));
+        stage_coefficients(t - 1);  // (COEF; while the poll is on its way)
       } else {
 #pragma unroll
         for (int ks = 0; ks < NK; ++ks) {
@@ -593,7 +641,13 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
 #endif
       XS_QTICK(7);
       if (gate_reset) st = CellState{0.0f, 0.0f, 0.0f, 0.0f};
-      slstm_pointwise(raw0, raw1, raw2, raw3, st);
+      if constexpr (COEF) {
+        kept_c = st.c; kept_n = st.n; kept_f = raw1;
+        slstm_pointwise_keep(raw0, raw1, raw2, raw3, st, kept);
+        kept_y = st.y;
+      } else {
+        slstm_pointwise(raw0, raw1, raw2, raw3, st);
+      }
       const float y = st.y;
 #ifdef XS_PROFILE
       asm volatile("" :: "v"(y));
@@ -615,6 +669,7 @@ __global__ __launch_bounds__(kThreads + 64 * max_prefetch_waves(NCH)) void slstm
         asm volatile("" :: "v"(areg[ks].x), "v"(areg[ks].y), "v"(areg[ks].z), "v"(areg[ks].w));
       XS_QTICK(4);
     }
+    if (COEF && p.T > 0) stage_coefficients(p.T - 1);
     for (int j = NIT; j < NITpad; ++j) lds_barrier();  // padding iterations of the feeder
     lds_barrier();                                     // final barrier
 #ifdef XS_PROFILE

@@ -61,6 +61,28 @@ def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
     return None
 
 
+class CoefficientsUnsupported(EngineError):
+    """A forward call was asked to leave the backward pass its coefficients and is not one of those that can."""
+
+
+def backward_coefficients_buffer(wx: torch.Tensor, num_heads: int) -> Optional[torch.Tensor]:
+    """The tensor a training forward (``slstm_forward(..., coef_out=)``) leaves the backward pass's coefficients in, or
+    ``None`` where the forward cannot: it takes bfloat16 inputs, a head dim of 128 or 256 and a batch whose row tiles of
+    4 rows fit the device in the forward (``ceil(B/4) * NH * dh/16`` workgroups) and, with their prefetching workgroups,
+    in the backward.  36 bytes per step and element, held from the forward to the backward (the reference keeps the
+    states and gate values of every step instead, ``slstm.cc:79-108``); without it the backward pass recomputes them."""
+    B, T = int(wx.shape[0]), int(wx.shape[1])
+    H = int(wx.shape[2]) // 4
+    dh = H // num_heads
+    if wx.dtype != torch.bfloat16 or dh not in (128, 256) or B < 1 or T < 2:
+        return None
+    cus = _compute_units(wx.device)
+    groups4 = num_heads * ((B + 3) // 4)
+    if (groups4 + 7) // 8 * 8 * (dh // 16) > cus or (groups4 + 7) // 8 * 8 * (dh // 64) + 8 > cus:
+        return None
+    return torch.empty((T, (B + 3) // 4 * 4, 9, H), dtype=torch.float32, device=wx.device)
+
+
 def slstm_backward(
     wx: torch.Tensor,
     r: torch.Tensor,
@@ -74,6 +96,7 @@ def slstm_backward(
     split_override: Optional[bool] = None,
     spin_limit: int = 0,
     row_tile_override: Optional[int] = None,
+    coef: Optional[torch.Tensor] = None,
     recurrent_cut: bool = False,
     recurrent_clipval: Optional[float] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -92,6 +115,7 @@ def slstm_backward(
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel), in row tiles of 4 rows where four times the workgroups fit (bfloat16, head dims up to 256;
     ``row_tile_override`` = 16 or 4 forces either); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
+    ``coef``: what a training forward left (``slstm_forward(..., coef_out=)``); the forward walk is then skipped.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
     to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
     clipped to +-value before ``d_h`` is added, ``slstm_pointwise.cu:136-143``).
@@ -107,6 +131,9 @@ def slstm_backward(
     if tuple(h_out.shape) != (T, B, H) or tuple(d_h.shape) != (T, B, H):
         raise ValueError(f"h_out and d_h must be [S, B, H] = {(T, B, H)}")
     dh_k = backward_kernel_head_dim(dh, wx.dtype)
+    if coef is not None and (dh_k != dh or not bf16 or tuple(coef.shape) != (T, (B + 3) // 4 * 4, 9, H)
+                             or coef.dtype != torch.float32 or not coef.is_contiguous()):
+        raise ValueError("coef must be the tensor that the forward call of the same inputs filled")
     if dh_k is None:
         raise EngineError(f"xlstm_amd: no backward kernel for head dim {dh} with {wx.dtype} inputs "
                           f"(up to 512 with bfloat16, up to 256 with float32)")
@@ -138,7 +165,7 @@ def slstm_backward(
     # The kernel that spreads a head over dh/64 compute units needs all its workgroups on the device at once.  A batch
     # with more row tiles than that runs in slices of rows (rows do not meet in the backward pass but in the sums for
     # R and the bias), rather than with one workgroup per head, which takes 7 times as long per step.
-    if split_override is not False:
+    if split_override is not False and coef is None:
         room = (_compute_units(dev) - 8) // (8 * (dh // 64)) * 8      # groups per launch, the prefetching workgroups kept
         tiles_per_launch = room // NH
         if tiles_per_launch >= 1 and (B + 15) // 16 > tiles_per_launch:
@@ -182,8 +209,14 @@ def slstm_backward(
             and (reset_mask is None or 3 * reset_mask.stride(0) + T < 2 ** 31 - 256))
     if row_tile_override is not None:
         quad = split and row_tile_override == 4
+    if coef is not None:
+        if not (split and quad):
+            raise EngineError("xlstm_amd: coefficients from the forward call go with the reverse kernel for row tiles of 4 rows, "
+                              "which this call does not run")
     # (the split kernels read the coefficients in pieces of a row tile: the buffer covers whole row tiles)
-    coef = torch.empty((T, ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else B, 9, H), dtype=torch.float32, device=dev)
+    coef_given = coef is not None
+    if not coef_given:
+        coef = torch.empty((T, ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else B, 9, H), dtype=torch.float32, device=dev)
     if quad:
         # R transposed with K ordered (unit, gate), tiled as the MFMA B operands of the workgroup that owns the output
         # columns and of the wave that owns the eighth of K: [NH][S][8 waves][k-steps of a wave][4 column blocks][k / 8 % 4][column % 16][k % 8]
@@ -238,6 +271,11 @@ def slstm_backward(
     marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
+            if coef_given and fn is lib.xs_slstm_backward_prepare:
+                if timings is not None:
+                    marks.append(torch.cuda.Event(enable_timing=True))
+                    marks[-1].record()
+                continue
             if timings is not None:
                 marks.append(torch.cuda.Event(enable_timing=True))
                 marks[-1].record()
@@ -294,8 +332,13 @@ def slstm_forward(
     s_out: Optional[torch.Tensor] = None,
     spin_limit: int = 0,
     h_prev: Optional[torch.Tensor] = None,
+    coef_out: Optional[torch.Tensor] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Runs the cell over ``wx`` and returns ``(h[S,B,H] in wx.dtype, state[4,B,H] float32)``.
+
+    ``coef_out`` (a training forward; a float32 tensor from ``backward_coefficients_buffer``): the kernel also leaves
+    the coefficients of the backward pass there, and ``slstm_backward(..., coef=coef_out)`` skips its own forward walk.
+    Raises ``CoefficientsUnsupported`` (nothing has run) for calls that cannot: see ``backward_coefficients_buffer``.
 
     ``reset_mask[B,S]`` (bool/uint8) marks document starts: the row's state is
     zeroed before that step.  ``step=True`` uses the decode entry point (S == 1).
@@ -378,9 +421,18 @@ def slstm_forward(
         if h_prev.dtype != torch.bfloat16 or h_prev.numel() != B * H or not h_prev.is_contiguous():
             raise ValueError(f"h_prev must be a contiguous bfloat16 tensor of {B * H} elements")
         a.h_prev = h_prev.data_ptr()
+    a.coef_out = None
+    if coef_out is not None:
+        if step:
+            raise CoefficientsUnsupported("xlstm_amd: a decode step keeps no coefficients")
+        if coef_out.dtype != torch.float32 or not coef_out.is_contiguous() or coef_out.numel() != T * ((B + 3) // 4 * 4) * 9 * H:
+            raise ValueError("coef_out must be the tensor backward_coefficients_buffer returns for this call")
+        a.coef_out = coef_out.data_ptr()
     with torch.cuda.device(dev):
         rc = (lib.xs_slstm_step if step else lib.xs_slstm_forward)(ctypes.byref(a))
     if rc != 0:
+        if coef_out is not None and rc == _lib.XS_ERR_UNSUPPORTED:
+            raise CoefficientsUnsupported(f"xlstm_amd error {rc}: {_lib.last_error()}")
         raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
     return h_out, s_out
 
