@@ -570,62 +570,98 @@ __global__ __launch_bounds__(256) void slstm_bwd_arm_kernel(uint4 *xch, long lon
     for (int i = threadIdx.x; i < nwords; i += blockDim.x) words[i] = 0u;
 }
 
-// One workgroup per XCD that brings what the XCD's groups will read from memory - coefficients and d_h - into the XCD's
+// Prefetching workgroups: they bring what an XCD's groups will read from memory - coefficients and d_h - into the XCD's
 // L2, a few steps ahead of them.  A compute unit returns its loads in the order they were issued, whichever wave issued
 // them: a miss that goes to HBM holds up every poll of the exchange ring behind it, and a step took 2.7 us at config 2
 // with the inputs fetched by the workgroup itself (by its polling waves or by others, one step ahead or two) against
-// 2.0 us with inputs that were already in the L2.  So another compute unit takes the misses.  Nothing depends on
-// these workgroups: they follow the groups' progress words at a distance, and stop when those stop.
-constexpr int kBwdAhead = 12;  // steps the prefetch may run ahead (1.2 MiB of a 4 MiB L2 at config 2)
-template <bool BF16, int ROWS = 16>  // ROWS: batch rows of a row tile
-__device__ __forceinline__ void bwd_prefetch(const BwdSplitParams &p, int xcd) {
+// 2.0 us with inputs that were already in the L2.  So other compute units take the misses.  Nothing depends on these
+// workgroups: they follow the groups' progress words at a distance, and stop when those stop.
+//
+// `which` of the `of` prefetching workgroups of this XCD (a compute unit draws some 65 GB/s from memory: the host
+// launches as many as the XCD's groups need); they share a step's lines by position.  The groups' progress words are
+// read by the lanes of one wave side by side, the lines of a step - the coefficients and d_h of all groups of the XCD -
+// are dealt out over the threads as one flat range, and a workgroup that has fallen behind what the feeder waves have
+// already asked for skips ahead.  (An earlier version, one workgroup per XCD with a call per group and tensor and the
+// progress words read one after the other, took longer than the compute units take for the step once an XCD held more
+// than two or three groups; the feeder waves then missed to HBM, every poll of their compute unit came back behind those
+// misses, and at the end the prefetch kept the kernel alive for as long again: 5 us per step at B 64 x 4 heads of 256
+// instead of 2, 16 at B 192.)
+constexpr int kBwdAhead = 12;  // steps the prefetch may run ahead at most (1.2 MiB of a 4 MiB L2 at config 2)
+// ROWS: batch rows of a row tile; DEPTH: steps the feeder waves ask ahead
+template <bool BF16, int S, int ROWS, int DEPTH>
+__device__ __forceinline__ void bwd_tile_prefetch(const BwdSplitParams &p, int xcd, int which, int of) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  const int S = p.dh >> 6, H = p.NH * p.dh, NT = (p.B + ROWS - 1) / ROWS, ngroups = p.NH * NT;
-  const int tid = threadIdx.x, nthreads = blockDim.x;
-  if (xcd >= ngroups) return;
+  constexpr int dh = 64 * S;
+  constexpr int PIECE = ROWS * 9 * 64 * 4;          // bytes of a workgroup's coefficients of one step
+  constexpr int CL = S * PIECE / 128;               // lines of a group's coefficients of one step (its S workgroups' pieces lie in a row)
+  constexpr int PER_ROW = dh * ESZ / 128;           // lines of a row of d_h
+  constexpr int DL = ROWS * PER_ROW;
+  const int H = p.NH * dh, ntiles = (p.B + ROWS - 1) / ROWS, ngroups = p.NH * ntiles;
+  const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63;
+  if (xcd >= ngroups || of < 1) return;
+  const int G = (ngroups - xcd + 7) >> 3;           // groups of this XCD: xcd, xcd + 8, ...
+  // steps the prefetch may run ahead of the groups' progress: about 2 MiB of the XCD's 4 MiB L2, and more than the
+  // feeder waves run ahead
+  int ahead = (2 << 20) / (G * (CL + DL) * 128);
+  ahead = ahead > kBwdAhead ? kBwdAhead : (ahead < DEPTH + 2 ? DEPTH + 2 : ahead);
   // A touch is a load that writes LDS, not a register: nothing waits for these loads before the end, and a register
   // that a load in flight is going to write would be handed out again by the compiler in the meantime.  Every touch of
   // every wave lands in the same kilobyte, which nobody reads.
   __shared__ uint4 dump[64];
   const uint32_t dump_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dump);
-  auto touch_lines = [&](const char *base, int bytes, int first_line, int lines, int line_stride_lines, int per_run) {
-    // lines first_line + tid, + nthreads, ... of `lines`; line l is at base + ((l / per_run) * line_stride_lines + l % per_run) * 128
-    const unsigned long long b = reinterpret_cast<unsigned long long>(base);
-    const u32x4_t rs = {uniform((uint32_t)b), uniform((uint32_t)(b >> 32) & 0xFFFFu), (uint32_t)bytes, 0x00020000u};
-    for (int l0 = first_line; l0 < lines; l0 += nthreads) {  // (uniform trip count: lanes past the end ask past the buffer's end)
-      const int l = l0 + tid;
-      const int off = l < lines ? ((l / per_run) * line_stride_lines + l % per_run) * 128 : 0x7FFFFF00;
-      lds_direct_fetch_b128(rs, uniform(dump_lds), off);
-    }
-  };
-  __shared__ int stop;
-  if (tid == 0) stop = 0;
-  __syncthreads();
-  for (int m0 = 0; m0 < p.T; m0 += 4) {
-    if (m0 >= kBwdAhead) {
-      if (tid == 0) {
-        for (int g = xcd; g < ngroups && !stop; g += 8) {
-          int spins = 0;
-          while ((int)__hip_atomic_load(p.progress + g, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + kBwdAhead < m0) {
-            if (++spins > (1 << 16) || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) { stop = 1; break; }
-            __builtin_amdgcn_s_sleep(8);
+  __shared__ int slowest;      // the least progress among the XCD's groups; -1: stop
+  const long long coef_step = (long long)ngroups * S * PIECE;  // bytes of one step's coefficients, all groups
+  const long long dh_step = (long long)p.B * H * ESZ;
+  for (int m = 0; m < p.T; ++m) {
+    if (m >= ahead && (m & 1) == 0) {  // (every other step: the groups' progress is read through the L2)
+      if (tid == 0) slowest = 0x7FFFFFFF;
+      __syncthreads();
+      if (tid < 64) {
+        int spins = 0;
+        for (;;) {
+          int least = 0x7FFFFFFF;
+          for (int j = lane; j < G; j += 64) {
+            const int at = (int)__hip_atomic_load(p.progress + xcd + 8 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            least = at < least ? at : least;
           }
+          if (__builtin_amdgcn_ballot_w64(least < m - ahead) == 0ull) {  // (lanes without a group: the largest int)
+            if (lane < G) atomicMin(&slowest, least);
+            break;
+          }
+          if (++spins > (1 << 16) || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
+            if (lane == 0) slowest = -1;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
         }
       }
       __syncthreads();
-      if (stop) break;
+      const int at = slowest;
+      if (at < 0) break;
+      // (fallen behind what the feeder waves have already asked for: skip to where a touch can still come first)
+      if (m < at + DEPTH + 1) m = (at + DEPTH + 1) & ~1;
+      if (m >= p.T) break;
     }
-    for (int m = m0; m < m0 + 4 && m < p.T; ++m) {
-      const int t = p.T - 1 - m;
-      for (int g = xcd; g < ngroups; g += 8) {
-        const int head = g % p.NH, tile = g / p.NH, row0 = tile * ROWS;
-        const int piece_lines = ROWS * 9 * 64 * 4 / 128;
-        const char *cbase = reinterpret_cast<const char *>(p.coef) + ((((long long)t * NT + tile) * p.NH + head) * S) * (piece_lines * 128ll);
-        touch_lines(cbase, S * piece_lines * 128, 0, S * piece_lines, 1, 1);
-        const int rows = p.B - row0 < ROWS ? p.B - row0 : ROWS, per_row = p.dh * ESZ / 128;
-        const char *dbase = reinterpret_cast<const char *>(p.d_h) + (((long long)t * p.B + row0) * H + (long long)head * p.dh) * ESZ;
-        touch_lines(dbase, ((rows - 1) * H + p.dh) * ESZ, 0, rows * per_row, H * ESZ / 128, per_row);
-      }
+    const int t = p.T - 1 - m;
+    const unsigned long long cb = reinterpret_cast<unsigned long long>(p.coef) + (unsigned long long)(t * coef_step);
+    const unsigned long long db = reinterpret_cast<unsigned long long>(p.d_h) + (unsigned long long)(t * dh_step);
+    const u32x4_t crs = {uniform((uint32_t)cb), uniform((uint32_t)(cb >> 32) & 0xFFFFu), uniform((uint32_t)coef_step), 0x00020000u};
+    const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), uniform((uint32_t)dh_step), 0x00020000u};
+    // (uniform trip counts: lanes past the end ask past the buffer's end)
+    for (int i0 = which * nthreads; i0 < G * CL; i0 += of * nthreads) {
+      const int i = i0 + tid;
+      const int j = i / CL, l = i - j * CL;
+      const int g = xcd + 8 * j, head = g % p.NH, tile = g / p.NH;
+      const uint32_t coff = i < G * CL ? (uint32_t)(((tile * p.NH + head) * S) * PIECE + l * 128) : 0xFFFFFF00u;
+      bwd_fetch_to_lds_b128(crs, uniform(dump_lds), coff);
+    }
+    for (int i0 = which * nthreads; i0 < G * DL; i0 += of * nthreads) {
+      const int i = i0 + tid;
+      const int j = i / DL, l = i - j * DL;
+      const int g = xcd + 8 * j, head = g % p.NH, tile = g / p.NH;
+      const int row = tile * ROWS + l / PER_ROW;
+      const uint32_t doff = (i < G * DL && row < p.B) ? (uint32_t)(((long long)row * H + head * dh) * ESZ + (l % PER_ROW) * 128) : 0xFFFFFF00u;
+      bwd_fetch_to_lds_b128(drs, uniform(dump_lds), doff);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -681,7 +717,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
   const int ngroups = p.NH * ((p.B + 15) / 16);
   const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
   if (local >= p.main_locals) {
-    bwd_prefetch<BF16>(p, xcd);
+    bwd_tile_prefetch<BF16, S, 16, 2>(p, xcd, local - p.main_locals, (int)(gridDim.x >> 3) - p.main_locals);
     return;
   }
   const int group = (local / S) * 8 + xcd, s = local % S;

@@ -40,87 +40,6 @@ constexpr int bwd_quad_lds_bytes() { return 2 * 8 * kBwdQuadPart * 4 + kBwdQuadS
 // so does every cycle slept past the arrival.
 constexpr int kBwdQuadSleepIdle = 8, kBwdQuadSleepPublished = 2;
 
-// The prefetching workgroup of an XCD (see bwd_prefetch) for row tiles of 4 rows.  Four times the groups of the 16-row
-// kernel and a shorter step: the groups' progress words are read by the lanes of one wave side by side, and the lines of
-// a step - the coefficients and d_h of all groups of the XCD - are dealt out over the threads as one flat range (a call
-// per group and tensor, with its address arithmetic, took this workgroup longer than the compute units take for the
-// step once an XCD held more than two groups; the feeder waves then missed to HBM, and every poll of their compute unit
-// came back behind those misses).
-template <int S>
-__device__ __forceinline__ void bwd_quad_prefetch(const BwdSplitParams &p, int xcd, int which, int of) {
-  // `which` of the `of` prefetching workgroups of this XCD (a compute unit draws some 65 GB/s from memory: the host
-  // launches as many as the XCD's groups need); they share a step's lines by position
-  constexpr int dh = 64 * S;
-  constexpr int CL = S * kBwdQuadCoefBytes / 128;  // lines of a group's coefficients of one step (its S workgroups' pieces lie in a row)
-  constexpr int DL = 4 * S;                        // lines of its d_h: 4 rows of dh bf16
-  const int H = p.NH * dh, ntiles = (p.B + 3) >> 2, ngroups = p.NH * ntiles;
-  const int tid = threadIdx.x, nthreads = blockDim.x, lane = tid & 63;
-  if (xcd >= ngroups) return;
-  const int G = (ngroups - xcd + 7) >> 3;          // groups of this XCD: xcd, xcd + 8, ...
-  // steps the prefetch may run ahead of the groups' progress: about 2 MiB of the XCD's 4 MiB L2, and more than the
-  // feeder waves run ahead
-  int ahead = (2 << 20) / (G * (CL + DL) * 128);
-  ahead = ahead > kBwdAhead ? kBwdAhead : (ahead < kBwdQuadDepth + 2 ? kBwdQuadDepth + 2 : ahead);
-  __shared__ uint4 dump[64];   // (every touch lands here; nobody reads it)
-  const uint32_t dump_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)dump);
-  __shared__ int slowest;      // the least progress among the XCD's groups; -1: stop
-  const long long coef_step = (long long)ngroups * S * kBwdQuadCoefBytes;  // bytes of one step's coefficients, all groups
-  const long long dh_step = (long long)p.B * H * 2;
-  for (int m = 0; m < p.T; ++m) {
-    if (m >= ahead && (m & 1) == 0) {  // (every other step: the groups' progress is read through the L2)
-      if (tid == 0) slowest = 0x7FFFFFFF;
-      __syncthreads();
-      if (tid < 64) {
-        int spins = 0;
-        for (;;) {
-          int least = 0x7FFFFFFF;
-          for (int j = lane; j < G; j += 64) {
-            const int at = (int)__hip_atomic_load(p.progress + xcd + 8 * j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            least = at < least ? at : least;
-          }
-          if (__builtin_amdgcn_ballot_w64(least < m - ahead) == 0ull) {  // (lanes without a group: the largest int)
-            if (lane < G) atomicMin(&slowest, least);
-            break;
-          }
-          if (++spins > (1 << 16) || __hip_atomic_load(p.abort_word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) {
-            if (lane == 0) slowest = -1;
-            break;
-          }
-          __builtin_amdgcn_s_sleep(8);
-        }
-      }
-      __syncthreads();
-      const int at = slowest;
-      if (at < 0) break;
-      // (fallen behind what the feeder waves have already asked for: skip to where a touch can still come first)
-      if (m < at + kBwdQuadDepth + 1) m = (at + kBwdQuadDepth + 1) & ~1;
-      if (m >= p.T) break;
-    }
-    const int t = p.T - 1 - m;
-    const unsigned long long cb = reinterpret_cast<unsigned long long>(p.coef) + (unsigned long long)(t * coef_step);
-    const unsigned long long db = reinterpret_cast<unsigned long long>(p.d_h) + (unsigned long long)(t * dh_step);
-    const u32x4_t crs = {uniform((uint32_t)cb), uniform((uint32_t)(cb >> 32) & 0xFFFFu), uniform((uint32_t)coef_step), 0x00020000u};
-    const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), uniform((uint32_t)dh_step), 0x00020000u};
-    // (uniform trip counts: lanes past the end ask past the buffer's end)
-    for (int i0 = which * nthreads; i0 < G * CL; i0 += of * nthreads) {
-      const int i = i0 + tid;
-      const int j = i / CL, l = i - j * CL;
-      const int g = xcd + 8 * j, head = g % p.NH, tile = g / p.NH;
-      const uint32_t coff = i < G * CL ? (uint32_t)(((tile * p.NH + head) * S) * kBwdQuadCoefBytes + l * 128) : 0xFFFFFF00u;
-      bwd_fetch_to_lds_b128(crs, uniform(dump_lds), coff);
-    }
-    for (int i0 = which * nthreads; i0 < G * DL; i0 += of * nthreads) {
-      const int i = i0 + tid;
-      const int j = i / DL, l = i - j * DL;
-      const int g = xcd + 8 * j, head = g % p.NH, tile = g / p.NH;
-      const int row = tile * 4 + l / S;
-      const uint32_t doff = (i < G * DL && row < p.B) ? (uint32_t)(((long long)row * H + head * dh) * 2 + (l % S) * 128) : 0xFFFFFF00u;
-      bwd_fetch_to_lds_b128(drs, uniform(dump_lds), doff);
-    }
-  }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
-
 template <int S>  // S workgroups per group, dh = 64 S
 __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSplitParams p) {
   constexpr int UW = 64;
@@ -139,7 +58,7 @@ __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSpli
   const long long wg_start = wall_clock64();
 #endif
   if (local >= p.main_locals) {
-    bwd_quad_prefetch<S>(p, xcd, local - p.main_locals, (int)(gridDim.x >> 3) - p.main_locals);
+    bwd_tile_prefetch<true, S, 4, kBwdQuadDepth>(p, xcd, local - p.main_locals, (int)(gridDim.x >> 3) - p.main_locals);
     return;
   }
   const int group = (local / S) * 8 + xcd, s = local % S;

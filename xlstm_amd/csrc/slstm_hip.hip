@@ -514,7 +514,18 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       if (((uintptr_t)a->exchange % 16)) return fail(XS_ERR_ALIGN, "exchange must be 16-byte aligned");
       q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1; q.placement = a->counters + 1 + ngroups;
       q.main_locals = (int)(grid / 8);
-      const bool prefetchers = grid + 8 <= device_cus();  // (one more workgroup per XCD, where there is room)
+      // prefetching workgroups per XCD, as for the row tiles of 4 rows below: one per 40 KB that the XCD's groups read
+      // per step, as far as there are compute units left
+      int prefetchers = 0;
+      {
+        const long long groups_per_xcd = (ngroups + 7) / 8;
+        const long long step_bytes = groups_per_xcd * S * (kBwdCoefBytes + 16 * 64 * (bf16 ? 2 : 4));
+        long long want = (step_bytes + 39999) / 40000;
+        const long long room = (device_cus() - grid) / 8;
+        if (want > room) want = room;
+        if (want > 8) want = 8;
+        prefetchers = (int)(want < 0 ? 0 : want);
+      }
       q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;  // (negative: every wait gives up at once)
       q.cut = a->recurrent_cut != 0; q.clip = clip;
       const long long n16 = (long long)kBwdRing * ngroups * 16 * 4 * a->dh * (bf16 ? 2 : 4) / 16;
@@ -532,7 +543,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
         const int rc = ensure_dynamic_lds((const void *)ks, (size_t)lds);
         if (rc != XS_OK) return rc;
       }
-      hipLaunchKernelGGL(ks, dim3((unsigned)(grid + (prefetchers ? 8 : 0))), dim3(feed ? 768 : 512), lds, stream, q);
+      hipLaunchKernelGGL(ks, dim3((unsigned)(grid + 8 * prefetchers)), dim3(feed ? 768 : 512), lds, stream, q);
       const hipError_t es = hipGetLastError();
       if (es != hipSuccess) return fail(XS_ERR_LAUNCH, "backward kernel launch failed: %s", hipGetErrorString(es));
       return XS_OK;
