@@ -21,7 +21,7 @@
 namespace {
 
 constexpr int kBwdQuadCoefBytes = 4 * 9 * 64 * 4;  // a step's coefficients of a workgroup: 4 rows, 9 of them, 64 units
-// a slot of the feeder wave: the coefficients, d_h (4 rows of 128 bytes in a landing zone of 1 KiB), the reset flags of the
+// a slot of the feeder waves: the coefficients, d_h (4 rows of 128 bytes in a landing zone of 1 KiB), the reset flags of the
 // 4 rows as words (in a landing zone of 256 bytes)
 constexpr int kBwdQuadSlot = kBwdQuadCoefBytes + 1024 + 256;
 constexpr int kBwdQuadSlots = 8;
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSpli
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
   char *const feed = reinterpret_cast<char *>(part + 2 * 8 * PART);
   bwd_note_placement(p, group);
-  // look_step[w]: 1 + the step of the call whose first look compute wave w has issued (for the feeder wave, see there)
+  // look_step[w]: 1 + the step of the call whose first look compute wave w has issued (for the feeder waves, see there)
   __shared__ volatile int look_step[8];
   if (tid < 8) look_step[tid] = 0;
   const int rows_there = p.B - row0 < 4 ? p.B - row0 : 4;
