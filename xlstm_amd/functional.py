@@ -187,8 +187,12 @@ def slstm_backward(
     bias = bias.to(torch.float32).contiguous()
     if s0 is not None:
         s0 = s0.to(torch.float32).contiguous()
-    if reset_mask is not None:
-        reset_mask = (reset_mask != 0).to(torch.uint8).contiguous()
+    if reset_mask is not None:  # (bytes, any non-zero value marks a document start: as the forward takes it)
+        if reset_mask.dtype == torch.bool:
+            reset_mask = reset_mask.view(torch.uint8) if reset_mask.is_contiguous() else reset_mask.to(torch.uint8)
+        elif reset_mask.dtype != torch.uint8:
+            reset_mask = (reset_mask != 0).to(torch.uint8)
+        reset_mask = reset_mask.contiguous()
     r32 = r.to(torch.float32)
     if bf16:
         r32 = r32.bfloat16().float()  # (the forward rounds R to bf16)
