@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 12
+#define XS_ABI_VERSION 13
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -281,7 +281,7 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  * unit k = g*dh + a) of head h is the reference's external view recurrent_kernel[h][d][g][a] (cell.py:234-242) -
  * tiled as MFMA operands: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC] with EPC = 16 bytes of elements (8 bf16, 4 f32)
  * and KC = 4*EPC, so that what the 64 lanes of a wave load for one k-step is 1 KiB in a row.  Head dims: 64, 128, 256
- * (512 with bf16 and split).
+ * (512 with bf16 and split; up to 1024 with bf16 and 512 with f32 with split == 3, one launch per step).
  * The caller owns every buffer; both calls only enqueue kernels on `stream`.
  */
 typedef struct xs_slstm_bwd_args {
@@ -313,7 +313,15 @@ typedef struct xs_slstm_bwd_args {
    * shorter step; for batches whose NH * ceil(B/4) * dh/64 workgroups fit the device.  Then K is ordered k = 4*a + g,
    * r_t is tiled the same way, coef is [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units], exchange has
    * 4 * NH * ceil(B/4) * 4 * 4*dh elements and counters 1 + 2 * NH * ceil(B/4) words.
-   * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once. */
+   * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once.
+   * split == 3 (both calls; head dims 512 to 1024 with XS_BF16, 256 to 512 with XS_F32, in steps of 64: up to what the
+   * forward entry points cover): ONE LAUNCH PER STEP instead of one per call, the reference's own decomposition
+   * (slstm_backward.cu:291-319), for head dims whose slice of R transposed no compute unit can keep in registers.
+   * prepare runs the decode step kernel T times (h_out is not read), the backward call T + 1 launches of a kernel that
+   * multiplies the gate deltas of the step behind by R transposed and forms the step's gradient.  Then coef is
+   * [T,B,9,H], r_t is plain R transposed [NH][dh][4*dh] (element (d, k = g*dh + a), K contiguous), counters is not
+   * used, nothing waits and nothing can give up, and exchange is a 16-byte aligned buffer of at least
+   * 256 + 32*B*H + B*H*sizeof(dtype) bytes that carries states and deltas from launch to launch. */
   int32_t split;
   void *exchange;
   uint32_t *counters;

@@ -248,7 +248,7 @@ def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=
     m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
     dsf_t = torch.from_numpy(d_sf).to(dev) if d_sf is not None else None
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
-    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override", "row_tile_override")}
+    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override", "row_tile_override", "stepwise_override")}
     d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), dsf_t, **kw)
     torch.cuda.synchronize()
     okw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval")}
@@ -387,7 +387,7 @@ def test_cell_config_gradient_recurrent_cut_and_clipval():
 
 
 @pytest.mark.parametrize("bf16,B,T,NH,dh,split", [(False, 5, 9, 2, 64, True), (True, 16, 12, 4, 256, True), (False, 4, 10, 2, 128, False),
-                                                  (True, 14, 12, 4, 256, 4)])
+                                                  (True, 14, 12, 4, 256, 4), (True, 3, 6, 1, 1024, "step"), (False, 66, 3, 1, 512, "step")])
 def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     """A caller without torch arithmetic - the binding a maintainer would put in place of the reference's
     ``sLSTMFunc.backward`` (slstm.cc:137-221, which returns {dx, ds0, dR, db} from one native call): forward, then the
@@ -416,7 +416,10 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     # R transposed in the reverse kernel's operand order (include/xlstm_amd.h), by numpy
     epc = 8 if bf16 else 4
     tile_rows = 4 if split == 4 and split is not True else 16  # (split: False, True = row tiles of 16 rows, 4 = of 4 rows)
-    if tile_rows == 4:
+    stepwise = split == "step"                                 # ("step": one launch per step, the largest head dims)
+    if stepwise:
+        r_t = r_k.transpose(0, 2, 1)                                          # plain R transposed [NH, dh, 4 dh]
+    elif tile_rows == 4:
         S, ksteps = dh // 64, 4 * dh // 8 // 32                               # K ordered (unit, gate)
         r_t = (r_k.reshape(NH, 4, dh, dh).transpose(0, 2, 1, 3).reshape(NH, 4 * dh, dh)
                .reshape(NH, 8, ksteps, 4, 8, S, 4, 16).transpose(0, 5, 1, 2, 6, 3, 7, 4))
@@ -432,7 +435,7 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     dh_t, dsf_t = dev_t(d_h, tdt), dev_t(d_sf)
     h, _ = F.slstm_forward(wx_t, r_fwd if bf16 else dev_t(r_k), b_t, s0_t, m_t)
     groups = NH * ((B + tile_rows - 1) // tile_rows)
-    rows = (B + tile_rows - 1) // tile_rows * tile_rows if split else B
+    rows = (B + tile_rows - 1) // tile_rows * tile_rows if split and not stepwise else B
     coef = torch.empty(T * rows * 9 * H, dtype=torch.float32, device=dev)
     d_wx = torch.empty(B, T, 4 * H, dtype=torch.float32, device=dev)
     d_s0 = torch.empty(4, B, H, dtype=torch.float32, device=dev)
@@ -440,6 +443,8 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     d_b = torch.empty(NH, 4, dh, dtype=torch.float32, device=dev)
     exchange = torch.empty(4 * groups * tile_rows * 4 * dh, dtype=tdt, device=dev)
     counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
+    if stepwise:  # (states and deltas from launch to launch; no counters: nothing waits)
+        exchange = torch.empty(256 + 32 * B * H + B * H * (2 if bf16 else 4), dtype=torch.uint8, device=dev)
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
     a.wx, a.wx_stride_b, a.wx_stride_t = wx_t.data_ptr(), wx_t.stride(0), wx_t.stride(1)
@@ -449,13 +454,15 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     a.d_wx, a.d_wx_stride_b, a.d_wx_stride_t, a.d_s0 = d_wx.data_ptr(), d_wx.stride(0), d_wx.stride(1), d_s0.data_ptr()
     a.d_r, a.d_bias = d_r.data_ptr(), d_b.data_ptr()
     a.stream = torch.cuda.current_stream().cuda_stream
-    a.split = (2 if tile_rows == 4 else 1) if split else 0
+    a.split = 3 if stepwise else ((2 if tile_rows == 4 else 1) if split else 0)
     a.exchange, a.counters = (exchange.data_ptr(), counters.data_ptr()) if split else (None, None)
+    if stepwise:
+        a.counters = None
     for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
         rc = fn(ctypes.byref(a))
         assert rc == 0, _lib.last_error()
     torch.cuda.synchronize()
-    if split:
+    if split and not stepwise:
         assert int(counters[0]) == 0
     o_wx, o_r, o_b, o_s0 = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf)
     tol = 2e-2 if bf16 else 1e-5

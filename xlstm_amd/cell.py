@@ -170,7 +170,7 @@ class sLSTMCellConfig:
         self.num_states = rnn_function_registry[self.function]["states"]
 
 
-BACKWARD_MAX_HEAD_DIM = {torch.float32: 256, torch.bfloat16: 512}  # what xs_slstm_backward covers (smaller head dims padded up)
+BACKWARD_MAX_HEAD_DIM = {torch.float32: 512, torch.bfloat16: 1024}  # what xs_slstm_backward covers: the forward's range
 
 
 class _ForwardOnly(torch.autograd.Function):
@@ -184,7 +184,7 @@ class _ForwardOnly(torch.autograd.Function):
     @staticmethod
     def backward(ctx, *grads):
         raise RuntimeError(
-            "sLSTMCell backend 'hip' has a backward pass for head dims up to 256 (float32) and 512 (bfloat16) only; "
+            "sLSTMCell backend 'hip' has a backward pass for head dims up to 512 (float32) and 1024 (bfloat16) only; "
             "use the reference's 'cuda' or 'vanilla' backend to train this shape"
         )
 

@@ -35,6 +35,7 @@
 #include "slstm_layer_kernels.h"
 #include "slstm_backward_kernels.h"
 #include "slstm_backward_quad_kernel.h"
+#include "slstm_backward_step_kernel.h"
 #include "slstm_backward_params_kernel.h"
 #include "slstm_serial_bound.h"
 
@@ -393,19 +394,104 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   return XS_OK;
 }
 
+// ---- backward pass with one launch per step (split == 3): the forward walk is the decode step kernel in its variant
+// that leaves the coefficients, the reverse pass slstm_bwd_step_kernel.  Both keep what a step hands to the next in
+// the caller's `exchange` buffer: 256 bytes that the step kernel's status words go to, two states [4,B,H] float32 that
+// the forward walk alternates between, one [B,H] row of outputs in the type of the operands that nobody reads; the
+// reverse pass two sets of gate deltas [B,NH,4 dh] in the type of the operands.
+int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
+  const bool bf16 = a->dtype == XS_BF16;
+  const int esz = bf16 ? 2 : 4;
+  const int B = a->B, T = a->T, NH = a->NH, dh = a->dh;
+  const long long H = (long long)NH * dh, BH = (long long)B * H;
+  hipStream_t stream = (hipStream_t)a->stream;
+  if (!a->exchange) return fail(XS_ERR_NULL, "exchange is required with one launch per step");
+  if (((uintptr_t)a->exchange % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "exchange and coef must be 16-byte aligned");
+  if (prepare) {
+    if (!a->wx || !a->r || !a->bias) return fail(XS_ERR_NULL, "wx, r and bias are required");
+    if (a->wx_stride_t < 4 * H || (B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");
+    if (((uintptr_t)a->wx % 16) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16))
+      return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
+    if (((uintptr_t)a->r % 16) || ((uintptr_t)a->s0 % 16) || ((uintptr_t)a->bias % 16)) return fail(XS_ERR_ALIGN, "r, s0 and bias must be 16-byte aligned");
+    const int epc = bf16 ? 8 : 4;
+    int nch = 1;
+    while (nch * 16 * epc < dh) nch *= 2;
+    int nch_log2 = 0;
+    while ((1 << nch_log2) < nch) ++nch_log2;
+    char *const ws = (char *)a->exchange;
+    float *const states[2] = {(float *)(ws + 256), (float *)(ws + 256 + 16 * BH)};
+    StepParams p;
+    p.r = a->r; p.r_bf16 = bf16; p.bias = a->bias;
+    p.reset_sb = a->reset_stride_b;
+    p.h_out = ws + 256 + 32 * BH;
+    p.status = (xs_slstm_status *)ws;
+    p.B = B; p.NH = NH; p.dh = dh;
+    p.n_unit_tiles = (dh + 31) / 32;
+    p.n_row_tiles = (B + 63) / 64;
+    p.h_prev = nullptr; p.spin_limit = 0; p.wx_sb = a->wx_stride_b;
+    const long long nwg = (long long)NH * p.n_unit_tiles * p.n_row_tiles;
+    if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
+    void (*kern)(StepParams, int) = bf16 ? slstm_step_tile_kernel<true, 2, false, false, false, true>
+                                         : slstm_step_tile_kernel<false, 2, false, false, false, true>;
+    const size_t lds = (size_t)2 * (64 + 128) * (2 * 64 + 16);
+    for (int t = 0; t < T; ++t) {
+      p.wx = (const char *)a->wx + (long long)t * a->wx_stride_t * esz;
+      p.s0 = t == 0 ? a->s0 : states[(t - 1) & 1];
+      p.s_out = states[t & 1];
+      p.reset = a->reset ? a->reset + t : nullptr;
+      p.coef = a->coef + (long long)t * 9 * BH;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), lds, stream, p, nch_log2);
+    }
+  } else {
+    if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
+    if (((uintptr_t)a->r_t % 16) || ((uintptr_t)a->d_h % 16) || ((uintptr_t)a->d_s0 % 16) || ((uintptr_t)a->d_s_final % 16))
+      return fail(XS_ERR_ALIGN, "r_t, d_h, d_s0 and d_s_final must be 16-byte aligned");
+    if (((uintptr_t)a->d_wx % 16) || (a->d_wx_stride_b % 4) || (a->d_wx_stride_t % 4))
+      return fail(XS_ERR_ALIGN, "d_wx and its row/step strides must be 16-byte aligned");
+    if (a->d_wx_stride_t < 4 * H || (B > 1 && a->d_wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "d_wx strides overlap the innermost 4*H elements");
+    BwdStepParams q;
+    q.B = B; q.T = T; q.NH = NH; q.dh = dh;
+    q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_t = a->r_t;
+    q.reset = a->reset; q.reset_sb = a->reset_stride_b;
+    q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+    q.cut = a->recurrent_cut != 0;
+    q.clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
+    char *const deltas[2] = {(char *)a->exchange, (char *)a->exchange + 4 * BH * esz};
+    const long long nwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
+    if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
+    void (*kern)(BwdStepParams) = bf16 ? slstm_bwd_step_kernel<true> : slstm_bwd_step_kernel<false>;
+    for (int t = T - 1; t >= -1; --t) {
+      q.t = t; q.first = t == T - 1;
+      q.delta_out = deltas[(t + 1) & 1];
+      q.delta_in = deltas[t & 1];  // (what the launch of step t + 1 wrote)
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBwdStepThreads), bwd_step_lds_bytes(), stream, q);
+    }
+  }
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "backward step kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 // ---- backward pass: the forward walk that leaves the coefficients, and the reverse-time kernel
 int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
   if (a->B < 0 || a->T < 0 || a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims B=%d T=%d NH=%d dh=%d", a->B, a->T, a->NH, a->dh);
   if (a->dtype != XS_F32 && a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
-  if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && a->dtype == XS_BF16 && (prepare || a->split)))
-    return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256; 512 in bf16 over several compute units)", a->dh);
+  if (a->split == 3) {
+    // one launch per step: the head dims the forward covers beyond those of the persistent kernels, and those next below
+    const int lo = a->dtype == XS_BF16 ? 512 : 256;
+    if (a->dh % 64 != 0 || a->dh < lo || a->dh > 2 * lo)
+      return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d not supported (%d to %d in steps of 64)", a->dh, lo, 2 * lo);
+  } else if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && a->dtype == XS_BF16 && (prepare || a->split)))
+    return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256; 512 in bf16 over several compute units; "
+                "up to 1024 in bf16 and 512 in float32 with one launch per step, split = 3)", a->dh);
   if (a->B == 0 || a->T == 0) return XS_OK;
   const bool bf16 = a->dtype == XS_BF16;
   const long long H = (long long)a->NH * a->dh;
   if (!a->coef) return fail(XS_ERR_NULL, "coef is required");
   if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
   hipStream_t stream = (hipStream_t)a->stream;
+  if (a->split == 3) return run_backward_stepwise(a, prepare);
   if (prepare) {
     if (!a->wx || !a->r || !a->h_out || !a->bias) return fail(XS_ERR_NULL, "wx, r, h_out and bias are required");
     if (a->wx_stride_t < 4 * H || (a->B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");

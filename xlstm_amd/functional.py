@@ -53,12 +53,22 @@ def _compute_units(dev) -> int:
 
 
 def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
-    """The head dim that the backward kernels run a head dim ``dh`` as (64, 128, 256, and 512 with bfloat16 inputs; sizes in
-    between are padded up by ``slstm_backward``), or None when there is none."""
+    """The head dim that the backward kernels run a head dim ``dh`` as: 64, 128, 256 (and 512 with bfloat16 inputs) for
+    the kernels that take one launch for all steps, beyond those any multiple of 64 up to the forward's range (1024 with
+    bfloat16, 512 with float32) for the kernels that take one launch per step; sizes in between are padded up by
+    ``slstm_backward``.  None when there is none."""
+    bf16 = dtype == torch.bfloat16
     for size in (64, 128, 256, 512):
-        if dh <= size and (size < 512 or dtype == torch.bfloat16):
+        if dh <= size and (size < 512 or bf16):
             return size
+    if dh <= (1024 if bf16 else 512):
+        return (dh + 63) // 64 * 64
     return None
+
+
+def backward_runs_stepwise(dh_kernel: int, dtype: torch.dtype) -> bool:
+    """Whether the backward pass of that (kernel) head dim takes one launch per step (``split == 3`` of the C ABI)."""
+    return dh_kernel > (512 if dtype == torch.bfloat16 else 256)
 
 
 class CoefficientsUnsupported(EngineError):
@@ -99,6 +109,7 @@ def slstm_backward(
     coef: Optional[torch.Tensor] = None,
     recurrent_cut: bool = False,
     recurrent_clipval: Optional[float] = None,
+    stepwise_override: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -115,6 +126,9 @@ def slstm_backward(
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel), in row tiles of 4 rows where four times the workgroups fit (bfloat16, head dims up to 256;
     ``row_tile_override`` = 16 or 4 forces either); ``spin_limit`` bounds those waits, and a wait that runs out raises ``EngineError``.
+    Head dims beyond those (up to 1024 with bfloat16, 512 with float32: the forward's range) take one launch per step,
+    forward walk and reverse pass alike (``stepwise_override=True`` forces that for head dim 512 in bfloat16 and 256 in
+    float32, which both ways cover).
     ``coef``: what a training forward left (``slstm_forward(..., coef_out=)``); the forward walk is then skipped.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
     to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
@@ -136,7 +150,7 @@ def slstm_backward(
         raise ValueError("coef must be the tensor that the forward call of the same inputs filled")
     if dh_k is None:
         raise EngineError(f"xlstm_amd: no backward kernel for head dim {dh} with {wx.dtype} inputs "
-                          f"(up to 512 with bfloat16, up to 256 with float32)")
+                          f"(up to 1024 with bfloat16, up to 512 with float32)")
     if dh_k != dh:
         # A head dim between the kernels' sizes runs as the next size up with units that are not there: their W.x, bias
         # and rows and columns of R are zero, so they neither see nor touch the real units, and their results are cut off.
@@ -156,7 +170,8 @@ def slstm_backward(
         dsf_p = widen(d_s_final, (4, B_)).reshape(4, B_, NH * dh_k) if d_s_final is not None else None
         d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
                                                  split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
-                                                 recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval)
+                                                 recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval,
+                                                 stepwise_override=stepwise_override)
         return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
                 d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
                 d_bias[..., :dh].contiguous(),
@@ -165,7 +180,12 @@ def slstm_backward(
     # The kernel that spreads a head over dh/64 compute units needs all its workgroups on the device at once.  A batch
     # with more row tiles than that runs in slices of rows (rows do not meet in the backward pass but in the sums for
     # R and the bias), rather than with one workgroup per head, which takes 7 times as long per step.
-    if split_override is not False and coef is None:
+    stepwise = backward_runs_stepwise(dh, wx.dtype)
+    if stepwise_override and dh == (512 if bf16 else 256):
+        stepwise = True
+    if stepwise and coef is not None:
+        raise EngineError("xlstm_amd: coefficients from the forward call do not go with the backward pass of one launch per step")
+    if split_override is not False and coef is None and not stepwise:
         room = (_compute_units(dev) - 8) // (8 * (dh // 64)) * 8      # groups per launch, the prefetching workgroups kept
         tiles_per_launch = room // NH
         if tiles_per_launch >= 1 and (B + 15) // 16 > tiles_per_launch:
@@ -207,12 +227,15 @@ def slstm_backward(
     split = (dh in (64, 128, 256) or (dh == 512 and bf16)) and (groups + 7) // 8 * 8 * S <= _compute_units(dev)
     if split_override is not None:
         split = bool(split_override)
+    if stepwise:
+        split = False
     # row tiles of 4 rows (bf16, head dims up to 256) where four times the workgroups still fit, with the prefetching ones
     groups4 = NH * ((B + 3) // 4)
     quad = (split and bf16 and dh <= 256 and (groups4 + 7) // 8 * 8 * S + 8 <= _compute_units(dev)
             and (reset_mask is None or 3 * reset_mask.stride(0) + T < 2 ** 31 - 256))
     if row_tile_override is not None:
         quad = split and row_tile_override == 4
+    quad = quad and not stepwise
     if coef is not None:
         if not (split and quad):
             raise EngineError("xlstm_amd: coefficients from the forward call go with the reverse kernel for row tiles of 4 rows, "
@@ -238,6 +261,11 @@ def slstm_backward(
                .view(NH, 8, ksteps, 4, epc, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
         exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=wx.dtype, device=dev)
         counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
+    elif stepwise:
+        # plain R transposed [NH, dh (d), 4*dh (k)]; what the launches of a call hand to each other goes through `exchange`
+        r_t = r32.transpose(1, 2).to(wx.dtype).contiguous()
+        exchange = torch.empty(256 + 32 * B * H + B * H * esz, dtype=torch.uint8, device=dev)
+        counters = None
     else:
         # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
         r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
@@ -266,9 +294,9 @@ def slstm_backward(
     a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
     a.d_s0 = d_s0.data_ptr()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
-    a.split = (2 if quad else 1) if split else 0
-    a.exchange = exchange.data_ptr() if split else None
-    a.counters = counters.data_ptr() if split else None
+    a.split = 3 if stepwise else ((2 if quad else 1) if split else 0)
+    a.exchange = exchange.data_ptr() if exchange is not None else None
+    a.counters = counters.data_ptr() if counters is not None else None
     a.spin_limit = int(spin_limit)
     a.recurrent_cut = 1 if recurrent_cut else 0
     a.recurrent_clipval = float(recurrent_clipval) if recurrent_clipval is not None else 0.0
