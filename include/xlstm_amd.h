@@ -319,9 +319,11 @@ typedef struct xs_slstm_bwd_args {
    * (slstm_backward.cu:291-319), for head dims whose slice of R transposed no compute unit can keep in registers.
    * prepare runs the decode step kernel T times (h_out is not read), the backward call T + 1 launches of a kernel that
    * multiplies the gate deltas of the step behind by R transposed and forms the step's gradient.  Then coef is
-   * [T,B,9,H], r_t is plain R transposed [NH][dh][4*dh] (element (d, k = g*dh + a), K contiguous), counters is not
-   * used, nothing waits and nothing can give up, and exchange is a 16-byte aligned buffer of at least
-   * 256 + 32*B*H + B*H*sizeof(dtype) bytes that carries states and deltas from launch to launch. */
+   * [T,B,9,H]; r_t is R transposed (element (d, k = g*dh + a)) in slabs of 256 bytes of K per tile of 32 input units,
+   * [NH][d/32][k/KS][d%32][k%KS] with KS = 128 (bf16) or 64 (f32), so that what a workgroup stages per slab is 8 KiB in
+   * a row; counters is not used, nothing waits and nothing can give up; and exchange is a 16-byte aligned buffer of at
+   * least max(256 + 32*B*H + B*H*sizeof(dtype), 8*ceil(B/64)*64*H*sizeof(dtype)) bytes that carries states (prepare)
+   * and gate deltas (backward) from launch to launch. */
   int32_t split;
   void *exchange;
   uint32_t *counters;

@@ -418,7 +418,8 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     tile_rows = 4 if split == 4 and split is not True else 16  # (split: False, True = row tiles of 16 rows, 4 = of 4 rows)
     stepwise = split == "step"                                 # ("step": one launch per step, the largest head dims)
     if stepwise:
-        r_t = r_k.transpose(0, 2, 1)                                          # plain R transposed [NH, dh, 4 dh]
+        ks = 128 if bf16 else 64                                              # R transposed in slabs of 256 bytes of K
+        r_t = r_k.transpose(0, 2, 1).reshape(NH, dh // 32, 32, 4 * dh // ks, ks).transpose(0, 1, 3, 2, 4)
     elif tile_rows == 4:
         S, ksteps = dh // 64, 4 * dh // 8 // 32                               # K ordered (unit, gate)
         r_t = (r_k.reshape(NH, 4, dh, dh).transpose(0, 2, 1, 3).reshape(NH, 4 * dh, dh)
@@ -444,7 +445,8 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     exchange = torch.empty(4 * groups * tile_rows * 4 * dh, dtype=tdt, device=dev)
     counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     if stepwise:  # (states and deltas from launch to launch; no counters: nothing waits)
-        exchange = torch.empty(256 + 32 * B * H + B * H * (2 if bf16 else 4), dtype=torch.uint8, device=dev)
+        esz = 2 if bf16 else 4
+        exchange = torch.empty(max(256 + 32 * B * H + B * H * esz, 8 * ((B + 63) // 64 * 64) * H * esz), dtype=torch.uint8, device=dev)
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
     a.wx, a.wx_stride_b, a.wx_stride_t = wx_t.data_ptr(), wx_t.stride(0), wx_t.stride(1)

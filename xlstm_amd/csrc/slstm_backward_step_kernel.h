@@ -7,8 +7,10 @@
 // forms what reaches y_t through the recurrence - the gate deltas of step t + 1 (left in memory by the launch before,
 // in the type of the operands) times R transposed - and then the gradient of step t from it, its nine coefficients
 // and d_h, element by element.  A workgroup owns 64 batch rows x 32 hidden units: K = 4 dh gate units are walked in
-// slabs of 256 bytes per row that go through LDS (two buffers, one barrier per slab, the loads of four slabs in flight
-// in registers); the product is formed transposed (units on the MFMA M axis), so a lane ends with 4 consecutive units
+// slabs of 256 bytes per row that four feeder waves bring straight into a ring of LDS slots, several slabs ahead of
+// the four waves that multiply, one barrier per slab (both operands lie in memory slab by slab, so a slab of a tile is
+// one piece of 8 or 16 KiB; with the loads in registers of the multiplying waves, whose waits the compiler places, a
+// slab took a whole memory latency: 73 us per step at 4 heads of 1024 instead of the figures below); the product is formed transposed (units on the MFMA M axis), so a lane ends with 4 consecutive units
 // of one batch row and everything pointwise moves as 16-byte accesses, asked for in front of the K loop.  What the
 // steps hand on besides the deltas - the gradients of c and n - lives in planes 1 and 2 of d_s0 between the launches
 // (each element is read and written by the same lane of the same workgroup of every launch); a last launch (t = -1)
@@ -24,8 +26,11 @@ struct BwdStepParams {
   const float *coef;         // [T,B,9,H]
   const void *d_h;           // [T,B,H] in the type of the operands
   const float *d_s_final;    // [4,B,H] or null
-  const void *r_t;           // [NH][dh][4 dh]: R transposed, element (input unit d, gate unit k = g dh + a), K contiguous
-  const void *delta_in;      // [B][NH][4 dh] in the type of the operands: the gate deltas of step t + 1
+  const void *r_t;           // R transposed, element (input unit d, gate unit k = g dh + a) of head h, in slabs of 256 bytes of K:
+                             // [NH][d / 32][k / KS][d % 32][k % KS], KS = 128 (bf16) or 64 (float32) - what a workgroup
+                             // stages per slab is 8 KiB in a row (rows of K, 8 or 16 KiB apart, all fall on one memory channel)
+  const void *delta_in;      // the gate deltas of step t + 1 in the type of the operands, tiled the same way:
+                             // [ceil(B / 64)][NH][k / KS][b % 64][k % KS]
   void *delta_out;           // ... of step t
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
@@ -36,18 +41,16 @@ struct BwdStepParams {
   float clip;
 };
 
-constexpr int kBwdStepThreads = 256;
-constexpr int kBwdStepRow = 256 + 16;   // bytes of an LDS row: a slab's 256 bytes and padding (conflict-free 16-byte reads)
-constexpr int kBwdStepRing = 4;         // slabs whose loads are in flight
-constexpr int bwd_step_lds_bytes() { return 2 * (64 + 32) * kBwdStepRow; }
+constexpr int kBwdStepThreads = 512;    // waves 0-3: MFMAs and the gradient; waves 4-7: bring the operands to LDS
+constexpr int kBwdStepSlots = 6;        // slabs in LDS: one being multiplied, the others landing
+constexpr int kBwdStepSlot = (64 + 32) * 256;  // bytes of a slab in LDS: the deltas of 64 rows, R transposed of 32 units
+constexpr int bwd_step_lds_bytes() { return kBwdStepSlots * kBwdStepSlot; }
 
 template <bool BF16>
 __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStepParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  constexpr int RS = kBwdStepRow;
-  extern __shared__ __attribute__((aligned(16))) unsigned char bstep_lds[];
-  unsigned char(*dbuf)[64 * RS] = reinterpret_cast<unsigned char(*)[64 * RS]>(bstep_lds);
-  unsigned char(*rbuf)[32 * RS] = reinterpret_cast<unsigned char(*)[32 * RS]>(bstep_lds + 2 * 64 * RS);
+  constexpr int D = kBwdStepSlots;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char bstep_lds[];
   const int dh = p.dh, NH = p.NH;
   const int H = NH * dh;
   const long long BH = (long long)p.B * H;
@@ -71,53 +74,62 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     }
   }
   const int a0 = (tile % n_ut) * 32, rowbase = (tile / n_ut) * 64;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
-  const int wr = wave >> 1, wu = wave & 1;
+  const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
+  const int wave = (int)uniform((uint32_t)(tid >> 6));
   const int t = p.t;
   const bool last_launch = t < 0;
   const bool multiply = !p.first && !p.cut;
-
-  // ---- staging roles: consecutive lanes take consecutive 16-byte pieces of a row (16 pieces a slab)
-  const unsigned char *dsrc[4], *rsrc[2];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int idx = tid + 256 * j, row = rowbase + (idx >> 4);
-    const int rowc = row < p.B ? row : p.B - 1;  // (rows past the batch read a row that is there; their results are dropped)
-    dsrc[j] = reinterpret_cast<const unsigned char *>(p.delta_in) + ((long long)rowc * NH + head) * KB + (idx & 15) * 16;
-  }
-#pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int idx = tid + 256 * j;
-    rsrc[j] = reinterpret_cast<const unsigned char *>(p.r_t) + ((long long)head * dh + a0 + (idx >> 4)) * KB + (idx & 15) * 16;
-  }
-  uint4 dring[kBwdStepRing][4], rring[kBwdStepRing][2];
-  auto load_slab = [&](int s, uint4 (&d)[4], uint4 (&r)[2]) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) d[j] = *reinterpret_cast<const uint4 *>(dsrc[j] + (long long)s * 256);
-#pragma unroll
-    for (int j = 0; j < 2; ++j) r[j] = *reinterpret_cast<const uint4 *>(rsrc[j] + (long long)s * 256);
-  };
-  auto store_slab = [&](int buf, const uint4 (&d)[4], const uint4 (&r)[2]) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int idx = tid + 256 * j;
-      *reinterpret_cast<uint4 *>(&dbuf[buf][(idx >> 4) * RS + (idx & 15) * 16]) = d[j];
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const int idx = tid + 256 * j;
-      *reinterpret_cast<uint4 *>(&rbuf[buf][(idx >> 4) * RS + (idx & 15) * 16]) = r[j];
-    }
-  };
   const int nslab = (int)(KB >> 8);
-  if (multiply) {
+  const long long dtile = ((long long)(rowbase >> 6) * NH + head) * nslab * (64 * 256);  // this row tile's deltas of the head
+  const uint32_t lds0 = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)bstep_lds);
+
+  if (wave >= 4) {
+    // ---- a feeder wave: per slab 4 of the 16 KiB of deltas and 2 of the 8 KiB of R transposed, 1 KiB (4 rows of 256
+    //      bytes) per load, straight into LDS.  Such a load fills consecutive LDS, so the rows cannot be padded: piece
+    //      g of row r (16 bytes) sits at position g ^ (r & 7) of the row, which keeps the 16-byte reads of the MFMA
+    //      waves (8 consecutive rows, one piece) free of bank conflicts.  Slab s is asked for D - 1 slabs ahead, into
+    //      the slot that the MFMA waves left before the barrier just passed; the waits are for a constant count
+    //      (slabs past the end are asked for like the others - the last slab again, into a slot that nobody reads).
+    if (!multiply) return;
+    const int f = wave - 4, sub = lane >> 4, pos = lane & 15;
+    const unsigned long long db = reinterpret_cast<unsigned long long>(p.delta_in) + dtile;
+    const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_t) + ((long long)head * (dh >> 5) + (a0 >> 5)) * nslab * (32 * 256);
+    const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), (uint32_t)(nslab * (64 * 256)), 0x00020000u};
+    const u32x4_t rrs = {uniform((uint32_t)rb), uniform((uint32_t)(rb >> 32) & 0xFFFFu), (uint32_t)(nslab * (32 * 256)), 0x00020000u};
+    uint32_t dvo[4], rvo[2];
 #pragma unroll
-    for (int u = 0; u < kBwdStepRing; ++u)
-      if (u < nslab) load_slab(u, dring[u], rring[u]);
+    for (int k = 0; k < 4; ++k) {
+      const int row = 4 * (4 * f + k) + sub;
+      dvo[k] = (uint32_t)(row * 256 + ((pos ^ (row & 7)) << 4));
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int row = 4 * (2 * f + k) + sub;
+      rvo[k] = (uint32_t)(row * 256 + ((pos ^ (row & 7)) << 4));
+    }
+    auto request = [&](int s) {
+      const int sc = s < nslab ? s : nslab - 1;
+      const uint32_t slot = lds0 + (uint32_t)(s % D) * kBwdStepSlot;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        bwd_fetch_to_lds_b128(drs, uniform(slot + (4 * f + k) * 1024), dvo[k] + (uint32_t)sc * (64 * 256));
+#pragma unroll
+      for (int k = 0; k < 2; ++k)
+        bwd_fetch_to_lds_b128(rrs, uniform(slot + 64 * 256 + (2 * f + k) * 1024), rvo[k] + (uint32_t)sc * (32 * 256));
+    };
+    for (int s = 0; s < D - 1; ++s) request(s);
+    for (int s = 0; s < nslab; ++s) {
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(6 * (D - 2)) : "memory");  // (slab s has landed)
+      lds_barrier();
+      request(s + D - 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (nothing may land in LDS that another workgroup has been given)
+    return;
   }
+  const int wr = wave >> 1, wu = wave & 1;
 
   // ---- what the gradient of the step needs of this lane's elements: batch rows rowbase + 32 wr + 16 ut + r16,
-  //      units a0 + 16 wu + 4 q .. + 3; asked for behind the first operands
+  //      units a0 + 16 wu + 4 q .. + 3; asked for in front of the K loop
   const int ua = a0 + 16 * wu + 4 * q;
   f32x4 cf[2][9], dhv[2], dcv[2], dnv[2], dyv[2];
   bool there[2], restart[2], cut_off[2];
@@ -153,39 +165,36 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
   // ---- delta_{t+1} [64 rows x K] . R^T [K x 32 units], transposed: acc[ut][i] = unit ua + i, row 32 wr + 16 ut + r16
   f32x4 acc[2] = {f32x4{0.0f, 0.0f, 0.0f, 0.0f}, f32x4{0.0f, 0.0f, 0.0f, 0.0f}};
   if (multiply) {
-    store_slab(0, dring[0], rring[0]);
-    __syncthreads();
-    for (int s0i = 0; s0i < nslab; s0i += kBwdStepRing) {
+    // this lane's pieces of a slab: k-step ch, lane group q -> piece 4 ch + q of the row, at position piece ^ (row & 7)
+    // (all rows this lane reads have row & 7 == r16 & 7)
+    int swz[4];
 #pragma unroll
-      for (int u = 0; u < kBwdStepRing; ++u) {
-        const int sidx = s0i + u;
-        if (sidx < nslab) {
-          const int buf = sidx & 1;
+    for (int ch = 0; ch < 4; ++ch) swz[ch] = ((4 * ch + q) ^ (r16 & 7)) << 4;
+    const int drow[2] = {(32 * wr + r16) * 256, (32 * wr + 16 + r16) * 256};
+    const int rrow = 64 * 256 + (16 * wu + r16) * 256;
+    for (int s = 0; s < nslab; ++s) {
+      lds_barrier();  // (slab s is in LDS; the feeder waves may overwrite the slot of slab s - 1)
+      const unsigned char *slot = bstep_lds + (s % D) * kBwdStepSlot;
+      uint4 rv[4], dv[2][4];
 #pragma unroll
-          for (int ch = 0; ch < 4; ++ch) {
-            const uint4 rv = *reinterpret_cast<const uint4 *>(&rbuf[buf][(16 * wu + r16) * RS + ch * 64 + q * 16]);
+      for (int ch = 0; ch < 4; ++ch) {
+        rv[ch] = *reinterpret_cast<const uint4 *>(slot + rrow + swz[ch]);
 #pragma unroll
-            for (int ut = 0; ut < 2; ++ut) {
-              const uint4 dv = *reinterpret_cast<const uint4 *>(&dbuf[buf][(32 * wr + 16 * ut + r16) * RS + ch * 64 + q * 16]);
-              if (BF16) {
-                acc[ut] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv), __builtin_bit_cast(bf16x8, dv), acc[ut], 0, 0, 0);
-              } else {
-                const uint32_t rw[4] = {rv.x, rv.y, rv.z, rv.w}, dw[4] = {dv.x, dv.y, dv.z, dv.w};
+        for (int ut = 0; ut < 2; ++ut) dv[ut][ch] = *reinterpret_cast<const uint4 *>(slot + drow[ut] + swz[ch]);
+      }
 #pragma unroll
-                for (int e = 0; e < 4; ++e)
-                  acc[ut] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(dw[e]), acc[ut], 0, 0, 0);
-              }
-            }
-          }
-          // slab sidx went to LDS one iteration ago: its ring entry takes the loads of slab sidx + kBwdStepRing
-          if (sidx + kBwdStepRing < nslab) load_slab(sidx + kBwdStepRing, dring[u], rring[u]);
-          if (sidx + 1 < nslab) {
-            const int un = (u + 1) % kBwdStepRing;
-            store_slab((sidx + 1) & 1, dring[un], rring[un]);  // (the other buffer was last read before the previous barrier)
-            __syncthreads();
+      for (int ch = 0; ch < 4; ++ch)
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut) {
+          if (BF16) {
+            acc[ut] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[ch]), __builtin_bit_cast(bf16x8, dv[ut][ch]), acc[ut], 0, 0, 0);
+          } else {
+            const uint32_t rw[4] = {rv[ch].x, rv[ch].y, rv[ch].z, rv[ch].w}, dw[4] = {dv[ut][ch].x, dv[ut][ch].y, dv[ut][ch].z, dv[ut][ch].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              acc[ut] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(dw[e]), acc[ut], 0, 0, 0);
           }
         }
-      }
     }
   }
 
@@ -217,17 +226,19 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     }
     const int row = rowbase + 32 * wr + 16 * ut + r16;
     float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + head * dh + ua;
-    unsigned char *dout = reinterpret_cast<unsigned char *>(p.delta_out) + ((long long)row * NH + head) * KB;
+    unsigned char *dout = reinterpret_cast<unsigned char *>(p.delta_out) + dtile + (row & 63) * 256;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       __builtin_nontemporal_store(delta[g], reinterpret_cast<f32x4 *>(dw + (long long)g * H));
+      const int kb = (g * dh + ua) * ESZ;  // byte of the row of K: slab kb / 256, inside it kb % 256
+      unsigned char *dst = dout + (long long)(kb >> 8) * (64 * 256) + (kb & 255);
       if (BF16) {
         uint2 w;
         w.x = pack_bf16x2(delta[g][0], delta[g][1]);
         w.y = pack_bf16x2(delta[g][2], delta[g][3]);
-        *reinterpret_cast<uint2 *>(dout + ((long long)g * dh + ua) * 2) = w;
+        *reinterpret_cast<uint2 *>(dst) = w;
       } else {
-        *reinterpret_cast<f32x4 *>(dout + ((long long)g * dh + ua) * 4) = delta[g];
+        *reinterpret_cast<f32x4 *>(dst) = delta[g];
       }
     }
     *reinterpret_cast<f32x4 *>(p.d_s0 + BH + eo[ut]) = dc_prev;

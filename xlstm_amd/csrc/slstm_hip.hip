@@ -398,7 +398,7 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
 // that leaves the coefficients, the reverse pass slstm_bwd_step_kernel.  Both keep what a step hands to the next in
 // the caller's `exchange` buffer: 256 bytes that the step kernel's status words go to, two states [4,B,H] float32 that
 // the forward walk alternates between, one [B,H] row of outputs in the type of the operands that nobody reads; the
-// reverse pass two sets of gate deltas [B,NH,4 dh] in the type of the operands.
+// reverse pass two sets of gate deltas in the type of the operands, in tiles of 64 rows.
 int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   const bool bf16 = a->dtype == XS_BF16;
   const int esz = bf16 ? 2 : 4;
@@ -456,10 +456,14 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
     q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
     q.cut = a->recurrent_cut != 0;
     q.clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
-    char *const deltas[2] = {(char *)a->exchange, (char *)a->exchange + 4 * BH * esz};
+    char *const deltas[2] = {(char *)a->exchange, (char *)a->exchange + 4ll * ((B + 63) / 64 * 64) * H * esz};  // (tiles of 64 rows)
     const long long nwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
     if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
     void (*kern)(BwdStepParams) = bf16 ? slstm_bwd_step_kernel<true> : slstm_bwd_step_kernel<false>;
+    {
+      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)bwd_step_lds_bytes());
+      if (rc != XS_OK) return rc;
+    }
     for (int t = T - 1; t >= -1; --t) {
       q.t = t; q.first = t == T - 1;
       q.delta_out = deltas[(t + 1) & 1];

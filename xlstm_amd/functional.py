@@ -66,6 +66,12 @@ def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
     return None
 
 
+def stepwise_exchange_bytes(B: int, H: int, esz: int) -> int:
+    """Bytes of the ``exchange`` buffer of a backward pass of one launch per step: the forward walk keeps 256 bytes of
+    status words, two states and a row of outputs there, the reverse pass two sets of gate deltas in tiles of 64 rows."""
+    return max(256 + 32 * B * H + B * H * esz, 8 * ((B + 63) // 64 * 64) * H * esz)
+
+
 def backward_runs_stepwise(dh_kernel: int, dtype: torch.dtype) -> bool:
     """Whether the backward pass of that (kernel) head dim takes one launch per step (``split == 3`` of the C ABI)."""
     return dh_kernel > (512 if dtype == torch.bfloat16 else 256)
@@ -262,9 +268,11 @@ def slstm_backward(
         exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=wx.dtype, device=dev)
         counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     elif stepwise:
-        # plain R transposed [NH, dh (d), 4*dh (k)]; what the launches of a call hand to each other goes through `exchange`
-        r_t = r32.transpose(1, 2).to(wx.dtype).contiguous()
-        exchange = torch.empty(256 + 32 * B * H + B * H * esz, dtype=torch.uint8, device=dev)
+        # R transposed [NH, dh (d), 4*dh (k)] in slabs of 256 bytes of K per tile of 32 input units:
+        # [NH][d / 32][k / KS][d % 32][k % KS]; what the launches of a call hand to each other goes through `exchange`
+        ks = 256 // esz
+        r_t = (r32.transpose(1, 2).to(wx.dtype).reshape(NH, dh // 32, 32, 4 * dh // ks, ks).permute(0, 1, 3, 2, 4).contiguous())
+        exchange = torch.empty(stepwise_exchange_bytes(B, H, esz), dtype=torch.uint8, device=dev)
         counters = None
     else:
         # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
