@@ -446,7 +446,7 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     if stepwise:  # (states and deltas from launch to launch; no counters: nothing waits)
         esz = 2 if bf16 else 4
-        exchange = torch.empty(max(256 + 32 * B * H + B * H * esz, 8 * ((B + 63) // 64 * 64) * H * esz), dtype=torch.uint8, device=dev)
+        exchange = torch.empty(max(16 * B * H + 4 * NH * dh * dh * esz, 8 * ((B + 63) // 64 * 64) * H * esz), dtype=torch.uint8, device=dev)
     a = _lib.SlstmBwdArgs()
     a.B, a.T, a.NH, a.dh, a.dtype = B, T, NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32
     a.wx, a.wx_stride_b, a.wx_stride_t = wx_t.data_ptr(), wx_t.stride(0), wx_t.stride(1)

@@ -18,13 +18,13 @@ CASES = [
     (True, 3, 9, 2, 1024, True),      # config 5's cell, a few rows and steps
     (True, 2, 1, 1, 1024, False),     # one step: the first launch and the one for the initial state only
     (True, 70, 4, 1, 1024, True),     # two row tiles, the second ragged
-    (True, 5, 6, 2, 768, True),       # a multiple of 64 between the sizes runs as it is
+    (True, 5, 6, 2, 768, True),       # a multiple of 128 between the sizes runs as it is
     (True, 4, 5, 1, 600, True),       # padded up to 640
     (False, 3, 8, 2, 512, True),
     (False, 66, 3, 1, 512, False),
     (False, 4, 6, 2, 320, True),
     (False, 2, 5, 1, 296, True),      # padded up to 320
-    (True, 9, 40, 8, 576, True),      # eight heads: one per XCD
+    (True, 9, 40, 8, 640, True),      # eight heads: one per XCD
 ]
 
 

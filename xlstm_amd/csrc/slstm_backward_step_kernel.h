@@ -1,20 +1,31 @@
-// The reverse pass with ONE LAUNCH PER STEP, for the head dims whose slice of R transposed no compute unit can keep in
-// its registers (1024 in bf16, 512 in float32: 4 dh x 64 operands are 512 KiB, the whole register file), where the
+// The backward pass with ONE LAUNCH PER STEP, for the head dims whose slice of R no compute unit can keep in its
+// registers (1024 in bf16, 512 in float32: 4 dh x 64 operands are 512 KiB, the whole register file), where the
 // persistent kernels of slstm_backward_kernels.h do not reach.  Included by slstm_hip.hip only.
 //
 // It is the reference's own decomposition (slstm_backward.cu:291-319: per timestep one pointwise launch and one
-// strided-batched GEMM with R transposed), fused into one kernel per step and turned round: the launch of step t first
-// forms what reaches y_t through the recurrence - the gate deltas of step t + 1 (left in memory by the launch before,
-// in the type of the operands) times R transposed - and then the gradient of step t from it, its nine coefficients
-// and d_h, element by element.  A workgroup owns 64 batch rows x 32 hidden units: K = 4 dh gate units are walked in
-// slabs of 256 bytes per row that four feeder waves bring straight into a ring of LDS slots, several slabs ahead of
-// the four waves that multiply, one barrier per slab (both operands lie in memory slab by slab, so a slab of a tile is
-// one piece of 8 or 16 KiB; with the loads in registers of the multiplying waves, whose waits the compiler places, a
-// slab took a whole memory latency: 73 us per step at 4 heads of 1024 instead of the figures below); the product is formed transposed (units on the MFMA M axis), so a lane ends with 4 consecutive units
-// of one batch row and everything pointwise moves as 16-byte accesses, asked for in front of the K loop.  What the
-// steps hand on besides the deltas - the gradients of c and n - lives in planes 1 and 2 of d_s0 between the launches
-// (each element is read and written by the same lane of the same workgroup of every launch); a last launch (t = -1)
-// forms what reaches the y of the initial state.  No launch waits for another workgroup: nothing here can give up.
+// strided-batched GEMM with R transposed; the forward that fills its caches likewise, slstm_forward.cu:176-182), each
+// step fused into one kernel:
+//
+//   slstm_fwd_walk_kernel   the forward walk (what slstm_bwd_prepare_kernel does for the smaller head dims): the launch
+//                           of step t multiplies the outputs of step t - 1, which the forward call stored, by R, adds
+//                           W.x and the bias, runs the forward's update on the state that the walk keeps in memory, and
+//                           leaves the step's nine coefficients.
+//   slstm_bwd_step_kernel   the reverse pass: the launch of step t first forms what reaches y_t through the recurrence -
+//                           the gate deltas of step t + 1 (left in memory by the launch before, in the type of the
+//                           operands) times R transposed - and then the gradient of step t from it, its nine
+//                           coefficients and d_h, element by element.  What the steps hand on besides the deltas - the
+//                           gradients of c and n - lives in planes 1 and 2 of d_s0 between the launches; a last launch
+//                           (t = -1) forms what reaches the y of the initial state.
+//
+// Both: a workgroup owns 64 batch rows x 32 hidden units (the walk: x 4 gates).  K is walked in slabs of 256 bytes per
+// row that four feeder waves bring straight into a ring of LDS slots, slabs ahead of the four waves that multiply, one
+// barrier per slab; R lies in memory slab by slab, so a slab of a tile is one piece.  (With the loads in registers of
+// the multiplying waves, whose waits the compiler places, a slab took a whole memory latency: 73 us per step of the
+// reverse pass at 4 heads of 1024 instead of 19, 29 us per step of the walk.)  The product is formed transposed (units
+// on the MFMA M axis), so a lane ends with 4 consecutive units of one batch row and everything pointwise moves as
+// 16-byte accesses, asked for in front of the K loop.  Each element of what the launches hand to each other is read
+// and written by the same lane of the same workgroup of every launch.  No launch waits for another workgroup: nothing
+// here can give up.
 #pragma once
 
 namespace {
@@ -243,6 +254,234 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     }
     *reinterpret_cast<f32x4 *>(p.d_s0 + BH + eo[ut]) = dc_prev;
     *reinterpret_cast<f32x4 *>(p.d_s0 + 2 * BH + eo[ut]) = dn_prev;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+struct FwdWalkParams {
+  int B, T, NH, dh;
+  int t;
+  const void *wx;            // [B,T,4,NH,dh], strides in elements
+  long long wx_sb, wx_st;
+  const void *r_tiled;       // R in the type of the operands, in slabs of 256 bytes of K per tile of 32 units:
+                             // [NH][a / 32][k / KS][gate][a % 32][k % KS], KS = 128 (bf16) or 64 (float32)
+  const void *h_prev;        // [B][H] in the type of the operands: the outputs of step t - 1 (step 0: the y of the initial
+                             // state in that type), or null: zeros
+  const float *bias;         // [NH,4,dh]
+  const float *state_in;     // [4,B,H]: planes 1-3 are c, n, m in front of the step (step 0: the initial state), or null: zeros
+  float *state;              // [4,B,H]: planes 1-3 take c, n, m behind the step
+  const uint8_t *reset;      // [B,T] or null
+  long long reset_sb;
+  float *coef;               // [T,B,9,H]
+};
+
+constexpr int kFwdWalkSlots = 3;
+constexpr int kFwdWalkSlot = (64 + 128) * 256;  // bytes of a slab in LDS: the outputs of 64 rows, R of 4 gates x 32 units
+constexpr int fwd_walk_lds_bytes() { return kFwdWalkSlots * kFwdWalkSlot; }
+
+// R [NH][4 dh][dh] into the walk's slabs, and the y plane of the initial state into the type of the operands
+template <bool BF16>
+__global__ __launch_bounds__(256) void slstm_fwd_walk_init_kernel(const void *r, void *r_tiled, const float *s0, void *h_init, int B, int NH, int dh) {
+  constexpr int ESZ = BF16 ? 2 : 4;
+  const int nslab = dh * ESZ >> 8;
+  const long long pieces = (long long)NH * 4 * dh * nslab * 16;  // 16-byte pieces of R
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < pieces; i += stride) {
+    const int piece = (int)(i & 15);
+    long long v = i >> 4;
+    const int j = (int)(v & 31); v >>= 5;
+    const int g = (int)(v & 3); v >>= 2;
+    const int slab = (int)(v % nslab); v /= nslab;
+    const int ut = (int)(v % (dh >> 5));
+    const int head = (int)(v / (dh >> 5));
+    const char *src = reinterpret_cast<const char *>(r) + (((long long)head * 4 + g) * dh + ut * 32 + j) * dh * ESZ + slab * 256 + piece * 16;
+    reinterpret_cast<uint4 *>(r_tiled)[i] = *reinterpret_cast<const uint4 *>(src);
+  }
+  const long long BH = (long long)B * NH * dh;
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < BH; i += stride) {
+    const float y = s0 ? s0[i] : 0.0f;
+    if (BF16) reinterpret_cast<uint16_t *>(h_init)[i] = (uint16_t)(pack_bf16x2(y, 0.0f) & 0xFFFFu);
+    else reinterpret_cast<float *>(h_init)[i] = y;
+  }
+}
+
+template <bool BF16>
+__global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalkParams p) {
+  constexpr int ESZ = BF16 ? 2 : 4;
+  constexpr int D = kFwdWalkSlots;
+  extern __shared__ __attribute__((aligned(1024))) unsigned char fwalk_lds[];
+  const int dh = p.dh, NH = p.NH;
+  const int H = NH * dh;
+  const long long BH = (long long)p.B * H;
+  const int n_ut = dh >> 5, n_rt = (p.B + 63) >> 6;
+  int head, tile;  // (placed as in slstm_bwd_step_kernel)
+  {
+    const int i = blockIdx.x, tiles = n_ut * n_rt;
+    if (NH % 8 == 0) {
+      const int hpx = NH / 8, m = i >> 3;
+      head = (i & 7) * hpx + m % hpx;
+      tile = m / hpx;
+    } else if (8 % NH == 0 && tiles % (8 / NH) == 0) {
+      head = (i & 7) % NH;
+      tile = (i >> 3) * (8 / NH) + (i & 7) / NH;
+    } else {
+      head = i / tiles;
+      tile = i - head * tiles;
+    }
+  }
+  const int a0 = (tile % n_ut) * 32, rowbase = (tile / n_ut) * 64;
+  const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
+  const int wave = (int)uniform((uint32_t)(tid >> 6));
+  const int t = p.t;
+  const int nslab = dh * ESZ >> 8;
+  const uint32_t lds0 = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)fwalk_lds);
+
+  if (wave >= 4) {
+    // ---- a feeder wave: per slab 4 of the 16 KiB of outputs and 8 of the 32 KiB of R, 1 KiB (4 rows of 256 bytes) per
+    //      load, straight into LDS, piece g of row r at position g ^ (r & 7) (see slstm_bwd_step_kernel).  Rows past
+    //      the batch, rows that start a document at this step and a walk without an initial state ask out of range:
+    //      the loads return zeros.
+    const int f = wave - 4, sub = lane >> 4, pos = lane & 15;
+    const unsigned long long hb = reinterpret_cast<unsigned long long>(p.h_prev ? p.h_prev : p.r_tiled);
+    const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_tiled) + ((long long)head * n_ut + (a0 >> 5)) * nslab * (128 * 256);
+    const u32x4_t hrs = {uniform((uint32_t)hb), uniform((uint32_t)(hb >> 32) & 0xFFFFu), (uint32_t)(BH * ESZ), 0x00020000u};
+    const u32x4_t rrs = {uniform((uint32_t)rb), uniform((uint32_t)(rb >> 32) & 0xFFFFu), (uint32_t)(nslab * (128 * 256)), 0x00020000u};
+    uint32_t hvo[4], rvo[8];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int row = 4 * (4 * f + k) + sub, brow = rowbase + row;
+      bool zero = brow >= p.B || !p.h_prev;
+      if (!zero && p.reset) zero = p.reset[(long long)brow * p.reset_sb + t] != 0;
+      hvo[k] = zero ? 0x80000000u : (uint32_t)(((long long)brow * H + head * dh) * ESZ + ((pos ^ (row & 7)) << 4));
+    }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int row = 4 * (8 * f + k) + sub;  // gate row / 32, unit row % 32 of the tile
+      rvo[k] = (uint32_t)(row * 256 + ((pos ^ (row & 7)) << 4));
+    }
+    auto request = [&](int s) {
+      const int sc = s < nslab ? s : nslab - 1;
+      const uint32_t slot = lds0 + (uint32_t)(s % D) * kFwdWalkSlot;
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+        bwd_fetch_to_lds_b128(hrs, uniform(slot + (4 * f + k) * 1024), hvo[k] + (uint32_t)sc * 256u);
+#pragma unroll
+      for (int k = 0; k < 8; ++k)
+        bwd_fetch_to_lds_b128(rrs, uniform(slot + 64 * 256 + (8 * f + k) * 1024), rvo[k] + (uint32_t)sc * (128 * 256));
+    };
+    for (int s = 0; s < D - 1; ++s) request(s);
+    for (int s = 0; s < nslab; ++s) {
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(12 * (D - 2)) : "memory");  // (slab s has landed)
+      lds_barrier();
+      request(s + D - 1);
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    return;
+  }
+  const int wr = wave >> 1, wu = wave & 1;
+
+  // ---- pointwise operands of this lane's elements (rows rowbase + 32 wr + 16 ut + r16, units a0 + 16 wu + 4 q .. + 3)
+  const int ua = a0 + 16 * wu + 4 * q;
+  f32x4 bias4[4], wx4[2][4], cv[2], nv[2], mv[2];
+  bool there[2], restart[2];
+  long long eo[2];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) bias4[g] = *reinterpret_cast<const f32x4 *>(p.bias + ((long long)head * 4 + g) * dh + ua);
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    const int row = rowbase + 32 * wr + 16 * ut + r16;
+    there[ut] = row < p.B;
+    const int rowc = there[ut] ? row : p.B - 1;
+    eo[ut] = (long long)rowc * H + head * dh + ua;
+    restart[ut] = !p.state_in || (p.reset && p.reset[(long long)rowc * p.reset_sb + t] != 0);
+    const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    cv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + BH + eo[ut]) : zero;
+    nv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + 2 * BH + eo[ut]) : zero;
+    mv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + 3 * BH + eo[ut]) : zero;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const long long o = (long long)rowc * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + head * dh + ua;
+      if (BF16) {
+        typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+        const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(reinterpret_cast<const uint16_t *>(p.wx) + o));
+        wx4[ut][g] = f32x4{bf16_bits_to_float(w.x & 0xFFFFu), bf16_bits_to_float(w.x >> 16), bf16_bits_to_float(w.y & 0xFFFFu), bf16_bits_to_float(w.y >> 16)};
+      } else {
+        wx4[ut][g] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.wx) + o));
+      }
+    }
+  }
+
+  // ---- R [4 x 32 units x K] . y_{t-1} [64 rows x K], transposed: acc[ut][g][i] = gate g of unit ua + i, row 32 wr + 16 ut + r16
+  f32x4 acc[2][4];
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+  {
+    int swz[4];
+#pragma unroll
+    for (int ch = 0; ch < 4; ++ch) swz[ch] = ((4 * ch + q) ^ (r16 & 7)) << 4;
+    const int hrow[2] = {(32 * wr + r16) * 256, (32 * wr + 16 + r16) * 256};
+    const int rrow = 64 * 256 + (16 * wu + r16) * 256;  // (gate g: 32 rows further each)
+    for (int s = 0; s < nslab; ++s) {
+      lds_barrier();
+      const unsigned char *slot = fwalk_lds + (s % D) * kFwdWalkSlot;
+#pragma unroll
+      for (int ch = 0; ch < 4; ++ch) {
+        uint4 rv[4], hv[2];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) rv[g] = *reinterpret_cast<const uint4 *>(slot + rrow + g * (32 * 256) + swz[ch]);
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut) hv[ut] = *reinterpret_cast<const uint4 *>(slot + hrow[ut] + swz[ch]);
+#pragma unroll
+        for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            if (BF16) {
+              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
+            } else {
+              const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w}, hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+            }
+          }
+      }
+    }
+  }
+
+  // ---- the forward's update with the gate values kept, and the nine coefficients of the step's gradient
+#pragma unroll
+  for (int ut = 0; ut < 2; ++ut) {
+    if (!there[ut]) continue;
+    f32x4 cf[9], cn, nn, mn;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float raw[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) raw[g] = (wx4[ut][g][i] + acc[ut][g][i]) + bias4[g][i];
+      CellState st{0.0f, restart[ut] ? 0.0f : cv[ut][i], restart[ut] ? 0.0f : nv[ut][i], restart[ut] ? 0.0f : mv[ut][i]};
+      const float c_old = st.c, n_old = st.n;
+      GateValues k;
+      slstm_pointwise_keep(raw[0], raw[1], raw[2], raw[3], st, k);
+      const float omf = __builtin_amdgcn_rcpf(1.0f + __expf(raw[1]));  // 1 - sigmoid(f)
+      cf[0][i] = k.og * k.rn;
+      cf[1][i] = st.y * k.rn;
+      cf[2][i] = k.ig * k.tz;
+      cf[3][i] = k.ig;
+      cf[4][i] = k.fg * omf * c_old;
+      cf[5][i] = k.fg * omf * n_old;
+      cf[6][i] = k.ig * (1.0f - k.tz * k.tz);
+      cf[7][i] = (1.0f - k.og) * st.y;
+      cf[8][i] = k.fg;
+      cn[i] = st.c; nn[i] = st.n; mn[i] = st.m;
+    }
+    float *cd = p.coef + ((long long)t * p.B + (rowbase + 32 * wr + 16 * ut + r16)) * 9 * H + head * dh + ua;
+#pragma unroll
+    for (int j = 0; j < 9; ++j) __builtin_nontemporal_store(cf[j], reinterpret_cast<f32x4 *>(cd + (long long)j * H));
+    *reinterpret_cast<f32x4 *>(p.state + BH + eo[ut]) = cn;
+    *reinterpret_cast<f32x4 *>(p.state + 2 * BH + eo[ut]) = nn;
+    *reinterpret_cast<f32x4 *>(p.state + 3 * BH + eo[ut]) = mn;
   }
 }
 

@@ -394,11 +394,10 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   return XS_OK;
 }
 
-// ---- backward pass with one launch per step (split == 3): the forward walk is the decode step kernel in its variant
-// that leaves the coefficients, the reverse pass slstm_bwd_step_kernel.  Both keep what a step hands to the next in
-// the caller's `exchange` buffer: 256 bytes that the step kernel's status words go to, two states [4,B,H] float32 that
-// the forward walk alternates between, one [B,H] row of outputs in the type of the operands that nobody reads; the
-// reverse pass two sets of gate deltas in the type of the operands, in tiles of 64 rows.
+// ---- backward pass with one launch per step (split == 3): slstm_fwd_walk_kernel and slstm_bwd_step_kernel.  Both keep
+// what a step hands to the next in the caller's `exchange` buffer: the forward walk a state [4,B,H] float32 (its y
+// plane holds the y of the initial state in the type of the operands) and R in the walk's slabs; the reverse pass two
+// sets of gate deltas in the type of the operands, in tiles of 64 rows.
 int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   const bool bf16 = a->dtype == XS_BF16;
   const int esz = bf16 ? 2 : 4;
@@ -407,40 +406,37 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   hipStream_t stream = (hipStream_t)a->stream;
   if (!a->exchange) return fail(XS_ERR_NULL, "exchange is required with one launch per step");
   if (((uintptr_t)a->exchange % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "exchange and coef must be 16-byte aligned");
+  if ((dh * esz) % 256 != 0) return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d is not a multiple of %d", dh, 256 / esz);
+  const long long nwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
+  if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
   if (prepare) {
-    if (!a->wx || !a->r || !a->bias) return fail(XS_ERR_NULL, "wx, r and bias are required");
+    if (!a->wx || !a->r || !a->bias || !a->h_out) return fail(XS_ERR_NULL, "wx, r, bias and h_out are required");
     if (a->wx_stride_t < 4 * H || (B > 1 && a->wx_stride_b < 4 * H)) return fail(XS_ERR_SHAPE, "wx strides overlap the innermost 4*H elements");
     if (((uintptr_t)a->wx % 16) || ((a->wx_stride_b * esz) % 16) || ((a->wx_stride_t * esz) % 16))
       return fail(XS_ERR_ALIGN, "wx and its row/step strides must be 16-byte aligned");
-    if (((uintptr_t)a->r % 16) || ((uintptr_t)a->s0 % 16) || ((uintptr_t)a->bias % 16)) return fail(XS_ERR_ALIGN, "r, s0 and bias must be 16-byte aligned");
-    const int epc = bf16 ? 8 : 4;
-    int nch = 1;
-    while (nch * 16 * epc < dh) nch *= 2;
-    int nch_log2 = 0;
-    while ((1 << nch_log2) < nch) ++nch_log2;
+    if (((uintptr_t)a->r % 16) || ((uintptr_t)a->s0 % 16) || ((uintptr_t)a->bias % 16) || ((uintptr_t)a->h_out % 16))
+      return fail(XS_ERR_ALIGN, "r, s0, bias and h_out must be 16-byte aligned");
+    if (BH * esz >= (1ll << 31)) return fail(XS_ERR_UNSUPPORTED, "a step's outputs of 2 GiB or more");
     char *const ws = (char *)a->exchange;
-    float *const states[2] = {(float *)(ws + 256), (float *)(ws + 256 + 16 * BH)};
-    StepParams p;
-    p.r = a->r; p.r_bf16 = bf16; p.bias = a->bias;
-    p.reset_sb = a->reset_stride_b;
-    p.h_out = ws + 256 + 32 * BH;
-    p.status = (xs_slstm_status *)ws;
-    p.B = B; p.NH = NH; p.dh = dh;
-    p.n_unit_tiles = (dh + 31) / 32;
-    p.n_row_tiles = (B + 63) / 64;
-    p.h_prev = nullptr; p.spin_limit = 0; p.wx_sb = a->wx_stride_b;
-    const long long nwg = (long long)NH * p.n_unit_tiles * p.n_row_tiles;
-    if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
-    void (*kern)(StepParams, int) = bf16 ? slstm_step_tile_kernel<true, 2, false, false, false, true>
-                                         : slstm_step_tile_kernel<false, 2, false, false, false, true>;
-    const size_t lds = (size_t)2 * (64 + 128) * (2 * 64 + 16);
+    float *const state = (float *)ws;              // [4,B,H]; the y plane: the y of the initial state in the type of the operands
+    char *const r_tiled = ws + 16 * BH;
+    void (*init)(const void *, void *, const float *, void *, int, int, int) = bf16 ? slstm_fwd_walk_init_kernel<true> : slstm_fwd_walk_init_kernel<false>;
+    hipLaunchKernelGGL(init, dim3(1024), dim3(256), 0, stream, a->r, (void *)r_tiled, a->s0, (void *)state, B, NH, dh);
+    FwdWalkParams p;
+    p.B = B; p.T = T; p.NH = NH; p.dh = dh;
+    p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
+    p.r_tiled = r_tiled; p.bias = a->bias; p.state = state;
+    p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
+    void (*kern)(FwdWalkParams) = bf16 ? slstm_fwd_walk_kernel<true> : slstm_fwd_walk_kernel<false>;
+    {
+      const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)fwd_walk_lds_bytes());
+      if (rc != XS_OK) return rc;
+    }
     for (int t = 0; t < T; ++t) {
-      p.wx = (const char *)a->wx + (long long)t * a->wx_stride_t * esz;
-      p.s0 = t == 0 ? a->s0 : states[(t - 1) & 1];
-      p.s_out = states[t & 1];
-      p.reset = a->reset ? a->reset + t : nullptr;
-      p.coef = a->coef + (long long)t * 9 * BH;
-      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(256), lds, stream, p, nch_log2);
+      p.t = t;
+      p.h_prev = t == 0 ? (a->s0 ? (const void *)state : nullptr) : (const void *)((const char *)a->h_out + (long long)(t - 1) * BH * esz);
+      p.state_in = t == 0 ? a->s0 : state;
+      hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBwdStepThreads), fwd_walk_lds_bytes(), stream, p);
     }
   } else {
     if (!a->d_h || !a->r_t || !a->d_wx || !a->d_s0) return fail(XS_ERR_NULL, "d_h, r_t, d_wx and d_s0 are required");
@@ -457,8 +453,6 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
     q.cut = a->recurrent_cut != 0;
     q.clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
     char *const deltas[2] = {(char *)a->exchange, (char *)a->exchange + 4ll * ((B + 63) / 64 * 64) * H * esz};  // (tiles of 64 rows)
-    const long long nwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
-    if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
     void (*kern)(BwdStepParams) = bf16 ? slstm_bwd_step_kernel<true> : slstm_bwd_step_kernel<false>;
     {
       const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)bwd_step_lds_bytes());
@@ -484,8 +478,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (a->split == 3) {
     // one launch per step: the head dims the forward covers beyond those of the persistent kernels, and those next below
     const int lo = a->dtype == XS_BF16 ? 512 : 256;
-    if (a->dh % 64 != 0 || a->dh < lo || a->dh > 2 * lo)
-      return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d not supported (%d to %d in steps of 64)", a->dh, lo, 2 * lo);
+    if (a->dh % (lo / 4) != 0 || a->dh < lo || a->dh > 2 * lo)
+      return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d not supported (%d to %d in steps of %d)", a->dh, lo, 2 * lo, lo / 4);
   } else if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && a->dtype == XS_BF16 && (prepare || a->split)))
     return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256; 512 in bf16 over several compute units; "
                 "up to 1024 in bf16 and 512 in float32 with one launch per step, split = 3)", a->dh);

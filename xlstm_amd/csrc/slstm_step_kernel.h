@@ -39,7 +39,6 @@ struct StepParams {
   int n_unit_tiles, n_row_tiles;
   const void *h_prev;  // optional bf16 copy of the y plane of s0 (see the HB variant)
   int spin_limit;      // bound of the waits between the waves of a workgroup (the pipelined kernel)
-  float *coef;         // COEF variants: [B][9][H], the step's nine coefficients of the backward pass (see slstm_bwd_prepare_kernel)
 };
 
 // Workgroup i runs on XCD i % 8.  The workgroups of one head share its h rows and its R, so they
@@ -87,12 +86,9 @@ __device__ __forceinline__ void step_tile_of(const StepParams &p, int i, int &he
 // Measured slower or equal: the gating waves fetching and staging the second K half (it then arrives later and
 // the MFMA waves wait for it), the gating waves fetching row tile 1's operands late and handing them over
 // through LDS, streaming loads for the once-read operands.
-// COEF (the backward pass of the head dims that only this kernel covers walks forward with it, one launch per step):
-// the step also leaves the nine coefficients of its gradient in StepParams::coef.
-template <bool BF16, int SLABCH, bool FULL, bool HB = false, bool SPLIT = false, bool COEF = false>
+template <bool BF16, int SLABCH, bool FULL, bool HB = false, bool SPLIT = false>
 __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(StepParams p, int nch_log2) {
   static_assert(!HB || (BF16 && FULL), "the bf16 operand hint is a steady-state bf16 path");
-  static_assert(!COEF || (!FULL && !SPLIT), "the coefficients come from the general variant");
   static_assert(!SPLIT || SLABCH >= 4, "two roles only with the whole K range in one slab");
   constexpr int HBYTES = HB ? 2 : 4;          // bytes per element of the recurrent operand as it is read
   constexpr int EPC = BF16 ? 8 : 4;
@@ -310,7 +306,6 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
     const float nin[4] = {n4[ut].x, n4[ut].y, n4[ut].z, n4[ut].w};
     const float min_[4] = {m4[ut].x, m4[ut].y, m4[ut].z, m4[ut].w};
     float yv[4], cv[4], nv[4], mv[4];
-    float cf[COEF ? 9 : 1][4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       float raw[4];
@@ -328,33 +323,11 @@ __global__ __launch_bounds__(SPLIT ? 512 : 256) void slstm_step_tile_kernel(Step
         raw[g] = (wxv + tot[ut][g][i]) + bf[i];
       }
       CellState st{0.0f, reset_row ? 0.0f : cin[i], reset_row ? 0.0f : nin[i], reset_row ? 0.0f : min_[i]};
-      if constexpr (COEF) {
-        const float c_old = st.c, n_old = st.n;
-        GateValues k;
-        slstm_pointwise_keep(raw[0], raw[1], raw[2], raw[3], st, k);
-        const float omf = __builtin_amdgcn_rcpf(1.0f + __expf(raw[1]));  // 1 - sigmoid(f)
-        cf[0][i] = k.og * k.rn;
-        cf[1][i] = st.y * k.rn;
-        cf[2][i] = k.ig * k.tz;
-        cf[3][i] = k.ig;
-        cf[4][i] = k.fg * omf * c_old;
-        cf[5][i] = k.fg * omf * n_old;
-        cf[6][i] = k.ig * (1.0f - k.tz * k.tz);
-        cf[7][i] = (1.0f - k.og) * st.y;
-        cf[8][i] = k.fg;
-      } else {
-        slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
-      }
+      slstm_pointwise(raw[0], raw[1], raw[2], raw[3], st);
       yv[i] = st.y; cv[i] = st.c; nv[i] = st.n; mv[i] = st.m;
     }
     if (FULL || (brow < p.B && ua < dh)) {
       const long long o = (long long)brow * H + head * dh + ua;
-      if constexpr (COEF) {
-#pragma unroll
-        for (int j = 0; j < 9; ++j)
-          __builtin_nontemporal_store(f32x4{cf[j][0], cf[j][1], cf[j][2], cf[j][3]},
-                                      reinterpret_cast<f32x4 *>(p.coef + ((long long)brow * 9 + j) * H + head * dh + ua));
-      }
       // streaming stores: the lines leave the L2 while the kernel still runs instead of being
       // written back when it ends (measured: 0.65 us per step at B = 256, D = 2048)
       __builtin_nontemporal_store(f32x4{yv[0], yv[1], yv[2], yv[3]}, reinterpret_cast<f32x4 *>(p.s_out + o));

@@ -54,22 +54,24 @@ def _compute_units(dev) -> int:
 
 def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
     """The head dim that the backward kernels run a head dim ``dh`` as: 64, 128, 256 (and 512 with bfloat16 inputs) for
-    the kernels that take one launch for all steps, beyond those any multiple of 64 up to the forward's range (1024 with
-    bfloat16, 512 with float32) for the kernels that take one launch per step; sizes in between are padded up by
-    ``slstm_backward``.  None when there is none."""
+    the kernels that take one launch for all steps; beyond those, up to the forward's range (1024 with bfloat16, 512 with
+    float32), the next multiple of 128 (bfloat16) or 64 (float32) for the kernels that take one launch per step.  Sizes
+    in between are padded up by ``slstm_backward``.  None when there is none."""
     bf16 = dtype == torch.bfloat16
     for size in (64, 128, 256, 512):
         if dh <= size and (size < 512 or bf16):
             return size
     if dh <= (1024 if bf16 else 512):
-        return (dh + 63) // 64 * 64
+        step = 128 if bf16 else 64
+        return (dh + step - 1) // step * step
     return None
 
 
-def stepwise_exchange_bytes(B: int, H: int, esz: int) -> int:
-    """Bytes of the ``exchange`` buffer of a backward pass of one launch per step: the forward walk keeps 256 bytes of
-    status words, two states and a row of outputs there, the reverse pass two sets of gate deltas in tiles of 64 rows."""
-    return max(256 + 32 * B * H + B * H * esz, 8 * ((B + 63) // 64 * 64) * H * esz)
+def stepwise_exchange_bytes(B: int, NH: int, dh: int, esz: int) -> int:
+    """Bytes of the ``exchange`` buffer of a backward pass of one launch per step: the forward walk keeps a state
+    ``[4,B,H]`` and R in its own order there, the reverse pass two sets of gate deltas in tiles of 64 rows."""
+    H = NH * dh
+    return max(16 * B * H + 4 * NH * dh * dh * esz, 8 * ((B + 63) // 64 * 64) * H * esz)
 
 
 def backward_runs_stepwise(dh_kernel: int, dtype: torch.dtype) -> bool:
@@ -272,7 +274,7 @@ def slstm_backward(
         # [NH][d / 32][k / KS][d % 32][k % KS]; what the launches of a call hand to each other goes through `exchange`
         ks = 256 // esz
         r_t = (r32.transpose(1, 2).to(wx.dtype).reshape(NH, dh // 32, 32, 4 * dh // ks, ks).permute(0, 1, 3, 2, 4).contiguous())
-        exchange = torch.empty(stepwise_exchange_bytes(B, H, esz), dtype=torch.uint8, device=dev)
+        exchange = torch.empty(stepwise_exchange_bytes(B, NH, dh, esz), dtype=torch.uint8, device=dev)
         counters = None
     else:
         # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
