@@ -317,6 +317,58 @@ def bench_backward(device, iters=3):
                          "traffic_source": "profiles/traffic_bwd_cfg2.json (rocprofv3 counters of a separate run, not of this one)"}}
 
 
+def bench_backward_large(device, T=4096, iters=2):
+    """The backward pass at BASELINE config 5's shape (B=64, 4 heads of 1024, bf16): the kernels of one launch per step
+    (``split == 3`` of the C ABI), the whole call and its three parts by HIP events.  Per step the walk and the reverse
+    pass each read R once (32 MiB: it does not stay in any cache level below the Infinity Cache) and the operand rows
+    once per tile of 32 units; the roofline line prices those bytes of the reverse kernel against the HBM peak."""
+    import numpy as np
+    import torch
+
+    from xlstm_amd import functional as F
+
+    B, NH, dh = 64, 4, 1024
+    H = NH * dh
+    g = torch.Generator(device=device).manual_seed(11)
+    wx = torch.empty(B, T, 4 * H, dtype=torch.bfloat16, device=device)
+    for row in range(B):
+        wx[row] = torch.randn(T, 4 * H, generator=g, device=device).bfloat16()
+    r = (torch.rand(NH, 4 * dh, dh, generator=g, device=device) * 2 - 1) / float(np.sqrt(H))
+    bias = torch.zeros(NH, 4, dh, device=device)
+    bias[:, 1] = torch.linspace(3.0, 6.0, dh, device=device)
+    h, _ = F.slstm_forward(wx, r, bias)
+    d_h = torch.empty(T, B, H, dtype=torch.bfloat16, device=device)
+    for t0 in range(0, T, 256):
+        d_h[t0:t0 + 256] = torch.randn(min(256, T - t0), B, H, generator=g, device=device).bfloat16()
+    total, prep, rev, par = [], [], [], []
+    for i in range(iters + 1):
+        tm = {}
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = F.slstm_backward(wx, r, bias, None, None, h, d_h, timings=tm)
+        torch.cuda.synchronize()
+        if i:
+            total.append((time.perf_counter() - t0) * 1e3)
+            ev = tm["events"]
+            prep.append(ev[0].elapsed_time(ev[1]))
+            rev.append(ev[1].elapsed_time(ev[2]))
+            par.append(ev[2].elapsed_time(ev[3]))
+        finite = bool(torch.isfinite(out[0][:, -1]).all() and torch.isfinite(out[3]).all())
+        del out
+    rev_ms = float(np.median(rev))
+    # a launch of the reverse kernel: R transposed once, nine coefficients in and four gate deltas out per element in
+    # float32, the deltas in bf16 out and (the step behind's) in, d_h in bf16, the gradients of c and n in and out
+    nbytes = NH * 4 * dh * dh * 2 + (9 * 4 + 4 * 4 + 2 + 2 + 2 + 4 * 4) * B * H
+    return {"workload": "backward pass at config 5's shape: B=64 T=%d D=4096 NH=4 bf16, one launch per step" % T,
+            "ms": float(np.median(total)), "forward_walk_ms": float(np.median(prep)), "reverse_ms": rev_ms,
+            "parameter_gradient_kernel_ms": float(np.median(par)),
+            "us_per_step": {"forward_walk": float(np.median(prep)) * 1e3 / T, "reverse": rev_ms * 1e3 / (T + 1)},
+            "finite": finite,
+            "roofline": {"bound": "hbm", "achieved": nbytes / (rev_ms / (T + 1) * 1e-3) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": nbytes / (rev_ms / (T + 1) * 1e-3) / 1e9 / HBM_PEAK_GBS, "traffic": None,
+                         "kernel": "slstm_bwd_step_kernel<bf16>", "algorithmic_bytes_per_launch": nbytes}}
+
+
 def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
     """Times one forward call of the cell at another BASELINE shape (median of `iters`)."""
     import numpy as np
@@ -617,6 +669,9 @@ def main():
                     help="only time the sequence kernel at B = 1, 2, 4 (head dims 128 and 256) and the reference test's shape")
     ap.add_argument("--backward-only", action="store_true",
                     help="only time the backward pass at config 2 (its own JSON line)")
+    ap.add_argument("--backward-large-only", action="store_true",
+                    help="only the backward pass at config 5's shape (4 heads of 1024: one launch per step)")
+    ap.add_argument("--backward-large-steps", type=int, default=4096, help="sequence length of --backward-large-only")
     ap.add_argument("--phase-profile", action="store_true",
                     help="per-phase cycle tables of the sequence kernels from the measurement build of the library "
                          "(python -m xlstm_amd.build -DXS_PROFILE -o xlstm_amd/lib/libxlstm_amd_profile.so)")
@@ -666,6 +721,10 @@ def main():
         return
     if args.backward_only:
         print(json.dumps({"backward": bench_backward(device, iters=max(1, min(args.steps, 5)))}))
+        return
+    if args.backward_large_only:
+        print(json.dumps({"backward_config5_shape": bench_backward_large(device, T=args.backward_large_steps,
+                                                                           iters=max(1, min(args.steps, 3)))}))
         return
     if args.config5_only:
         c5 = bench_config(device, CONFIG5_NAME, 64, 4096, 4, 1024, True, 0, iters=max(1, min(args.steps, 5)))
@@ -771,6 +830,7 @@ def main():
             bench_config(device, "reference test shape: B=1 T=1 NH=4 dh=16 fp32 (one step, the step kernel)", 1, 1, 4, 16, False, 0, iters=20),
         ]
         out["backward"] = bench_backward(device)
+        out["backward_config5_shape"] = bench_backward_large(device)
     if args.config4:
         out["config4"] = bench_config4(device)
     if args.layer:

@@ -103,6 +103,7 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     //      (slabs past the end are asked for like the others - the last slab again, into a slot that nobody reads).
     if (!multiply) return;
     const int f = wave - 4, sub = lane >> 4, pos = lane & 15;
+    const bool live = rowbase + 16 * f < p.B;  // (this wave's 16 rows of deltas: not fetched when the batch ends in front of them)
     const unsigned long long db = reinterpret_cast<unsigned long long>(p.delta_in) + dtile;
     const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_t) + ((long long)head * (dh >> 5) + (a0 >> 5)) * nslab * (32 * 256);
     const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), (uint32_t)(nslab * (64 * 256)), 0x00020000u};
@@ -121,16 +122,19 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     auto request = [&](int s) {
       const int sc = s < nslab ? s : nslab - 1;
       const uint32_t slot = lds0 + (uint32_t)(s % D) * kBwdStepSlot;
+      if (live) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        bwd_fetch_to_lds_b128(drs, uniform(slot + (4 * f + k) * 1024), dvo[k] + (uint32_t)sc * (64 * 256));
+        for (int k = 0; k < 4; ++k)
+          bwd_fetch_to_lds_b128(drs, uniform(slot + (4 * f + k) * 1024), dvo[k] + (uint32_t)sc * (64 * 256));
+      }
 #pragma unroll
       for (int k = 0; k < 2; ++k)
         bwd_fetch_to_lds_b128(rrs, uniform(slot + 64 * 256 + (2 * f + k) * 1024), rvo[k] + (uint32_t)sc * (32 * 256));
     };
     for (int s = 0; s < D - 1; ++s) request(s);
     for (int s = 0; s < nslab; ++s) {
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(6 * (D - 2)) : "memory");  // (slab s has landed)
+      if (live) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(6 * (D - 2)) : "memory");  // (slab s has landed)
+      else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * (D - 2)) : "memory");
       lds_barrier();
       request(s + D - 1);
     }
@@ -342,6 +346,7 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalk
     //      the batch, rows that start a document at this step and a walk without an initial state ask out of range:
     //      the loads return zeros.
     const int f = wave - 4, sub = lane >> 4, pos = lane & 15;
+    const bool live = rowbase + 16 * f < p.B;  // (this wave's 16 rows of outputs: not fetched when the batch ends in front of them)
     const unsigned long long hb = reinterpret_cast<unsigned long long>(p.h_prev ? p.h_prev : p.r_tiled);
     const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_tiled) + ((long long)head * n_ut + (a0 >> 5)) * nslab * (128 * 256);
     const u32x4_t hrs = {uniform((uint32_t)hb), uniform((uint32_t)(hb >> 32) & 0xFFFFu), (uint32_t)(BH * ESZ), 0x00020000u};
@@ -362,16 +367,19 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalk
     auto request = [&](int s) {
       const int sc = s < nslab ? s : nslab - 1;
       const uint32_t slot = lds0 + (uint32_t)(s % D) * kFwdWalkSlot;
+      if (live) {
 #pragma unroll
-      for (int k = 0; k < 4; ++k)
-        bwd_fetch_to_lds_b128(hrs, uniform(slot + (4 * f + k) * 1024), hvo[k] + (uint32_t)sc * 256u);
+        for (int k = 0; k < 4; ++k)
+          bwd_fetch_to_lds_b128(hrs, uniform(slot + (4 * f + k) * 1024), hvo[k] + (uint32_t)sc * 256u);
+      }
 #pragma unroll
       for (int k = 0; k < 8; ++k)
         bwd_fetch_to_lds_b128(rrs, uniform(slot + 64 * 256 + (8 * f + k) * 1024), rvo[k] + (uint32_t)sc * (128 * 256));
     };
     for (int s = 0; s < D - 1; ++s) request(s);
     for (int s = 0; s < nslab; ++s) {
-      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(12 * (D - 2)) : "memory");  // (slab s has landed)
+      if (live) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(12 * (D - 2)) : "memory");  // (slab s has landed)
+      else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(8 * (D - 2)) : "memory");
       lds_barrier();
       request(s + D - 1);
     }
