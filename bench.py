@@ -822,6 +822,7 @@ def main():
         out["backward"]["roofline"] = bw["roofline"]
         if "with_forward_coefficients" in bw:
             out["backward"]["with_forward_coefficients"] = bw["with_forward_coefficients"]
+        out["backward_config5_shape"] = bench_backward_large(device, iters=1)
     if args.all_configs:
         out["all_configs"] = [
             bench_config(device, "config 1: B=4 T=256 D=512 NH=4 fp32, no resets", 4, 256, 4, 128, False, 0),
