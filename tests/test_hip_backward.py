@@ -544,8 +544,22 @@ def test_calls_that_cannot_leave_coefficients_say_so_before_anything_runs():
     assert bool(torch.isfinite(h.float()).all())
 
 
-def test_cell_that_keeps_the_backward_coefficients_has_the_same_gradients():
+def test_cell_that_keeps_the_backward_coefficients_has_the_same_gradients(monkeypatch):
+    """The cell's default (a training forward leaves the coefficients, the backward call skips its forward walk) against
+    ``keep_backward_coefficients = False``; the backward calls are watched to see that each ran the way it was meant to."""
     from tests.test_hip_cell import _cell_from
+    from xlstm_amd import cell as cell_module
+    from xlstm_amd import functional as F
+
+    assert cell_module.sLSTMCell_hip.keep_backward_coefficients is True
+    seen = []
+    plain_backward = F.slstm_backward
+
+    def watched(*a, **kw):
+        seen.append(kw.get("coef") is not None)
+        return plain_backward(*a, **kw)
+
+    monkeypatch.setattr(cell_module.F_hip, "slstm_backward", watched)
 
     B, T, NH, dh = 8, 16, 2, 128
     wx, r, b, s0 = make_problem(360, B, T, NH, dh, rscale=2.0, bf16=True, with_state=True)
@@ -561,5 +575,6 @@ def test_cell_that_keeps_the_backward_coefficients_has_the_same_gradients():
         out, _ = cell(x, st, reset_mask=mask)
         (out.float() * w).sum().backward()
         grads.append((x.grad.float(), cell._recurrent_kernel_.grad.float(), cell._bias_.grad.float(), st.grad.float()))
+    assert seen == [False, True]
     for a, g in zip(grads[1], grads[0]):
         assert float((a - g).abs().max()) <= 2e-3 * max(1.0, float(g.abs().max()))

@@ -250,9 +250,9 @@ class sLSTMCell_hip(nn.Module):
     #: Training: let the forward call leave the backward pass its coefficients (36 bytes per step and element, held
     #: until the backward has run) where it can - bfloat16 inputs, head dim 128 or 256, a batch whose row tiles of 4
     #: rows fit the device - instead of having the backward pass recompute them in a forward walk of its own.  The
-    #: reference's native forward always keeps its states and gate values (slstm.cc:79-108); here the default keeps
-    #: nothing.  The gradients are the same either way.
-    keep_backward_coefficients: bool = False
+    #: reference's native forward always keeps its states and gate values when it trains (slstm.cc:79-108); set this to
+    #: False to keep nothing (the memory then goes to the backward call alone).  The gradients are the same either way.
+    keep_backward_coefficients: bool = True
 
     def __init__(self, config: sLSTMCellConfig, skip_backend_init: bool = False):
         super().__init__()
