@@ -73,12 +73,17 @@ SPLIT_CASES = [
 ]
 
 
-def _row_tile_of(kernel, bf16, dh):
+def _row_tile_of(kernel):
     """``kernel``: "one-unit" (one workgroup per head), "split" (a head over dh/64 compute units, row tiles of 16 rows),
     "quad" (the same in row tiles of 4 rows: bf16, head dims up to 256).  Returns (split_override, row_tile_override)."""
-    if kernel == "quad" and (not bf16 or dh > 256):
-        pytest.skip("row tiles of 4 rows: bf16 and head dims up to 256")
     return kernel != "one-unit", {"one-unit": None, "split": 16, "quad": 4}[kernel]
+
+
+def _kernels_of(bf16, dh):
+    """The reverse kernels that cover a case: head dim 512 (and what is padded up to it) has the split kernel only, row
+    tiles of 4 rows go with bf16 and head dims up to 256."""
+    dh_k = (dh + 63) // 64 * 64
+    return (["one-unit"] if dh_k <= 256 else []) + ["split"] + (["quad"] if bf16 and dh_k <= 256 else [])
 
 
 QUAD_CASES = [
@@ -90,14 +95,12 @@ QUAD_CASES = [
 ]
 
 
-@pytest.mark.parametrize("kernel", ["one-unit", "split", "quad"])
-@pytest.mark.parametrize("bf16,B,T,NH,dh,masked", CASES + SPLIT_CASES + PADDED_CASES + QUAD_CASES)
+@pytest.mark.parametrize("bf16,B,T,NH,dh,masked,kernel", [c + (k,) for c in CASES + SPLIT_CASES + PADDED_CASES + QUAD_CASES
+                                                          for k in _kernels_of(c[0], c[4])])
 def test_backward_against_the_oracle(bf16, B, T, NH, dh, masked, kernel):
     from xlstm_amd import functional as F
 
-    split, row_tile = _row_tile_of(kernel, bf16, (dh + 63) // 64 * 64)
-    if not split and dh > 256:
-        pytest.skip("head dim 512 (and what is padded up to it) has the split kernel only")
+    split, row_tile = _row_tile_of(kernel)
     print("case backward", bf16, B, T, NH, dh, masked, kernel, flush=True)
     H = NH * dh
     wx, r, b, s0 = make_problem(91, B, T, NH, dh, rscale=2.0, bf16=bf16, with_state=masked)

@@ -680,6 +680,9 @@ int run_backward_params(const xs_slstm_bwd_args *a) {
       return fail(XS_ERR_ALIGN, "d_wx and its row/step strides must be 16-byte aligned");
     if (((uintptr_t)a->h_out % 16) || ((uintptr_t)a->s0 % 16)) return fail(XS_ERR_ALIGN, "h_out and s0 must be 16-byte aligned");
     if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
+    // (a chunk of 32 steps is read through one buffer descriptor: its offsets are 31-bit)
+    if (32ll * a->d_wx_stride_t * 4 >= (1ll << 31) || 32ll * a->B * H * (bf16 ? 2 : 4) >= (1ll << 31))
+      return fail(XS_ERR_UNSUPPORTED, "32 steps of d_wx or of the outputs span 2 GiB or more: run the batch in slices of rows");
   }
   // (the slices of K are added into the results: they start at zero)
   hipLaunchKernelGGL(fill_u32_kernel, dim3(256), dim3(256), 0, stream, (uint32_t *)a->d_r, nr, 0u);
@@ -696,7 +699,10 @@ int run_backward_params(const xs_slstm_bwd_args *a) {
     const long long nchunks = (long long)a->B * p.tchunks;
     // slices of K: enough workgroups for two per compute unit, no slice shorter than four chunks
     const int cus = device_cus() > 0 ? device_cus() : 256;
-    long long ks = (2ll * cus + (long long)a->NH * tiles - 1) / ((long long)a->NH * tiles);
+    long long ks = (2ll * cus + (long long)a->NH * tiles - 1) / ((long long)a->NH * tiles);  // (4 or 8 per compute unit: 10 to 30 % slower)
+    // (head, slice) groups are dealt out over the XCDs, group i on XCD i % 8: a multiple of 8 of them keeps every XCD
+    // busy (4 heads of 1024 are 512 tiles and one slice each by the rule above: four XCDs idle, twice the time)
+    while ((a->NH * ks) % 8 != 0 && a->NH * ks < 64) ++ks;
     if (ks > nchunks / 4) ks = nchunks / 4;
     if (ks < 1) ks = 1;
     p.ksplit = (int)ks;
