@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 13
+#define XS_ABI_VERSION 14
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -362,6 +362,16 @@ int xs_slstm_backward(const xs_slstm_bwd_args *args);
  *   the order the compute units finish in.
  */
 int xs_slstm_backward_params(const xs_slstm_bwd_args *args);
+
+/*
+ * xs_slstm_backward_tile_r   brings the recurrent matrix into the operand order of the reverse kernel that `split`
+ *   names: reads r ([NH,4*dh,dh] in dtype, the forward's layout) and writes r_t (NH*4*dh*dh elements of dtype) as
+ *   described at xs_slstm_bwd_args above, so that a caller need not know the tilings.  The reference hands its GEMM R
+ *   as it lies and a transpose flag (slstm_backward.cu:308-319); here the kernels keep R transposed in registers or read
+ *   it slab by slab, in an order of their own.  Uses NH, dh, dtype, split, r, r_t, stream.  Call it once per change of
+ *   the parameters, in front of xs_slstm_backward.
+ */
+int xs_slstm_backward_tile_r(const xs_slstm_bwd_args *args);
 
 /*
  * Measurement (no counterpart in the reference): one stage of the dependency chain of a timestep of the sequence

@@ -46,6 +46,19 @@ def test_backward_argument_errors_without_touching_the_gpu():
     assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -1  # coef missing
     a.dtype = 5
     assert lib.xs_slstm_backward(ctypes.byref(a)) == -3
+    # the tiling of R for the reverse kernels
+    assert lib.xs_slstm_backward_tile_r(None) == -1
+    t = _lib.SlstmBwdArgs()
+    t.NH, t.dh, t.dtype, t.split = 2, 64, _lib.XS_F32, 0
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -1 and b"r and r_t" in lib.xs_last_error()
+    buf = (ctypes.c_char * 64)()
+    t.r = t.r_t = ctypes.addressof(buf)
+    t.split = 2
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5  # row tiles of 4 rows: bf16
+    t.split, t.dh = 3, 96
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5
+    t.split = 7
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5
 
 
 def test_backward_alignment_errors_without_touching_the_gpu():

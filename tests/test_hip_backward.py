@@ -395,7 +395,8 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     """A caller without torch arithmetic - the binding a maintainer would put in place of the reference's
     ``sLSTMFunc.backward`` (slstm.cc:137-221, which returns {dx, ds0, dR, db} from one native call): forward, then the
     three backward entry points, through ctypes with buffers the caller owns; the recurrent matrix is brought into the
-    reverse kernel's operand order with numpy on the host.  All four gradients against the oracle."""
+    reverse kernel's operand order with numpy on the host or by ``xs_slstm_backward_tile_r``.  All four gradients against
+    the oracle."""
     import ctypes
 
     from xlstm_amd import _lib
@@ -463,6 +464,10 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     a.exchange, a.counters = (exchange.data_ptr(), counters.data_ptr()) if split else (None, None)
     if stepwise:
         a.counters = None
+    if stepwise or tile_rows == 4:  # (these cases let the library bring R into the reverse kernel's order)
+        rt_lib = torch.empty(r_fwd.numel(), dtype=tdt, device=dev)
+        a.r_t = rt_lib.data_ptr()
+        assert lib.xs_slstm_backward_tile_r(ctypes.byref(a)) == 0, _lib.last_error()
     for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
         rc = fn(ctypes.byref(a))
         assert rc == 0, _lib.last_error()
@@ -581,3 +586,41 @@ def test_cell_that_keeps_the_backward_coefficients_has_the_same_gradients(monkey
     assert seen == [False, True]
     for a, g in zip(grads[1], grads[0]):
         assert float((a - g).abs().max()) <= 2e-3 * max(1.0, float(g.abs().max()))
+
+
+@pytest.mark.parametrize("bf16,NH,dh,split", [(True, 2, 256, 0), (False, 2, 128, 0), (True, 2, 512, 1), (False, 3, 256, 1), (True, 4, 256, 2),
+                                              (True, 1, 64, 2), (True, 2, 1024, 3), (True, 1, 640, 3), (False, 2, 512, 3), (False, 1, 320, 3)])
+def test_the_library_tiles_r_as_the_header_describes(bf16, NH, dh, split):
+    """``xs_slstm_backward_tile_r`` against the layouts of ``r_t`` in ``include/xlstm_amd.h`` written out with numpy, for
+    every reverse kernel (``split`` 0 to 3), bit for bit."""
+    import ctypes
+
+    from xlstm_amd import _lib
+
+    lib = _lib.load()
+    rng = np.random.default_rng(370)
+    r_k = rng.standard_normal((NH, 4 * dh, dh)).astype(np.float32)          # [NH, k = g dh + a, d]
+    epc = 8 if bf16 else 4
+    if split == 0:
+        want = r_k.transpose(0, 2, 1).reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).transpose(0, 1, 3, 4, 2, 5)
+    elif split == 3:
+        ks = 128 if bf16 else 64
+        want = r_k.transpose(0, 2, 1).reshape(NH, dh // 32, 32, 4 * dh // ks, ks).transpose(0, 1, 3, 2, 4)
+    else:
+        S, ksteps = dh // 64, 4 * dh // 8 // (4 * epc)
+        if split == 2:                                                       # K ordered (unit, gate)
+            rp = r_k.reshape(NH, 4, dh, dh).transpose(0, 2, 1, 3).reshape(NH, 4 * dh, dh)
+        else:                                                                # K ordered (owner slice, gate, unit % 64)
+            rp = r_k.reshape(NH, 4, S, 64, dh).transpose(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh)
+        want = rp.reshape(NH, 8, ksteps, 4, epc, S, 4, 16).transpose(0, 5, 1, 2, 6, 3, 7, 4)
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    r_dev = torch.from_numpy(r_k).cuda().to(tdt)
+    out = torch.empty(r_dev.numel(), dtype=tdt, device="cuda")
+    a = _lib.SlstmBwdArgs()
+    a.NH, a.dh, a.dtype, a.split = NH, dh, _lib.XS_BF16 if bf16 else _lib.XS_F32, split
+    a.r, a.r_t = r_dev.data_ptr(), out.data_ptr()
+    a.stream = torch.cuda.current_stream().cuda_stream
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(a)) == 0, _lib.last_error()
+    torch.cuda.synchronize()
+    want_t = torch.from_numpy(np.ascontiguousarray(want)).to(tdt).reshape(-1)
+    assert torch.equal(out.cpu(), want_t)

@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 XS_F32, XS_BF16 = 0, 1
 XS_ERR_UNSUPPORTED = -5
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 EXPORTS = (
     "xs_abi_version",
@@ -27,6 +27,7 @@ EXPORTS = (
     "xs_slstm_backward_prepare",
     "xs_slstm_backward",
     "xs_slstm_backward_params",
+    "xs_slstm_backward_tile_r",
     "xs_causal_conv_silu",
     "xs_headwise_gates",
     "xs_headwise_group_norm",
@@ -195,7 +196,7 @@ def load() -> ctypes.CDLL:
         fn = getattr(lib, name)
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmArgs)]
-    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params):
+    for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params, lib.xs_slstm_backward_tile_r):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmBwdArgs)]
     lib.xs_causal_conv_silu.restype = ctypes.c_int

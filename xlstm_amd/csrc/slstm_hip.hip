@@ -660,6 +660,71 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   return XS_OK;
 }
 
+// ---- backward pass: R in the operand order of the reverse kernels (xs_slstm_bwd_args::r_t), one thread per element of
+// the result: its place says which (gate unit k = g dh + a, input unit d) it holds, and R[h][k][d] is read from the
+// forward's layout.  mode = xs_slstm_bwd_args::split.
+template <typename T>
+__global__ __launch_bounds__(256) void slstm_bwd_tile_r_kernel(const T *r, T *r_t, int NH, int dh, int mode, int epc) {
+  const long long per_head = 4ll * dh * dh, n = (long long)NH * per_head;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long o = (long long)blockIdx.x * blockDim.x + threadIdx.x; o < n; o += stride) {
+    const int h = (int)(o / per_head);
+    long long v = o - (long long)h * per_head;
+    int k, d;
+    if (mode == 0) {         // [d / 16][k / KC][(k % KC) / EPC][d % 16][k % EPC], KC = 4 EPC
+      const int e = (int)(v % epc); v /= epc;
+      const int r16 = (int)(v & 15); v >>= 4;
+      const int c = (int)(v & 3); v >>= 2;
+      const int nkc = 4 * dh / (4 * epc);
+      const int kc = (int)(v % nkc); v /= nkc;
+      k = (kc * 4 + c) * epc + e;
+      d = (int)v * 16 + r16;
+    } else if (mode == 3) {  // [d / 32][k / KS][d % 32][k % KS], KS = 32 EPC / 2 (256 bytes)
+      const int ks = 16 * epc;
+      const int e = (int)(v % ks); v /= ks;
+      const int r32 = (int)(v & 31); v >>= 5;
+      const int nsl = 4 * dh / ks;
+      const int sl = (int)(v % nsl); v /= nsl;
+      k = sl * ks + e;
+      d = (int)v * 32 + r32;
+    } else {                 // [dh / 64][8 waves][k-steps of a wave][4 column blocks][4][16 columns][EPC], K reordered
+      const int ksteps = 4 * dh / 8 / (4 * epc);
+      const int e = (int)(v % epc); v /= epc;
+      const int r16 = (int)(v & 15); v >>= 4;
+      const int c = (int)(v & 3); v >>= 2;
+      const int cb = (int)(v & 3); v >>= 2;
+      const int kst = (int)(v % ksteps); v /= ksteps;
+      const int w = (int)(v & 7); v >>= 3;
+      const int kk = ((w * ksteps + kst) * 4 + c) * epc + e;  // the kernel's K index
+      d = ((int)v * 4 + cb) * 16 + r16;
+      if (mode == 1) k = ((kk & 255) >> 6) * dh + (kk >> 8) * 64 + (kk & 63);  // kk = 256 (a / 64) + 64 g + a % 64
+      else k = (kk & 3) * dh + (kk >> 2);                                     // kk = 4 a + g
+    }
+    r_t[o] = r[((long long)h * 4 * dh + k) * dh + d];
+  }
+}
+
+int run_backward_tile_r(const xs_slstm_bwd_args *a) {
+  if (!a) return fail(XS_ERR_NULL, "args is NULL");
+  if (a->NH <= 0 || a->dh <= 0) return fail(XS_ERR_SHAPE, "bad dims NH=%d dh=%d", a->NH, a->dh);
+  if (a->dtype != XS_F32 && a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
+  if (a->split < 0 || a->split > 3) return fail(XS_ERR_UNSUPPORTED, "split = %d", a->split);
+  if (!a->r || !a->r_t) return fail(XS_ERR_NULL, "r and r_t are required");
+  const bool bf16 = a->dtype == XS_BF16;
+  const int epc = bf16 ? 8 : 4;
+  if (a->split == 2 && !bf16) return fail(XS_ERR_UNSUPPORTED, "row tiles of 4 rows go with XS_BF16");
+  if (a->dh % 64 != 0 || (a->split == 3 && (a->dh * (bf16 ? 2 : 4)) % 256 != 0))
+    return fail(XS_ERR_UNSUPPORTED, "head dim %d is not one of the backward kernels'", a->dh);
+  hipStream_t stream = (hipStream_t)a->stream;
+  const long long n = 4ll * a->NH * a->dh * a->dh;
+  const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (bf16) hipLaunchKernelGGL(slstm_bwd_tile_r_kernel<uint16_t>, dim3(blocks), dim3(256), 0, stream, (const uint16_t *)a->r, (uint16_t *)a->r_t, a->NH, a->dh, a->split, epc);
+  else hipLaunchKernelGGL(slstm_bwd_tile_r_kernel<uint32_t>, dim3(blocks), dim3(256), 0, stream, (const uint32_t *)a->r, (uint32_t *)a->r_t, a->NH, a->dh, a->split, epc);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "tiling kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
+}
+
 // ---- backward pass: the gradients of R and the bias from the gate deltas and the forward's outputs
 int run_backward_params(const xs_slstm_bwd_args *a) {
   if (!a) return fail(XS_ERR_NULL, "args is NULL");
@@ -1011,6 +1076,11 @@ int xs_measure_stage(const xs_measure_args *args) {
 int xs_slstm_backward_params(const xs_slstm_bwd_args *args) {
   g_err[0] = 0;
   return run_backward_params(args);
+}
+
+int xs_slstm_backward_tile_r(const xs_slstm_bwd_args *args) {
+  g_err[0] = 0;
+  return run_backward_tile_r(args);
 }
 
 int xs_causal_conv_silu(const xs_conv_args *args) {

@@ -129,7 +129,7 @@ def slstm_backward(
     Three kernels of the engine: ``xs_slstm_backward_prepare`` (a forward walk over the stored outputs that leaves nine
     coefficients per step and element), ``xs_slstm_backward`` (the reverse pass) and ``xs_slstm_backward_params`` (the
     gradients of R and the bias, sums over all steps of products of the gate deltas with the outputs); what torch does
-    here is allocating the buffers and bringing R into the kernels' operand order.  ``timings`` (a dict) receives four
+    here is allocating the buffers (R is brought into the reverse kernel's operand order by ``xs_slstm_backward_tile_r``).  ``timings`` (a dict) receives four
     events around the three kernels.  Where the head dim allows it (64, 128, 256; 512 in bfloat16) and the workgroups fit the device at once,
     a head is spread over ``dh/64`` compute units that wait for each other every step (``split_override`` forces either
     kernel), in row tiles of 4 rows where four times the workgroups fit (bfloat16, head dims up to 256;
@@ -221,10 +221,7 @@ def slstm_backward(
         elif reset_mask.dtype != torch.uint8:
             reset_mask = (reset_mask != 0).to(torch.uint8)
         reset_mask = reset_mask.contiguous()
-    r32 = r.to(torch.float32)
-    if bf16:
-        r32 = r32.bfloat16().float()  # (the forward rounds R to bf16)
-    r_fwd = r32.to(wx.dtype).contiguous()  # R as the forward multiplies by it: the prepare kernel recomputes R.y_{t-1} from it
+    r_fwd = r.to(wx.dtype).contiguous()  # R as the forward multiplies by it (the forward rounds R to bf16)
     h_c = h_out if h_out.is_contiguous() and h_out.dtype == wx.dtype else h_out.to(wx.dtype).contiguous()
     d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
     d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
@@ -252,35 +249,18 @@ def slstm_backward(
     coef_given = coef is not None
     if not coef_given:
         coef = torch.empty((T, ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else B, 9, H), dtype=torch.float32, device=dev)
+    # R transposed in the operand order of the reverse kernel (xs_slstm_backward_tile_r), and what the kernels of a call
+    # hand to each other
+    r_t = torch.empty(NH * 4 * dh * dh, dtype=wx.dtype, device=dev)
+    exchange = counters = None
     if quad:
-        # R transposed with K ordered (unit, gate), tiled as the MFMA B operands of the workgroup that owns the output
-        # columns and of the wave that owns the eighth of K: [NH][S][8 waves][k-steps of a wave][4 column blocks][k / 8 % 4][column % 16][k % 8]
-        ksteps = 4 * dh // 8 // 32
-        r_t = (r32.view(NH, 4, dh, dh).permute(0, 2, 1, 3).reshape(NH, 4 * dh, dh).to(wx.dtype)           # [NH, k, d]
-               .view(NH, 8, ksteps, 4, 8, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
         exchange = torch.empty(4 * groups4 * 4 * 4 * dh, dtype=wx.dtype, device=dev)
         counters = torch.empty(1 + 2 * groups4, dtype=torch.int32, device=dev)
     elif split:
-        # R transposed with K ordered (owner slice, gate, unit % 64), tiled as the MFMA B operands of the workgroup
-        # that owns the output columns and of the wave that owns the eighth of K:
-        # [NH][S][8 waves][chunks of a wave][4 column blocks][k chunk of 4][column % 16][k % EPC]
-        ksteps = 4 * dh // 8 // (4 * epc)
-        r_t = (r32.view(NH, 4, S, 64, dh).permute(0, 2, 1, 3, 4).reshape(NH, 4 * dh, dh).to(wx.dtype)   # [NH, k, d]
-               .view(NH, 8, ksteps, 4, epc, S, 4, 16).permute(0, 5, 1, 2, 6, 3, 7, 4).contiguous())
         exchange = torch.empty(4 * groups * 16 * 4 * dh, dtype=wx.dtype, device=dev)
         counters = torch.empty(1 + 2 * groups, dtype=torch.int32, device=dev)
     elif stepwise:
-        # R transposed [NH, dh (d), 4*dh (k)] in slabs of 256 bytes of K per tile of 32 input units:
-        # [NH][d / 32][k / KS][d % 32][k % KS]; what the launches of a call hand to each other goes through `exchange`
-        ks = 256 // esz
-        r_t = (r32.transpose(1, 2).to(wx.dtype).reshape(NH, dh // 32, 32, 4 * dh // ks, ks).permute(0, 1, 3, 2, 4).contiguous())
         exchange = torch.empty(stepwise_exchange_bytes(B, NH, dh, esz), dtype=torch.uint8, device=dev)
-        counters = None
-    else:
-        # R transposed, tiled as the MFMA operands of the reverse kernel: [NH][d/16][k/KC][(k%KC)/EPC][d%16][k%EPC]
-        r_t = (r32.transpose(1, 2).to(wx.dtype)                              # [NH, dh (d), 4*dh (k)]
-               .reshape(NH, dh // 16, 16, 4 * dh // (4 * epc), 4, epc).permute(0, 1, 3, 4, 2, 5).contiguous())
-        exchange = counters = None
     d_h = d_h.to(wx.dtype).contiguous()
     if d_s_final is not None:
         d_s_final = d_s_final.to(torch.float32).contiguous()
@@ -312,6 +292,9 @@ def slstm_backward(
     a.recurrent_clipval = float(recurrent_clipval) if recurrent_clipval is not None else 0.0
     marks = []  # (measurement: events around the two kernels, read by the caller after a synchronisation)
     with torch.cuda.device(dev):
+        rc = lib.xs_slstm_backward_tile_r(ctypes.byref(a))
+        if rc != 0:
+            raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
         for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward):
             if coef_given and fn is lib.xs_slstm_backward_prepare:
                 if timings is not None:
