@@ -25,6 +25,7 @@ CASES = [
     (False, 4, 6, 2, 320, True),
     (False, 2, 5, 1, 296, True),      # padded up to 320
     (True, 9, 40, 8, 640, True),      # eight heads: one per XCD
+    (False, 5, 4, 3, 320, True),      # three heads: tiles dealt out head by head
 ]
 
 
