@@ -17,9 +17,11 @@ What differs, on purpose:
   * the stabiliser uses the native kernel's per-element ``n == 0`` rule
     (slstm_pointwise.cu:79), which equals the vanilla rule for every state the
     cell itself can produce;
-  * training: the forward stores nothing for it; ``loss.backward()`` recomputes what it needs and runs the engine's
-    backward kernels (``functional.slstm_backward``), with the reference's ``gradient_recurrent_cut`` and
-    ``gradient_recurrent_clipval``.  Head dims beyond the backward kernels' range raise in ``backward``;
+  * training: ``loss.backward()`` runs the engine's backward kernels (``functional.slstm_backward``), with the
+    reference's ``gradient_recurrent_cut`` and ``gradient_recurrent_clipval``, for every head dim the forward runs.
+    A forward call that is asked for a gradient leaves the backward pass nine coefficients per step and element
+    where its kernel can (``keep_backward_coefficients``); otherwise it stores nothing and the backward call
+    recomputes them;
   * a call with S == 1 -- what the reference's ``sLSTMLayer.step`` makes for every decoded
     token (layer.py:113-115) -- runs the single-token step kernel, bit-identical to the same
     step inside a longer call.
