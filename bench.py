@@ -280,7 +280,7 @@ def bench_backward(device, iters=3):
     keep = {}
     coef = F.backward_coefficients_buffer(wx, NH)
     if coef is not None:
-        fwd_plain, fwd_keep, tot_keep = [], [], []
+        fwd_plain, fwd_keep, tot_keep, tot_cell = [], [], [], []
         for i in range(iters + 1):
             e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
             e[0].record()
@@ -292,13 +292,20 @@ def bench_backward(device, iters=3):
             t0 = time.perf_counter()
             out2 = F.slstm_backward(wx, r, bias, None, mask, h, d_h, coef=coef)
             torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            # ... and with the gate deltas returned in the input's type, as sLSTMCell_hip asks for them
+            out3 = F.slstm_backward(wx, r, bias, None, mask, h, d_h, coef=coef, d_wx_dtype=torch.bfloat16)
+            torch.cuda.synchronize()
             if i:
-                tot_keep.append((time.perf_counter() - t0) * 1e3)
+                tot_cell.append((time.perf_counter() - t1) * 1e3)
+                tot_keep.append((t1 - t0) * 1e3)
                 fwd_plain.append(e[0].elapsed_time(e[1]))
                 fwd_keep.append(e[1].elapsed_time(e[2]))
         keep = {"with_forward_coefficients": {
             "backward_ms": float(np.median(tot_keep)), "forward_ms": float(np.median(fwd_keep)),
             "plain_forward_ms": float(np.median(fwd_plain)),
+            "backward_ms_with_bf16_gate_deltas": float(np.median(tot_cell)),
+            "bf16_gate_deltas_are_the_float32_ones_rounded": bool(torch.equal(out3[0], out2[0].bfloat16())),
             "same_gradients": bool(torch.allclose(out2[0], out[0], rtol=0, atol=2e-3 * float(out[0].abs().max())))}}
     # what the reverse kernel has to move per step and element: nine coefficients and the four gate deltas in float32,
     # the output gradient in bf16; R transposed once (the gate deltas that the compute units of a head exchange stay in the L2)

@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 14
+#define XS_ABI_VERSION 15
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -298,7 +298,7 @@ typedef struct xs_slstm_bwd_args {
   const void *d_h;           /* [T,B,H]: gradient with respect to h_out (backward) */
   const float *d_s_final;    /* [4,B,H] or NULL: gradient with respect to the final state; y, c, n are used (backward) */
   const void *r_t;           /* (backward) */
-  float *d_wx;               /* [B,T,4,NH,dh], strides in elements (backward) */
+  void *d_wx;                /* [B,T,4,NH,dh] float32 (or bf16: d_wx_dtype below), strides in elements (backward, params) */
   int64_t d_wx_stride_b, d_wx_stride_t;
   float *d_s0;               /* [4,B,H] (backward) */
   void *stream;
@@ -346,6 +346,11 @@ typedef struct xs_slstm_bwd_args {
   const void *r;             /* [NH,4*dh,dh] in dtype, the forward's layout (prepare) */
   float *d_r;                /* [NH,4*dh,dh] float32: gradient of r in that layout (params) */
   float *d_bias;             /* [NH,4,dh] float32 (params) */
+  /* the type of d_wx: XS_F32 (0, the default), or XS_BF16 with dtype == XS_BF16 - the gate deltas are then written
+   * rounded to bf16, as the reference returns dx in the type of its kernels (slstm.cc:137-221), the reverse kernel
+   * writes and xs_slstm_backward_params reads half the bytes, and a caller whose input is bf16 needs no conversion
+   * (d_wx must then be 16-byte aligned and its strides multiples of 8 elements) */
+  int32_t d_wx_dtype;
 } xs_slstm_bwd_args;
 
 int xs_slstm_backward_prepare(const xs_slstm_bwd_args *args);

@@ -33,7 +33,7 @@ def test_abi_version_and_struct_mirror():
     assert ctypes.sizeof(_lib.GatesArgs) == 16 + 11 * 8
     assert ctypes.sizeof(_lib.NormArgs) == 24 + 7 * 8  # 5 int32 + float, then 7 8-byte fields
     # 5 int32 (+4), 17 8-byte fields, int32 (+4), 3 more, int32 + float, 4 pointers
-    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8 + 8 + 4 * 8
+    assert ctypes.sizeof(_lib.SlstmBwdArgs) == 24 + 17 * 8 + 8 + 3 * 8 + 8 + 4 * 8 + 8
 
 
 def test_backward_argument_errors_without_touching_the_gpu():
@@ -46,6 +46,9 @@ def test_backward_argument_errors_without_touching_the_gpu():
     assert lib.xs_slstm_backward_prepare(ctypes.byref(a)) == -1  # coef missing
     a.dtype = 5
     assert lib.xs_slstm_backward(ctypes.byref(a)) == -3
+    # d_wx in bf16 goes with bf16 operands
+    a.dtype, a.d_wx_dtype = _lib.XS_F32, _lib.XS_BF16
+    assert lib.xs_slstm_backward(ctypes.byref(a)) == -3 and lib.xs_slstm_backward_params(ctypes.byref(a)) in (-1, -3)
     # the tiling of R for the reverse kernels
     assert lib.xs_slstm_backward_tile_r(None) == -1
     t = _lib.SlstmBwdArgs()

@@ -251,7 +251,7 @@ def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=
     m_t = torch.from_numpy(reset).to(dev) if reset is not None else None
     dsf_t = torch.from_numpy(d_sf).to(dev) if d_sf is not None else None
     h, _ = F.slstm_forward(wx_t, r_t, b_t, s0_t, m_t)
-    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override", "row_tile_override", "stepwise_override")}
+    kw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval", "split_override", "row_tile_override", "stepwise_override", "d_wx_dtype")}
     d_wx, d_r, d_b, d_s0 = F.slstm_backward(wx_t, r_t, b_t, s0_t, m_t, h, torch.from_numpy(d_h).to(dev), dsf_t, **kw)
     torch.cuda.synchronize()
     okw = {k: v for k, v in opts.items() if k in ("recurrent_cut", "recurrent_clipval")}
@@ -259,7 +259,7 @@ def _run_both(bf16, B, T, NH, dh, seed, masked, with_state, mean_len=None, d_sf=
     if key not in _ORACLE_RESULTS:  # (the same problem through several kernels: the oracle runs once)
         _ORACLE_RESULTS[key] = so.slstm_backward(wx, r, b, s0, reset, d_h, d_sf, **okw)
     o_wx, o_r, o_b, o_s0 = _ORACLE_RESULTS[key]
-    errs = dict(d_wx=_rel(d_wx.cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
+    errs = dict(d_wx=_rel(d_wx.float().cpu().numpy(), o_wx), d_r=_rel(d_r.cpu().numpy(), r_ext_to_kernel(torch.from_numpy(o_r)).numpy()),
                 d_b=_rel(d_b.cpu().numpy(), o_b), d_s0=_rel(d_s0.cpu().numpy(), o_s0))
     return errs, (d_wx, d_r, d_b, d_s0), (o_wx, o_r, o_b, o_s0)
 
@@ -624,3 +624,26 @@ def test_the_library_tiles_r_as_the_header_describes(bf16, NH, dh, split):
     torch.cuda.synchronize()
     want_t = torch.from_numpy(np.ascontiguousarray(want)).to(tdt).reshape(-1)
     assert torch.equal(out.cpu(), want_t)
+
+
+@pytest.mark.parametrize("B,T,NH,dh,kernel", [(6, 9, 2, 128, "one-unit"), (20, 7, 2, 256, "split"), (9, 6, 2, 512, "split"),
+                                              (16, 12, 4, 256, "quad"), (7, 5, 3, 64, "quad"), (5, 6, 1, 1024, "step"), (70, 3, 2, 640, "step")])
+def test_gate_deltas_in_bfloat16(B, T, NH, dh, kernel):
+    """``d_wx_dtype = XS_BF16``: every reverse kernel writes the gate deltas rounded to bf16 - exactly the float32 ones
+    rounded - and the parameter kernel reads them in that type: all four gradients against the oracle as before."""
+    print("case d_wx in bf16", B, T, NH, dh, kernel, flush=True)
+    H = NH * dh
+    d_sf = np.random.default_rng(381).standard_normal((4, B, H)).astype(np.float32)
+    d_sf[3] = 0.0
+    if kernel == "step":
+        kw = {}
+    else:
+        split, row_tile = _row_tile_of(kernel)
+        kw = dict(split_override=split, row_tile_override=row_tile)
+    errs, got, _ = _run_both(True, B, T, NH, dh, 380, masked=True, with_state=True, d_sf=d_sf, d_wx_dtype=torch.bfloat16, **kw)
+    print(errs, flush=True)
+    assert got[0].dtype == torch.bfloat16
+    assert all(np.isfinite(v) and v <= 2e-2 for v in errs.values()), errs
+    _, ref, _ = _run_both(True, B, T, NH, dh, 380, masked=True, with_state=True, d_sf=d_sf, **kw)
+    assert torch.equal(got[0], ref[0].bfloat16())
+    assert torch.equal(got[3], ref[3])

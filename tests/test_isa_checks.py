@@ -99,7 +99,8 @@ def test_the_backward_kernel_with_feeder_waves_keeps_its_registers_and_polls_wit
     seen = 0
     for entry in re.split(r"\n  - ", meta)[1:]:
         name = re.search(r"\.name:\s+(\S+)", entry)
-        if not name or "slstm_bwd_split_kernel" not in name.group(1) or not name.group(1).endswith("ELb1EEEvNS_14BwdSplitParamsE"):
+        # (template arguments: bf16, S, feeder waves, gate deltas in bf16)
+        if not name or not re.search(r"slstm_bwd_split_kernelILb[01]ELi\d+ELb1ELb[01]EEEvNS_14BwdSplitParamsE$", name.group(1)):
             continue
         seen += 1
         assert int(re.search(r"\.vgpr_count:\s*(\d+)", entry).group(1)) <= 168, name.group(1)
@@ -110,4 +111,4 @@ def test_the_backward_kernel_with_feeder_waves_keeps_its_registers_and_polls_wit
         assert polls, name.group(1)
         for i in polls:
             assert not any("v_readfirstlane" in line for line in body[max(0, i - 6): i]), (name.group(1), body[i - 6: i + 1])
-    assert seen == 5  # bf16 at head dims 64, 128, 256; float32 at 64, 128
+    assert seen == 8  # bf16 at head dims 64, 128, 256 with the gate deltas in float32 and in bf16; float32 at 64, 128

@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 XS_F32, XS_BF16 = 0, 1
 XS_ERR_UNSUPPORTED = -5
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 EXPORTS = (
     "xs_abi_version",
@@ -90,6 +90,7 @@ class SlstmBwdArgs(ctypes.Structure):
         ("r", ctypes.c_void_p),
         ("d_r", ctypes.c_void_p),
         ("d_bias", ctypes.c_void_p),
+        ("d_wx_dtype", ctypes.c_int32),
     ]
 
 

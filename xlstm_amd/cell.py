@@ -211,7 +211,8 @@ class _CellFunction(torch.autograd.Function):
         NH, dh = ctx.num_heads, r.shape[2]
         d_wx, d_r, d_bias, d_s0 = F_hip.slstm_backward(
             x.detach(), r.detach(), bias.detach().view(NH, 4, dh), None if state is None else state.detach(), ctx.mask,
-            h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval, coef=ctx.coef)
+            h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval, coef=ctx.coef,
+            d_wx_dtype=torch.bfloat16 if x.dtype == torch.bfloat16 else None)  # (the input's gradient in the input's type)
         ctx.coef = None
         return (d_wx.to(x.dtype), d_r.to(r.dtype), d_bias.reshape(bias.shape).to(bias.dtype),
                 None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None, None)

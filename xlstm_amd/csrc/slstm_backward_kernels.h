@@ -347,8 +347,9 @@ struct BwdParams {
                              // of 16 bytes, KC = 4 EPC (the 64 lanes' operands of one MFMA k-step are 1 KiB in a row)
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
-  float *d_wx;               // [B,T,4,NH,dh] float32, strides in elements
+  float *d_wx;               // [B,T,4,NH,dh] float32 (bf16 with d_wx_bf16), strides in elements
   long long d_wx_sb, d_wx_st;
+  int d_wx_bf16;
   float *d_s0;               // [4,B,H]
   int cut;                   // no gradient from a step to the y it started from (slstm_backward_cut.cu:265-312)
   float clip;                // > 0: that gradient is clipped to +-clip before d_h is added (slstm_pointwise.cu:136-143); 0: not
@@ -448,9 +449,12 @@ __global__ __launch_bounds__(NW * 64) void slstm_bwd_kernel(BwdParams p) {
             // (a row that starts a document at t took nothing from the step before)
             dc[nb][i] = restart[ii] ? 0.0f : cf[ii][nb][8] * dct;
             dn[nb][i] = restart[ii] ? 0.0f : cf[ii][nb][8] * dnt;
-            float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + head * dh + unit;
+            const long long wo = (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + head * dh + unit;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) dw[(long long)g * H] = delta[g];
+            for (int g = 0; g < 4; ++g) {
+              if (p.d_wx_bf16) reinterpret_cast<uint16_t *>(p.d_wx)[wo + (long long)g * H] = (uint16_t)(pack_bf16x2(delta[g], 0.0f) & 0xFFFFu);
+              else p.d_wx[wo + (long long)g * H] = delta[g];
+            }
           }
 #pragma unroll
           for (int g = 0; g < 4; ++g) {
@@ -547,7 +551,7 @@ struct BwdSplitParams {
                              // [NH][S][8 waves][KSTEPS][4 column blocks][64 lanes][16 bytes]
   const uint8_t *reset;
   long long reset_sb;
-  float *d_wx;
+  float *d_wx;               // (bf16 in the DWX16 variants of the kernels)
   long long d_wx_sb, d_wx_st;
   float *d_s0;
   void *xch;                 // [kBwdRing][groups][K / KC][16][4][16 bytes], all ones at the start
@@ -699,9 +703,13 @@ constexpr int bwd_split_lds_bytes(bool feed, bool bf16) {
 // With feeders a step has two barriers: B', behind which the slot that the step's inputs were read from is free for
 // the inputs of the step after the next, and A, in front of which the wave's partial tile is written and the next
 // step's inputs have landed.  (Without: one barrier, two sets of partial tiles.)
-template <bool BF16, int S, bool FEED>  // eight compute waves; S workgroups per group, dh = 64 S (S = 1: one workgroup
+// DWX16: d_wx takes the gate deltas rounded to bf16.  (A template flag, not a branch on a kernel argument: with the
+// branch in the step the compiler kept the exchange ring's descriptor in vector registers and wrapped every poll in a
+// loop over the lanes' values.)
+template <bool BF16, int S, bool FEED, bool DWX16 = false>  // eight compute waves; S workgroups per group, dh = 64 S (S = 1: one workgroup
                                         // per head and row tile, the same step with nobody else to wait for)
 __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSplitParams p) {
+  static_assert(!DWX16 || BF16, "gate deltas in bf16 go with bf16 operands");
   constexpr int ESZ = BF16 ? 2 : 4;
   constexpr int EPC = 16 / ESZ;               // elements of a 16-byte chunk
   constexpr int KC = 4 * EPC;                 // K of one chunk row: what one MFMA (bf16) or four (float32) take
@@ -734,7 +742,7 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
     const int f = (int)uniform((uint32_t)wave) - 8;
     const uint32_t feed_lds = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)feed);
     const int rows_there = p.B - row0 < 16 ? p.B - row0 : 16;
-    const uint32_t dh_records = (uint32_t)(((long long)(rows_there - 1) * H + 64) * ESZ);
+    const uint32_t dh_records = uniform((uint32_t)(((long long)(rows_there - 1) * H + 64) * ESZ));
     // d_h: a load covers 8 rows of 128 bytes (bf16; the waves' two halves twice over) or 4 rows of 256 bytes
     const int dh_part = BF16 ? (f & 1) : f;
     const int dh_voff = BF16 ? ((dh_part * 8 + (lane >> 3)) * H * 2 + (lane & 7) * 16) : ((dh_part * 4 + (lane >> 4)) * H * 4 + (lane & 15) * 16);
@@ -744,10 +752,10 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
       const u32x4_t crs = {uniform((uint32_t)cb), uniform((uint32_t)(cb >> 32) & 0xFFFFu), (uint32_t)kBwdCoefBytes, 0x00020000u};
       const uint32_t slot = feed_lds + (n & 1) * FSLOT;
 #pragma unroll
-      for (int k = 0; k < 9; ++k) lds_direct_fetch_b128(crs, uniform(slot + (f * 9 + k) * 1024), (f * 9 + k) * 1024 + lane * 16);
+      for (int k = 0; k < 9; ++k) bwd_fetch_to_lds_b128(crs, uniform(slot + (f * 9 + k) * 1024), (uint32_t)((f * 9 + k) * 1024 + lane * 16));
       const unsigned long long db = reinterpret_cast<unsigned long long>(p.d_h) + (unsigned long long)((((long long)t * p.B + row0) * H + (long long)head * dh + s * UW) * ESZ);
       const u32x4_t drs = {uniform((uint32_t)db), uniform((uint32_t)(db >> 32) & 0xFFFFu), dh_records, 0x00020000u};
-      lds_direct_fetch_b128(drs, uniform(slot + kBwdCoefBytes + dh_part * 1024), dh_voff);
+      bwd_fetch_to_lds_b128(drs, uniform(slot + kBwdCoefBytes + dh_part * 1024), (uint32_t)dh_voff);  // (with the wait states behind the descriptor's scalar writes)
     };
     // Slot n % 2 is free behind barrier B'(n), but the inputs of step n + 2 are asked for only behind barrier A(n),
     // when the compute waves add up, read LDS and do arithmetic: right behind B' they publish and poll, and 38 KiB
@@ -883,9 +891,12 @@ __global__ __launch_bounds__(FEED ? 768 : 512) void slstm_bwd_split_kernel(BwdSp
     if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
     if (FEED && there && p.reset && t > 0) restart_raw = p.reset[(long long)row * p.reset_sb + t - 1];  // (used by the next step)
     if (there) {
-      float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
+      const long long wo = (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) *reinterpret_cast<f32x2 *>(dw + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
+      for (int g = 0; g < 4; ++g) {
+        if constexpr (DWX16) *reinterpret_cast<uint32_t *>(reinterpret_cast<uint16_t *>(p.d_wx) + wo + (long long)g * H) = pack_bf16x2(delta[g][0], delta[g][1]);
+        else *reinterpret_cast<f32x2 *>(p.d_wx + wo + (long long)g * H) = f32x2{delta[g][0], delta[g][1]};
+      }
     }
     if (cut) {
       if (!FEED) fetch_step(in, t - 2);

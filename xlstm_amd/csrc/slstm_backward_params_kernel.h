@@ -26,8 +26,9 @@ namespace {
 
 struct BwdParamParams {
   int B, T, NH, dh;
-  const float *d_wx;         // [B,T,4,NH,dh] float32, strides in elements: the gate deltas
+  const float *d_wx;         // [B,T,4,NH,dh] float32 (bf16 with d_wx_bf16), strides in elements: the gate deltas
   long long d_wx_sb, d_wx_st;
+  int d_wx_bf16;
   const void *h_out;         // [T,B,H] in the operand type: the forward's outputs
   const float *s0;           // [4,B,H] or null
   const uint8_t *reset;      // [B,T] or null
@@ -84,6 +85,7 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
   const int yk = tid / NROWTHREADS, yn = (tid % NROWTHREADS) * 8;
   const bool y_thread = tid < kParamKC * NROWTHREADS;  // (NT 64: 256 threads cover the chunk)
   float bsum[8] = {0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f};
+  const bool dbf16 = BF16 && p.d_wx_bf16 != 0;  // the deltas lie in bf16 (only with bf16 operands)
 
   struct Staged { float4 d[2]; uint4 y[YPASS < 1 ? 1 : YPASS][BF16 ? 1 : 2]; uint32_t flag[YPASS < 1 ? 1 : YPASS]; };
   // The loads of a chunk have no branch around them: they go through buffer descriptors that end where the chunk's
@@ -95,12 +97,14 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
     const int b = (int)(c / p.tchunks), t0 = (int)(c % p.tchunks) * kParamKC;
     const int nrows = p.T - t0 < kParamKC ? p.T - t0 : kParamKC;  // (>= 1)
     {  // delta: rows t0 .. of the batch row, this thread's 8 m of row dk
-      const float *base = p.d_wx + (long long)b * p.d_wx_sb + (long long)t0 * p.d_wx_st;
+      const int dsz = dbf16 ? 2 : 4;
+      const char *base = reinterpret_cast<const char *>(p.d_wx) + ((long long)b * p.d_wx_sb + (long long)t0 * p.d_wx_st) * dsz;
       const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-          const_cast<float *>(base), 0, (int)(((long long)(nrows - 1) * p.d_wx_st + 4ll * H) * 4), 0x00020000);
-      const int vo = (int)(((long long)dk * p.d_wx_st + d_off) * 4);
+          const_cast<char *>(base), 0, (int)(((long long)(nrows - 1) * p.d_wx_st + 4ll * H) * dsz), 0x00020000);
+      const int vo = (int)(((long long)dk * p.d_wx_st + d_off) * dsz);
       s.d[0] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rs, vo, 0, 0));
-      s.d[1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rs, vo + 16, 0, 0));
+      // (deltas in bf16: the thread's 8 values are the first 16 bytes; the second load asks past the end and reads zeros)
+      s.d[1] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(rs, dbf16 ? (int)0x80000000 : vo + 16, 0, 0));
     }
     // y_{t-1}: the outputs of steps t0 - 1 .. (row -1, in front of step 0, lies in front of the descriptor: zeros)
     const int tb = t0 > 0 ? t0 - 1 : 0;  // the step the descriptor starts at
@@ -130,9 +134,9 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
       const int b = b0 + dk;
       s.d[0] = s.d[1] = float4{0.0f, 0.0f, 0.0f, 0.0f};
       if (b < p.B) {
-        const float *src = p.d_wx + (long long)b * p.d_wx_sb + d_off;
+        const char *src = reinterpret_cast<const char *>(p.d_wx) + ((long long)b * p.d_wx_sb + d_off) * (dbf16 ? 2 : 4);
         s.d[0] = *reinterpret_cast<const float4 *>(src);
-        s.d[1] = *reinterpret_cast<const float4 *>(src + 4);
+        if (!dbf16) s.d[1] = *reinterpret_cast<const float4 *>(src + 16);
       }
     }
 #pragma unroll
@@ -155,7 +159,12 @@ __global__ __launch_bounds__(512) void slstm_bwd_param_kernel(BwdParamParams p) 
     }
   };
   auto stage = [&](const Staged &s, int buf, bool count_bias = true) {
-    const float dv[8] = {s.d[0].x, s.d[0].y, s.d[0].z, s.d[0].w, s.d[1].x, s.d[1].y, s.d[1].z, s.d[1].w};
+    float dv[8] = {s.d[0].x, s.d[0].y, s.d[0].z, s.d[0].w, s.d[1].x, s.d[1].y, s.d[1].z, s.d[1].w};
+    if (dbf16) {  // (8 bf16 in the first 16 bytes)
+      const uint32_t w[4] = {__float_as_uint(s.d[0].x), __float_as_uint(s.d[0].y), __float_as_uint(s.d[0].z), __float_as_uint(s.d[0].w)};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) { dv[2 * j] = bf16_bits_to_float(w[j] & 0xFFFFu); dv[2 * j + 1] = bf16_bits_to_float(w[j] >> 16); }
+    }
     if (n0 == 0 && count_bias) {
 #pragma unroll
       for (int j = 0; j < 8; ++j) bsum[j] += dv[j];

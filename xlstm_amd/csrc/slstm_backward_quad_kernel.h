@@ -40,7 +40,7 @@ constexpr int bwd_quad_lds_bytes() { return 2 * 8 * kBwdQuadPart * 4 + kBwdQuadS
 // so does every cycle slept past the arrival.
 constexpr int kBwdQuadSleepIdle = 8, kBwdQuadSleepPublished = 2;
 
-template <int S>  // S workgroups per group, dh = 64 S
+template <int S, bool DWX16 = false>  // S workgroups per group, dh = 64 S; DWX16: d_wx takes the gate deltas rounded to bf16
 __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSplitParams p) {
   constexpr int UW = 64;
   constexpr int dh = S * UW;
@@ -248,9 +248,12 @@ __global__ __launch_bounds__(kBwdQuadThreads) void slstm_bwd_quad_kernel(BwdSpli
       //      kernel took 2.33 ms at config 2 instead of 2.20: the look then waits for the stores behind it as well)
       if (s == 0 && tid == 0) p.progress[group] = (unsigned int)n;
       if (there) {
-        float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
+        const long long wo = (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + ecol;
 #pragma unroll
-        for (int g = 0; g < 4; ++g) dw[(long long)g * H] = delta[g];
+        for (int g = 0; g < 4; ++g) {
+          if constexpr (DWX16) reinterpret_cast<uint16_t *>(p.d_wx)[wo + (long long)g * H] = (uint16_t)(pack_bf16x2(delta[g], 0.0f) & 0xFFFFu);
+          else p.d_wx[wo + (long long)g * H] = delta[g];
+        }
       }
       if (n + 1 < p.T) read_inputs(n + 1);
       if (!cut && S > 1) __builtin_amdgcn_s_sleep(kBwdQuadSleepPublished);

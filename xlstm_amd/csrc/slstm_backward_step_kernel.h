@@ -45,8 +45,9 @@ struct BwdStepParams {
   void *delta_out;           // ... of step t
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
-  float *d_wx;               // [B,T,4,NH,dh] float32, strides in elements
+  float *d_wx;               // [B,T,4,NH,dh] float32 (bf16 with d_wx_bf16), strides in elements
   long long d_wx_sb, d_wx_st;
+  int d_wx_bf16;
   float *d_s0;               // [4,B,H]
   int cut;
   float clip;
@@ -243,17 +244,18 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
       dn_prev[i] = restart[ut] ? 0.0f : cf[ut][8][i] * dnt;
     }
     const int row = rowbase + 32 * wr + 16 * ut + r16;
-    float *dw = p.d_wx + (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + head * dh + ua;
+    const long long wo = (long long)row * p.d_wx_sb + (long long)t * p.d_wx_st + head * dh + ua;
     unsigned char *dout = reinterpret_cast<unsigned char *>(p.delta_out) + dtile + (row & 63) * 256;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      __builtin_nontemporal_store(delta[g], reinterpret_cast<f32x4 *>(dw + (long long)g * H));
       const int kb = (g * dh + ua) * ESZ;  // byte of the row of K: slab kb / 256, inside it kb % 256
       unsigned char *dst = dout + (long long)(kb >> 8) * (64 * 256) + (kb & 255);
+      if (!BF16 || !p.d_wx_bf16) __builtin_nontemporal_store(delta[g], reinterpret_cast<f32x4 *>(p.d_wx + wo + (long long)g * H));
       if (BF16) {
         uint2 w;
         w.x = pack_bf16x2(delta[g][0], delta[g][1]);
         w.y = pack_bf16x2(delta[g][2], delta[g][3]);
+        if (p.d_wx_bf16) *reinterpret_cast<uint2 *>(reinterpret_cast<uint16_t *>(p.d_wx) + wo + (long long)g * H) = w;
         *reinterpret_cast<uint2 *>(dst) = w;
       } else {
         *reinterpret_cast<f32x4 *>(dst) = delta[g];

@@ -394,6 +394,17 @@ int run_forward(const xs_slstm_args *a, size_t *need = nullptr) {
   return XS_OK;
 }
 
+// the type of d_wx that a backward call asks for
+int d_wx_type(const xs_slstm_bwd_args *a, int *is_bf16) {
+  *is_bf16 = 0;
+  if (a->d_wx_dtype == XS_F32) return XS_OK;
+  if (a->d_wx_dtype != XS_BF16 || a->dtype != XS_BF16) return fail(XS_ERR_DTYPE, "d_wx_dtype must be XS_F32, or XS_BF16 with dtype XS_BF16");
+  if (a->d_wx && (((uintptr_t)a->d_wx % 16) || (a->d_wx_stride_b % 8) || (a->d_wx_stride_t % 8)))
+    return fail(XS_ERR_ALIGN, "d_wx in bf16 must be 16-byte aligned and its strides multiples of 8 elements");
+  *is_bf16 = 1;
+  return XS_OK;
+}
+
 // ---- backward pass with one launch per step (split == 3): slstm_fwd_walk_kernel and slstm_bwd_step_kernel.  Both keep
 // what a step hands to the next in the caller's `exchange` buffer: the forward walk a state [4,B,H] float32 (its y
 // plane holds the y of the initial state in the type of the operands) and R in the walk's slabs; the reverse pass two
@@ -404,6 +415,11 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   const int B = a->B, T = a->T, NH = a->NH, dh = a->dh;
   const long long H = (long long)NH * dh, BH = (long long)B * H;
   hipStream_t stream = (hipStream_t)a->stream;
+  int dwx_bf16 = 0;
+  {
+    const int rc = d_wx_type(a, &dwx_bf16);
+    if (rc != XS_OK) return rc;
+  }
   if (!a->exchange) return fail(XS_ERR_NULL, "exchange is required with one launch per step");
   if (((uintptr_t)a->exchange % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "exchange and coef must be 16-byte aligned");
   if ((dh * esz) % 256 != 0) return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d is not a multiple of %d", dh, 256 / esz);
@@ -449,7 +465,7 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
     q.B = B; q.T = T; q.NH = NH; q.dh = dh;
     q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_t = a->r_t;
     q.reset = a->reset; q.reset_sb = a->reset_stride_b;
-    q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+    q.d_wx = (float *)a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_wx_bf16 = dwx_bf16; q.d_s0 = a->d_s0;
     q.cut = a->recurrent_cut != 0;
     q.clip = (a->recurrent_clipval > 0.0f && a->recurrent_clipval < __builtin_inff()) ? a->recurrent_clipval : 0.0f;
     char *const deltas[2] = {(char *)a->exchange, (char *)a->exchange + 4ll * ((B + 63) / 64 * 64) * H * esz};  // (tiles of 64 rows)
@@ -486,6 +502,11 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (a->B == 0 || a->T == 0) return XS_OK;
   const bool bf16 = a->dtype == XS_BF16;
   const long long H = (long long)a->NH * a->dh;
+  int dwx_bf16 = 0;
+  if (!prepare) {
+    const int rc = d_wx_type(a, &dwx_bf16);
+    if (rc != XS_OK) return rc;
+  }
   if (!a->coef) return fail(XS_ERR_NULL, "coef is required");
   if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
   hipStream_t stream = (hipStream_t)a->stream;
@@ -545,7 +566,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.B = a->B; q.T = a->T; q.NH = a->NH; q.dh = a->dh;
       q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
       q.reset = a->reset; q.reset_sb = a->reset_stride_b;
-      q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+      q.d_wx = (float *)a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
       q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1; q.placement = a->counters + 1 + ngroups;
       q.main_locals = (int)(grid / 8);
       // prefetching workgroups per XCD: one per 40 KB that the XCD's groups read per step (a compute unit draws some
@@ -572,6 +593,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       hipLaunchKernelGGL(slstm_bwd_arm_kernel, dim3((unsigned)((n16 + 255) / 256 < 1024 ? (n16 + 255) / 256 : 1024)), dim3(256), 0, stream,
                          (uint4 *)a->exchange, n16, a->counters, (int)(1 + 2 * ngroups));
       void (*kq)(BwdSplitParams) = a->dh == 64 ? slstm_bwd_quad_kernel<1> : (a->dh == 128 ? slstm_bwd_quad_kernel<2> : slstm_bwd_quad_kernel<4>);
+      if (dwx_bf16) kq = a->dh == 64 ? slstm_bwd_quad_kernel<1, true> : (a->dh == 128 ? slstm_bwd_quad_kernel<2, true> : slstm_bwd_quad_kernel<4, true>);
       const int lds = bwd_quad_lds_bytes();
       {
         const int rc = ensure_dynamic_lds((const void *)kq, (size_t)lds);
@@ -594,7 +616,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       q.B = a->B; q.T = a->T; q.NH = a->NH; q.dh = a->dh;
       q.coef = a->coef; q.d_h = a->d_h; q.d_s_final = a->d_s_final; q.r_ts = a->r_t;
       q.reset = a->reset; q.reset_sb = a->reset_stride_b;
-      q.d_wx = a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
+      q.d_wx = (float *)a->d_wx; q.d_wx_sb = a->d_wx_stride_b; q.d_wx_st = a->d_wx_stride_t; q.d_s0 = a->d_s0;
       if (((uintptr_t)a->exchange % 16)) return fail(XS_ERR_ALIGN, "exchange must be 16-byte aligned");
       q.xch = a->exchange; q.abort_word = a->counters; q.progress = a->counters + 1; q.placement = a->counters + 1 + ngroups;
       q.main_locals = (int)(grid / 8);
@@ -622,6 +644,12 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
       else if (a->dh == 256 && bf16) ks = slstm_bwd_split_kernel<true, 4, true>;
       else if (a->dh == 256) { ks = slstm_bwd_split_kernel<false, 4, false>; feed = false; }
       else { ks = slstm_bwd_split_kernel<true, 8, false>; feed = false; }
+      if (dwx_bf16) {
+        if (a->dh == 64) ks = slstm_bwd_split_kernel<true, 1, true, true>;
+        else if (a->dh == 128) ks = slstm_bwd_split_kernel<true, 2, true, true>;
+        else if (a->dh == 256) ks = slstm_bwd_split_kernel<true, 4, true, true>;
+        else ks = slstm_bwd_split_kernel<true, 8, false, true>;
+      }
       const int lds = bwd_split_lds_bytes(feed, bf16);
       {
         const int rc = ensure_dynamic_lds((const void *)ks, (size_t)lds);
@@ -636,7 +664,7 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
     p.coef = a->coef; p.d_h = a->d_h; p.d_s_final = a->d_s_final; p.r_t = a->r_t;
     p.reset = a->reset; p.reset_sb = a->reset_stride_b;
-    p.d_wx = a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t; p.d_s0 = a->d_s0;
+    p.d_wx = (float *)a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t; p.d_wx_bf16 = dwx_bf16; p.d_s0 = a->d_s0;
     p.cut = a->recurrent_cut != 0; p.clip = clip;
     void (*kern)(BwdParams) = nullptr;
     int waves = 0;
@@ -734,6 +762,11 @@ int run_backward_params(const xs_slstm_bwd_args *a) {
   if (!a->d_r || !a->d_bias) return fail(XS_ERR_NULL, "d_r and d_bias are required");
   const bool bf16 = a->dtype == XS_BF16;
   const long long H = (long long)a->NH * a->dh;
+  int dwx_bf16 = 0;
+  {
+    const int rc = d_wx_type(a, &dwx_bf16);
+    if (rc != XS_OK) return rc;
+  }
   hipStream_t stream = (hipStream_t)a->stream;
   const size_t nr = (size_t)a->NH * 4 * a->dh * a->dh, nb = (size_t)4 * H;
   if (((uintptr_t)a->d_r % 4) || ((uintptr_t)a->d_bias % 4)) return fail(XS_ERR_ALIGN, "d_r and d_bias must be 4-byte aligned");
@@ -746,7 +779,7 @@ int run_backward_params(const xs_slstm_bwd_args *a) {
     if (((uintptr_t)a->h_out % 16) || ((uintptr_t)a->s0 % 16)) return fail(XS_ERR_ALIGN, "h_out and s0 must be 16-byte aligned");
     if (a->reset && a->reset_stride_b < a->T) return fail(XS_ERR_SHAPE, "reset row stride %lld < T", (long long)a->reset_stride_b);
     // (a chunk of 32 steps is read through one buffer descriptor: its offsets are 31-bit)
-    if (32ll * a->d_wx_stride_t * 4 >= (1ll << 31) || 32ll * a->B * H * (bf16 ? 2 : 4) >= (1ll << 31))
+    if (32ll * a->d_wx_stride_t * (dwx_bf16 ? 2 : 4) >= (1ll << 31) || 32ll * a->B * H * (bf16 ? 2 : 4) >= (1ll << 31))
       return fail(XS_ERR_UNSUPPORTED, "32 steps of d_wx or of the outputs span 2 GiB or more: run the batch in slices of rows");
   }
   // (the slices of K are added into the results: they start at zero)
@@ -755,7 +788,7 @@ int run_backward_params(const xs_slstm_bwd_args *a) {
   if (!empty) {
     BwdParamParams p;
     p.B = a->B; p.T = a->T; p.NH = a->NH; p.dh = a->dh;
-    p.d_wx = a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t;
+    p.d_wx = (const float *)a->d_wx; p.d_wx_sb = a->d_wx_stride_b; p.d_wx_st = a->d_wx_stride_t; p.d_wx_bf16 = dwx_bf16;
     p.h_out = a->h_out; p.s0 = a->s0; p.reset = a->reset; p.reset_sb = a->reset_stride_b;
     p.d_r = a->d_r; p.d_bias = a->d_bias;
     p.tchunks = (a->T + kParamKC - 1) / kParamKC;

@@ -118,6 +118,7 @@ def slstm_backward(
     recurrent_cut: bool = False,
     recurrent_clipval: Optional[float] = None,
     stepwise_override: Optional[bool] = None,
+    d_wx_dtype: Optional[torch.dtype] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -137,6 +138,8 @@ def slstm_backward(
     Head dims beyond those (up to 1024 with bfloat16, 512 with float32: the forward's range) take one launch per step,
     forward walk and reverse pass alike (``stepwise_override=True`` forces that for head dim 512 in bfloat16 and 256 in
     float32, which both ways cover).
+    ``d_wx_dtype=torch.bfloat16`` (bfloat16 inputs only): ``d_wx`` comes back in bfloat16, as the reference returns its
+    input gradient in the type of its kernels; the reverse kernel then writes and the parameter kernel reads half the bytes.
     ``coef``: what a training forward left (``slstm_forward(..., coef_out=)``); the forward walk is then skipped.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
     to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
@@ -179,7 +182,7 @@ def slstm_backward(
         d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
                                                  split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
                                                  recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval,
-                                                 stepwise_override=stepwise_override)
+                                                 stepwise_override=stepwise_override, d_wx_dtype=d_wx_dtype)
         return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
                 d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
                 d_bias[..., :dh].contiguous(),
@@ -205,7 +208,7 @@ def slstm_backward(
                     wx[b0:b1], r, bias, None if s0 is None else s0[:, b0:b1], None if reset_mask is None else reset_mask[b0:b1],
                     h_out[:, b0:b1], d_h[:, b0:b1], None if d_s_final is None else d_s_final[:, b0:b1],
                     timings=None, split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
-                    recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval))
+                    recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval, d_wx_dtype=d_wx_dtype))
             return (torch.cat([q[0] for q in parts], 0), sum(q[1] for q in parts), sum(q[2] for q in parts),
                     torch.cat([q[3] for q in parts], 1))
     esz = wx.element_size()
@@ -223,7 +226,9 @@ def slstm_backward(
         reset_mask = reset_mask.contiguous()
     r_fwd = r.to(wx.dtype).contiguous()  # R as the forward multiplies by it (the forward rounds R to bf16)
     h_c = h_out if h_out.is_contiguous() and h_out.dtype == wx.dtype else h_out.to(wx.dtype).contiguous()
-    d_wx = torch.empty((B, T, 4 * H), dtype=torch.float32, device=dev)
+    if d_wx_dtype not in (None, torch.float32) and not (d_wx_dtype == torch.bfloat16 and bf16):
+        raise TypeError("d_wx_dtype: float32, or bfloat16 with bfloat16 inputs")
+    d_wx = torch.empty((B, T, 4 * H), dtype=d_wx_dtype or torch.float32, device=dev)
     d_s0 = torch.empty((4, B, H), dtype=torch.float32, device=dev)
     epc = 8 if bf16 else 4
     groups = NH * ((B + 15) // 16)
@@ -282,6 +287,7 @@ def slstm_backward(
     a.r_t = r_t.data_ptr()
     a.d_wx = d_wx.data_ptr()
     a.d_wx_stride_b, a.d_wx_stride_t = d_wx.stride(0), d_wx.stride(1)
+    a.d_wx_dtype = _DTYPE_CODE[d_wx.dtype]
     a.d_s0 = d_s0.data_ptr()
     a.stream = torch.cuda.current_stream(dev).cuda_stream
     a.split = 3 if stepwise else ((2 if quad else 1) if split else 0)
