@@ -273,7 +273,7 @@ int xs_headwise_group_norm(const xs_norm_args *args);
  *   outputs h_out of the forward call (y_{-1} the y plane of s0; zero where reset[b,t] is set) and r, and writes nine
  *   float32 coefficients per step and element into coef [T,B,9,H] (with split != 0: T * ceil(B/16)*16 * 9 * H floats,
  *   in the order the split kernel reads them).
- * xs_slstm_backward          one launch for all T steps, reverse in time: d_wx [B,T,4,NH,dh] (float32, the gradient
+ * xs_slstm_backward          one launch for all T steps, reverse in time: d_wx [B,T,4,NH,dh] (float32, or bf16 with d_wx_dtype; the gradient
  *   with respect to the raw gates: the gradient of wx, and with the outputs what the gradients of R and the bias are
  *   sums of, slstm_backward.cu:381-386, 52-108) and d_s0 [4,B,H] (the m part is zero).
  *
