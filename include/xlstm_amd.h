@@ -314,11 +314,11 @@ typedef struct xs_slstm_bwd_args {
    * r_t is tiled the same way, coef is [T][ceil(B/4)][NH][dh/64][4 rows][9][64 units], exchange has
    * 4 * NH * ceil(B/4) * 4 * 4*dh elements and counters 1 + 2 * NH * ceil(B/4) words.
    * The call is refused (XS_ERR_DEVICE) when its workgroups do not all fit the device at once.
-   * split == 3 (both calls; head dims 512 to 1024 in steps of 128 with XS_BF16, 256 to 512 in steps of 64 with XS_F32:
+   * split == 3 (both calls; head dims 512 to 1024 with XS_BF16, 256 to 512 with XS_F32, in steps of 64:
    * up to what the forward entry points cover): ONE LAUNCH PER STEP instead of one per call, the reference's own
    * decomposition (slstm_backward.cu:291-319), for head dims whose slice of R no compute unit can keep in registers.
-   * prepare launches T times a kernel that multiplies the outputs of the step before (h_out) by r and runs the
-   * forward's update, the backward call T + 1 times a kernel that multiplies the gate deltas of the step behind by R
+   * prepare launches, once per four steps, a kernel that multiplies the outputs of the steps before (h_out) by r in one
+   * pass over r and runs the forward's update step by step, the backward call T + 1 times a kernel that multiplies the gate deltas of the step behind by R
    * transposed and forms the step's gradient.  Then coef is [T,B,9,H]; r_t is R transposed (element (d, k = g*dh + a))
    * in slabs of 256 bytes of K per tile of 32 input units, [NH][d/32][k/KS][d%32][k%KS] with KS = 128 (bf16) or 64
    * (f32), so that what a workgroup stages per slab is 8 KiB in a row; counters is not used, nothing waits and nothing

@@ -267,43 +267,50 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// The forward walk.  What a step multiplies by R is known in advance - the outputs that the forward call stored - so
+// only the pointwise part of the walk is a chain in time: a launch covers kFwdWalkSteps steps, multiplies their
+// operand rows (64 batch rows x the steps) by R in ONE pass over R, keeps the sums of all its steps in registers and
+// then walks through the steps.  R is read from memory once per kFwdWalkSteps steps instead of once per step (14.2 us
+// a step at B 64 x 4 heads of 1024 with one step per launch).
 struct FwdWalkParams {
   int B, T, NH, dh;
-  int t;
+  int t;                     // the first step of this launch
+  int nsteps;                // its steps: kFwdWalkSteps, fewer at the end of the sequence
   const void *wx;            // [B,T,4,NH,dh], strides in elements
   long long wx_sb, wx_st;
-  const void *r_tiled;       // R in the type of the operands, in slabs of 256 bytes of K per tile of 32 units:
-                             // [NH][a / 32][k / KS][gate][a % 32][k % KS], KS = 128 (bf16) or 64 (float32)
-  const void *h_prev;        // [B][H] in the type of the operands: the outputs of step t - 1 (step 0: the y of the initial
-                             // state in that type), or null: zeros
+  const void *r_tiled;       // R in the type of the operands, in slabs of 128 bytes of K per tile of 32 units:
+                             // [NH][a / 32][k / KS][gate][a % 32][k % KS], KS = 64 (bf16) or 32 (float32)
+  const void *h_out;         // [T,B,H] in the type of the operands: the forward's outputs
+  const void *h_init;        // [B,H] in that type: the y of the initial state, or null: zeros
   const float *bias;         // [NH,4,dh]
-  const float *state_in;     // [4,B,H]: planes 1-3 are c, n, m in front of the step (step 0: the initial state), or null: zeros
-  float *state;              // [4,B,H]: planes 1-3 take c, n, m behind the step
+  const float *state_in;     // [4,B,H]: planes 1-3 are c, n, m in front of step t (step 0: the initial state), or null: zeros
+  float *state;              // [4,B,H]: planes 1-3 take c, n, m behind the launch's last step
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
   float *coef;               // [T,B,9,H]
 };
 
+constexpr int kFwdWalkSteps = 4;
 constexpr int kFwdWalkSlots = 3;
-constexpr int kFwdWalkSlot = (64 + 128) * 256;  // bytes of a slab in LDS: the outputs of 64 rows, R of 4 gates x 32 units
+constexpr int kFwdWalkSlot = (128 + kFwdWalkSteps * 64) * 128;  // bytes of a slab in LDS: R of 4 gates x 32 units, the outputs of 64 rows x the steps
 constexpr int fwd_walk_lds_bytes() { return kFwdWalkSlots * kFwdWalkSlot; }
 
 // R [NH][4 dh][dh] into the walk's slabs, and the y plane of the initial state into the type of the operands
 template <bool BF16>
 __global__ __launch_bounds__(256) void slstm_fwd_walk_init_kernel(const void *r, void *r_tiled, const float *s0, void *h_init, int B, int NH, int dh) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  const int nslab = dh * ESZ >> 8;
-  const long long pieces = (long long)NH * 4 * dh * nslab * 16;  // 16-byte pieces of R
+  const int nslab = dh * ESZ >> 7;
+  const long long pieces = (long long)NH * 4 * dh * nslab * 8;  // 16-byte pieces of R
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < pieces; i += stride) {
-    const int piece = (int)(i & 15);
-    long long v = i >> 4;
+    const int piece = (int)(i & 7);
+    long long v = i >> 3;
     const int j = (int)(v & 31); v >>= 5;
     const int g = (int)(v & 3); v >>= 2;
     const int slab = (int)(v % nslab); v /= nslab;
     const int ut = (int)(v % (dh >> 5));
     const int head = (int)(v / (dh >> 5));
-    const char *src = reinterpret_cast<const char *>(r) + (((long long)head * 4 + g) * dh + ut * 32 + j) * dh * ESZ + slab * 256 + piece * 16;
+    const char *src = reinterpret_cast<const char *>(r) + (((long long)head * 4 + g) * dh + ut * 32 + j) * dh * ESZ + slab * 128 + piece * 16;
     reinterpret_cast<uint4 *>(r_tiled)[i] = *reinterpret_cast<const uint4 *>(src);
   }
   const long long BH = (long long)B * NH * dh;
@@ -317,7 +324,7 @@ __global__ __launch_bounds__(256) void slstm_fwd_walk_init_kernel(const void *r,
 template <bool BF16>
 __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalkParams p) {
   constexpr int ESZ = BF16 ? 2 : 4;
-  constexpr int D = kFwdWalkSlots;
+  constexpr int D = kFwdWalkSlots, TB = kFwdWalkSteps;
   extern __shared__ __attribute__((aligned(1024))) unsigned char fwalk_lds[];
   const int dh = p.dh, NH = p.NH;
   const int H = NH * dh;
@@ -341,50 +348,49 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalk
   const int a0 = (tile % n_ut) * 32, rowbase = (tile / n_ut) * 64;
   const int tid = threadIdx.x, lane = tid & 63, q = lane >> 4, r16 = lane & 15;
   const int wave = (int)uniform((uint32_t)(tid >> 6));
-  const int t = p.t;
-  const int nslab = dh * ESZ >> 8;
+  const int t0 = p.t;
+  const int nslab = dh * ESZ >> 7;
   const uint32_t lds0 = (uint32_t)(unsigned long long)((__attribute__((address_space(3))) unsigned char *)fwalk_lds);
 
   if (wave >= 4) {
-    // ---- a feeder wave: per slab 4 of the 16 KiB of outputs and 8 of the 32 KiB of R, 1 KiB (4 rows of 256 bytes) per
-    //      load, straight into LDS, piece g of row r at position g ^ (r & 7) (see slstm_bwd_step_kernel).  Rows past
-    //      the batch, rows that start a document at this step and a walk without an initial state ask out of range:
-    //      the loads return zeros.
-    const int f = wave - 4, sub = lane >> 4, pos = lane & 15;
-    const bool live = rowbase + 16 * f < p.B;  // (this wave's 16 rows of outputs: not fetched when the batch ends in front of them)
-    const unsigned long long hb = reinterpret_cast<unsigned long long>(p.h_prev ? p.h_prev : p.r_tiled);
-    const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_tiled) + ((long long)head * n_ut + (a0 >> 5)) * nslab * (128 * 256);
+    // ---- feeder wave f: per slab the 8 KiB of operand rows of step t0 + f (64 rows x 128 bytes) and 4 of the 16 KiB
+    //      of R, 1 KiB (8 rows of 128 bytes) per load, straight into LDS, piece g of row r (16 bytes) at position
+    //      g ^ (r & 7) of the row.  Rows past the batch, rows that start a document at that step, a step past the
+    //      end and a walk without an initial state ask out of range: the loads return zeros.
+    const int f = wave - 4, sub = lane >> 3, pos = lane & 7;
+    const int tt = t0 + f;  // this wave's step
+    const void *hsrc = tt == 0 ? p.h_init : reinterpret_cast<const void *>(reinterpret_cast<const char *>(p.h_out) + (long long)(tt - 1) * BH * ESZ);
+    const bool step_there = f < p.nsteps && hsrc != nullptr;
+    const unsigned long long hb = reinterpret_cast<unsigned long long>(step_there ? hsrc : p.r_tiled);
+    const unsigned long long rb = reinterpret_cast<unsigned long long>(p.r_tiled) + ((long long)head * n_ut + (a0 >> 5)) * nslab * (128 * 128);
     const u32x4_t hrs = {uniform((uint32_t)hb), uniform((uint32_t)(hb >> 32) & 0xFFFFu), (uint32_t)(BH * ESZ), 0x00020000u};
-    const u32x4_t rrs = {uniform((uint32_t)rb), uniform((uint32_t)(rb >> 32) & 0xFFFFu), (uint32_t)(nslab * (128 * 256)), 0x00020000u};
-    uint32_t hvo[4], rvo[8];
+    const u32x4_t rrs = {uniform((uint32_t)rb), uniform((uint32_t)(rb >> 32) & 0xFFFFu), (uint32_t)(nslab * (128 * 128)), 0x00020000u};
+    uint32_t hvo[8], rvo[4];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      const int row = 4 * (4 * f + k) + sub, brow = rowbase + row;
-      bool zero = brow >= p.B || !p.h_prev;
-      if (!zero && p.reset) zero = p.reset[(long long)brow * p.reset_sb + t] != 0;
+    for (int k = 0; k < 8; ++k) {
+      const int row = 8 * k + sub, brow = rowbase + row;
+      bool zero = brow >= p.B || !step_there;
+      if (!zero && p.reset) zero = p.reset[(long long)brow * p.reset_sb + tt] != 0;
       hvo[k] = zero ? 0x80000000u : (uint32_t)(((long long)brow * H + head * dh) * ESZ + ((pos ^ (row & 7)) << 4));
     }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int row = 4 * (8 * f + k) + sub;  // gate row / 32, unit row % 32 of the tile
-      rvo[k] = (uint32_t)(row * 256 + ((pos ^ (row & 7)) << 4));
+    for (int k = 0; k < 4; ++k) {
+      const int row = 8 * (4 * f + k) + sub;  // gate row / 32, unit row % 32 of the tile
+      rvo[k] = (uint32_t)(row * 128 + ((pos ^ (row & 7)) << 4));
     }
     auto request = [&](int s) {
       const int sc = s < nslab ? s : nslab - 1;
       const uint32_t slot = lds0 + (uint32_t)(s % D) * kFwdWalkSlot;
-      if (live) {
 #pragma unroll
-        for (int k = 0; k < 4; ++k)
-          bwd_fetch_to_lds_b128(hrs, uniform(slot + (4 * f + k) * 1024), hvo[k] + (uint32_t)sc * 256u);
-      }
+      for (int k = 0; k < 4; ++k)
+        bwd_fetch_to_lds_b128(rrs, uniform(slot + (4 * f + k) * 1024), rvo[k] + (uint32_t)sc * (128 * 128));
 #pragma unroll
       for (int k = 0; k < 8; ++k)
-        bwd_fetch_to_lds_b128(rrs, uniform(slot + 64 * 256 + (8 * f + k) * 1024), rvo[k] + (uint32_t)sc * (128 * 256));
+        bwd_fetch_to_lds_b128(hrs, uniform(slot + 128 * 128 + (8 * f + k) * 1024), hvo[k] + (uint32_t)sc * 128u);
     };
     for (int s = 0; s < D - 1; ++s) request(s);
     for (int s = 0; s < nslab; ++s) {
-      if (live) asm volatile("s_waitcnt vmcnt(%0)" :: "n"(12 * (D - 2)) : "memory");  // (slab s has landed)
-      else asm volatile("s_waitcnt vmcnt(%0)" :: "n"(8 * (D - 2)) : "memory");
+      asm volatile("s_waitcnt vmcnt(%0)" :: "n"(12 * (D - 2)) : "memory");  // (slab s has landed)
       lds_barrier();
       request(s + D - 1);
     }
@@ -395,106 +401,156 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalk
 
   // ---- pointwise operands of this lane's elements (rows rowbase + 32 wr + 16 ut + r16, units a0 + 16 wu + 4 q .. + 3)
   const int ua = a0 + 16 * wu + 4 * q;
-  f32x4 bias4[4], wx4[2][4], cv[2], nv[2], mv[2];
-  bool there[2], restart[2];
-  long long eo[2];
+  f32x4 cv[2], nv[2], mv[2];
+  bool there[2];
+  uint32_t restart_bits = 0u;  // bit 2 j + ut: the row starts from nothing at step t0 + j
+  long long eo[2], wo[2];
+  typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
+  struct StepWx { typename std::conditional<BF16, u32x2_t, f32x4>::type g[2][4]; };
+  auto load_wx = [&](int j, StepWx &w) {
 #pragma unroll
-  for (int g = 0; g < 4; ++g) bias4[g] = *reinterpret_cast<const f32x4 *>(p.bias + ((long long)head * 4 + g) * dh + ua);
+    for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const long long o = wo[ut] + (long long)(t0 + j) * p.wx_st + (long long)g * H;
+        if constexpr (BF16) w.g[ut][g] = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(reinterpret_cast<const uint16_t *>(p.wx) + o));
+        else w.g[ut][g] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.wx) + o));
+      }
+  };
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
     const int row = rowbase + 32 * wr + 16 * ut + r16;
     there[ut] = row < p.B;
     const int rowc = there[ut] ? row : p.B - 1;
     eo[ut] = (long long)rowc * H + head * dh + ua;
-    restart[ut] = !p.state_in || (p.reset && p.reset[(long long)rowc * p.reset_sb + t] != 0);
+    wo[ut] = (long long)rowc * p.wx_sb + head * dh + ua;
+#pragma unroll
+    for (int j = 0; j < TB; ++j) {
+      const bool rs = (j == 0 && !p.state_in) || (p.reset && j < p.nsteps && p.reset[(long long)rowc * p.reset_sb + t0 + j] != 0);
+      restart_bits |= rs ? (1u << (2 * j + ut)) : 0u;
+    }
     const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     cv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + BH + eo[ut]) : zero;
     nv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + 2 * BH + eo[ut]) : zero;
     mv[ut] = p.state_in ? *reinterpret_cast<const f32x4 *>(p.state_in + 3 * BH + eo[ut]) : zero;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const long long o = (long long)rowc * p.wx_sb + (long long)t * p.wx_st + (long long)g * H + head * dh + ua;
-      if (BF16) {
-        typedef unsigned int u32x2_t __attribute__((ext_vector_type(2)));
-        const u32x2_t w = __builtin_nontemporal_load(reinterpret_cast<const u32x2_t *>(reinterpret_cast<const uint16_t *>(p.wx) + o));
-        wx4[ut][g] = f32x4{bf16_bits_to_float(w.x & 0xFFFFu), bf16_bits_to_float(w.x >> 16), bf16_bits_to_float(w.y & 0xFFFFu), bf16_bits_to_float(w.y >> 16)};
-      } else {
-        wx4[ut][g] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(reinterpret_cast<const float *>(p.wx) + o));
-      }
-    }
   }
+  // (float32: one set of W.x registers, asked for per step - two sets did not fit beside the sums of four steps)
+  StepWx wxa, wxb;
+  if constexpr (BF16) load_wx(0, wxa);
 
-  // ---- R [4 x 32 units x K] . y_{t-1} [64 rows x K], transposed: acc[ut][g][i] = gate g of unit ua + i, row 32 wr + 16 ut + r16
-  f32x4 acc[2][4];
+  // ---- R [4 x 32 units x K] . y_{t-1} [64 rows x K] for every step of the launch, transposed:
+  //      acc[j][ut][g][i] = gate g of unit ua + i, row 32 wr + 16 ut + r16, step t0 + j
+  f32x4 acc[TB][2][4];
 #pragma unroll
-  for (int ut = 0; ut < 2; ++ut)
+  for (int j = 0; j < TB; ++j)
 #pragma unroll
-    for (int g = 0; g < 4; ++g) acc[ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int ut = 0; ut < 2; ++ut)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) acc[j][ut][g] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
   {
-    int swz[4];
-#pragma unroll
-    for (int ch = 0; ch < 4; ++ch) swz[ch] = ((4 * ch + q) ^ (r16 & 7)) << 4;
-    const int hrow[2] = {(32 * wr + r16) * 256, (32 * wr + 16 + r16) * 256};
-    const int rrow = 64 * 256 + (16 * wu + r16) * 256;  // (gate g: 32 rows further each)
+    // this lane's pieces of a slab: k-step ch, lane group q -> piece 4 ch + q of the row, at position piece ^ (row & 7)
+    // (all rows this lane reads have row & 7 == r16 & 7)
+    const int swz[2] = {((0 + q) ^ (r16 & 7)) << 4, ((4 + q) ^ (r16 & 7)) << 4};
+    const int rrow = (16 * wu + r16) * 128;                 // (gate g: 32 rows further each)
+    const int hrow = 128 * 128 + (32 * wr + r16) * 128;     // (row tile ut: 16 rows further, step j: 64 rows further)
     for (int s = 0; s < nslab; ++s) {
       lds_barrier();
       const unsigned char *slot = fwalk_lds + (s % D) * kFwdWalkSlot;
 #pragma unroll
-      for (int ch = 0; ch < 4; ++ch) {
-        uint4 rv[4], hv[2];
+      for (int ch = 0; ch < 2; ++ch) {
+        uint4 rv[4];
 #pragma unroll
-        for (int g = 0; g < 4; ++g) rv[g] = *reinterpret_cast<const uint4 *>(slot + rrow + g * (32 * 256) + swz[ch]);
+        for (int g = 0; g < 4; ++g) rv[g] = *reinterpret_cast<const uint4 *>(slot + rrow + g * (32 * 128) + swz[ch]);
 #pragma unroll
-        for (int ut = 0; ut < 2; ++ut) hv[ut] = *reinterpret_cast<const uint4 *>(slot + hrow[ut] + swz[ch]);
+        for (int j = 0; j < TB; ++j) {
+          uint4 hv[2];
 #pragma unroll
-        for (int ut = 0; ut < 2; ++ut)
+          for (int ut = 0; ut < 2; ++ut) hv[ut] = *reinterpret_cast<const uint4 *>(slot + hrow + (j * 64 + 16 * ut) * 128 + swz[ch]);
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            if (BF16) {
-              acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[ut][g], 0, 0, 0);
-            } else {
-              const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w}, hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
+          for (int ut = 0; ut < 2; ++ut)
 #pragma unroll
-              for (int e = 0; e < 4; ++e)
-                acc[ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[ut][g], 0, 0, 0);
+            for (int g = 0; g < 4; ++g) {
+              if (BF16) {
+                acc[j][ut][g] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, rv[g]), __builtin_bit_cast(bf16x8, hv[ut]), acc[j][ut][g], 0, 0, 0);
+              } else {
+                const uint32_t rw[4] = {rv[g].x, rv[g].y, rv[g].z, rv[g].w}, hw[4] = {hv[ut].x, hv[ut].y, hv[ut].z, hv[ut].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  acc[j][ut][g] = __builtin_amdgcn_mfma_f32_16x16x4f32(__uint_as_float(rw[e]), __uint_as_float(hw[e]), acc[j][ut][g], 0, 0, 0);
+              }
             }
-          }
+        }
       }
     }
   }
 
-  // ---- the forward's update with the gate values kept, and the nine coefficients of the step's gradient
+  // ---- the walk through the launch's steps: the forward's update with the gate values kept, and the nine
+  //      coefficients of each step's gradient (W.x of the next step is asked for while this one is worked)
+  f32x4 bias4[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) bias4[g] = *reinterpret_cast<const f32x4 *>(p.bias + ((long long)head * 4 + g) * dh + ua);
+  auto one_step = [&](int j, const StepWx &w) {
+#pragma unroll
+    for (int ut = 0; ut < 2; ++ut) {
+      const bool restart = (restart_bits >> (2 * j + ut)) & 1u;
+      f32x4 cf[9];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float raw[4];
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          float wv;
+          if constexpr (BF16) {
+            const uint32_t wd = i < 2 ? w.g[ut][g][0] : w.g[ut][g][1];
+            wv = bf16_bits_to_float((i & 1) ? (wd >> 16) : (wd & 0xFFFFu));
+          } else {
+            wv = w.g[ut][g][i];
+          }
+          raw[g] = (wv + acc[j][ut][g][i]) + bias4[g][i];
+        }
+        CellState st{0.0f, restart ? 0.0f : cv[ut][i], restart ? 0.0f : nv[ut][i], restart ? 0.0f : mv[ut][i]};
+        const float c_old = st.c, n_old = st.n;
+        GateValues k;
+        slstm_pointwise_keep(raw[0], raw[1], raw[2], raw[3], st, k);
+        const float omf = __builtin_amdgcn_rcpf(1.0f + __expf(raw[1]));  // 1 - sigmoid(f)
+        cf[0][i] = k.og * k.rn;
+        cf[1][i] = st.y * k.rn;
+        cf[2][i] = k.ig * k.tz;
+        cf[3][i] = k.ig;
+        cf[4][i] = k.fg * omf * c_old;
+        cf[5][i] = k.fg * omf * n_old;
+        cf[6][i] = k.ig * (1.0f - k.tz * k.tz);
+        cf[7][i] = (1.0f - k.og) * st.y;
+        cf[8][i] = k.fg;
+        cv[ut][i] = st.c; nv[ut][i] = st.n; mv[ut][i] = st.m;
+      }
+      if (there[ut]) {
+        float *cd = p.coef + ((long long)(t0 + j) * p.B + (rowbase + 32 * wr + 16 * ut + r16)) * 9 * H + head * dh + ua;
+#pragma unroll
+        for (int jj = 0; jj < 9; ++jj) __builtin_nontemporal_store(cf[jj], reinterpret_cast<f32x4 *>(cd + (long long)jj * H));
+      }
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < TB; ++j) {
+    if (j < p.nsteps) {
+      if constexpr (BF16) {
+        StepWx &cur = (j & 1) ? wxb : wxa;
+        StepWx &nxt = (j & 1) ? wxa : wxb;
+        if (j + 1 < p.nsteps) load_wx(j + 1, nxt);
+        one_step(j, cur);
+      } else {
+        load_wx(j, wxa);
+        one_step(j, wxa);
+      }
+    }
+  }
 #pragma unroll
   for (int ut = 0; ut < 2; ++ut) {
     if (!there[ut]) continue;
-    f32x4 cf[9], cn, nn, mn;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float raw[4];
-#pragma unroll
-      for (int g = 0; g < 4; ++g) raw[g] = (wx4[ut][g][i] + acc[ut][g][i]) + bias4[g][i];
-      CellState st{0.0f, restart[ut] ? 0.0f : cv[ut][i], restart[ut] ? 0.0f : nv[ut][i], restart[ut] ? 0.0f : mv[ut][i]};
-      const float c_old = st.c, n_old = st.n;
-      GateValues k;
-      slstm_pointwise_keep(raw[0], raw[1], raw[2], raw[3], st, k);
-      const float omf = __builtin_amdgcn_rcpf(1.0f + __expf(raw[1]));  // 1 - sigmoid(f)
-      cf[0][i] = k.og * k.rn;
-      cf[1][i] = st.y * k.rn;
-      cf[2][i] = k.ig * k.tz;
-      cf[3][i] = k.ig;
-      cf[4][i] = k.fg * omf * c_old;
-      cf[5][i] = k.fg * omf * n_old;
-      cf[6][i] = k.ig * (1.0f - k.tz * k.tz);
-      cf[7][i] = (1.0f - k.og) * st.y;
-      cf[8][i] = k.fg;
-      cn[i] = st.c; nn[i] = st.n; mn[i] = st.m;
-    }
-    float *cd = p.coef + ((long long)t * p.B + (rowbase + 32 * wr + 16 * ut + r16)) * 9 * H + head * dh + ua;
-#pragma unroll
-    for (int j = 0; j < 9; ++j) __builtin_nontemporal_store(cf[j], reinterpret_cast<f32x4 *>(cd + (long long)j * H));
-    *reinterpret_cast<f32x4 *>(p.state + BH + eo[ut]) = cn;
-    *reinterpret_cast<f32x4 *>(p.state + 2 * BH + eo[ut]) = nn;
-    *reinterpret_cast<f32x4 *>(p.state + 3 * BH + eo[ut]) = mn;
+    *reinterpret_cast<f32x4 *>(p.state + BH + eo[ut]) = cv[ut];
+    *reinterpret_cast<f32x4 *>(p.state + 2 * BH + eo[ut]) = nv[ut];
+    *reinterpret_cast<f32x4 *>(p.state + 3 * BH + eo[ut]) = mv[ut];
   }
 }
 

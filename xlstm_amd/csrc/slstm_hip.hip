@@ -406,8 +406,9 @@ int d_wx_type(const xs_slstm_bwd_args *a, int *is_bf16) {
 }
 
 // ---- backward pass with one launch per step (split == 3): slstm_fwd_walk_kernel and slstm_bwd_step_kernel.  Both keep
-// what a step hands to the next in the caller's `exchange` buffer: the forward walk a state [4,B,H] float32 (its y
-// plane holds the y of the initial state in the type of the operands) and R in the walk's slabs; the reverse pass two
+// what a launch hands to the next in the caller's `exchange` buffer: the forward walk (a launch per kFwdWalkSteps
+// steps) a state [4,B,H] float32 (its y plane holds the y of the initial state in the type of the operands) and R in
+// the walk's slabs; the reverse pass two
 // sets of gate deltas in the type of the operands, in tiles of 64 rows.
 int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   const bool bf16 = a->dtype == XS_BF16;
@@ -422,7 +423,6 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
   }
   if (!a->exchange) return fail(XS_ERR_NULL, "exchange is required with one launch per step");
   if (((uintptr_t)a->exchange % 16) || ((uintptr_t)a->coef % 16)) return fail(XS_ERR_ALIGN, "exchange and coef must be 16-byte aligned");
-  if ((dh * esz) % 256 != 0) return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d is not a multiple of %d", dh, 256 / esz);
   const long long nwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
   if (nwg > 0x7FFFFFFF) return fail(XS_ERR_UNSUPPORTED, "too many tiles for one step launch");
   if (prepare) {
@@ -442,15 +442,16 @@ int run_backward_stepwise(const xs_slstm_bwd_args *a, bool prepare) {
     p.B = B; p.T = T; p.NH = NH; p.dh = dh;
     p.wx = a->wx; p.wx_sb = a->wx_stride_b; p.wx_st = a->wx_stride_t;
     p.r_tiled = r_tiled; p.bias = a->bias; p.state = state;
+    p.h_out = a->h_out; p.h_init = a->s0 ? (const void *)state : nullptr;
     p.reset = a->reset; p.reset_sb = a->reset_stride_b; p.coef = a->coef;
     void (*kern)(FwdWalkParams) = bf16 ? slstm_fwd_walk_kernel<true> : slstm_fwd_walk_kernel<false>;
     {
       const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(kern), (size_t)fwd_walk_lds_bytes());
       if (rc != XS_OK) return rc;
     }
-    for (int t = 0; t < T; ++t) {
+    for (int t = 0; t < T; t += kFwdWalkSteps) {  // (a launch covers kFwdWalkSteps steps: one pass over R for all of them)
       p.t = t;
-      p.h_prev = t == 0 ? (a->s0 ? (const void *)state : nullptr) : (const void *)((const char *)a->h_out + (long long)(t - 1) * BH * esz);
+      p.nsteps = T - t < kFwdWalkSteps ? T - t : kFwdWalkSteps;
       p.state_in = t == 0 ? a->s0 : state;
       hipLaunchKernelGGL(kern, dim3((unsigned)nwg), dim3(kBwdStepThreads), fwd_walk_lds_bytes(), stream, p);
     }
@@ -494,8 +495,8 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
   if (a->split == 3) {
     // one launch per step: the head dims the forward covers beyond those of the persistent kernels, and those next below
     const int lo = a->dtype == XS_BF16 ? 512 : 256;
-    if (a->dh % (lo / 4) != 0 || a->dh < lo || a->dh > 2 * lo)
-      return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d not supported (%d to %d in steps of %d)", a->dh, lo, 2 * lo, lo / 4);
+    if (a->dh % 64 != 0 || a->dh < lo || a->dh > 2 * lo)
+      return fail(XS_ERR_UNSUPPORTED, "backward pass with one launch per step: head dim %d not supported (%d to %d in steps of 64)", a->dh, lo, 2 * lo);
   } else if (a->dh != 64 && a->dh != 128 && a->dh != 256 && !(a->dh == 512 && a->dtype == XS_BF16 && (prepare || a->split)))
     return fail(XS_ERR_UNSUPPORTED, "backward pass: head dim %d not supported (64, 128, 256; 512 in bf16 over several compute units; "
                 "up to 1024 in bf16 and 512 in float32 with one launch per step, split = 3)", a->dh);

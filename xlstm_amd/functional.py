@@ -55,15 +55,14 @@ def _compute_units(dev) -> int:
 def backward_kernel_head_dim(dh: int, dtype: torch.dtype) -> Optional[int]:
     """The head dim that the backward kernels run a head dim ``dh`` as: 64, 128, 256 (and 512 with bfloat16 inputs) for
     the kernels that take one launch for all steps; beyond those, up to the forward's range (1024 with bfloat16, 512 with
-    float32), the next multiple of 128 (bfloat16) or 64 (float32) for the kernels that take one launch per step.  Sizes
-    in between are padded up by ``slstm_backward``.  None when there is none."""
+    float32), the next multiple of 64 for the kernels that take one launch per step.  Sizes in between are padded up by
+    ``slstm_backward``.  None when there is none."""
     bf16 = dtype == torch.bfloat16
     for size in (64, 128, 256, 512):
         if dh <= size and (size < 512 or bf16):
             return size
     if dh <= (1024 if bf16 else 512):
-        step = 128 if bf16 else 64
-        return (dh + step - 1) // step * step
+        return (dh + 63) // 64 * 64
     return None
 
 
