@@ -294,7 +294,7 @@ typedef struct xs_slstm_bwd_args {
   const float *s0;           /* [4,B,H] or NULL (prepare) */
   const uint8_t *reset;      /* [B,T] or NULL, row stride reset_stride_b bytes (both) */
   int64_t reset_stride_b;
-  float *coef;               /* [T,B,9,H] ([T,ceil(B/16)*16,9,H] with split, [T,ceil(B/4)*4,9,H] with split == 2): written by prepare, read by backward */
+  float *coef;               /* [T,B,9,H] ([T,ceil(B/16)*16,9,H] with split, [T,ceil(B/4)*4,9,H] with split == 2, [T,ceil(B/64)*64,9,H] with split == 3): written by prepare, read by backward */
   const void *d_h;           /* [T,B,H]: gradient with respect to h_out (backward) */
   const float *d_s_final;    /* [4,B,H] or NULL: gradient with respect to the final state; y, c, n are used (backward) */
   const void *r_t;           /* (backward) */
@@ -319,7 +319,8 @@ typedef struct xs_slstm_bwd_args {
    * decomposition (slstm_backward.cu:291-319), for head dims whose slice of R no compute unit can keep in registers.
    * prepare launches, once per four steps, a kernel that multiplies the outputs of the steps before (h_out) by r in one
    * pass over r and runs the forward's update step by step, the backward call T + 1 times a kernel that multiplies the gate deltas of the step behind by R
-   * transposed and forms the step's gradient.  Then coef is [T,B,9,H]; r_t is R transposed (element (d, k = g*dh + a))
+   * transposed and forms the step's gradient.  Then coef has T * ceil(B/64)*64 * 9 * H floats, in the order the walk's
+   * waves write and the reverse pass's read them; r_t is R transposed (element (d, k = g*dh + a))
    * in slabs of 256 bytes of K per tile of 32 input units, [NH][d/32][k/KS][d%32][k%KS] with KS = 128 (bf16) or 64
    * (f32), so that what a workgroup stages per slab is 8 KiB in a row; counters is not used, nothing waits and nothing
    * can give up; and exchange is a 16-byte aligned buffer of at least

@@ -440,7 +440,7 @@ def test_all_four_gradients_through_the_c_abi(bf16, B, T, NH, dh, split):
     dh_t, dsf_t = dev_t(d_h, tdt), dev_t(d_sf)
     h, _ = F.slstm_forward(wx_t, r_fwd if bf16 else dev_t(r_k), b_t, s0_t, m_t)
     groups = NH * ((B + tile_rows - 1) // tile_rows)
-    rows = (B + tile_rows - 1) // tile_rows * tile_rows if split and not stepwise else B
+    rows = (B + tile_rows - 1) // tile_rows * tile_rows if split and not stepwise else ((B + 63) // 64 * 64 if stepwise else B)
     coef = torch.empty(T * rows * 9 * H, dtype=torch.float32, device=dev)
     d_wx = torch.empty(B, T, 4 * H, dtype=torch.float32, device=dev)
     d_s0 = torch.empty(4, B, H, dtype=torch.float32, device=dev)

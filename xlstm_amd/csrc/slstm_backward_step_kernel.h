@@ -34,7 +34,7 @@ struct BwdStepParams {
   int B, T, NH, dh;
   int t;                     // the step of this launch; -1: only the gradient of the initial state's y
   int first;                 // the call's last step (its first launch): what reaches y comes from d_s_final
-  const float *coef;         // [T,B,9,H]
+  const float *coef;         // [T][ceil(B/64)][NH][dh/32][2 row tiles of a wave][4 waves][9][64 lanes][4]: as the walk's waves wrote them
   const void *d_h;           // [T,B,H] in the type of the operands
   const float *d_s_final;    // [4,B,H] or null
   const void *r_t;           // R transposed, element (input unit d, gate unit k = g dh + a) of head h, in slabs of 256 bytes of K:
@@ -169,9 +169,11 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_bwd_step_kernel(BwdStep
     const float *carry = p.first ? p.d_s_final : p.d_s0;
     dcv[ut] = carry ? *reinterpret_cast<const f32x4 *>(carry + BH + eo[ut]) : zero;
     dnv[ut] = carry ? *reinterpret_cast<const f32x4 *>(carry + 2 * BH + eo[ut]) : zero;
-    const float *cs = p.coef + ((long long)t * p.B + rowc) * 9 * H + head * dh + ua;
+    // (the coefficients lie as the walk's waves wrote them: per tile, row tile of the wave, wave and coefficient the 64
+    // lanes' 16 bytes in a row - a load is 1 KiB in one piece; the lanes of rows past the batch ask for nothing)
+    const float *cs = p.coef + ((((long long)t * n_rt * NH * n_ut + ((long long)(rowbase >> 6) * NH + head) * n_ut + (a0 >> 5)) * 2 + ut) * 4 + wave) * (9 * 256) + lane * 4;
 #pragma unroll
-    for (int j = 0; j < 9; ++j) cf[ut][j] = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(cs + (long long)j * H));
+    for (int j = 0; j < 9; ++j) cf[ut][j] = there[ut] ? *reinterpret_cast<const f32x4 *>(cs + j * 256) : zero;
     const long long ho = (long long)t * BH + eo[ut];
     if (BF16) {
       const uint2 w = *reinterpret_cast<const uint2 *>(reinterpret_cast<const uint16_t *>(p.d_h) + ho);
@@ -287,7 +289,7 @@ struct FwdWalkParams {
   float *state;              // [4,B,H]: planes 1-3 take c, n, m behind the launch's last step
   const uint8_t *reset;      // [B,T] or null
   long long reset_sb;
-  float *coef;               // [T,B,9,H]
+  float *coef;               // [T][ceil(B/64)][NH][dh/32][2 row tiles of a wave][4 waves][9][64 lanes][4] (the lanes' 4 units)
 };
 
 constexpr int kFwdWalkSteps = 4;
@@ -525,12 +527,11 @@ __global__ __launch_bounds__(kBwdStepThreads) void slstm_fwd_walk_kernel(FwdWalk
         cv[ut][i] = st.c; nv[ut][i] = st.n; mv[ut][i] = st.m;
       }
       if (there[ut]) {
-        float *cd = p.coef + ((long long)(t0 + j) * p.B + (rowbase + 32 * wr + 16 * ut + r16)) * 9 * H + head * dh + ua;
+        float *cd = p.coef + ((((long long)(t0 + j) * n_rt * NH * n_ut + ((long long)(rowbase >> 6) * NH + head) * n_ut + (a0 >> 5)) * 2 + ut) * 4 + wave) * (9 * 256) + lane * 4;
 #pragma unroll
-        // (plain stores: two waves share each 128-byte line of a coefficient plane, which streaming stores write as
-        // halves - 11.0 instead of 10.0 us per step at B 64 x 4 heads of 1024; nor do the feeder waves help by taking
-        // half of the walk over through LDS: 11.7)
-        for (int jj = 0; jj < 9; ++jj) *reinterpret_cast<f32x4 *>(cd + (long long)jj * H) = cf[jj];
+        // (a store is 1 KiB in one piece: with the coefficients in planes of H floats per batch row two waves shared each
+        // 128-byte line of a plane)
+        for (int jj = 0; jj < 9; ++jj) *reinterpret_cast<f32x4 *>(cd + jj * 256) = cf[jj];
       }
     }
   };

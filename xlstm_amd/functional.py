@@ -252,7 +252,8 @@ def slstm_backward(
     # (the split kernels read the coefficients in pieces of a row tile: the buffer covers whole row tiles)
     coef_given = coef is not None
     if not coef_given:
-        coef = torch.empty((T, ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else B, 9, H), dtype=torch.float32, device=dev)
+        rows = ((B + 3) // 4 * 4 if quad else (B + 15) // 16 * 16) if split else ((B + 63) // 64 * 64 if stepwise else B)
+        coef = torch.empty((T, rows, 9, H), dtype=torch.float32, device=dev)
     # R transposed in the operand order of the reverse kernel (xs_slstm_backward_tile_r), and what the kernels of a call
     # hand to each other
     r_t = torch.empty(NH * 4 * dh * dh, dtype=wx.dtype, device=dev)
