@@ -220,6 +220,17 @@ def test_a_wait_between_compute_units_that_runs_out_is_reported(row_tile):
     assert bool(torch.isnan(got[3][:3]).all())
     again = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, **kw)  # the next call is unaffected
     assert torch.equal(again[0], good[0]) and torch.equal(again[3], good[3])
+    # the way the cell's autograd function calls it: the abort word goes to the cell's status ring, nothing
+    # synchronises or raises in the call, the cell reports it afterwards
+    from tests.test_hip_cell import _cell_from
+
+    cell = _cell_from(r, b, dtype="bfloat16")
+    got = F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, spin_limit=-1, abort_sink=cell._watch_word, **kw)
+    with pytest.raises(F.EngineError, match="gave up"):
+        cell.check_status()
+    assert bool(torch.isnan(got[3][:3]).all())
+    F.slstm_backward(wx_t, r_t, b_t, None, None, h, d_h, abort_sink=cell._watch_word, **kw)
+    cell.check_status()  # (a good call leaves nothing to report)
 
 
 _ORACLE_RESULTS = {}

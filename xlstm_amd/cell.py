@@ -198,10 +198,11 @@ class _CellFunction(torch.autograd.Function):
     what the forward call returned for ``x, r, bias, state, mask``; nothing else is stored for the backward."""
 
     @staticmethod
-    def forward(ctx, x, r, bias, state, h, s, mask, num_heads, cut, clipval, coef):
+    def forward(ctx, x, r, bias, state, h, s, mask, num_heads, cut, clipval, coef, abort_sink):
         ctx.save_for_backward(x, r, bias, h, *(() if state is None else (state,)))
         ctx.mask, ctx.num_heads, ctx.cut, ctx.clipval = mask, num_heads, cut, clipval
         ctx.coef = coef  # (what a training forward left for the backward pass, or None: see keep_backward_coefficients)
+        ctx.abort_sink = abort_sink  # (takes the backward call's abort word: the cell looks at it later, without a synchronisation)
         return h.view_as(h), s.view_as(s)
 
     @staticmethod
@@ -212,10 +213,11 @@ class _CellFunction(torch.autograd.Function):
         d_wx, d_r, d_bias, d_s0 = F_hip.slstm_backward(
             x.detach(), r.detach(), bias.detach().view(NH, 4, dh), None if state is None else state.detach(), ctx.mask,
             h, d_h, d_s, recurrent_cut=ctx.cut, recurrent_clipval=ctx.clipval, coef=ctx.coef,
-            d_wx_dtype=torch.bfloat16 if x.dtype == torch.bfloat16 else None)  # (the input's gradient in the input's type)
+            d_wx_dtype=torch.bfloat16 if x.dtype == torch.bfloat16 else None,  # (the input's gradient in the input's type)
+            abort_sink=ctx.abort_sink)
         ctx.coef = None
         return (d_wx.to(x.dtype), d_r.to(r.dtype), d_bias.reshape(bias.shape).to(bias.dtype),
-                None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None, None)
+                None if state is None else d_s0.to(state.dtype), None, None, None, None, None, None, None, None)
 
 
 class _Runtime:
@@ -434,6 +436,11 @@ class sLSTMCell_hip(nn.Module):
         """Queues a copy of the call's ``aborted`` word to pinned host memory behind the kernel and looks at the
         words of earlier calls that have arrived: a sequence call whose wait between compute units ran out
         (its outputs are NaN by then) raises here, at the next call, or in :meth:`check_status`."""
+        self._watch_word(workspace[:4].view(torch.int32))
+
+    def _watch_word(self, word: torch.Tensor) -> None:
+        """The same for any call's abort word (one int32 on the device): the backward pass hands its own here, so a
+        backward call does not synchronise the host either."""
         if torch.cuda.is_current_stream_capturing():
             return
         ring = self._rt.status_ring
@@ -446,7 +453,7 @@ class sLSTMCell_hip(nn.Module):
         if ring["events"][i] is not None:  # the ring is full of calls still running: wait for the oldest
             ring["events"][i].synchronize()
             self._poll_status(block=False)
-        ring["host"][i:i + 1].copy_(workspace[:4].view(torch.int32), non_blocking=True)
+        ring["host"][i:i + 1].copy_(word, non_blocking=True)
         ev = torch.cuda.Event()
         ev.record()
         ring["events"][i] = ev
@@ -468,8 +475,8 @@ class sLSTMCell_hip(nn.Module):
             bad |= int(ring["host"][i]) != 0
         if bad:
             raise F_hip.EngineError(
-                "an earlier sLSTM sequence call on the hip backend gave up waiting for some of its compute units "
-                "(they were held by other work on the GPU); its outputs were set to NaN"
+                "an earlier sLSTM sequence call (forward or backward) on the hip backend gave up waiting for some of its "
+                "compute units (they were held by other work on the GPU); its outputs were set to NaN"
             )
 
     def check_status(self) -> None:
@@ -522,7 +529,7 @@ class sLSTMCell_hip(nn.Module):
             if x.is_cuda and self.head_dim <= BACKWARD_MAX_HEAD_DIM.get(x.dtype, 0):
                 h, s = _CellFunction.apply(x, self._recurrent_kernel_, self._bias_, state, h, s, reset_mask,
                                            self.config.num_heads, bool(self.config.gradient_recurrent_cut),
-                                           self.config.gradient_recurrent_clipval, coef)
+                                           self.config.gradient_recurrent_clipval, coef, self._watch_word)
             else:
                 h, s = _ForwardOnly.apply(h, s, input, self._recurrent_kernel_, self._bias_)
         output = self._permute_output(h)

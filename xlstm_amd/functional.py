@@ -118,6 +118,7 @@ def slstm_backward(
     recurrent_clipval: Optional[float] = None,
     stepwise_override: Optional[bool] = None,
     d_wx_dtype: Optional[torch.dtype] = None,
+    abort_sink=None,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     """Gradients of the cell, by the rule of the reference's native kernel (the stabiliser is a constant of the
     differentiation, ``slstm_pointwise.cu:118-196``).
@@ -139,6 +140,8 @@ def slstm_backward(
     float32, which both ways cover).
     ``d_wx_dtype=torch.bfloat16`` (bfloat16 inputs only): ``d_wx`` comes back in bfloat16, as the reference returns its
     input gradient in the type of its kernels; the reverse kernel then writes and the parameter kernel reads half the bytes.
+    ``abort_sink``: a callable that takes the call's abort word (an int32 tensor of one element on the device) instead
+    of this function reading it, which synchronises the host; the cell queues an asynchronous copy and raises at a later call.
     ``coef``: what a training forward left (``slstm_forward(..., coef_out=)``); the forward walk is then skipped.
     ``recurrent_cut`` and ``recurrent_clipval`` are the reference's ``gradient_recurrent_cut`` (no gradient from a step
     to the y it started from, ``slstm_backward_cut.cu:265-312``) and ``gradient_recurrent_clipval`` (that gradient
@@ -181,7 +184,7 @@ def slstm_backward(
         d_wx, d_r, d_bias, d_s0 = slstm_backward(wx_p, r_p, bias_p, s0_p, reset_mask, h_p, dh_p, dsf_p, timings=timings,
                                                  split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
                                                  recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval,
-                                                 stepwise_override=stepwise_override, d_wx_dtype=d_wx_dtype)
+                                                 stepwise_override=stepwise_override, d_wx_dtype=d_wx_dtype, abort_sink=abort_sink)
         return (d_wx.view(B_, T_, 4, NH, dh_k)[..., :dh].reshape(B_, T_, 4 * H),
                 d_r.view(NH, 4, dh_k, dh_k)[:, :, :dh, :dh].reshape(NH, 4 * dh, dh),
                 d_bias[..., :dh].contiguous(),
@@ -207,7 +210,7 @@ def slstm_backward(
                     wx[b0:b1], r, bias, None if s0 is None else s0[:, b0:b1], None if reset_mask is None else reset_mask[b0:b1],
                     h_out[:, b0:b1], d_h[:, b0:b1], None if d_s_final is None else d_s_final[:, b0:b1],
                     timings=None, split_override=split_override, spin_limit=spin_limit, row_tile_override=row_tile_override,
-                    recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval, d_wx_dtype=d_wx_dtype))
+                    recurrent_cut=recurrent_cut, recurrent_clipval=recurrent_clipval, d_wx_dtype=d_wx_dtype, abort_sink=abort_sink))
             return (torch.cat([q[0] for q in parts], 0), sum(q[1] for q in parts), sum(q[2] for q in parts),
                     torch.cat([q[3] for q in parts], 1))
     esz = wx.element_size()
@@ -328,7 +331,9 @@ def slstm_backward(
         if timings is not None:
             marks.append(torch.cuda.Event(enable_timing=True))
             marks[-1].record()  # parameter gradients = [2] -> [3]
-    if split and timings is None and int(counters[0].item()):  # (a synchronisation; training calls are not latency-bound)
+    if split and abort_sink is not None:  # (the caller looks at the call's abort word later: no synchronisation here)
+        abort_sink(counters[:1])
+    elif split and timings is None and int(counters[0].item()):  # (a synchronisation)
         raise EngineError("xlstm_amd: a wait between the compute units of a head ran out in the backward pass "
                           "(other work held compute units, or the workgroups of a head were not placed on one XCD); "
                           "the gradients are invalid")
