@@ -20,7 +20,7 @@
 extern "C" {
 #endif
 
-#define XS_ABI_VERSION 15
+#define XS_ABI_VERSION 16
 
 /* element types */
 enum { XS_F32 = 0, XS_BF16 = 1 };
@@ -101,6 +101,13 @@ enum {
  *                             launched (call again without it and use
  *                             xs_slstm_backward_prepare).  h_out and s_out are bit for bit
  *                             those of a call without it.
+ *   r_tiled                   optional, xs_slstm_step only: r in the element type of wx as
+ *                             xs_slstm_tile_r_for_steps lays it out, made once per change
+ *                             of the parameters.  With it a step at a head dim beyond 256
+ *                             (bf16; with h_prev) or 128 (f32), a multiple of 64, runs a
+ *                             kernel whose operands are brought to LDS by waves of their
+ *                             own (13 -> 8 us a step at 4 heads of 512); the result is bit
+ *                             for bit the same.  Ignored elsewhere.  Not in the reference.
  */
 typedef struct xs_slstm_args {
   int32_t B, T, NH, dh;
@@ -120,6 +127,7 @@ typedef struct xs_slstm_args {
   int64_t spin_limit;
   const void *h_prev;
   float *coef_out;
+  const void *r_tiled;
 } xs_slstm_args;
 
 /* Status block at the start of the workspace, written by the kernels. */
@@ -187,6 +195,14 @@ int xs_slstm_forward_static(const xs_slstm_args *args);
  * calls the cell's forward with S = 1).
  */
 int xs_slstm_step(const xs_slstm_args *args);
+
+/*
+ * xs_slstm_tile_r_for_steps   r ([NH, 4*dh, dh] in dtype, the forward's layout; dh a multiple of 64) into the slabs that
+ *   xs_slstm_step reads it in when xs_slstm_args::r_tiled is given: [NH][unit/32][k/KS][gate][unit%32][k%KS] with KS
+ *   = 128 bytes of K (NH*4*dh*dh elements).  No counterpart in the reference, whose step GEMM reads R as it lies
+ *   (slstm_forward.cu:176-182).
+ */
+int xs_slstm_tile_r_for_steps(const void *r, void *r_tiled, int32_t NH, int32_t dh, int32_t dtype, void *stream);
 
 /*
  * The operations around the cell inside an sLSTM layer (bf16 only; the layer keeps its

@@ -26,7 +26,7 @@ def test_abi_version_and_struct_mirror():
     lib = _lib.load()
     assert lib.xs_abi_version() == _lib.ABI_VERSION
     # xs_slstm_args: 6 int32, pointers/int64 after -> 8-byte aligned, 15 more 8-byte fields
-    assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 16 * 8
+    assert ctypes.sizeof(_lib.SlstmArgs) == 24 + 17 * 8
     assert ctypes.sizeof(_lib.SlstmStatus) == 64
     # xs_conv_args: 5 int32 (+4 padding), then 12 8-byte fields; xs_gates_args: 4 int32, then 11 8-byte fields
     assert ctypes.sizeof(_lib.ConvArgs) == 24 + 12 * 8

@@ -343,3 +343,69 @@ def test_cell_forward_decode_loop_uses_the_previous_h_when_the_state_comes_back_
             assert used_hint == (t not in (0, 5)), (t, used_hint)
         assert torch.equal(s, st)
 
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("bf16,B,NH,dh", [(True, 64, 4, 512), (True, 70, 2, 1024), (True, 5, 3, 320), (True, 256, 4, 512),
+                                          (False, 9, 2, 256), (False, 66, 2, 512), (False, 4, 1, 192)])
+def test_step_kernel_with_r_in_slabs_gives_the_same_bits(bf16, B, NH, dh):
+    """Head dims whose K range the step kernel walks in slabs: a plan hands the library R slab by slab
+    (``xs_slstm_tile_r_for_steps``) and the steps run the kernel whose feeder waves bring the slabs to LDS.  Five steps of
+    a chain - the first without a state, one with a reset mask through the generic call - against the step kernel that
+    reads R as it lies, and the chain against ONE sequence call: bit for bit."""
+    import torch
+
+    from xlstm_amd import functional as F
+
+    print("case step kernel with R in slabs", bf16, B, NH, dh, flush=True)
+    dev = torch.device("cuda:0")
+    torch.manual_seed(11)
+    H = NH * dh
+    tdt = torch.bfloat16 if bf16 else torch.float32
+    r = ((torch.rand(NH, 4 * dh, dh, device=dev) - 0.5) * 0.2).to(tdt)
+    bias = torch.randn(NH, 4, dh, device=dev)
+    T = 5
+    wx = torch.randn(B, T, 4 * H, device=dev).to(tdt)
+    s0 = torch.randn(4, B, H, device=dev)
+    s0[2] = s0[2].abs() + 0.5
+    plan = F.StepPlan(B, r, bias, wx_dtype=tdt)
+    assert plan.r_tiled is not None
+    h_seq, s_seq = F.slstm_forward(wx, r, bias, s0)
+    a, b = s0.clone(), torch.empty_like(s0)
+    hs = [s0[0].to(tdt).contiguous(), torch.empty(B, H, dtype=tdt, device=dev)]
+    ref = s0.clone()
+    for t in range(T):
+        x_t = wx[:, t:t + 1].contiguous()
+        plan(x_t, a, b, hs[(t + 1) & 1], h_prev=hs[t & 1] if bf16 else None)
+        h_ref, ref = F.slstm_forward(x_t, r, bias, ref, None, step=True)     # (no r_tiled: the kernel that reads R as it lies)
+        a, b = b, a
+        torch.cuda.synchronize()
+        assert torch.equal(hs[(t + 1) & 1].view(1, B, H), h_ref) and torch.equal(a, ref), t
+        assert torch.equal(h_ref[0], h_seq[t]), t
+    assert torch.equal(a, s_seq)
+    # the kernel ran: with the plan's argument block, minus r_tiled, the status says the tile kernel; here it says nothing
+    # else either, so look at the one thing that differs - time is no test - by running the C entry without a state and
+    # with a mask through the same block
+    import ctypes
+
+    from xlstm_amd import _lib
+
+    mask = (torch.rand(B, 1, device=dev) < 0.4).to(torch.uint8)
+    args = plan._args
+    x_t = wx[:, :1].contiguous()
+    out_h, out_s = torch.empty(B, H, dtype=tdt, device=dev), torch.empty_like(s0)
+    args.wx, args.s0, args.s_out, args.h_out = x_t.data_ptr(), s0.data_ptr(), out_s.data_ptr(), out_h.data_ptr()
+    args.h_prev = hs[0].data_ptr() if bf16 else None
+    hs[0].copy_(s0[0].to(tdt))
+    args.reset, args.reset_stride_b = mask.data_ptr(), 1
+    args.stream = torch.cuda.current_stream().cuda_stream
+    assert _lib.load().xs_slstm_step(ctypes.byref(args)) == 0, _lib.last_error()
+    h_ref, s_ref = F.slstm_forward(x_t, r, bias, s0, mask, step=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out_h.view(1, B, H), h_ref) and torch.equal(out_s, s_ref)
+    args.s0, args.h_prev = None, None
+    assert _lib.load().xs_slstm_step(ctypes.byref(args)) == 0, _lib.last_error()
+    h_ref, s_ref = F.slstm_forward(x_t, r, bias, None, mask, step=True)
+    torch.cuda.synchronize()
+    assert torch.equal(out_h.view(1, B, H), h_ref) and torch.equal(out_s, s_ref)
+    args.reset, args.reset_stride_b = None, 0

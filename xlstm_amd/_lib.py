@@ -15,7 +15,7 @@ LIB_PATH = os.environ.get("XLSTM_AMD_LIB", os.path.join(PKG, "lib", "libxlstm_am
 XS_F32, XS_BF16 = 0, 1
 XS_ERR_UNSUPPORTED = -5
 STATIC_SCRATCH_BYTES = (4 << 20) + (64 << 10)
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 EXPORTS = (
     "xs_abi_version",
@@ -24,6 +24,7 @@ EXPORTS = (
     "xs_slstm_forward",
     "xs_slstm_step",
     "xs_slstm_forward_static",
+    "xs_slstm_tile_r_for_steps",
     "xs_slstm_backward_prepare",
     "xs_slstm_backward",
     "xs_slstm_backward_params",
@@ -56,6 +57,7 @@ class SlstmArgs(ctypes.Structure):
         ("spin_limit", ctypes.c_int64),
         ("h_prev", ctypes.c_void_p),
         ("coef_out", ctypes.c_void_p),
+        ("r_tiled", ctypes.c_void_p),
     ]
 
 
@@ -200,6 +202,8 @@ def load() -> ctypes.CDLL:
     for fn in (lib.xs_slstm_backward_prepare, lib.xs_slstm_backward, lib.xs_slstm_backward_params, lib.xs_slstm_backward_tile_r):
         fn.restype = ctypes.c_int
         fn.argtypes = [ctypes.POINTER(SlstmBwdArgs)]
+    lib.xs_slstm_tile_r_for_steps.restype = ctypes.c_int
+    lib.xs_slstm_tile_r_for_steps.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int32, ctypes.c_int32, ctypes.c_int32, ctypes.c_void_p]
     lib.xs_causal_conv_silu.restype = ctypes.c_int
     lib.xs_causal_conv_silu.argtypes = [ctypes.POINTER(ConvArgs)]
     lib.xs_headwise_gates.restype = ctypes.c_int

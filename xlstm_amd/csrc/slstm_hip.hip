@@ -36,6 +36,7 @@
 #include "slstm_backward_kernels.h"
 #include "slstm_backward_quad_kernel.h"
 #include "slstm_backward_step_kernel.h"
+#include "slstm_step_feed_kernel.h"
 #include "slstm_backward_params_kernel.h"
 #include "slstm_serial_bound.h"
 
@@ -217,6 +218,26 @@ int run_step(const xs_slstm_args *a) {
     const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(pk), plds);
     if (rc != XS_OK) return rc;
     hipLaunchKernelGGL(pk, grid, dim3(kStepPipeThreads), plds, stream, p);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
+    return XS_OK;
+  }
+  // R prepared in slabs (xs_slstm_tile_r_for_steps) and the recurrent operand in the type of the operands: the kernel
+  // whose feeder waves bring the slabs to LDS, for the head dims whose K range is walked in slabs
+  if (a->r_tiled && slabch == 2 && dh % 64 == 0 && (!bf16 || a->h_prev || !a->s0) && (long long)B * NH * dh * (bf16 ? 2 : 4) < (1ll << 31)) {
+    StepFeedParams q;
+    q.B = B; q.NH = NH; q.dh = dh; q.nch = nch;
+    q.wx = a->wx; q.wx_sb = a->wx_stride_b;
+    q.r_tiled = a->r_tiled;
+    q.h_prev = a->s0 ? (bf16 ? a->h_prev : (const void *)a->s0) : nullptr;
+    q.bias = a->bias; q.s0 = a->s0; q.reset = a->reset; q.reset_sb = a->reset_stride_b;
+    q.h_out = a->h_out; q.s_out = a->s_out; q.status = (xs_slstm_status *)a->workspace;
+    if (((uintptr_t)a->r_tiled % 16) || ((uintptr_t)q.h_prev % 16)) return fail(XS_ERR_ALIGN, "r_tiled and h_prev must be 16-byte aligned");
+    void (*fk)(StepFeedParams) = bf16 ? slstm_step_feed_kernel<true> : slstm_step_feed_kernel<false>;
+    const int rc = ensure_dynamic_lds(reinterpret_cast<const void *>(fk), (size_t)step_feed_lds_bytes());
+    if (rc != XS_OK) return rc;
+    const long long fwg = (long long)NH * (dh / 32) * ((B + 63) / 64);
+    hipLaunchKernelGGL(fk, dim3((unsigned)fwg), dim3(512), step_feed_lds_bytes(), stream, q);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "step kernel launch failed: %s", hipGetErrorString(e));
     return XS_OK;
@@ -1110,6 +1131,19 @@ int xs_measure_stage(const xs_measure_args *args) {
 int xs_slstm_backward_params(const xs_slstm_bwd_args *args) {
   g_err[0] = 0;
   return run_backward_params(args);
+}
+
+int xs_slstm_tile_r_for_steps(const void *r, void *r_tiled, int32_t NH, int32_t dh, int32_t dtype, void *stream) {
+  g_err[0] = 0;
+  if (!r || !r_tiled) return fail(XS_ERR_NULL, "r and r_tiled are required");
+  if (NH <= 0 || dh <= 0 || dh % 64 != 0) return fail(XS_ERR_SHAPE, "bad dims NH=%d dh=%d (a multiple of 64)", NH, dh);
+  if (dtype != XS_F32 && dtype != XS_BF16) return fail(XS_ERR_DTYPE, "dtype must be XS_F32 or XS_BF16");
+  if (((uintptr_t)r % 16) || ((uintptr_t)r_tiled % 16)) return fail(XS_ERR_ALIGN, "r and r_tiled must be 16-byte aligned");
+  void (*init)(const void *, void *, const float *, void *, int, int, int) = dtype == XS_BF16 ? slstm_fwd_walk_init_kernel<true> : slstm_fwd_walk_init_kernel<false>;
+  hipLaunchKernelGGL(init, dim3(1024), dim3(256), 0, (hipStream_t)stream, r, r_tiled, (const float *)nullptr, (void *)nullptr, 0, NH, dh);
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(XS_ERR_LAUNCH, "tiling kernel launch failed: %s", hipGetErrorString(e));
+  return XS_OK;
 }
 
 int xs_slstm_backward_tile_r(const xs_slstm_bwd_args *args) {

@@ -518,6 +518,17 @@ class StepPlan:
         a.reset, a.reset_stride_b = None, 0
         a.workspace, a.workspace_bytes = self.workspace.data_ptr(), self.workspace.numel()
         a.spin_limit = 0
+        # Head dims whose K range the step kernel walks in slabs (beyond 256 in bfloat16, 128 in float32): R once more, slab
+        # by slab, for the kernel whose feeder waves bring the slabs to LDS (bfloat16: when the caller passes ``h_prev``)
+        self.r_tiled = None
+        if dh % 64 == 0 and dh > (256 if wx_dtype == torch.bfloat16 else 128):
+            self.r_tiled = torch.empty_like(self.r)
+            with torch.cuda.device(self.device):
+                rc = lib.xs_slstm_tile_r_for_steps(self.r.data_ptr(), self.r_tiled.data_ptr(), NH, dh, _DTYPE_CODE[wx_dtype],
+                                                   torch.cuda.current_stream(self.device).cuda_stream)
+            if rc != 0:
+                raise EngineError(f"xlstm_amd error {rc}: {_lib.last_error()}")
+            a.r_tiled = self.r_tiled.data_ptr()
         self._args, self._ref, self._fn = a, ctypes.byref(a), lib.xs_slstm_step
         self._wx_numel, self._s_numel = self.B * 4 * self.H, 4 * self.B * self.H
 
