@@ -376,6 +376,49 @@ def bench_backward_large(device, T=4096, iters=2):
                          "kernel": "slstm_bwd_step_kernel<bf16>", "algorithmic_bytes_per_launch": nbytes}}
 
 
+def bench_decode_other_head_dims(device, steps=300):
+    """Decode steps at the head dims that `slstm_step_feed_kernel` takes (beyond 256 in bf16): eager launches back to
+    back through a `StepPlan` with the previous step's h handed on, us per step; `r_tiled_off` the same plan without R
+    in slabs (the tile kernel that reads R as it lies)."""
+    import numpy as np
+    import torch
+
+    from xlstm_amd import functional as F
+
+    rows = []
+    for B, NH, dh in ((256, 4, 512), (64, 4, 1024)):
+        H = NH * dh
+        g = torch.Generator(device=device).manual_seed(5)
+        r = ((torch.rand(NH, 4 * dh, dh, generator=g, device=device) * 2 - 1) / float(np.sqrt(H))).bfloat16()
+        bias = torch.zeros(NH, 4, dh, device=device)
+        bias[:, 1] = torch.linspace(3.0, 6.0, dh, device=device)
+        wx = torch.randn(B, 1, 4 * H, generator=g, device=device).bfloat16()
+        row = {"workload": "decode step B=%d NH=%d dh=%d bf16" % (B, NH, dh)}
+        for key in ("us_per_step", "r_tiled_off_us_per_step"):
+            plan = F.StepPlan(B, r, bias, wx_dtype=torch.bfloat16)
+            if key != "us_per_step":
+                plan._args.r_tiled = None
+            s = [torch.zeros(4, B, H, device=device), torch.zeros(4, B, H, device=device)]
+            s[0][1:3] = 0.1
+            h = [torch.zeros(B, H, device=device, dtype=torch.bfloat16) for _ in range(2)]
+            for i in range(20):
+                plan(wx, s[i & 1], s[(i + 1) & 1], h[(i + 1) & 1], h_prev=h[i & 1])
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(steps):
+                plan(wx, s[i & 1], s[(i + 1) & 1], h[(i + 1) & 1], h_prev=h[i & 1])
+            e1.record()
+            torch.cuda.synchronize()
+            row[key] = e0.elapsed_time(e1) * 1e3 / steps
+            row["finite"] = bool(torch.isfinite(s[steps & 1]).all())
+        nbytes = NH * 4 * dh * dh * 2 + B * H * (4 * 2 + 7 * 4 + 2 + 2)  # R, W.x, state in (c, n, m) and out, h in and out
+        row["roofline"] = {"bound": "hbm", "achieved": nbytes / row["us_per_step"] / 1e3, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": nbytes / row["us_per_step"] / 1e3 / HBM_PEAK_GBS, "kernel": "slstm_step_feed_kernel<bf16>",
+                           "algorithmic_bytes_per_launch": nbytes}
+        rows.append(row)
+    return rows
+
+
 def bench_config(device, name, B, T, NH, dh, bf16, mean_doc, iters=5):
     """Times one forward call of the cell at another BASELINE shape (median of `iters`)."""
     import numpy as np
@@ -845,6 +888,8 @@ def main():
         out["layer"] = bench_layer(device, args.layer_iters, args.layer_decode_steps)
     if not args.no_decode:
         out["decode"] = bench_decode(device)
+        if not lean:
+            out["decode"]["other_head_dims"] = bench_decode_other_head_dims(device)
         if not lean:
             # a decode step is one dependent launch: its floor is the launch itself plus the step's bytes at the HBM peak
             launch = out["roofline"]["serial_bound_stages_us"].get("dependent_launch_us")
