@@ -127,9 +127,9 @@ __global__ __launch_bounds__(512) void slstm_step_feed_kernel(StepFeedParams p) 
     eo[ut] = (long long)rowc * H + head * dh + ua;
     restart[ut] = !has_s0 || (p.reset && p.reset[(long long)rowc * p.reset_sb] != 0);
     const f32x4 zero = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-    c4[ut] = has_s0 ? *reinterpret_cast<const f32x4 *>(p.s0 + BH + eo[ut]) : zero;
-    n4[ut] = has_s0 ? *reinterpret_cast<const f32x4 *>(p.s0 + 2 * BH + eo[ut]) : zero;
-    m4[ut] = has_s0 ? *reinterpret_cast<const f32x4 *>(p.s0 + 3 * BH + eo[ut]) : zero;
+    c4[ut] = has_s0 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.s0 + BH + eo[ut])) : zero;
+    n4[ut] = has_s0 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.s0 + 2 * BH + eo[ut])) : zero;
+    m4[ut] = has_s0 ? __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(p.s0 + 3 * BH + eo[ut])) : zero;
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       const long long o = (long long)rowc * p.wx_sb + (long long)g * H + head * dh + ua;
