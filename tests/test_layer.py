@@ -148,12 +148,12 @@ def test_prefill_then_steps_equals_one_forward(dtype):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("B,D,NH", [(8, 256, 4), (64, 512, 4), (5, 96, 3)],
-                         ids=["engine-ops", "engine-ops-operand-hint", "torch-ops"])
+@pytest.mark.parametrize("B,D,NH", [(8, 256, 4), (64, 512, 4), (5, 96, 3), (16, 2048, 4)],
+                         ids=["engine-ops", "engine-ops-operand-hint", "torch-ops", "head-dim-512-r-in-slabs"])
 def test_graphed_decoder_replays_equal_eager_steps(B, D, NH):
     """Two alternating HIP graphs of layer.step against the eager loop, with host work between replays.
     (64, 512, 4) is a shape where the step kernel takes the previous h as its bf16 operand; (5, 96, 3)
-    one where the ops around the cell are PyTorch's."""
+    one where the ops around the cell are PyTorch's; (16, 2048, 4) one where the step kernel reads R in slabs."""
     from xlstm_amd.decode import GraphedLayerDecoder
     from xlstm_amd.layer import sLSTMLayer, sLSTMLayerConfig
 
