@@ -764,7 +764,9 @@ def main():
         print(json.dumps({"serial_bound": serial_bound(device)}))
         return
     if args.decode_only:
-        print(json.dumps({"decode": bench_decode(device)}))
+        dec = bench_decode(device)
+        dec["other_head_dims"] = bench_decode_other_head_dims(device)
+        print(json.dumps({"decode": dec}))
         return
     if args.small_batch_only:
         print(json.dumps({"small_batch": bench_small_batch(device)}))
