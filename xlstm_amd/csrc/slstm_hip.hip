@@ -603,12 +603,6 @@ int run_backward(const xs_slstm_bwd_args *a, bool prepare) {
         if (want > 8) want = 8;
         prefetchers = (int)(want < 0 ? 0 : want);
       }
-#ifdef XS_BQ_NOPF
-      prefetchers = 0;
-#endif
-#ifdef XS_BQ_PF
-      if (prefetchers > XS_BQ_PF) prefetchers = XS_BQ_PF;
-#endif
       q.spin_limit = a->spin_limit != 0 ? a->spin_limit : kDefaultSpinLimit;
       q.cut = a->recurrent_cut != 0; q.clip = clip;
       const long long n16 = (long long)kBwdRing * ngroups * 4 * 4 * a->dh * 2 / 16;
