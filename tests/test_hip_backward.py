@@ -92,6 +92,7 @@ QUAD_CASES = [
     (True, 7, 4, 3, 256, True),       # a ragged second row tile, as many steps as feeder slots
     (True, 6, 5, 2, 64, True),
     (True, 16, 300, 16, 64, True),    # 64 groups, eight per XCD, long enough for the prefetching workgroups to follow and skip
+    (True, 64, 6, 4, 256, True),      # 256 workgroups: the whole device, no room for prefetching workgroups
 ]
 
 
