@@ -59,7 +59,7 @@ def test_backward_argument_errors_without_touching_the_gpu():
     t.split = 2
     assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5  # row tiles of 4 rows: bf16
     t.split, t.dh = 3, 96
-    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5
+    assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5  # (not a multiple of 64)
     t.split = 7
     assert lib.xs_slstm_backward_tile_r(ctypes.byref(t)) == -5
 

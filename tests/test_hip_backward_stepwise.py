@@ -26,6 +26,8 @@ CASES = [
     (False, 2, 5, 1, 296, True),      # padded up to 320
     (True, 9, 40, 8, 640, True),      # eight heads: one per XCD
     (False, 5, 4, 3, 320, True),      # three heads: tiles dealt out head by head
+    (True, 129, 3, 1, 576, True),     # a head dim whose rows of K are no whole number of 256-byte slabs in the walk; three row tiles
+    (False, 1, 9, 3, 384, True),      # one batch row
 ]
 
 

@@ -757,8 +757,7 @@ int run_backward_tile_r(const xs_slstm_bwd_args *a) {
   const bool bf16 = a->dtype == XS_BF16;
   const int epc = bf16 ? 8 : 4;
   if (a->split == 2 && !bf16) return fail(XS_ERR_UNSUPPORTED, "row tiles of 4 rows go with XS_BF16");
-  if (a->dh % 64 != 0 || (a->split == 3 && (a->dh * (bf16 ? 2 : 4)) % 256 != 0))
-    return fail(XS_ERR_UNSUPPORTED, "head dim %d is not one of the backward kernels'", a->dh);
+  if (a->dh % 64 != 0) return fail(XS_ERR_UNSUPPORTED, "head dim %d is not one of the backward kernels'", a->dh);
   hipStream_t stream = (hipStream_t)a->stream;
   const long long n = 4ll * a->NH * a->dh * a->dh;
   const unsigned blocks = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
